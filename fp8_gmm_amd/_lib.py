@@ -1,0 +1,160 @@
+"""ctypes binding of ``libfp8gmm_hip.so`` (the C ABI declared in ``include/fp8gmm.h``).
+
+This plays the role of ``import fp8_gmm_backend`` in the reference
+(fp8_gmm/backend.py:1, pybind module defined in csrc/ops.cu:9-16).  There is no
+fallback: if the shared library is missing or does not export the expected
+symbols, importing the backend raises.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libfp8gmm_hip.so")
+
+E4M3 = 0
+E5M2 = 1
+OUT_BF16 = 2
+EPI_GELU = 1
+
+OP_QUANTIZE = 0
+OP_SCALE_MUL = 1
+OP_PAD_TRANSPOSE = 2
+OP_PAD_CAST_TRANSPOSE = 3
+OP_PAD_CAST_TRANSPOSE_DGELU = 4
+
+# struct fp8gmm_tensor_desc (64 bytes)
+TENSOR_DESC = np.dtype(
+    [
+        ("in", "<u8"),
+        ("in2", "<u8"),
+        ("out", "<u8"),
+        ("out_t", "<u8"),
+        ("scale", "<u8"),
+        ("amax", "<u8"),
+        ("rows", "<i4"),
+        ("cols", "<i4"),
+        ("rows_padded", "<i4"),
+        ("block_begin", "<i4"),
+    ],
+    align=False,
+)
+
+# struct fp8gmm_gemm_problem (96 bytes)
+GEMM_PROBLEM = np.dtype(
+    [
+        ("a", "<u8"),
+        ("b", "<u8"),
+        ("c", "<u8"),
+        ("aux", "<u8"),
+        ("a_scale_inv", "<u8"),
+        ("b_scale_inv", "<u8"),
+        ("c_scale", "<u8"),
+        ("c_amax", "<u8"),
+        ("m", "<i4"),
+        ("n", "<i4"),
+        ("k", "<i4"),
+        ("lda", "<i4"),
+        ("ldb", "<i4"),
+        ("ldc", "<i4"),
+        ("tile_begin", "<i4"),
+        ("tiles_n", "<i4"),
+    ],
+    align=False,
+)
+
+EXPORTS = (
+    "fp8gmm_version",
+    "fp8gmm_status_string",
+    "fp8gmm_sizeof_tensor_desc",
+    "fp8gmm_sizeof_gemm_problem",
+    "fp8gmm_gemm_tile_shape",
+    "fp8gmm_plan_multi_tensor",
+    "fp8gmm_plan_grouped_gemm",
+    "fp8gmm_multi_quantize",
+    "fp8gmm_multi_scale_mul",
+    "fp8gmm_multi_pad_transpose",
+    "fp8gmm_multi_pad_cast_transpose",
+    "fp8gmm_multi_pad_cast_transpose_dgelu",
+    "fp8gmm_grouped_gemm",
+)
+
+
+class Fp8GmmError(RuntimeError):
+    """Raised when a C-ABI call returns a non-zero status (the reference raises RuntimeError via TORCH_CHECK)."""
+
+
+_lib = None
+
+
+def load():
+    """Load the shared library once; raise loudly when it is absent or incomplete."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: the HIP extension is not built. "
+            "Run `make -C fp8_gmm_amd/csrc -j8` (or `python -c 'import __graft_entry__ as g; g.build()'`)."
+        )
+    L = ctypes.CDLL(LIB_PATH)
+    missing = [s for s in EXPORTS if not hasattr(L, s)]
+    if missing:
+        raise ImportError(f"{LIB_PATH} does not export {missing}")
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    ip = ctypes.POINTER(ctypes.c_int)
+    L.fp8gmm_version.restype = ci
+    L.fp8gmm_version.argtypes = []
+    L.fp8gmm_status_string.restype = ctypes.c_char_p
+    L.fp8gmm_status_string.argtypes = [ci]
+    L.fp8gmm_sizeof_tensor_desc.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_tensor_desc.argtypes = []
+    L.fp8gmm_sizeof_gemm_problem.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_gemm_problem.argtypes = []
+    L.fp8gmm_gemm_tile_shape.restype = None
+    L.fp8gmm_gemm_tile_shape.argtypes = [ip, ip]
+    L.fp8gmm_plan_multi_tensor.restype = ci
+    L.fp8gmm_plan_multi_tensor.argtypes = [vp, ci, ci, ip]
+    L.fp8gmm_plan_grouped_gemm.restype = ci
+    L.fp8gmm_plan_grouped_gemm.argtypes = [vp, ci, ip]
+    L.fp8gmm_multi_quantize.restype = ci
+    L.fp8gmm_multi_quantize.argtypes = [vp, ci, ci, ci, vp]
+    L.fp8gmm_multi_scale_mul.restype = ci
+    L.fp8gmm_multi_scale_mul.argtypes = [vp, ci, ci, vp]
+    L.fp8gmm_multi_pad_transpose.restype = ci
+    L.fp8gmm_multi_pad_transpose.argtypes = [vp, ci, ci, vp]
+    L.fp8gmm_multi_pad_cast_transpose.restype = ci
+    L.fp8gmm_multi_pad_cast_transpose.argtypes = [vp, ci, ci, ci, vp]
+    L.fp8gmm_multi_pad_cast_transpose_dgelu.restype = ci
+    L.fp8gmm_multi_pad_cast_transpose_dgelu.argtypes = [vp, ci, ci, ci, vp]
+    L.fp8gmm_grouped_gemm.restype = ci
+    L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
+    if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize:
+        raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
+    _lib = L
+    return L
+
+
+def check(status):
+    if status != 0:
+        raise Fp8GmmError(f"fp8gmm error {status}: {load().fp8gmm_status_string(status).decode()}")
+
+
+def plan_multi_tensor(table, op):
+    """Validate + schedule a host table (numpy structured array of TENSOR_DESC). Returns total workgroups."""
+    total = ctypes.c_int(0)
+    check(load().fp8gmm_plan_multi_tensor(table.ctypes.data, len(table), op, ctypes.byref(total)))
+    return total.value
+
+
+def plan_grouped_gemm(table):
+    total = ctypes.c_int(0)
+    check(load().fp8gmm_plan_grouped_gemm(table.ctypes.data, len(table), ctypes.byref(total)))
+    return total.value
+
+
+def gemm_tile_shape():
+    tm, tn = ctypes.c_int(0), ctypes.c_int(0)
+    load().fp8gmm_gemm_tile_shape(ctypes.byref(tm), ctypes.byref(tn))
+    return tm.value, tn.value

@@ -1,0 +1,173 @@
+// Device-side helpers shared by the gfx950 kernels: bf16 / fp8 conversions, the
+// deterministic tanh used by the GELU paths, wave64 reductions and the amax merge.
+// Counterpart of the reference's csrc/utils.cuh, re-thought for 64-wide wavefronts.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/fp8gmm.h"
+
+namespace fp8gmm {
+
+constexpr int kWaveSize = 64;
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float bf16_lo_to_f32(uint32_t packed) { return __uint_as_float(packed << 16); }
+__device__ __forceinline__ float bf16_hi_to_f32(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  uint32_t nan = (u >> 16) | 0x0040u;
+  return ((u & 0x7fffffffu) > 0x7f800000u) ? (nan & 0xffffu) : rounded;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+
+template <int FMT>
+struct Fp8Limits;
+template <>
+struct Fp8Limits<FP8GMM_E4M3> {
+  static constexpr float kMax = 448.0f;
+};
+template <>
+struct Fp8Limits<FP8GMM_E5M2> {
+  static constexpr float kMax = 57344.0f;
+};
+
+// Two fp32 -> two fp8 bytes in the low (HI = false) or high (HI = true) half of `old`.
+// Saturating round-to-nearest-even: |x| >= max (infinities included) -> max finite.
+// The median clamps; NaN inputs are patched by the caller (fp8_nan_fix) because the
+// median of (NaN, -max, max) is -max.
+template <int FMT, bool HI>
+__device__ __forceinline__ uint32_t cvt_pk_fp8_sat(float a, float b, uint32_t old) {
+  constexpr float mx = Fp8Limits<FMT>::kMax;
+  a = __builtin_amdgcn_fmed3f(a, -mx, mx);
+  b = __builtin_amdgcn_fmed3f(b, -mx, mx);
+  if constexpr (FMT == FP8GMM_E4M3) {
+    return __builtin_amdgcn_cvt_pk_fp8_f32(a, b, old, HI);
+  } else {
+    return __builtin_amdgcn_cvt_pk_bf8_f32(a, b, old, HI);
+  }
+}
+
+// Four scaled fp32 values -> one dword of fp8 bytes (element 0 in the low byte).
+// NaN becomes 0x7F (positive canonical NaN) whatever its sign.
+template <int FMT>
+__device__ __forceinline__ uint32_t cvt4_fp8(float v0, float v1, float v2, float v3) {
+  uint32_t w = 0;
+  w = cvt_pk_fp8_sat<FMT, false>(v0, v1, w);
+  w = cvt_pk_fp8_sat<FMT, true>(v2, v3, w);
+  if (__builtin_expect((v0 != v0) | (v1 != v1) | (v2 != v2) | (v3 != v3), 0)) {
+    if (v0 != v0) w = (w & 0xffffff00u) | 0x0000007fu;
+    if (v1 != v1) w = (w & 0xffff00ffu) | 0x00007f00u;
+    if (v2 != v2) w = (w & 0xff00ffffu) | 0x007f0000u;
+    if (v3 != v3) w = (w & 0x00ffffffu) | 0x7f000000u;
+  }
+  return w;
+}
+
+template <int FMT>
+__device__ __forceinline__ uint8_t cvt1_fp8(float v) {
+  return (uint8_t)(cvt4_fp8<FMT>(v, 0.f, 0.f, 0.f) & 0xffu);
+}
+
+// max(acc, |x|) that never lets a NaN in (fmaxf semantics of the reference's amax).
+__device__ __forceinline__ float amax_step(float acc, float x) { return fmaxf(acc, fabsf(x)); }
+
+// Wave-wide max of non-negative floats; every lane gets the result.
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = kWaveSize / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWaveSize));
+  return v;
+}
+
+// Merge a non-negative float into *addr with an integer atomic max on the bit
+// pattern (order-free, hence deterministic).  Vector-memory atomic.
+__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
+  atomicMax(reinterpret_cast<int*>(addr), __float_as_int(v));
+}
+
+// Block-wide amax merge for blocks of NWAVES waves. `stage` is NWAVES floats of LDS.
+template <int NWAVES>
+__device__ __forceinline__ void block_amax_merge(float local, float* amax, float* stage) {
+  float w = wave_max(local);
+  const int lane = threadIdx.x % kWaveSize;
+  const int wave = threadIdx.x / kWaveSize;
+  if (lane == 0) stage[wave] = w;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = stage[0];
+#pragma unroll
+    for (int i = 1; i < NWAVES; ++i) m = fmaxf(m, stage[i]);
+    if (amax != nullptr && m > 0.f) atomic_max_nonneg(amax, m);
+  }
+}
+
+// tanh from a fixed sequence of IEEE single-precision operations (mul, add, fma,
+// one correctly rounded division), so that a CPU following the same sequence gets
+// the same bits.  |error| < 2e-7.
+//   a = min(|u|, 9); z = a * 2/ln2; n = rne(z); f = z - n; e = 2^f * 2^n = exp(2a)
+//   tanh = (e - 1) / (e + 1), sign of u restored.
+__device__ __forceinline__ float det_tanh(float u) {
+  float a = fabsf(u);
+  a = (a > 9.0f) ? 9.0f : a;
+  float z = a * 2.8853900817779268f;
+  const float magic = 12582912.0f;
+  float zr = z + magic;
+  int n = (int)(__float_as_uint(zr) - __float_as_uint(magic));
+  float nf = zr - magic;
+  float f = z - nf;
+  float p = 1.5403530393381609e-4f;
+  p = __builtin_fmaf(p, f, 1.3333558146428443e-3f);
+  p = __builtin_fmaf(p, f, 9.6181291076284772e-3f);
+  p = __builtin_fmaf(p, f, 5.5504108664821580e-2f);
+  p = __builtin_fmaf(p, f, 2.4022650695910071e-1f);
+  p = __builtin_fmaf(p, f, 6.9314718055994531e-1f);
+  p = __builtin_fmaf(p, f, 1.0f);
+  float e = __uint_as_float(__float_as_uint(p) + ((uint32_t)n << 23));
+  float t = (e - 1.0f) / (e + 1.0f);
+  return __builtin_copysignf(t, u);
+}
+
+// d/dc of tanh-GELU with the constants of the reference (csrc/multi_pad_fusion.cu:39-44).
+__device__ __forceinline__ float dgelu(float c) {
+  float c2 = c * c;
+  float u = (0.79788456f * c) * __builtin_fmaf(0.044715f, c2, 1.0f);
+  float t = det_tanh(u);
+  float dt = __builtin_fmaf(-t, t, 1.0f);
+  float g = __builtin_fmaf(0.1070322243f, c2, 0.79788456f);
+  float left = (0.5f * c) * (dt * g);
+  float right = __builtin_fmaf(0.5f, t, 0.5f);
+  return left + right;
+}
+
+__device__ __forceinline__ float gelu_tanh(float v) {
+  float v2 = v * v;
+  float u = (0.79788456f * v) * __builtin_fmaf(0.044715f, v2, 1.0f);
+  float t = det_tanh(u);
+  return (0.5f * v) * (1.0f + t);
+}
+
+// Index of the last entry of a sorted device table whose key (read by `key(i)`) is <= x.
+// Uniform across the workgroup, so it compiles to scalar loads.
+template <typename KeyFn>
+__device__ __forceinline__ int upper_slot(int n, int x, KeyFn key) {
+  int lo = 0, hi = n - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (key(mid) <= x) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+}  // namespace fp8gmm

@@ -1,0 +1,129 @@
+// Multi-tensor element-wise kernels for gfx950: quantize (bf16 -> fp8 + amax) and
+// scale_mul (in-place bf16 *= s1 * s2).  One launch covers every tensor of the call;
+// each workgroup finds its tensor by a binary search over a device-side table.
+//
+// Replaces csrc/multi_pointwise.cu of the reference (multi_quantize_kernel :34-97,
+// multi_scale_mul_kernel :99-151).  HBM-bound: 2 B read + 1 B written per element
+// (quantize), 2 B + 2 B (scale_mul); every lane moves 32 bytes in and 16 bytes out per
+// step with 128-bit accesses, the wave reduces amax with cross-lane shuffles and the
+// workgroup issues a single integer atomic max.
+#include "device_utils.h"
+#include "tiling.h"
+
+namespace fp8gmm {
+namespace {
+
+template <int FMT>
+__global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(const fp8gmm_tensor_desc* __restrict__ descs,
+                                                                    int n) {
+  __shared__ float stage[kPwThreads / kWaveSize];
+  const int bid = blockIdx.x;
+  const int t = upper_slot(n, bid, [&](int i) { return descs[i].block_begin; });
+  const fp8gmm_tensor_desc d = descs[t];
+  const int64_t numel = (int64_t)d.rows * d.cols;
+  const int64_t base = (int64_t)(bid - d.block_begin) * kPwBlockElems;
+  const uint16_t* __restrict__ in = static_cast<const uint16_t*>(d.in);
+  uint8_t* __restrict__ out = static_cast<uint8_t*>(d.out);
+  const float scale = d.scale ? *d.scale : 1.f;
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  float mx = 0.f;
+
+#pragma unroll
+  for (int it = 0; it < kPwSteps; ++it) {
+    const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+    if (vec && off + kPwVec <= numel) {
+      const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + off));
+      const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + off + 8));
+      const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float x0 = bf16_lo_to_f32(w[2 * q]), x1 = bf16_hi_to_f32(w[2 * q]);
+        const float x2 = bf16_lo_to_f32(w[2 * q + 1]), x3 = bf16_hi_to_f32(w[2 * q + 1]);
+        mx = amax_step(amax_step(mx, x0), x1);
+        mx = amax_step(amax_step(mx, x2), x3);
+        o[q] = cvt4_fp8<FMT>(x0 * scale, x1 * scale, x2 * scale, x3 * scale);
+      }
+      const u32x4 ov = {o[0], o[1], o[2], o[3]};
+      __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(out + off));
+    } else if (off < numel) {
+      const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
+      for (int j = 0; j < cnt; ++j) {
+        const float x = bf16_to_f32(in[off + j]);
+        mx = amax_step(mx, x);
+        out[off + j] = cvt1_fp8<FMT>(x * scale);
+      }
+    }
+  }
+  block_amax_merge<kPwThreads / kWaveSize>(mx, d.amax, stage);
+}
+
+__global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gmm_tensor_desc* __restrict__ descs,
+                                                                     int n) {
+  const int bid = blockIdx.x;
+  const int t = upper_slot(n, bid, [&](int i) { return descs[i].block_begin; });
+  const fp8gmm_tensor_desc d = descs[t];
+  const int64_t numel = (int64_t)d.rows * d.cols;
+  const int64_t base = (int64_t)(bid - d.block_begin) * kPwBlockElems;
+  // in-place: `in` is the tensor being scaled
+  uint16_t* __restrict__ x = const_cast<uint16_t*>(static_cast<const uint16_t*>(d.in));
+  const float s1 = d.scale ? *d.scale : 1.f;
+  const float* s2p = static_cast<const float*>(d.in2);
+  const float s2 = s2p ? *s2p : 1.f;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+
+#pragma unroll
+  for (int it = 0; it < kPwSteps; ++it) {
+    const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+    if (vec && off + kPwVec <= numel) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        u32x4 a = *reinterpret_cast<const u32x4*>(x + off + 8 * h);
+        uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // left to right, as the reference: (x * s1) * s2
+          const float lo = bf16_lo_to_f32(w[q]) * s1 * s2;
+          const float hi = bf16_hi_to_f32(w[q]) * s1 * s2;
+          w[q] = pack_bf16x2(lo, hi);
+        }
+        const u32x4 o = {w[0], w[1], w[2], w[3]};
+        *reinterpret_cast<u32x4*>(x + off + 8 * h) = o;
+      }
+    } else if (off < numel) {
+      const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
+      for (int j = 0; j < cnt; ++j) x[off + j] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(x[off + j]) * s1 * s2);
+    }
+  }
+}
+
+}  // namespace
+}  // namespace fp8gmm
+
+extern "C" {
+
+int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+  if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (out_fmt != FP8GMM_E4M3 && out_fmt != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
+  if (n == 0 || total_blocks == 0) return FP8GMM_OK;
+  if (descs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (out_fmt == FP8GMM_E4M3)
+    hipLaunchKernelGGL(fp8gmm::multi_quantize_kernel<FP8GMM_E4M3>, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0, s,
+                       descs_dev, n);
+  else
+    hipLaunchKernelGGL(fp8gmm::multi_quantize_kernel<FP8GMM_E5M2>, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0, s,
+                       descs_dev, n);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream) {
+  if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (n == 0 || total_blocks == 0) return FP8GMM_OK;
+  if (descs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  hipLaunchKernelGGL(fp8gmm::multi_scale_mul_kernel, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0,
+                     static_cast<hipStream_t>(stream), descs_dev, n);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+}  // extern "C"

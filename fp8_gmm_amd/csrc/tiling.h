@@ -1,0 +1,22 @@
+// Work decomposition constants shared by the host planners and the kernels.
+#pragma once
+
+namespace fp8gmm {
+
+// ---- element-wise kernels (quantize, scale_mul) ----
+constexpr int kPwThreads = 256;                  // 4 wavefronts
+constexpr int kPwVec = 16;                       // elements per thread per step
+constexpr int kPwSteps = 4;                      // steps per workgroup
+constexpr int kPwBlockElems = kPwThreads * kPwVec * kPwSteps;  // 16384 elements per workgroup
+
+// ---- pad / cast / transpose kernels ----
+constexpr int kPtThreads = 256;
+constexpr int kPtTileRows = 128;                 // tile extent along the token (row) dimension
+constexpr int kPtTileCols = 128;                 // tile extent along the feature (column) dimension
+
+// ---- grouped GEMM ----
+constexpr int kGemmTileM = 256;                  // rows of c per workgroup tile
+constexpr int kGemmTileN = 256;                  // columns of c per workgroup tile
+constexpr int kGemmTileK = 128;                  // bytes of K consumed per main-loop step
+
+}  // namespace fp8gmm

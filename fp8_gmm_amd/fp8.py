@@ -1,0 +1,213 @@
+"""Per-tensor delayed-scaling FP8 metadata for the grouped modules.
+
+The reference inherits this machinery from TransformerEngine
+(``TransformerEngineBaseModule.prepare_forward`` / ``fp8_meta``, ``fp8_autocast``,
+``recipe.DelayedScaling``, ``get_fp8_te_dtype``; call sites grouped_linear.py:4-5,19,124,186,206,
+grouped_mlp.py:4-5,28,178,328,349, utils.py:78-96, example.py:156,159).  TransformerEngine
+is not a dependency here; this module provides the same names with the same
+meaning, sized for what the grouped modules use:
+
+* ``fp8_meta["scaling_fwd"]`` has 3 slots per GEMM (input, weight, output) and
+  ``fp8_meta["scaling_bwd"]`` 2 (grad_output, grad_input); each holds ``scale``,
+  ``scale_inv`` (fp32 ``[slots]``) and ``amax_history`` (fp32 ``[history, slots]``),
+  with the kernels writing amax into ``amax_history[0]``.
+* Update rule (applied at the start of a forward pass, from the second pass on):
+      amax      = max(amax_history, dim=0)        ("max")  or amax_history[0] ("most_recent")
+      new_scale = (fp8_max / amax) / 2**margin    where amax is finite and > 0, else the old scale
+      scale_inv = 1 / new_scale
+      amax_history = roll(amax_history, -1, dim=0);  amax_history[0] = 0
+  fp8_max is 448 for e4m3 and 57344 for e5m2.  HYBRID means e4m3 for forward tensors
+  and e5m2 for gradients.
+* Both directions are updated.  (The reference never enters TransformerEngine's
+  backward context, so its gradient scales stay at their initial value of 1; updating
+  them is a deliberate difference - e5m2 gradients need real scales.)
+
+No test vector of the reference pins TransformerEngine's update rule; the rule
+above is this package's own statement of it.
+"""
+import contextlib
+import threading
+from dataclasses import dataclass
+from enum import Enum
+
+import torch
+
+from .utils import DType
+
+FP8_MAX = {DType.kFloat8E4M3: 448.0, DType.kFloat8E5M2: 57344.0}
+
+
+class Format(Enum):
+    E4M3 = "e4m3"
+    E5M2 = "e5m2"
+    HYBRID = "hybrid"
+
+
+@dataclass
+class DelayedScaling:
+    """Delayed-scaling recipe (same fields and defaults the reference's example uses, example.py:156)."""
+
+    margin: int = 0
+    interval: int = 1
+    fp8_format: Format = Format.HYBRID
+    amax_history_len: int = 1024
+    amax_compute_algo: str = "max"
+
+    def __post_init__(self):
+        if self.amax_compute_algo not in ("max", "most_recent"):
+            raise ValueError(f"unsupported amax_compute_algo {self.amax_compute_algo!r}")
+        if self.amax_history_len < 1:
+            raise ValueError("amax_history_len must be >= 1")
+        if self.interval < 1:
+            raise ValueError("interval must be >= 1")
+
+
+class recipe:  # noqa: N801 - namespace with the spelling user code already has (`recipe.DelayedScaling`)
+    DelayedScaling = DelayedScaling
+    Format = Format
+
+
+def get_fp8_te_dtype(fp8_recipe, fprop_tensor=True):
+    """fp8 type of forward (``fprop_tensor``) or gradient tensors under a recipe."""
+    if fp8_recipe.fp8_format == Format.E4M3 or (fp8_recipe.fp8_format == Format.HYBRID and fprop_tensor):
+        return DType.kFloat8E4M3
+    return DType.kFloat8E5M2
+
+
+class _State(threading.local):
+    def __init__(self):
+        self.enabled = False
+        self.recipe = None
+
+
+_STATE = _State()
+
+
+@contextlib.contextmanager
+def fp8_autocast(enabled=True, fp8_recipe=None):
+    """Selects the recipe used by modules called inside the block."""
+    prev = (_STATE.enabled, _STATE.recipe)
+    _STATE.enabled = enabled
+    _STATE.recipe = (fp8_recipe or DelayedScaling()) if enabled else None
+    try:
+        yield
+    finally:
+        _STATE.enabled, _STATE.recipe = prev
+
+
+def current_recipe():
+    return _STATE.recipe if _STATE.enabled else None
+
+
+class Fp8MetaTensors:
+    """scale / scale_inv / amax_history of one direction."""
+
+    def __init__(self, slots, history_len, device):
+        self.scale = torch.ones(slots, dtype=torch.float32, device=device)
+        self.scale_inv = torch.ones(slots, dtype=torch.float32, device=device)
+        self.amax_history = torch.zeros(history_len, slots, dtype=torch.float32, device=device)
+
+    def state(self):
+        return {"scale": self.scale, "scale_inv": self.scale_inv, "amax_history": self.amax_history}
+
+    def load_state(self, state):
+        self.scale.copy_(state["scale"])
+        self.scale_inv.copy_(state["scale_inv"])
+        self.amax_history.copy_(state["amax_history"])
+
+
+def amax_and_scale_update(meta, fp8_max, fp8_recipe):
+    """Delayed-scaling update of one direction, in place (rule in the module docstring)."""
+    hist = meta.amax_history
+    if fp8_recipe.amax_compute_algo == "max":
+        amax = hist.max(dim=0).values
+    else:
+        amax = hist[0].clone()
+    sf = (fp8_max / amax) / (2.0 ** fp8_recipe.margin)
+    ok = (amax > 0) & torch.isfinite(amax)
+    meta.scale.copy_(torch.where(ok, sf, meta.scale))
+    meta.scale_inv.copy_(1.0 / meta.scale)
+    if hist.shape[0] > 1:
+        hist.copy_(torch.roll(hist, -1, 0))
+    hist[0].zero_()
+
+
+class Fp8GroupedModuleBase(torch.nn.Module):
+    """The slice of ``TransformerEngineBaseModule`` the grouped modules rely on."""
+
+    FWD_SLOTS_PER_GEMM = 3
+    BWD_SLOTS_PER_GEMM = 2
+
+    def __init__(self):
+        super().__init__()
+        self.fp8_meta = {}
+        self._fp8_steps = 0
+
+    def _init_fp8_meta(self, fp8_recipe, num_gemms, device):
+        meta = self.fp8_meta
+        same = (
+            meta.get("num_gemms") == num_gemms
+            and meta.get("recipe") == fp8_recipe
+            and "scaling_fwd" in meta
+            and meta["scaling_fwd"].scale.device == device
+        )
+        if same:
+            return
+        meta["recipe"] = fp8_recipe
+        meta["num_gemms"] = num_gemms
+        meta["scaling_fwd"] = Fp8MetaTensors(num_gemms * self.FWD_SLOTS_PER_GEMM, fp8_recipe.amax_history_len, device)
+        meta["scaling_bwd"] = Fp8MetaTensors(num_gemms * self.BWD_SLOTS_PER_GEMM, fp8_recipe.amax_history_len, device)
+        meta["fp8_max_fwd"] = FP8_MAX[get_fp8_te_dtype(fp8_recipe, True)]
+        meta["fp8_max_bwd"] = FP8_MAX[get_fp8_te_dtype(fp8_recipe, False)]
+        self._fp8_steps = 0
+
+    @contextlib.contextmanager
+    def prepare_forward(self, inp, is_first_microbatch, num_gemms=1):
+        """Makes ``self.fp8_meta`` ready for a forward pass of ``num_gemms`` GEMMs.
+
+        Outside ``fp8_autocast`` the default recipe is used (the modules are FP8-only).
+        In training mode every pass after the first starts with the delayed-scaling
+        update of both directions, every ``recipe.interval`` passes.
+        """
+        assert is_first_microbatch is None, "FP8 weight caching across micro-batches is not implemented"
+        fp8_recipe = current_recipe() or self.fp8_meta.get("recipe") or DelayedScaling()
+        self._init_fp8_meta(fp8_recipe, num_gemms, inp.device)
+        self._apply_pending_state()
+        if self.training and torch.is_grad_enabled():
+            if self._fp8_steps > 0 and self._fp8_steps % fp8_recipe.interval == 0:
+                with torch.no_grad():
+                    amax_and_scale_update(self.fp8_meta["scaling_fwd"], self.fp8_meta["fp8_max_fwd"], fp8_recipe)
+                    amax_and_scale_update(self.fp8_meta["scaling_bwd"], self.fp8_meta["fp8_max_bwd"], fp8_recipe)
+            self._fp8_steps += 1
+        yield
+
+    # checkpointing of the scaling state (TransformerEngine exposes it the same way)
+    def get_extra_state(self):
+        if "scaling_fwd" not in self.fp8_meta:
+            return None
+        return {
+            "num_gemms": self.fp8_meta["num_gemms"],
+            "steps": self._fp8_steps,
+            "scaling_fwd": {k: v.detach().cpu() for k, v in self.fp8_meta["scaling_fwd"].state().items()},
+            "scaling_bwd": {k: v.detach().cpu() for k, v in self.fp8_meta["scaling_bwd"].state().items()},
+        }
+
+    def set_extra_state(self, state):
+        if not state:
+            return
+        self._pending_extra_state = state
+
+    def _apply_pending_state(self):
+        state = getattr(self, "_pending_extra_state", None)
+        if state is None or "scaling_fwd" not in self.fp8_meta:
+            return
+        self._pending_extra_state = None
+        fwd, bwd = self.fp8_meta["scaling_fwd"], self.fp8_meta["scaling_bwd"]
+        if (
+            state["num_gemms"] != self.fp8_meta["num_gemms"]
+            or state["scaling_fwd"]["amax_history"].shape != fwd.amax_history.shape
+        ):
+            raise RuntimeError("saved FP8 scaling state does not match this module's recipe / expert count")
+        fwd.load_state(state["scaling_fwd"])
+        bwd.load_state(state["scaling_bwd"])
+        self._fp8_steps = state["steps"]

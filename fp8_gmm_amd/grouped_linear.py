@@ -1,0 +1,208 @@
+"""``GroupedLinear``: E expert linears on token-sorted rows, FP8 forward and backward.
+
+Same surface and data flow as the reference's ``fp8_gmm/grouped_linear.py``
+(``_GroupedLinear`` :11-183, ``GroupedLinear`` :186-214):
+
+forward   one multi-tensor cast(+transpose) launch over the E activation slices and
+          the E weights (e4m3 under HYBRID), then one grouped GEMM
+          ``out[rows_i] = x_fp8[rows_i] . w_fp8[i]^T * (x_scale_inv_i * w_scale_inv_i)``.
+backward  one cast(+transpose) launch over the E slices of grad_out (e5m2), a grouped
+          dgrad GEMM against the transposed weights, and a grouped wgrad GEMM
+          ``dW[i] = dY_i^T[N, Mpad_i] . X_i^T[K, Mpad_i]^T`` whose contraction runs over
+          the expert's tokens padded to a multiple of 16 with zeros.
+
+Differences from the reference: experts with zero tokens are allowed (their weight
+gradient is zero), wgrad is a single launch instead of a per-expert loop, and the
+grouped GEMM is the same HIP kernel whatever ``cutlass`` says (``cutlass=True`` keeps
+the two-rounding data flow of the reference's CUTLASS path, see ``backend.fp8_gmm``).
+"""
+import math
+
+import torch
+
+from .backend import fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
+from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
+from .utils import Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
+
+
+def row_slices(t, bounds):
+    """Per-expert row blocks of a token-major tensor."""
+    return [t[bounds[i]: bounds[i + 1]] for i in range(len(bounds) - 1)]
+
+
+def transposed_views(flat, bounds):
+    """Per-expert ``[features, tokens_i]`` views of a flat ``[sum(tokens_i), features]`` buffer.
+
+    Expert i owns the contiguous block of rows ``bounds[i]:bounds[i+1]``; the block is
+    reinterpreted as the transpose ``[features, bounds[i+1]-bounds[i]]``
+    (reference grouped_linear.py:36-52).
+    """
+    feat = flat.shape[1]
+    views = []
+    for i in range(len(bounds) - 1):
+        rows = bounds[i + 1] - bounds[i]
+        views.append(flat[bounds[i]: bounds[i + 1]].view(feat, rows) if rows > 0 else flat.new_empty((feat, 0)))
+    return views
+
+
+def alloc_transposed(features, padded, bounds, padded_bounds, dtype, device):
+    """Buffer + per-expert views for the transposed copy of a ``[tokens, features]`` operand."""
+    b = padded_bounds if padded else bounds
+    flat = torch.empty(b[-1], features, dtype=dtype, device=device)
+    return flat, transposed_views(flat, b)
+
+
+class _GroupedLinear(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, weight, group_sizes, fp8_meta, is_grad_enabled, cutlass):
+        wgrad_needed = is_grad_enabled and weight.requires_grad
+        dgrad_needed = is_grad_enabled and input.requires_grad
+        num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed
+        )
+        if cumsums[-1] != input.size(0):
+            raise RuntimeError("group_sizes must sum to the number of input rows")
+        meta = Fp8MetaWrapper(num_groups, fp8_meta)
+        fwd_dtype = get_fp8_te_dtype(fp8_meta["recipe"], fprop_tensor=True)
+        fp8_dtype = to_torch_dtype(fwd_dtype)
+        dev = input.device
+
+        plain = ([], [], [], [])            # inputs, outputs, scales, amaxes for cast only
+        with_t = ([], [], [], [], [])       # inputs, outputs, transposes, scales, amaxes
+
+        input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
+        input_t_fp8 = None
+        x_scales = meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kScale)
+        x_amaxes = meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kAmax)
+        if wgrad_needed:
+            input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums,
+                                                      fp8_dtype, dev)
+            with_t[0].extend(row_slices(input, cumsums))
+            with_t[1].extend(row_slices(input_fp8, cumsums))
+            with_t[2].extend(x_t_views)
+            with_t[3].extend(x_scales)
+            with_t[4].extend(x_amaxes)
+        else:
+            plain[0].extend(row_slices(input, cumsums))
+            plain[1].extend(row_slices(input_fp8, cumsums))
+            plain[2].extend(x_scales)
+            plain[3].extend(x_amaxes)
+
+        weight_fp8 = torch.empty(weight.shape, dtype=fp8_dtype, device=weight.device)
+        weight_t_fp8 = None
+        w_scales = meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kScale)
+        w_amaxes = meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kAmax)
+        if dgrad_needed:
+            weight_t_fp8 = torch.empty(num_groups, weight.size(2), weight.size(1), dtype=fp8_dtype,
+                                       device=weight.device)
+            with_t[0].extend(weight.unbind(0))
+            with_t[1].extend(weight_fp8.unbind(0))
+            with_t[2].extend(weight_t_fp8.unbind(0))
+            with_t[3].extend(w_scales)
+            with_t[4].extend(w_amaxes)
+        else:
+            plain[0].extend(weight.unbind(0))
+            plain[1].extend(weight_fp8.unbind(0))
+            plain[2].extend(w_scales)
+            plain[3].extend(w_amaxes)
+
+        if plain[0]:
+            multi_quantize(*plain)
+        if with_t[0]:
+            multi_cast_transpose(*with_t)
+
+        out = fp8_gmm(
+            input_fp8, weight_fp8, group_sizes,
+            meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kScaleInv),
+            meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kScaleInv),
+            backward=False, cutlass=cutlass,
+        )
+
+        if is_grad_enabled:
+            ctx.save_for_backward(input_t_fp8, weight_t_fp8)
+            ctx.group_sizes = group_sizes
+            meta.set_forward_scale_inv_cloned()
+            ctx.meta = meta
+            ctx.num_groups = num_groups
+            ctx.padded = padded
+            ctx.cumsums = cumsums
+            ctx.padded_cumsums = padded_cumsums
+            ctx.fp8_meta = fp8_meta
+            ctx.weight_shape = weight.shape
+            ctx.input_requires_grad = input.requires_grad
+            ctx.weight_requires_grad = weight.requires_grad
+            ctx.cutlass = cutlass
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        input_t_fp8, weight_t_fp8 = ctx.saved_tensors
+        meta = ctx.meta
+        cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
+        grad_dtype = to_torch_dtype(get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=False))
+        grad_out = grad_out.contiguous()
+        dev = grad_out.device
+
+        g_scales = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScale)
+        g_amaxes = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kAmax)
+        g_scale_invs = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScaleInv)
+        grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
+        g_t_views = None
+        if ctx.weight_requires_grad:
+            _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
+                                            dev)
+            multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
+                                 g_scales, g_amaxes)
+        else:
+            multi_quantize(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_scales, g_amaxes)
+
+        grad_input = None
+        if ctx.input_requires_grad:
+            grad_input = fp8_gmm(
+                grad_out_fp8, weight_t_fp8, ctx.group_sizes, g_scale_invs,
+                meta.get_meta_tensors(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
+                backward=True, cutlass=ctx.cutlass,
+            )
+
+        grad_weight = None
+        if ctx.weight_requires_grad:
+            grad_weight = torch.empty(ctx.weight_shape, dtype=torch.bfloat16, device=dev)
+            x_t_views = transposed_views(input_t_fp8, padded_cumsums if padded else cumsums)
+            grouped_gemm(
+                g_t_views, x_t_views, list(grad_weight.unbind(0)), g_scale_invs,
+                meta.get_meta_tensors(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv),
+            )
+        return grad_input, grad_weight, None, None, None, None
+
+
+class GroupedLinear(Fp8GroupedModuleBase):
+    """E independent ``in_features -> out_features`` linears (no bias) over token-sorted rows.
+
+    ``forward(input[tokens, in_features], group_sizes[E])`` where ``group_sizes`` is a CPU
+    int64 tensor (or list) of rows per expert, in order; returns ``[tokens, out_features]`` bf16.
+    """
+
+    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False):
+        super().__init__()
+        assert dtype == torch.bfloat16, "bfloat16 parameters only"
+        self.in_features = in_features
+        self.out_features = out_features
+        self.num_groups = num_groups
+        self.cutlass = cutlass
+        self.weight_tensor = torch.nn.Parameter(
+            torch.empty(num_groups, out_features, in_features, dtype=dtype, device=device)
+        )
+        bound = math.sqrt(1.0 / in_features)
+        torch.nn.init.uniform_(self.weight_tensor.data, -bound, bound)
+
+    def get_fp8_weights_scratchpad(self, is_first_microbatch):
+        assert is_first_microbatch is None
+        return [None, None]
+
+    def forward(self, input, group_sizes, is_first_microbatch=None):
+        with self.prepare_forward(input, is_first_microbatch, self.num_groups):
+            grad = torch.is_grad_enabled()
+            args = (input, self.weight_tensor, group_sizes, self.fp8_meta, grad, self.cutlass)
+            if grad:
+                return _GroupedLinear.apply(*args)
+            return _GroupedLinear.forward(None, *args)

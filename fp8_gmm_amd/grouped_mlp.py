@@ -1,0 +1,254 @@
+"""``GroupedMlp``: E expert MLPs (fc1 -> tanh-GELU -> fc2) on token-sorted rows in FP8.
+
+Same surface and data flow as the reference's ``fp8_gmm/grouped_mlp.py``
+(``_GroupedMlp`` :18-325, ``GroupedMlp`` :328-366).  ``GroupedMlp(in=H, out=F)`` owns
+``fc1_weight [E, F, H]`` and ``fc2_weight [E, H, F]``.
+
+forward   one cast(+transpose) launch over the E activation slices and 2E weights;
+          fc1 grouped GEMM with the GELU-aux epilogue (writes bf16 pre-GELU values and
+          the e4m3 GELU output scaled by the InputGroup2 scale, recording its amax);
+          fc2 grouped GEMM to bf16.
+backward  cast(+transpose) of grad_out to e5m2 and pad-transpose of the saved GELU
+          output; fc2 wgrad; fc2 dgrad; fused (dgelu * grad) cast(+transpose) under the
+          GradOutputGroup2 scale; fc1 dgrad (optionally all-reduced over a tensor-parallel
+          group, overlapped with fc1 wgrad); fc1 wgrad.
+
+Experts with zero tokens are allowed; each wgrad is one grouped launch.
+"""
+import math
+
+import torch
+
+from .backend import (
+    fp8_gmm,
+    grouped_gemm,
+    multi_cast_transpose,
+    multi_cast_transpose_dgelu,
+    multi_quantize,
+    multi_transpose,
+)
+from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
+from .grouped_linear import alloc_transposed, row_slices, transposed_views
+from .utils import Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
+
+_T = Fp8TensorType
+_M = MetaTensorType
+
+
+class _GroupedMlp(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, fc1_weight, fc2_weight, group_sizes, fp8_meta, is_grad_enabled, has_tp, tp_group):
+        input_requires_grad = input.requires_grad
+        weight_requires_grad = fc1_weight.requires_grad
+        wgrad_needed = is_grad_enabled and weight_requires_grad
+        # fc2's transposed weights feed the fc2 dgrad, which both the input and the fc1 weight gradients need
+        dgrad_needed = is_grad_enabled and (input_requires_grad or weight_requires_grad)
+        num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed
+        )
+        if cumsums[-1] != input.size(0):
+            raise RuntimeError("group_sizes must sum to the number of input rows")
+        meta = Fp8MetaWrapper(num_groups, fp8_meta)
+        fp8_dtype = to_torch_dtype(get_fp8_te_dtype(fp8_meta["recipe"], fprop_tensor=True))
+        dev = input.device
+        tokens, ffn = input.size(0), fc1_weight.size(1)
+
+        plain = ([], [], [], [])
+        with_t = ([], [], [], [], [])
+
+        input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
+        input_t_fp8 = None
+        x_scales = meta.get_meta_tensors(_T.kInputGroup1, _M.kScale)
+        x_amaxes = meta.get_meta_tensors(_T.kInputGroup1, _M.kAmax)
+        if wgrad_needed:
+            input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums, fp8_dtype, dev)
+            with_t[0].extend(row_slices(input, cumsums))
+            with_t[1].extend(row_slices(input_fp8, cumsums))
+            with_t[2].extend(x_t_views)
+            with_t[3].extend(x_scales)
+            with_t[4].extend(x_amaxes)
+        else:
+            plain[0].extend(row_slices(input, cumsums))
+            plain[1].extend(row_slices(input_fp8, cumsums))
+            plain[2].extend(x_scales)
+            plain[3].extend(x_amaxes)
+
+        fc1_weight_fp8 = torch.empty(fc1_weight.shape, dtype=fp8_dtype, device=dev)
+        fc2_weight_fp8 = torch.empty(fc2_weight.shape, dtype=fp8_dtype, device=dev)
+        fc1_weight_t_fp8 = fc2_weight_t_fp8 = None
+        w_scales = meta.get_meta_tensors(_T.kWeightGroup1, _M.kScale) + meta.get_meta_tensors(_T.kWeightGroup2, _M.kScale)
+        w_amaxes = meta.get_meta_tensors(_T.kWeightGroup1, _M.kAmax) + meta.get_meta_tensors(_T.kWeightGroup2, _M.kAmax)
+        w_in = list(fc1_weight.unbind(0)) + list(fc2_weight.unbind(0))
+        w_out = list(fc1_weight_fp8.unbind(0)) + list(fc2_weight_fp8.unbind(0))
+        if dgrad_needed:
+            fc1_weight_t_fp8 = torch.empty(num_groups, fc1_weight.size(2), fc1_weight.size(1), dtype=fp8_dtype,
+                                           device=dev)
+            fc2_weight_t_fp8 = torch.empty(num_groups, fc2_weight.size(2), fc2_weight.size(1), dtype=fp8_dtype,
+                                           device=dev)
+            with_t[0].extend(w_in)
+            with_t[1].extend(w_out)
+            with_t[2].extend(list(fc1_weight_t_fp8.unbind(0)) + list(fc2_weight_t_fp8.unbind(0)))
+            with_t[3].extend(w_scales)
+            with_t[4].extend(w_amaxes)
+        else:
+            plain[0].extend(w_in)
+            plain[1].extend(w_out)
+            plain[2].extend(w_scales)
+            plain[3].extend(w_amaxes)
+
+        if plain[0]:
+            multi_quantize(*plain)
+        if with_t[0]:
+            multi_cast_transpose(*with_t)
+
+        pre_gelu_out = torch.empty(tokens, ffn, dtype=torch.bfloat16, device=dev)
+        gelu_out_fp8 = torch.empty(tokens, ffn, dtype=fp8_dtype, device=dev)
+        # fc1: GELU-aux epilogue, fp8 output scaled for fc2 (slot InputGroup2)
+        fp8_gmm(
+            input_fp8, fc1_weight_fp8, group_sizes,
+            meta.get_meta_tensors(_T.kInputGroup1, _M.kScaleInv),
+            meta.get_meta_tensors(_T.kWeightGroup1, _M.kScaleInv),
+            c=gelu_out_fp8, pre_gelu_out=pre_gelu_out,
+            c_scales=meta.get_meta_tensors(_T.kInputGroup2, _M.kScale),
+            c_amaxes=meta.get_meta_tensors(_T.kInputGroup2, _M.kAmax),
+            backward=False, cutlass=False,
+        )
+        if not is_grad_enabled:
+            pre_gelu_out = None
+        out = fp8_gmm(
+            gelu_out_fp8, fc2_weight_fp8, group_sizes,
+            meta.get_meta_tensors(_T.kInputGroup2, _M.kScaleInv),
+            meta.get_meta_tensors(_T.kWeightGroup2, _M.kScaleInv),
+            backward=False, cutlass=False,
+        )
+        if not wgrad_needed:
+            gelu_out_fp8 = None
+
+        if is_grad_enabled:
+            ctx.save_for_backward(input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8, pre_gelu_out, gelu_out_fp8)
+            ctx.group_sizes = group_sizes
+            meta.set_forward_scale_inv_cloned()
+            ctx.meta = meta
+            ctx.num_groups = num_groups
+            ctx.padded = padded
+            ctx.cumsums = cumsums
+            ctx.padded_cumsums = padded_cumsums
+            ctx.fp8_meta = fp8_meta
+            ctx.fc1_weight_shape = fc1_weight.shape
+            ctx.fc2_weight_shape = fc2_weight.shape
+            ctx.input_requires_grad = input_requires_grad
+            ctx.weight_requires_grad = weight_requires_grad
+            ctx.has_tp = has_tp
+            if has_tp:
+                assert tp_group is not None
+            ctx.tp_group = tp_group
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
+        meta = ctx.meta
+        cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
+        t_bounds = padded_cumsums if padded else cumsums
+        grad_dtype = to_torch_dtype(get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=False))
+        grad_out = grad_out.contiguous()
+        dev = grad_out.device
+        wgrad = ctx.weight_requires_grad
+
+        g1_scales = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kScale)
+        g1_amaxes = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kAmax)
+        g1_scale_invs = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kScaleInv)
+        grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
+
+        grad_fc2_weight = None
+        if wgrad:
+            _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype, dev)
+            _, gelu_t_views = alloc_transposed(gelu_out_fp8.size(1), padded, cumsums, padded_cumsums,
+                                               gelu_out_fp8.dtype, dev)
+            multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
+                                 g1_scales, g1_amaxes)
+            multi_transpose(row_slices(gelu_out_fp8, cumsums), gelu_t_views)
+            # fc2 wgrad: dW2[i][H, F] = dY_i^T[H, Mpad] . gelu_i^T[F, Mpad]^T
+            grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev)
+            grouped_gemm(
+                g_t_views, gelu_t_views, list(grad_fc2_weight.unbind(0)), g1_scale_invs,
+                meta.get_meta_tensors(_T.kForwardInputGroup2, _M.kScaleInv),
+            )
+        else:
+            multi_quantize(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g1_scales, g1_amaxes)
+
+        # fc2 dgrad: d(gelu_out)[tokens, F]
+        grad_gelu_out = fp8_gmm(
+            grad_out_fp8, fc2_weight_t_fp8, ctx.group_sizes, g1_scale_invs,
+            meta.get_meta_tensors(_T.kForwardWeightGroup2, _M.kScaleInv),
+            backward=True, cutlass=False,
+        )
+
+        # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8 (+ padded transpose for fc1 wgrad)
+        grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
+        _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums, grad_dtype, dev)
+        multi_cast_transpose_dgelu(
+            row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums), row_slices(grad_pre_fp8, cumsums),
+            grad_pre_t_views,
+            meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kScale),
+            meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kAmax),
+        )
+        g2_scale_invs = meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kScaleInv)
+
+        grad_input = None
+        handle = None
+        if ctx.input_requires_grad:
+            grad_input = fp8_gmm(
+                grad_pre_fp8, fc1_weight_t_fp8, ctx.group_sizes, g2_scale_invs,
+                meta.get_meta_tensors(_T.kForwardWeightGroup1, _M.kScaleInv),
+                backward=True, cutlass=False,
+            )
+            if ctx.has_tp:
+                handle = torch.distributed.all_reduce(
+                    grad_input, op=torch.distributed.ReduceOp.SUM, group=ctx.tp_group, async_op=True
+                )
+
+        grad_fc1_weight = None
+        if wgrad:
+            # fc1 wgrad: dW1[i][F, H] = d(pre)_i^T[F, Mpad] . X_i^T[H, Mpad]^T
+            grad_fc1_weight = torch.empty(ctx.fc1_weight_shape, dtype=torch.bfloat16, device=dev)
+            grouped_gemm(
+                grad_pre_t_views, transposed_views(input_t_fp8, t_bounds), list(grad_fc1_weight.unbind(0)),
+                g2_scale_invs, meta.get_meta_tensors(_T.kForwardInputGroup1, _M.kScaleInv),
+            )
+        if handle is not None:
+            handle.wait()
+        return grad_input, grad_fc1_weight, grad_fc2_weight, None, None, None, None, None
+
+
+class GroupedMlp(Fp8GroupedModuleBase):
+    """E expert MLPs ``in_features -> out_features -> in_features`` with tanh-GELU, no biases.
+
+    ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None)``.
+    """
+
+    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda"):
+        super().__init__()
+        assert dtype == torch.bfloat16, "bfloat16 parameters only"
+        self.num_groups = num_groups
+        self.fc1_weight = torch.nn.Parameter(
+            torch.empty(num_groups, out_features, in_features, dtype=dtype, device=device)
+        )
+        self.fc2_weight = torch.nn.Parameter(
+            torch.empty(num_groups, in_features, out_features, dtype=dtype, device=device)
+        )
+        b1, b2 = math.sqrt(1.0 / in_features), math.sqrt(1.0 / out_features)
+        torch.nn.init.uniform_(self.fc1_weight.data, -b1, b1)
+        torch.nn.init.uniform_(self.fc2_weight.data, -b2, b2)
+
+    def get_fp8_weights_scratchpad(self, is_first_microbatch):
+        assert is_first_microbatch is None
+        return [None, None, None, None]
+
+    def forward(self, input, group_sizes, has_tp=False, tp_group=None, is_first_microbatch=None):
+        with self.prepare_forward(input, is_first_microbatch, self.num_groups * 2):
+            grad = torch.is_grad_enabled()
+            args = (input, self.fc1_weight, self.fc2_weight, group_sizes, self.fp8_meta, grad, has_tp, tp_group)
+            if grad:
+                return _GroupedMlp.apply(*args)
+            return _GroupedMlp.forward(None, *args)

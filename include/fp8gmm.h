@@ -1,0 +1,169 @@
+/*
+ * fp8gmm - C ABI of the MI355X (gfx950) FP8 grouped-GEMM library.
+ *
+ * This is the boundary that replaces the reference's pybind11 module
+ * `fp8_gmm_backend` (csrc/ops.cu:9-16).  Every function is `extern "C"`,
+ * takes plain pointers and integers, returns an int status (0 = success,
+ * negative = fp8gmm_status) and never throws, allocates, frees or synchronises.
+ * All device work is enqueued on the HIP stream passed in (`hipStream_t`,
+ * passed as `void*`; NULL = the default stream).
+ *
+ * Multi-tensor calls and the grouped GEMM read their work list from a table in
+ * DEVICE memory (no 64-tensor limit, unlike the reference's 4 KB by-value
+ * argument structs, csrc/multi_pointwise.cu:13, csrc/multi_pad_fusion.cu:14).
+ * The protocol is:
+ *   1. the caller fills an array of descriptors in host memory;
+ *   2. `fp8gmm_plan_*` validates it and fills the scheduling fields
+ *      (`block_begin` / `tile_begin`) and returns the launch size;
+ *   3. the caller copies the array to device memory on the same stream;
+ *   4. `fp8gmm_multi_*` / `fp8gmm_grouped_gemm` launches one kernel over the
+ *      device copy.
+ * The library never owns memory; outputs are written in place.
+ */
+#ifndef FP8GMM_H_
+#define FP8GMM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP8GMM_VERSION 1
+
+/* fp8 formats (OCP): e4m3fn = torch.float8_e4m3fn, e5m2 = torch.float8_e5m2 */
+#define FP8GMM_E4M3 0
+#define FP8GMM_E5M2 1
+/* output kind of the GEMM epilogue */
+#define FP8GMM_OUT_BF16 2
+
+typedef enum fp8gmm_status {
+  FP8GMM_OK = 0,
+  FP8GMM_ERR_NULL_POINTER = -1,   /* a required pointer is NULL */
+  FP8GMM_ERR_BAD_SHAPE = -2,      /* negative size, rows_padded < rows, size overflow */
+  FP8GMM_ERR_BAD_FORMAT = -3,     /* unknown fp8 format / unsupported format pair */
+  FP8GMM_ERR_ALIGNMENT = -4,      /* GEMM operand not 16-byte aligned / K or pitch not a multiple of 16 */
+  FP8GMM_ERR_LAUNCH = -5,         /* the HIP runtime rejected the launch */
+  FP8GMM_ERR_BAD_ARGUMENT = -6,   /* inconsistent scalar arguments (count < 0, total mismatch, ...) */
+  FP8GMM_ERR_NO_DEVICE = -7       /* no usable gfx950 device */
+} fp8gmm_status;
+
+/*
+ * One tensor of a multi-tensor call.  `rows x cols` row-major, contiguous.
+ *
+ *  op                              in         in2        out             out_t                       scale / amax
+ *  multi_quantize                  bf16       -          fp8 same shape  -                           read / max-merged
+ *  multi_scale_mul                 bf16 (rw)  -          -               -                           scale, scale2 read
+ *  multi_pad_transpose             fp8        -          -               fp8 [cols, rows_padded]     -
+ *  multi_pad_cast_transpose        bf16       -          fp8 (or NULL)   fp8 [cols, rows_padded]     read / max-merged
+ *  multi_pad_cast_transpose_dgelu  bf16 dy    bf16 pre   fp8 (or NULL)   fp8 [cols, rows_padded]     read / max-merged
+ *
+ * `scale` NULL means 1.0 (reference csrc/multi_pointwise.cu:51); `amax` NULL
+ * means "do not record" (csrc/multi_pad_fusion.cu:290).  `amax` is merged with
+ * its previous content by an integer atomic max and must hold a non-negative
+ * value on entry (csrc/utils.cuh:183-185).  For quantize / scale_mul, `cols`
+ * may carry the whole element count with rows = 1.
+ */
+typedef struct fp8gmm_tensor_desc {
+  const void* in;
+  const void* in2;      /* dgelu: pre-GELU input; scale_mul: second scale (const float*) */
+  void* out;
+  void* out_t;
+  const float* scale;
+  float* amax;
+  int32_t rows;
+  int32_t cols;
+  int32_t rows_padded;  /* second dimension of out_t, >= rows; ignored by ops without out_t */
+  int32_t block_begin;  /* filled by fp8gmm_plan_*: first workgroup of this tensor */
+} fp8gmm_tensor_desc;   /* 64 bytes */
+
+/* which multi-tensor kernel a plan is for */
+#define FP8GMM_OP_QUANTIZE 0
+#define FP8GMM_OP_SCALE_MUL 1
+#define FP8GMM_OP_PAD_TRANSPOSE 2
+#define FP8GMM_OP_PAD_CAST_TRANSPOSE 3
+#define FP8GMM_OP_PAD_CAST_TRANSPOSE_DGELU 4
+
+/*
+ * One GEMM of a grouped launch:  c[m, n] = epilogue( a[m, k] . b[n, k]^T ).
+ * Both operands are K-contiguous ("TN"), the only layout the reference uses
+ * (fp8_gmm/backend.py:25,57; csrc/fp8_gmm.h:7-11).  Pitches are in elements.
+ * a, b must be 16-byte aligned and k, lda, ldb multiples of 16 (the same
+ * divisibility cuBLASLt demands of the reference, grouped_linear.py:68).
+ * k == 0 is allowed and writes epilogue(0); m == 0 or n == 0 produce no work.
+ *
+ * Epilogue:  v = acc * (*a_scale_inv * *b_scale_inv)        (NULL scale = 1)
+ *   gelu off: r = v;   gelu on: r = gelu_tanh(v) and, if aux != NULL, aux = bf16(v)
+ *   out bf16: c = bf16(r)
+ *   out fp8 : c = fp8_saturate(r * *c_scale), *c_amax = max(*c_amax, max|r|)
+ * This is the behaviour the reference obtains from cuBLASLt through
+ * fp8_gmm/backend.py:26-54 (scaled TN GEMM, optional GELU-aux epilogue and fp8
+ * output with amax), and - with the scales folded in - what
+ * csrc/fp8_gmm.cu:163 + MultiScaleMul compute on the CUTLASS path.
+ */
+typedef struct fp8gmm_gemm_problem {
+  const void* a;
+  const void* b;
+  void* c;
+  void* aux;                 /* bf16 [m, n] pre-GELU output, pitch ldc, or NULL */
+  const float* a_scale_inv;
+  const float* b_scale_inv;
+  const float* c_scale;      /* fp8 output only */
+  float* c_amax;             /* fp8 output only, may be NULL */
+  int32_t m, n, k;
+  int32_t lda, ldb, ldc;
+  int32_t tile_begin;        /* filled by fp8gmm_plan_grouped_gemm */
+  int32_t tiles_n;           /* filled by fp8gmm_plan_grouped_gemm */
+} fp8gmm_gemm_problem;       /* 96 bytes */
+
+/* epilogue flags of fp8gmm_grouped_gemm */
+#define FP8GMM_EPI_GELU 1
+
+/* ---- library info ------------------------------------------------------------------------- */
+int fp8gmm_version(void);
+const char* fp8gmm_status_string(int status);
+size_t fp8gmm_sizeof_tensor_desc(void);   /* lets a binding check its struct layout */
+size_t fp8gmm_sizeof_gemm_problem(void);
+/* workgroup tile of the GEMM kernel (rows of c, columns of c), for callers that size grids */
+void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n);
+
+/* ---- planning (host only, no GPU needed) -------------------------------------------------- */
+/* Validates `descs[0..n)` for `op` (FP8GMM_OP_*), fills block_begin, returns the launch size
+ * in *total_blocks.  Replaces the host halves of MultiQuantize / MultiScaleMul /
+ * MultiPad* (csrc/multi_pointwise.cu:155-189,216-246; csrc/multi_pad_fusion.cu:442-488,505-559,587-644). */
+int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* total_blocks);
+
+/* Validates `probs[0..n)`, fills tile_begin / tiles_n, returns the tile count in *total_tiles.
+ * Replaces the host half of CutlassFp8GroupedGemm (csrc/fp8_gmm.cu:82-135). */
+int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles);
+
+/* ---- launches (descs_dev / probs_dev: DEVICE copies of planned tables) ------------------- */
+/* replaces MultiQuantize, csrc/multi_pointwise.cu:155 (pybind name multi_quantize, csrc/ops.cu:11) */
+int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream);
+/* replaces MultiScaleMul, csrc/multi_pointwise.cu:216 (multi_scale_mul, csrc/ops.cu:12) */
+int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream);
+/* replaces MultiPadTranspose, csrc/multi_pad_fusion.cu:442 (multi_pad_transpose, csrc/ops.cu:13) */
+int fp8gmm_multi_pad_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream);
+/* replaces MultiPadCastTranspose, csrc/multi_pad_fusion.cu:505 (multi_pad_cast_transpose, csrc/ops.cu:14) */
+int fp8gmm_multi_pad_cast_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+                                    void* stream);
+/* replaces MultiPadCastTransposeDgelu, csrc/multi_pad_fusion.cu:587 (multi_pad_cast_transpose_dgelu, csrc/ops.cu:15) */
+int fp8gmm_multi_pad_cast_transpose_dgelu(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+                                          void* stream);
+
+/*
+ * One persistent launch over all tiles of all problems.
+ * replaces Fp8GroupedGemm, csrc/fp8_gmm.cu:163 (pybind name fp8_gmm, csrc/ops.cu:10) and the
+ * per-expert cuBLASLt loop of fp8_gmm/backend.py:84-96 and grouped_linear.py:173-182.
+ *   a_fmt, b_fmt : FP8GMM_E4M3 / FP8GMM_E5M2 (e5m2 x e5m2 is rejected, as cuBLASLt does)
+ *   out_kind     : FP8GMM_OUT_BF16, or FP8GMM_E4M3 / FP8GMM_E5M2 for an fp8 `c`
+ *   epilogue     : 0 or FP8GMM_EPI_GELU
+ */
+int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int a_fmt, int b_fmt,
+                        int out_kind, int epilogue, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP8GMM_H_ */

@@ -1,0 +1,209 @@
+"""GroupedLinear / GroupedMlp forward + backward on the GPU against the CPU oracle's restatement.
+
+The reference has no module-level test at all (its test file stops at the backend entry
+points); these tests run the autograd modules for several steps of delayed scaling and
+compare outputs, gradients and the recorded scaling state.
+"""
+import pytest
+import torch
+
+from helpers import assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
+from oracle import modules as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _pkg():
+    import fp8_gmm_amd
+
+    return fp8_gmm_amd
+
+
+def _sync_meta(oracle_meta, gpu_meta):
+    oracle_meta.scale = gpu_meta.scale.detach().cpu().clone()
+    oracle_meta.scale_inv = gpu_meta.scale_inv.detach().cpu().clone()
+    oracle_meta.amax_history = gpu_meta.amax_history.detach().cpu().clone()
+
+
+def _check_amax(gpu_meta, oracle_meta, exact_slots, approx_slots, what):
+    g = gpu_meta.amax_history[0].detach().cpu()
+    o = oracle_meta.amax_history[0]
+    if exact_slots:
+        assert_scalar_bits_equal(g[exact_slots], o[exact_slots], f"{what} amax (cast of given tensors)")
+    if approx_slots:
+        assert torch.allclose(g[approx_slots], o[approx_slots], rtol=2e-2, atol=0), f"{what} amax (derived tensors)"
+
+
+LINEAR_CASES = {
+    "config1": ([137, 401, 59, 403], 256, 512),
+    "zero-rows": ([0, 48, 0, 5, 130], 128, 192),
+    "aligned": ([32, 64, 16], 64, 128),
+}
+
+
+@pytest.mark.parametrize("case", list(LINEAR_CASES))
+@pytest.mark.parametrize("cutlass", [False, True])
+def test_grouped_linear_fwd_bwd(dev, case, cutlass):
+    pkg = _pkg()
+    sizes, k, n = LINEAR_CASES[case]
+    e, m, hist = len(sizes), sum(sizes), 4
+    g = gen(1001)
+    w = randn_bf16((e, n, k), g, 0.02)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev, cutlass=cutlass)
+    module.weight_tensor.data.copy_(w)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
+    fwd, bwd = orc.Meta(3 * e, hist), orc.Meta(2 * e, hist)
+    tol = 2e-2 if cutlass else 1e-2  # the two-rounding path rounds the bf16 result twice
+    for step in range(3):
+        x = randn_bf16((m, k), g)
+        dy = randn_bf16((m, n), g, 1e-2)
+        if step > 0:
+            fwd.update(448.0)
+            bwd.update(57344.0)
+        o = orc.grouped_linear_step(x, w, sizes, dy, fwd, bwd)
+        xd = x.to(dev).requires_grad_()
+        module.weight_tensor.grad = None
+        with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
+            out = module(xd, torch.tensor(sizes, dtype=torch.int64))
+        out.backward(dy.to(dev))
+        torch.cuda.synchronize()
+        gm = module.fp8_meta
+        assert_scalar_bits_equal(gm["scaling_fwd"].scale, fwd.scale, f"step {step} fwd scale")
+        assert_scalar_bits_equal(gm["scaling_bwd"].scale, bwd.scale, f"step {step} bwd scale")
+        assert_scalar_bits_equal(gm["scaling_fwd"].amax_history, fwd.amax_history, f"step {step} fwd amax history")
+        assert_scalar_bits_equal(gm["scaling_bwd"].amax_history, bwd.amax_history, f"step {step} bwd amax history")
+        assert_gemm_close(out, o["out"].float(), tol, f"step {step} out")
+        assert_gemm_close(xd.grad, o["grad_input"].float(), tol, f"step {step} grad_input")
+        assert_gemm_close(module.weight_tensor.grad, o["grad_weight"].float(), tol, f"step {step} grad_weight")
+        for i, s in enumerate(sizes):
+            if s == 0:
+                assert not module.weight_tensor.grad[i].any(), "an expert without tokens has a zero weight gradient"
+
+
+def test_grouped_linear_inference_and_frozen_weight(dev):
+    """no_grad forward (cast-only path, multi_quantize) and a frozen weight (no wgrad, no padding)."""
+    pkg = _pkg()
+    sizes, k, n = [137, 401, 59, 403], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(1002)
+    w = randn_bf16((e, n, k), g, 0.02)
+    x = randn_bf16((m, k), g)
+    dy = randn_bf16((m, n), g, 1e-2)
+    fwd, bwd = orc.Meta(3 * e, 1), orc.Meta(2 * e, 1)
+    o = orc.grouped_linear_step(x, w, sizes, dy, fwd, bwd)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev)
+    module.weight_tensor.data.copy_(w)
+    gs = torch.tensor(sizes)
+    with torch.no_grad(), pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=1)):
+        out = module(x.to(dev), gs)
+    assert_gemm_close(out, o["out"].float(), 1e-2, "no_grad out")
+    module.weight_tensor.requires_grad_(False)
+    xd = x.to(dev).requires_grad_()
+    with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=1)):
+        out = module(xd, gs)
+    out.backward(dy.to(dev))
+    assert module.weight_tensor.grad is None
+    # scales were updated from the first pass: compare against the oracle run the same way
+    fwd.update(448.0)
+    bwd.update(57344.0)
+    o2 = orc.grouped_linear_step(x, w, sizes, dy, fwd, bwd)
+    assert_gemm_close(out, o2["out"].float(), 1e-2, "frozen-weight out")
+    assert_gemm_close(xd.grad, o2["grad_input"].float(), 1e-2, "frozen-weight grad_input")
+
+
+MLP_CASES = {
+    "small": ([137, 401, 59, 403], 256, 512),
+    "zero-rows": ([0, 48, 0, 5, 130], 128, 384),
+}
+
+
+@pytest.mark.parametrize("case", list(MLP_CASES))
+def test_grouped_mlp_fwd_bwd(dev, case):
+    pkg = _pkg()
+    sizes, h, f = MLP_CASES[case]
+    e, m, hist = len(sizes), sum(sizes), 3
+    g = gen(2001)
+    w1 = randn_bf16((e, f, h), g, 0.02)
+    w2 = randn_bf16((e, h, f), g, 0.02)
+    module = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+    module.fc1_weight.data.copy_(w1)
+    module.fc2_weight.data.copy_(w2)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
+    fwd, bwd = orc.Meta(3 * 2 * e, hist), orc.Meta(2 * 2 * e, hist)
+    live = [i for i, s in enumerate(sizes) if s > 0]
+    exact_fwd = [3 * i for i in live] + [3 * i + 1 for i in range(e)] + [3 * (e + i) + 1 for i in range(e)]
+    approx_fwd = [3 * (e + i) for i in live]
+    exact_bwd = [2 * i for i in live]
+    approx_bwd = [2 * (e + i) for i in live]
+    for step in range(3):
+        x = randn_bf16((m, h), g)
+        dy = randn_bf16((m, h), g, 1e-2)
+        if step > 0:
+            # derived amaxes (GELU output, dGELU product) depend on the accumulation order: take the
+            # GPU's state so that both sides quantise with identical scales, then update both
+            _sync_meta(fwd, module.fp8_meta["scaling_fwd"])
+            _sync_meta(bwd, module.fp8_meta["scaling_bwd"])
+            fwd.update(448.0)
+            bwd.update(57344.0)
+        o = orc.grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd)
+        xd = x.to(dev).requires_grad_()
+        module.fc1_weight.grad = None
+        module.fc2_weight.grad = None
+        with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
+            out = module(xd, torch.tensor(sizes, dtype=torch.int64))
+        out.backward(dy.to(dev))
+        torch.cuda.synchronize()
+        gm = module.fp8_meta
+        assert_scalar_bits_equal(gm["scaling_fwd"].scale, fwd.scale, f"step {step} fwd scale")
+        assert_scalar_bits_equal(gm["scaling_bwd"].scale, bwd.scale, f"step {step} bwd scale")
+        _check_amax(gm["scaling_fwd"], fwd, exact_fwd, approx_fwd, f"step {step} fwd")
+        _check_amax(gm["scaling_bwd"], bwd, exact_bwd, approx_bwd, f"step {step} bwd")
+        # every stage adds an fp8 re-quantisation of a slightly different bf16 value: widen the bound per stage
+        assert_gemm_close(out, o["out"].float(), 2e-2, f"step {step} out")
+        assert_gemm_close(module.fc2_weight.grad, o["grad_w2"].float(), 2e-2, f"step {step} grad_fc2")
+        assert_gemm_close(xd.grad, o["grad_input"].float(), 3e-2, f"step {step} grad_input")
+        assert_gemm_close(module.fc1_weight.grad, o["grad_w1"].float(), 3e-2, f"step {step} grad_fc1")
+        for i, s in enumerate(sizes):
+            if s == 0:
+                assert not module.fc1_weight.grad[i].any() and not module.fc2_weight.grad[i].any()
+
+
+def test_grouped_mlp_matches_bf16_autograd(dev):
+    """End-to-end sanity against plain torch autograd in fp32 (not the parity oracle): FP8 training
+    noise is a few percent, so outputs and gradients must correlate strongly with the fp32 model."""
+    pkg = _pkg()
+    sizes, h, f = [200, 333, 91], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(2002)
+    w1 = randn_bf16((e, f, h), g, 0.05)
+    w2 = randn_bf16((e, h, f), g, 0.05)
+    x = randn_bf16((m, h), g)
+    dy = randn_bf16((m, h), g, 1e-2)
+    module = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+    module.fc1_weight.data.copy_(w1)
+    module.fc2_weight.data.copy_(w2)
+    gs = torch.tensor(sizes)
+    for _ in range(2):  # second pass runs with real scales
+        xd = x.to(dev).requires_grad_()
+        module.zero_grad()
+        with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=2)):
+            out = module(xd, gs)
+        out.backward(dy.to(dev))
+    xr = x.float().requires_grad_()
+    w1r, w2r = w1.float().requires_grad_(), w2.float().requires_grad_()
+    outs, start = [], 0
+    for i, s in enumerate(sizes):
+        hdn = torch.nn.functional.gelu(xr[start: start + s] @ w1r[i].t(), approximate="tanh")
+        outs.append(hdn @ w2r[i].t())
+        start += s
+    ref_out = torch.cat(outs)
+    ref_out.backward(dy.float())
+
+    def cos(a, b):
+        a, b = a.detach().float().cpu().flatten(), b.detach().float().flatten()
+        return torch.dot(a, b) / (a.norm() * b.norm())
+
+    assert cos(out, ref_out) > 0.995
+    assert cos(xd.grad, xr.grad) > 0.99
+    assert cos(module.fc1_weight.grad, w1r.grad) > 0.99
+    assert cos(module.fc2_weight.grad, w2r.grad) > 0.99
