@@ -82,7 +82,12 @@ __device__ __forceinline__ uint8_t cvt1_fp8(float v) {
 }
 
 // max(acc, |x|) that never lets a NaN in (fmaxf semantics of the reference's amax).
-__device__ __forceinline__ float amax_step(float acc, float x) { return fmaxf(acc, fabsf(x)); }
+// A compare + select, not v_max_f32: in IEEE mode the hardware max returns a NaN when an
+// input is a signalling NaN (bf16 data can carry such patterns), which would erase `acc`.
+__device__ __forceinline__ float amax_step(float acc, float x) {
+  const float ax = fabsf(x);
+  return (ax > acc) ? ax : acc;
+}
 
 // Wave-wide max of non-negative floats; every lane gets the result.
 __device__ __forceinline__ float wave_max(float v) {
