@@ -1,0 +1,175 @@
+"""Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1]
+
+A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
+HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
+delayed-scaling update.  Prints ONE JSON line.
+
+  value     whole-step throughput in TFLOP/s: algorithmic GEMM flops of the step (unpadded rows,
+            2 * sum_i M_i * N * K per grouped GEMM) / wall time of the step
+  roofline  the dominant kernel (grouped GEMM): algorithmic flops per launch / mean launch
+            duration from HIP events recorded around every launch inside the timed region,
+            against the dense FP8 MFMA peak of 5.0 PFLOP/s
+  kernels   the same event timing for every kernel of the step (GB/s against 8 TB/s for the
+            cast / transpose / pad kernels)
+  cpu_baseline  the per-expert quantize-dequantize-fp32-matmul loop (oracle/cpu_baseline.py) on
+            a bounded sample, timed on this machine's host cores
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+FP8_PEAK_TFLOPS = 5000.0  # MI355X dense FP8 MFMA
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (module, experts, hidden, ffn, tokens, splitter)
+    "config1": ("linear", 4, 256, 512, 1000, "fixed"),
+    "config2": ("mlp", 8, 4096, 14336, 16384, "dirichlet"),
+    "config3": ("linear", 64, 2048, 1408, 24576, "zipf"),
+    "config4": ("mlp", 128, 2048, 768, 65536, "uniform"),
+}
+
+
+def splits(kind, experts, tokens, seed):
+    rng = np.random.default_rng(seed)
+    if kind == "fixed":
+        return [137, 401, 59, 403]
+    if kind == "dirichlet":
+        p = rng.dirichlet(np.ones(experts))
+    elif kind == "zipf":
+        p = 1.0 / np.arange(1, experts + 1) ** 1.1
+        p /= p.sum()
+    else:
+        p = np.full(experts, 1.0 / experts)
+    return [int(v) for v in rng.multinomial(tokens, p)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-events", action="store_true", help="skip per-kernel HIP events (pure wall time)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+
+    import fp8_gmm_amd as pkg
+    from fp8_gmm_amd.backend import kernel_timing
+
+    kind, experts, hidden, ffn, tokens, splitter = WORKLOADS[args.workload]
+    idx = int(args.workload[-1])
+    sizes = splits(splitter, experts, tokens, 1000 + idx)
+    dev = torch.device("cuda:0")
+    torch.manual_seed(1000 + idx)
+    if kind == "mlp":
+        module = pkg.GroupedMlp(hidden, ffn, experts, torch.bfloat16, device=dev)
+        module.fc1_weight.data.normal_(0, 0.02)
+        module.fc2_weight.data.normal_(0, 0.02)
+        out_features, gemms = hidden, 6
+    else:
+        module = pkg.GroupedLinear(hidden, ffn, experts, torch.bfloat16, device=dev)
+        module.weight_tensor.data.normal_(0, 0.02)
+        out_features, gemms = ffn, 3
+    x = torch.randn(tokens, hidden, device=dev, dtype=torch.bfloat16).requires_grad_()
+    dy = (torch.randn(tokens, out_features, device=dev) * 1e-2).to(torch.bfloat16)
+    gs = torch.tensor(sizes, dtype=torch.int64)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=16)
+    flops_per_gemm = 2.0 * tokens * hidden * ffn
+    flops_per_step = gemms * flops_per_gemm
+
+    def step():
+        module.zero_grad(set_to_none=True)
+        x.grad = None
+        with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
+            out = module(x, gs)
+        out.backward(dy)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timing = None
+    if args.no_kernel_events:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    else:
+        with kernel_timing() as timing:
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    value = flops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    roofline = None
+    kernels = {}
+    if timing is not None:
+        summ = timing.summary()
+        for name, d in summ.items():
+            if name == "grouped_gemm":
+                ach = flops_per_gemm / (d["ms"] * 1e-3) / 1e12
+                kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
+                                 "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4)}
+                roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
+                            "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),
+                            "traffic": None}
+            else:
+                gbs = d["work"] / (d["ms"] * 1e-3) / 1e9
+                kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
+                                 "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import cpu_baseline
+
+        cores = torch.get_num_threads()
+        sample_tokens = 16384
+        cpu_baseline.mlp_step_sample(64, hidden, ffn)  # warm-up of the thread pool
+        secs, fl = cpu_baseline.mlp_step_sample(sample_tokens, hidden, ffn)
+        cpu = {"value": round(fl / secs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+               "sample": f"all {sample_tokens} tokens through one expert, {hidden}->{ffn} MLP fwd+bwd (6 GEMMs, "
+                         f"{fl / 1e9:.0f} GFLOP) incl. weight quantisation, {secs:.1f} s"}
+
+    line = {
+        "metric": "FP8 grouped-GEMM TFLOP/s fwd+bwd, % of MI355X FP8 MFMA peak, E=8 MoE MLP",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "pct_of_fp8_mfma_peak": round(100.0 * value / FP8_PEAK_TFLOPS, 2),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: Grouped{'Mlp' if kind == 'mlp' else 'Linear'} fwd+bwd, E={experts}, "
+                               f"hidden={hidden}, ffn={ffn}, tokens={tokens}, split={splitter}",
+                   "group_sizes": sizes if experts <= 16 else f"{experts} experts, min {min(sizes)} max {max(sizes)}",
+                   "gemm_flops_per_step": flops_per_step},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "kernels": kernels,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

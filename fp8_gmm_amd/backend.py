@@ -27,6 +27,88 @@ def _fail(msg):
     raise RuntimeError(msg)
 
 
+class kernel_timing:
+    """Context manager that brackets every kernel launch of this module with HIP events.
+
+    The events are recorded on the stream the kernels are launched on (torch's current
+    stream).  ``records`` holds ``(kernel name, algorithmic work, start event, end event)``;
+    ``summary()`` synchronises and returns per-kernel launch counts, mean duration in ms and
+    the algorithmic work (flops for the GEMM, bytes for the other kernels) per launch.
+    """
+
+    _active = None
+
+    def __init__(self):
+        self.records = []
+
+    def __enter__(self):
+        kernel_timing._active = self
+        return self
+
+    def __exit__(self, *exc):
+        kernel_timing._active = None
+        return False
+
+    def summary(self):
+        torch.cuda.synchronize()
+        out = {}
+        for name, work, start, end in self.records:
+            d = out.setdefault(name, {"launches": 0, "ms": 0.0, "work": 0.0})
+            d["launches"] += 1
+            d["ms"] += start.elapsed_time(end)
+            d["work"] += work
+        for d in out.values():
+            d["ms"] /= d["launches"]
+            d["work"] /= d["launches"]
+        return out
+
+
+class _timed:
+    def __init__(self, name, work_fn):
+        self.rec = kernel_timing._active
+        if self.rec is not None:
+            self.name, self.work = name, float(work_fn())
+
+    def __enter__(self):
+        if self.rec is not None:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.start.record()
+
+    def __exit__(self, *exc):
+        if self.rec is not None:
+            end = torch.cuda.Event(enable_timing=True)
+            end.record()
+            self.rec.records.append((self.name, self.work, self.start, end))
+        return False
+
+
+_OP_NAMES = {
+    _lib.OP_QUANTIZE: "multi_quantize",
+    _lib.OP_SCALE_MUL: "multi_scale_mul",
+    _lib.OP_PAD_TRANSPOSE: "multi_pad_transpose",
+    _lib.OP_PAD_CAST_TRANSPOSE: "multi_pad_cast_transpose",
+    _lib.OP_PAD_CAST_TRANSPOSE_DGELU: "multi_pad_cast_transpose_dgelu",
+}
+
+
+def _algorithmic_bytes(op, table):
+    """HBM bytes an ideal kernel moves: every input element read once, every output element written once."""
+    rows = table["rows"].astype(np.int64)
+    cols = table["cols"].astype(np.int64)
+    rpad = table["rows_padded"].astype(np.int64)
+    if op == _lib.OP_QUANTIZE:
+        return int((rows * cols * 3).sum())
+    if op == _lib.OP_SCALE_MUL:
+        return int((rows * cols * 4).sum())
+    has_out = (table["out"] != 0).astype(np.int64)
+    in_bytes = {_lib.OP_PAD_TRANSPOSE: 1, _lib.OP_PAD_CAST_TRANSPOSE: 2, _lib.OP_PAD_CAST_TRANSPOSE_DGELU: 4}[op]
+    return int((cols * (rows * in_bytes + rows * has_out + rpad)).sum())
+
+
+def _algorithmic_flops(table):
+    return int((2 * table["m"].astype(np.int64) * table["n"].astype(np.int64) * table["k"].astype(np.int64)).sum())
+
+
 def _device_of(tensors):
     dev = None
     for t in tensors:
@@ -82,7 +164,7 @@ def _launch_multi(op, table, out_fmt, device):
     L = _lib.load()
     dev_table = _upload(table, device)
     n = len(table)
-    with torch.cuda.device(device):
+    with torch.cuda.device(device), _timed(_OP_NAMES[op], lambda: _algorithmic_bytes(op, table)):
         s = _stream(device)
         if op == _lib.OP_QUANTIZE:
             rc = L.fp8gmm_multi_quantize(dev_table.data_ptr(), n, total, out_fmt, s)
@@ -258,7 +340,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device):
     if total == 0:
         return
     dev_table = _upload(table, device)
-    with torch.cuda.device(device):
+    with torch.cuda.device(device), _timed("grouped_gemm", lambda: _algorithmic_flops(table)):
         rc = _lib.load().fp8gmm_grouped_gemm(
             dev_table.data_ptr(), len(table), total, _FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype],
             _lib.EPI_GELU if gelu else 0, _stream(device),

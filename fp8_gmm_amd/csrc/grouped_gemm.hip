@@ -345,10 +345,12 @@ int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles
     const bool has_work = p.m > 0 && p.n > 0;
     if (has_work) {
       if (p.c == nullptr) return FP8GMM_ERR_NULL_POINTER;
-      if (p.k > 0 && (p.a == nullptr || p.b == nullptr)) return FP8GMM_ERR_NULL_POINTER;
-      if ((p.k & 15) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
-      if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
-        return FP8GMM_ERR_ALIGNMENT;
+      if (p.k > 0) {  // with k == 0 the operands are never read
+        if (p.a == nullptr || p.b == nullptr) return FP8GMM_ERR_NULL_POINTER;
+        if ((p.k & 15) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
+        if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
+          return FP8GMM_ERR_ALIGNMENT;
+      }
     }
     const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;
     const int64_t tn = (p.n + fp8gmm::BN - 1) / fp8gmm::BN;

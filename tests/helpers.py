@@ -103,3 +103,27 @@ def scales_for(tensors, dtype):
         scales.append(s)
         invs.append((1.0 / s).to(torch.float32))
     return scales, invs
+
+
+def assert_close_multistage(c_gpu, ref_t, fro_tol=5e-3, what=""):
+    """Comparison for results that went through one or more fp8 RE-quantisations of computed values
+    (GroupedMlp): the GPU and the oracle accumulate in different orders, so a value that sits on an
+    fp8 rounding boundary may land one code step apart (6-12 % of that element) and move the few
+    outputs it feeds by several percent of the output rms.  The orchestration is what is under test
+    here (a wrong operand, scale or slot gives O(1) errors), so the bounds are:
+      * relative Frobenius error <= fro_tol
+      * every element within 0.02 |ref| + 0.25 rms(ref)
+    Stage-exact checks of each kernel live in the backend tests.
+    """
+    c = c_gpu.detach().float().cpu()
+    r = ref_t.float()
+    assert c.shape == r.shape, f"{what}: shape {c.shape} vs {r.shape}"
+    if r.numel() == 0:
+        return
+    assert torch.isfinite(c).all(), f"{what}: non-finite output"
+    err = c - r
+    fro = (err.norm() / r.norm().clamp_min(1e-30)).item()
+    assert fro <= fro_tol, f"{what}: relative Frobenius error {fro:.3e} > {fro_tol}"
+    rms = r.pow(2).mean().sqrt()
+    bad = err.abs() > 0.02 * r.abs() + 0.25 * rms
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements outside 0.02|ref| + 0.25 rms"

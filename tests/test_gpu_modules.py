@@ -7,7 +7,7 @@ compare outputs, gradients and the recorded scaling state.
 import pytest
 import torch
 
-from helpers import assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
+from helpers import assert_close_multistage, assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
 from oracle import modules as orc
 
 pytestmark = pytest.mark.gpu
@@ -103,12 +103,11 @@ def test_grouped_linear_inference_and_frozen_weight(dev):
         out = module(xd, gs)
     out.backward(dy.to(dev))
     assert module.weight_tensor.grad is None
-    # scales were updated from the first pass: compare against the oracle run the same way
-    fwd.update(448.0)
-    bwd.update(57344.0)
-    o2 = orc.grouped_linear_step(x, w, sizes, dy, fwd, bwd)
-    assert_gemm_close(out, o2["out"].float(), 1e-2, "frozen-weight out")
-    assert_gemm_close(xd.grad, o2["grad_input"].float(), 1e-2, "frozen-weight grad_input")
+    # a no_grad pass does not count as a training step, so this first training pass still runs with
+    # the initial scales: same oracle result
+    assert_gemm_close(out, o["out"].float(), 1e-2, "frozen-weight out")
+    assert_gemm_close(xd.grad, o["grad_input"].float(), 1e-2, "frozen-weight grad_input")
+    assert_scalar_bits_equal(module.fp8_meta["scaling_fwd"].amax_history[0], fwd.amax_history[0], "fwd amax")
 
 
 MLP_CASES = {
@@ -158,11 +157,10 @@ def test_grouped_mlp_fwd_bwd(dev, case):
         assert_scalar_bits_equal(gm["scaling_bwd"].scale, bwd.scale, f"step {step} bwd scale")
         _check_amax(gm["scaling_fwd"], fwd, exact_fwd, approx_fwd, f"step {step} fwd")
         _check_amax(gm["scaling_bwd"], bwd, exact_bwd, approx_bwd, f"step {step} bwd")
-        # every stage adds an fp8 re-quantisation of a slightly different bf16 value: widen the bound per stage
-        assert_gemm_close(out, o["out"].float(), 2e-2, f"step {step} out")
-        assert_gemm_close(module.fc2_weight.grad, o["grad_w2"].float(), 2e-2, f"step {step} grad_fc2")
-        assert_gemm_close(xd.grad, o["grad_input"].float(), 3e-2, f"step {step} grad_input")
-        assert_gemm_close(module.fc1_weight.grad, o["grad_w1"].float(), 3e-2, f"step {step} grad_fc1")
+        assert_close_multistage(out, o["out"], 5e-3, f"step {step} out")
+        assert_close_multistage(module.fc2_weight.grad, o["grad_w2"], 5e-3, f"step {step} grad_fc2")
+        assert_close_multistage(xd.grad, o["grad_input"], 1e-2, f"step {step} grad_input")
+        assert_close_multistage(module.fc1_weight.grad, o["grad_w1"], 1e-2, f"step {step} grad_fc1")
         for i, s in enumerate(sizes):
             if s == 0:
                 assert not module.fc1_weight.grad[i].any() and not module.fc2_weight.grad[i].any()
