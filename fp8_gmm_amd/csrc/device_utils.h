@@ -22,16 +22,14 @@ __device__ __forceinline__ float bf16_lo_to_f32(uint32_t packed) { return __uint
 __device__ __forceinline__ float bf16_hi_to_f32(uint32_t packed) { return __uint_as_float(packed & 0xffff0000u); }
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
-// fp32 -> bf16 bits, round-to-nearest-even, NaN kept quiet.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  uint32_t nan = (u >> 16) | 0x0040u;
-  return ((u & 0x7fffffffu) > 0x7f800000u) ? (nan & 0xffffu) : rounded;
-}
+// two fp32 -> packed bf16 (element 0 in the low half), round-to-nearest-even: one v_cvt_pk_bf16_f32
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 
 template <int FMT>
 struct Fp8Limits;
@@ -79,6 +77,13 @@ __device__ __forceinline__ uint32_t cvt4_fp8(float v0, float v1, float v2, float
 template <int FMT>
 __device__ __forceinline__ uint8_t cvt1_fp8(float v) {
   return (uint8_t)(cvt4_fp8<FMT>(v, 0.f, 0.f, 0.f) & 0xffu);
+}
+
+// Store through an explicit global-address-space pointer: a pointer loaded from a table is generic,
+// and a generic (flat) store also counts as an LDS operation in the wait counters.
+template <typename T>
+__device__ __forceinline__ void global_store(void* p, T v) {
+  *reinterpret_cast<__attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)) = v;
 }
 
 // max(acc, |x|) that never lets a NaN in (fmaxf semantics of the reference's amax).

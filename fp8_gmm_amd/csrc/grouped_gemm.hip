@@ -7,23 +7,34 @@
 //   c[m, n] = epilogue( sum_k a[m, k] * b[n, k] ),   a, b fp8 (K contiguous), fp32 accumulation
 //
 // Work decomposition
-//   * the output of every problem is cut into 256 x 256 tiles; all tiles of all
-//     problems form one list, walked by a persistent grid (one workgroup per CU);
-//     the list is split into 8 contiguous ranges, one per XCD, so that workgroups
-//     sharing an L2 work on neighbouring tiles (workgroup i runs on XCD i % 8);
-//   * a workgroup is 8 wavefronts (2 along m x 4 along n); a wavefront owns a
-//     128 x 64 sub-tile = 4 x 2 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4;
-//   * K is consumed 128 bytes per step through two LDS stages (2 x 64 KB): global
-//     loads for step s+1 are issued before the MFMAs of step s and written to the
-//     other stage afterwards - one barrier per step;
-//   * LDS rows are 128 bytes (one K step) with the 16-byte chunks XOR-swizzled by the
-//     row index so that the 16-byte fragment reads of 64 lanes spread over all banks;
-//   * the weight operand (b) is fed as MFMA source 0 and the token operand (a) as
-//     source 1: the accumulator layout then gives every lane 4 consecutive output
-//     columns of one output row, i.e. 8-byte bf16 stores without a shuffle.
+//   * the output of every problem is cut into 256 x 256 tiles; all tiles of all problems form
+//     one list walked by a persistent grid (one workgroup per CU).  The list is split into 8
+//     contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so that workgroups that
+//     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest, so
+//     neighbouring tiles share the weight slab.
+//   * a workgroup is 8 wavefronts (2 along m x 4 along n); a wavefront owns a 128 x 64
+//     sub-tile = 4 x 2 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4 (128 accumulator registers).
+//     The weight operand is MFMA source 0 and the token operand source 1: every lane then
+//     holds 4 consecutive output columns of one row (8-byte bf16 stores, no shuffle).
 //
-// Out-of-range rows / K tails are zero-filled on load, so m, n are arbitrary and k
-// only has to be a multiple of 16 bytes.
+// Data movement
+//   * operands go global -> LDS directly (`buffer_load_dwordx4 ... lds`), never through
+//     registers.  Buffer descriptors bound every operand, so rows past m / n and K tails read
+//     as zeros: m, n are arbitrary and k only has to be a multiple of 16.
+//   * LDS holds a ring of five 32 KB half-slots (all 160 KB); a half-slot is one K = 64 slice
+//     of the tile: 256 token rows + 256 weight rows of 64 bytes, the four 16-byte chunks of a
+//     row XOR-swizzled with (row >> 2) & 3, which makes the 16-byte fragment reads of a
+//     wavefront conflict-free.
+//   * every second step a wavefront issues the 8 loads of a K = 128 pair (the two 64-byte
+//     halves of each 128-byte line back to back, so the second half hits in L1) into the two
+//     half-slots that have just become free; the pair is first read three steps later.
+//   * the load stream, the fragment double buffer and the ring run CONTINUOUSLY across tile
+//     boundaries: while a tile's epilogue stores its result, the next tile's first two pairs
+//     are already in LDS and its first fragments in registers.
+//   * one s_barrier per K = 64 step.  After each barrier the MFMAs (whose fragments were
+//     fetched during the previous step) are issued first and the DMA issues / next-fragment
+//     LDS reads are interleaved between them (pinned with sched_barrier), so the MFMA pipe
+//     does not idle while the two wavefronts of a SIMD do their memory work.
 #include "device_utils.h"
 #include "tiling.h"
 
@@ -32,27 +43,27 @@ namespace {
 
 constexpr int BM = kGemmTileM;   // 256
 constexpr int BN = kGemmTileN;   // 256
-constexpr int BK = kGemmTileK;   // 128 bytes
+constexpr int HK = 64;           // bytes of K per half-slot / per MFMA
+constexpr int HS = (BM + BN) * HK;  // 32768 bytes per half-slot
+constexpr int RING = 5;
 constexpr int NTHREADS = 512;
-constexpr int WAVES_M = 2;
-constexpr int WAVES_N = 4;
-constexpr int WM = BM / WAVES_M;  // 128
-constexpr int WN = BN / WAVES_N;  // 64
+constexpr int WM = 128, WN = 64;  // wavefront sub-tile
 constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
 constexpr int NT = WN / 32;       // 2 MFMA tiles along n per wave
-constexpr int STAGE_BYTES = (BM + BN) * BK;  // 65536
-constexpr int A_LOADS = BM * (BK / 16) / NTHREADS;  // 4 x 16-byte chunks per thread
-constexpr int B_LOADS = BN * (BK / 16) / NTHREADS;  // 4
 constexpr int kNumXcd = 8;
+constexpr int kPairLoads = 8;     // buffer_load ... lds instructions per wavefront per K = 128 pair
+constexpr int kFastStores = MT * NT * 2;  // 16-byte stores per wavefront in the interior bf16 epilogue
+constexpr int kRelaxedWaits = 3;  // barriers after such an epilogue that need not wait for its stores
 
-// 16-byte chunk swizzle inside a 128-byte LDS row.
-__device__ __forceinline__ int swz(int row) { return row & 7; }
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-struct TileCoord {
-  int prob;
-  int m0;
-  int n0;
-};
+#define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
+#define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+#define FP8GMM_WAIT_VM_LGKM(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(n) : "memory")
+typedef unsigned u32pair __attribute__((ext_vector_type(2)));
+// global -> LDS: lane i's 16 bytes land at M0 + 16 i; out-of-range offsets deliver zeros
+#define FP8GMM_DMA(lds_addr, voff, rsrc) \
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
 
 template <int A_FMT, int B_FMT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
@@ -63,41 +74,203 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wave_m = wave / WAVES_N;  // 0..1
-  const int wave_n = wave % WAVES_N;  // 0..3
+  const int wave_m = wave >> 2;  // 0..1
+  const int wave_n = wave & 3;   // 0..3
   const int l32 = lane & 31;
-  const int khalf = lane >> 5;  // which 32-byte half of a 64-byte MFMA K slice this lane feeds
+  const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
-  // ---- global -> LDS staging map: chunk (row, c) of the 128-byte-wide stage ----
-  const int ld_c = tid & 7;     // 16-byte chunk in the K step
-  const int ld_r = tid >> 3;    // 0..63, rows ld_r + 64 i
-  const int st_off = ld_r * BK + ((ld_c ^ swz(ld_r)) << 4);  // same swizzle for rows ld_r + 64 i (64 % 8 == 0)
+  // DMA lane map: one wavefront instruction fills 16 rows x 64 B of a half-slot: lane -> row lane >> 2,
+  // slot chunk lane & 3.  With the swizzle (row >> 2) & 3 and row = 16 g + (lane >> 2) the GLOBAL chunk
+  // that has to land there is (lane & 3) ^ ((lane >> 4) & 3).
+  const int drow = lane >> 2;
+  const int dchunk = (lane & 3) ^ ((lane >> 4) & 3);
+  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 64 + 32 j + l32 (source 0)
+  const int fsw = (l32 >> 2) & 3;
+  const int fc0 = ((khalf * 2) ^ fsw) << 4;
+  const int fc1 = ((khalf * 2 + 1) ^ fsw) << 4;
+  const int fa_off = (wave_m * WM + l32) * HK;
+  const int fb_off = BM * HK + (wave_n * WN + l32) * HK;
 
-  // ---- LDS -> fragment map ----
-  // token rows (MFMA source 1):  wave_m * 128 + mt * 32 + l32 ; weight rows (source 0): wave_n * 64 + nt * 32 + l32
-  const int frag_row_off = l32 * BK;
-  const int frag_swz = swz(l32);
-
-  const int chunk = (total_tiles + kNumXcd - 1) / kNumXcd;
-  const int padded_total = chunk * kNumXcd;
-
-  for (int t = blockIdx.x; t < padded_total; t += gridDim.x) {
-    // XCD-aware order: consecutive workgroup ids land on different XCDs; give each XCD a contiguous range.
-    const int tile = (t % kNumXcd) * chunk + t / kNumXcd;
-    if (tile >= total_tiles) continue;
-
+  // ---- this workgroup's tile sequence (uniform) ----
+  // Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal COST
+  // (a tile of problem p costs ceil(k_p / 128) pair steps; k differs per problem in the wgrad form),
+  // and the workgroups of an XCD stride through that XCD's range.
+  const int xcd = blockIdx.x % kNumXcd;
+  const int wg_in_xcd = blockIdx.x / kNumXcd;
+  const int wgs_per_xcd = gridDim.x / kNumXcd;  // the launcher keeps gridDim.x a multiple of 8
+  int range_begin = total_tiles, range_end = total_tiles;
+  {
+    auto tile_cost = [&](int p) {
+      const int c = (probs[p].k + 127) / 128;
+      return (int64_t)(c > 0 ? c : 1);
+    };
+    int64_t total_cost = 0;
+    for (int p = 0; p < nprob; ++p) {
+      const int t_end = (p + 1 < nprob) ? probs[p + 1].tile_begin : total_tiles;
+      total_cost += (int64_t)(t_end - probs[p].tile_begin) * tile_cost(p);
+    }
+    const int64_t lo = (total_cost * xcd + kNumXcd - 1) / kNumXcd;
+    const int64_t hi = (total_cost * (xcd + 1) + kNumXcd - 1) / kNumXcd;
+    // first tile whose preceding cost is >= lo (resp. hi)
+    int64_t cum = 0;
+    bool have_lo = false, have_hi = false;
+    for (int p = 0; p < nprob && !have_hi; ++p) {
+      const int t_begin = probs[p].tile_begin;
+      const int t_end = (p + 1 < nprob) ? probs[p + 1].tile_begin : total_tiles;
+      const int64_t c = tile_cost(p);
+      const int64_t n_t = t_end - t_begin;
+      if (!have_lo && cum + n_t * c > lo - c) {  // some tile i of p has cum + i c >= lo
+        const int64_t i = lo > cum ? (lo - cum + c - 1) / c : 0;
+        if (i < n_t) {
+          range_begin = t_begin + (int)i;
+          have_lo = true;
+        }
+      }
+      if (cum + n_t * c > hi - c) {
+        const int64_t i = hi > cum ? (hi - cum + c - 1) / c : 0;
+        if (i < n_t) {
+          range_end = t_begin + (int)i;
+          have_hi = true;
+        }
+      }
+      cum += n_t * c;
+    }
+    if (!have_lo) range_begin = total_tiles;
+  }
+  auto next_tile = [&](int t) { return t < range_end ? t : -1; };
+  struct Geo {
+    int prob, m0, n0, nk;
+  };
+  auto geo_of = [&](int tile) {
     const int p = upper_slot(nprob, tile, [&](int i) { return probs[i].tile_begin; });
-    const fp8gmm_gemm_problem pr = probs[p];
-    const int local = tile - pr.tile_begin;
-    const int tiles_m = (pr.m + BM - 1) / BM;
-    const int tm = local % tiles_m;  // m fastest: neighbouring tiles share the weight slab
-    const int tn = local / tiles_m;
-    const int m0 = tm * BM;
-    const int n0 = tn * BN;
-    const int M = pr.m, N = pr.n, K = pr.k;
-    const uint8_t* __restrict__ A = static_cast<const uint8_t*>(pr.a);
-    const uint8_t* __restrict__ B = static_cast<const uint8_t*>(pr.b);
-    const int64_t lda = pr.lda, ldb = pr.ldb;
+    const int local = tile - probs[p].tile_begin;
+    const int tiles_m = (probs[p].m + BM - 1) / BM;
+    Geo g;
+    g.prob = p;
+    g.m0 = (local % tiles_m) * BM;  // m fastest: neighbouring tiles share the weight slab
+    g.n0 = (local / tiles_m) * BN;
+    g.nk = (probs[p].k + 127) / 128;  // K = 128 pairs; a K tail is zero-filled
+    return g;
+  };
+  const int t_stride = wgs_per_xcd;
+
+  int t_cp = next_tile(range_begin + wg_in_xcd);
+  if (t_cp < 0) return;
+
+  // ---- load side: runs two pairs ahead of the compute side, possibly in the next tile ----
+  int t_ld = t_cp;
+  int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
+  i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
+  uint32_t a_base[2], b_base[2];
+  uint32_t ok_mask = 0;  // bit part: rows of that part exist
+  auto load_setup = [&]() {
+    while (t_ld >= 0) {
+      const Geo g = geo_of(t_ld);
+      if (g.nk > 0) {
+        const fp8gmm_gemm_problem pr = probs[g.prob];
+        const uint64_t pa = (uint64_t)pr.a, pb = (uint64_t)pr.b;
+        const uint64_t sa = (uint64_t)pr.m * (uint64_t)pr.lda, sb = (uint64_t)pr.n * (uint64_t)pr.ldb;
+        rsrc_a[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pa);
+        rsrc_a[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pa >> 32));
+        rsrc_a[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sa > 0xffffffffull ? 0xffffffffull : sa));
+        rsrc_b[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pb);
+        rsrc_b[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pb >> 32));
+        rsrc_b[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sb > 0xffffffffull ? 0xffffffffull : sb));
+        ok_mask = 0;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int ar = g.m0 + (wave + 8 * j) * 16 + drow;
+          const int br = g.n0 + (wave + 8 * j) * 16 + drow;
+          if (ar < pr.m) ok_mask |= 1u << j;
+          if (br < pr.n) ok_mask |= 4u << j;
+          a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          b_base[j] = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
+        }
+        ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
+        ld_nk = g.nk;
+        ld_kt = 0;
+        return;
+      }
+      t_ld = next_tile(t_ld + t_stride);  // a tile without K work needs no loads
+    }
+  };
+  // One quarter of a pair: part 0, 1 = token row groups wave, wave + 8; part 2, 3 = weight row groups.
+  // Low 64-byte half into slot_lo, high half into slot_hi.  Past the end of the stream the loads are
+  // issued all the same with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
+  auto dma_part = [&](int slot_lo, int slot_hi, int part) {
+    const int j = part & 1;
+    const bool is_b = (part >> 1) != 0;
+    const int k0 = ld_kt * 128;
+    const bool rok = (t_ld >= 0) && ((ok_mask >> part) & 1);
+    const uint32_t base = is_b ? b_base[j] : a_base[j];
+    const uint32_t v_lo = (rok && k0 < ld_kmax) ? base + k0 : 0xffffffffu;
+    const uint32_t v_hi = (rok && k0 + 64 < ld_kmax) ? base + k0 + 64 : 0xffffffffu;
+    const uint32_t off = (is_b ? BM * HK : 0) + (wave + 8 * j) * 1024;
+    const uint32_t l_lo = __builtin_amdgcn_readfirstlane(lds_base + slot_lo * HS + off);
+    const uint32_t l_hi = __builtin_amdgcn_readfirstlane(lds_base + slot_hi * HS + off);
+    if (!is_b) {
+      FP8GMM_DMA(l_lo, v_lo, rsrc_a);
+      FP8GMM_DMA(l_hi, v_hi, rsrc_a);
+    } else {
+      FP8GMM_DMA(l_lo, v_lo, rsrc_b);
+      FP8GMM_DMA(l_hi, v_hi, rsrc_b);
+    }
+  };
+  auto dma_advance = [&]() {
+    if (t_ld < 0) return;
+    if (++ld_kt == ld_nk) {
+      t_ld = next_tile(t_ld + t_stride);
+      load_setup();
+    }
+  };
+  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
+
+  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: even / odd half-steps
+  auto read_frag = [&](i32x8& f, const uint8_t* base) {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc0);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc1);
+    f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+
+  // ---- fill: pairs 0 and 1 of the stream into half-slots 0..3, first fragments into registers ----
+  load_setup();
+#pragma unroll
+  for (int part = 0; part < 4; ++part) dma_part(0, 1, part);
+  dma_advance();
+#pragma unroll
+  for (int part = 0; part < 4; ++part) dma_part(2, 3, part);
+  dma_advance();
+  FP8GMM_WAIT_VM(kPairLoads);
+  __builtin_amdgcn_s_barrier();
+  {
+    const uint8_t* sa = lds + fa_off;
+    const uint8_t* sb = lds + fb_off;
+    read_frag(fb0[0], sb);
+    read_frag(fb0[1], sb + 32 * HK);
+    read_frag(fa0[0], sa);
+    read_frag(fa0[1], sa + 32 * HK);
+    read_frag(fa0[2], sa + 64 * HK);
+    read_frag(fa0[3], sa + 96 * HK);
+  }
+  int hs = 0;  // half-slot of the current even half-step
+  // vmcnt counts loads and stores in issue order.  A barrier needs the pair before the newest one, so it
+  // normally waits for "all but the newest 8".  Right after an interior epilogue the newest operations
+  // also include that epilogue's kFastStores stores, which nothing in LDS depends on: for the next
+  // kRelaxedWaits barriers the needed pair is older than those stores, so they may stay in flight.
+  int relaxed = 0;
+
+// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
+#define FP8GMM_MF0(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+#define FP8GMM_MF1(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+
+  for (; t_cp >= 0; t_cp = next_tile(t_cp + t_stride)) {
+    const Geo g = geo_of(t_cp);
+    const fp8gmm_gemm_problem pr = probs[g.prob];
+    const int M = pr.m, N = pr.n;
+    const int m0 = g.m0, n0 = g.n0;
 
     f32x16 acc[MT][NT];
 #pragma unroll
@@ -107,92 +280,69 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int nk = (K + BK - 1) / BK;
-
-    u32x4 ra[A_LOADS], rb[B_LOADS];
-    const uint8_t* a_ptr[A_LOADS];
-    const uint8_t* b_ptr[B_LOADS];
-    bool a_ok[A_LOADS], b_ok[B_LOADS];
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-      const int row = m0 + ld_r + 64 * i;
-      a_ok[i] = row < M;
-      a_ptr[i] = A + (int64_t)(a_ok[i] ? row : 0) * lda + ld_c * 16;
-    }
-#pragma unroll
-    for (int i = 0; i < B_LOADS; ++i) {
-      const int row = n0 + ld_r + 64 * i;
-      b_ok[i] = row < N;
-      b_ptr[i] = B + (int64_t)(b_ok[i] ? row : 0) * ldb + ld_c * 16;
-    }
-
-    auto load_global = [&](int kt) {
-      const int kbyte = kt * BK;
-      const bool k_ok = kbyte + ld_c * 16 < K;
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (a_ok[i] && k_ok) v = *reinterpret_cast<const u32x4*>(a_ptr[i] + kbyte);
-        ra[i] = v;
+    for (int kt = 0; kt < g.nk; ++kt) {
+      const int h1 = ring_inc(hs), h2 = ring_inc(h1);
+      // ---- even half-step: its fragments are in fa0 / fb0.  The barrier proves that every wavefront has
+      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed.
+      if (relaxed > 0) {
+        FP8GMM_WAIT_VM_LGKM(kPairLoads + kFastStores);
+        --relaxed;
+      } else {
+        FP8GMM_WAIT_VM_LGKM(kPairLoads);
       }
-#pragma unroll
-      for (int i = 0; i < B_LOADS; ++i) {
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (b_ok[i] && k_ok) v = *reinterpret_cast<const u32x4*>(b_ptr[i] + kbyte);
-        rb[i] = v;
+      __builtin_amdgcn_s_barrier();
+      {
+        const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
+        const int free_hi = hs;                                         // will hold half-step + 5
+        const uint8_t* qa = lds + h1 * HS + fa_off;
+        const uint8_t* qb = lds + h1 * HS + fb_off;
+        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 0);
+        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 2);
+        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 3);
+        dma_advance();
+        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
+        read_frag(fb1[0], qb);
+        read_frag(fb1[1], qb + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
+        read_frag(fa1[0], qa);
+        read_frag(fa1[1], qa + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_SB();
+        read_frag(fa1[2], qa + 64 * HK);
+        read_frag(fa1[3], qa + 96 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(3, 1); FP8GMM_SB();
       }
-    };
-    auto store_lds = [&](int stage) {
-      uint8_t* sa = lds + stage * STAGE_BYTES;
-      uint8_t* sb = sa + BM * BK;
-#pragma unroll
-      for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<u32x4*>(sa + st_off + i * 64 * BK) = ra[i];
-#pragma unroll
-      for (int i = 0; i < B_LOADS; ++i) *reinterpret_cast<u32x4*>(sb + st_off + i * 64 * BK) = rb[i];
-    };
-    auto compute = [&](int stage) {
-      const uint8_t* sa = lds + stage * STAGE_BYTES + (wave_m * WM) * BK + frag_row_off;
-      const uint8_t* sb = lds + stage * STAGE_BYTES + BM * BK + (wave_n * WN) * BK + frag_row_off;
-#pragma unroll
-      for (int ks = 0; ks < BK / 64; ++ks) {
-        const int c0 = ((ks * 4 + khalf * 2) ^ frag_swz) << 4;
-        const int c1 = ((ks * 4 + khalf * 2 + 1) ^ frag_swz) << 4;
-        i32x8 fa[MT], fb[NT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(sa + i * 32 * BK + c0);
-          const u32x4 hi = *reinterpret_cast<const u32x4*>(sa + i * 32 * BK + c1);
-          fa[i] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const u32x4 lo = *reinterpret_cast<const u32x4*>(sb + j * 32 * BK + c0);
-          const u32x4 hi = *reinterpret_cast<const u32x4*>(sb + j * 32 * BK + c1);
-          fb[j] = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-        }
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-            // source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[j], fa[i], acc[i][j], B_FMT, A_FMT, 0, 0,
-                                                                         0, 0);
+      // ---- odd half-step: fragments in fa1 / fb1; fetch the next even step's fragments early so that
+      // they have arrived long before the next barrier asks for lgkmcnt(0).
+      if (relaxed > 0) {
+        FP8GMM_WAIT_VM(kPairLoads + kFastStores);
+        --relaxed;
+      } else {
+        FP8GMM_WAIT_VM(kPairLoads);
       }
-    };
-
-    if (nk > 0) {
-      load_global(0);
-      store_lds(0);
+      __builtin_amdgcn_s_barrier();
+      {
+        const uint8_t* qa = lds + h2 * HS + fa_off;
+        const uint8_t* qb = lds + h2 * HS + fb_off;
+        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        read_frag(fb0[0], qb);
+        read_frag(fb0[1], qb + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        read_frag(fa0[0], qa);
+        read_frag(fa0[1], qa + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        read_frag(fa0[2], qa + 64 * HK);
+        read_frag(fa0[3], qa + 96 * HK);
+        FP8GMM_SB();
+        FP8GMM_MF1(1, 1); FP8GMM_MF1(2, 0); FP8GMM_MF1(2, 1); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1);
+        FP8GMM_SB();
+      }
+      hs = h2;
     }
-    __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-      const bool more = kt + 1 < nk;
-      if (more) load_global(kt + 1);
-      compute(kt & 1);
-      if (more) store_lds((kt + 1) & 1);
-      __syncthreads();
-    }
-
     // ---- epilogue ----
     const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
     const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
@@ -200,7 +350,37 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
     const int64_t ldc = pr.ldc;
     float amax = 0.f;
-    if (out_kind == FP8GMM_OUT_BF16) {
+    relaxed = 0;
+    const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
+    if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
+        ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
+      // Interior tile, plain bf16 output: straight-line code with an exact store count.  A lane holds
+      // columns 8 g + 4 khalf .. + 3 of its row for g = 0..3; swapping the upper lanes of the even-g
+      // registers with the lower lanes of the odd-g ones leaves 8 consecutive columns per lane:
+      // lanes 0-31 take g even, lanes 32-63 g odd.  One 16-byte store each.
+      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int m = m0 + wave_m * WM + i * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+#pragma unroll
+          for (int gp = 0; gp < 2; ++gp) {
+            const int ge = 8 * gp, go = 8 * gp + 4;  // accumulator index of g = 2 gp and g = 2 gp + 1
+            const uint32_t pe0 = pack_bf16x2(acc[i][j][ge + 0] * s, acc[i][j][ge + 1] * s);
+            const uint32_t pe1 = pack_bf16x2(acc[i][j][ge + 2] * s, acc[i][j][ge + 3] * s);
+            const uint32_t po0 = pack_bf16x2(acc[i][j][go + 0] * s, acc[i][j][go + 1] * s);
+            const uint32_t po1 = pack_bf16x2(acc[i][j][go + 2] * s, acc[i][j][go + 3] * s);
+            const u32pair r0 = __builtin_amdgcn_permlane32_swap(pe0, po0, false, false);
+            const u32pair r1 = __builtin_amdgcn_permlane32_swap(pe1, po1, false, false);
+            const u32x4 o = {r0.x, r1.x, r0.y, r1.y};
+            const int n = n0 + wave_n * WN + j * 32 + (2 * gp + khalf) * 8;
+            global_store(C + (int64_t)m * ldc + n, o);
+          }
+        }
+      }
+      relaxed = kRelaxedWaits;
+    } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
       const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) &&
@@ -223,17 +403,17 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
             const int64_t off = (int64_t)m * ldc + n;
             if (vec && n + 3 < N) {
               u32x2 o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
-              *reinterpret_cast<u32x2*>(C + off) = o;
+              global_store(C + off, o);
               if (gelu && AUX != nullptr) {
                 u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-                *reinterpret_cast<u32x2*>(AUX + off) = a;
+                global_store(AUX + off, a);
               }
             } else {
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
                 if (n + q < N) {
-                  C[off + q] = (uint16_t)f32_to_bf16_bits(r[q]);
-                  if (gelu && AUX != nullptr) AUX[off + q] = (uint16_t)f32_to_bf16_bits(v[q]);
+                  global_store(C + off + q, (uint16_t)f32_to_bf16_bits(r[q]));
+                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
                 }
               }
             }
@@ -270,17 +450,17 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
             }
             const int64_t off = (int64_t)m * ldc + n;
             if (vec && n + 3 < N) {
-              *reinterpret_cast<uint32_t*>(C + off) = w;
+              global_store(C + off, w);
               if (gelu && AUX != nullptr) {
                 u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-                *reinterpret_cast<u32x2*>(AUX + off) = a;
+                global_store(AUX + off, a);
               }
             } else {
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
                 if (n + q < N) {
-                  C[off + q] = (uint8_t)(w >> (8 * q));
-                  if (gelu && AUX != nullptr) AUX[off + q] = (uint16_t)f32_to_bf16_bits(v[q]);
+                  global_store(C + off + q, (uint8_t)(w >> (8 * q)));
+                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
                 }
               }
             }
@@ -292,16 +472,20 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         if (lane == 0 && amax > 0.f) atomic_max_nonneg(pr.c_amax, amax);
       }
     }
-    // all LDS reads of this tile are complete: the last main-loop barrier ordered them.
   }
+  // zero-fill loads issued past the end of the stream still target this workgroup's LDS
+  FP8GMM_WAIT_VM(0);
 }
+
+#undef FP8GMM_MF0
+#undef FP8GMM_MF1
 
 template <int A_FMT, int B_FMT>
 int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
            hipStream_t stream) {
   static int num_cu = 0;
   static bool attr_set = false;
-  const size_t lds_bytes = 2 * STAGE_BYTES;
+  const size_t lds_bytes = (size_t)RING * HS;
   auto kernel = grouped_gemm_kernel<A_FMT, B_FMT>;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -316,9 +500,11 @@ int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out
       return FP8GMM_ERR_NO_DEVICE;
     num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
-  const int chunk = (total_tiles + kNumXcd - 1) / kNumXcd;
-  int grid = chunk * kNumXcd;
-  if (grid > num_cu) grid = num_cu;
+  // one workgroup per CU, a multiple of 8 so that every XCD gets the same number of workgroups
+  int grid = (num_cu / kNumXcd) * kNumXcd;
+  if (grid < kNumXcd) grid = kNumXcd;
+  const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
+  if (grid > needed) grid = needed;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NTHREADS), lds_bytes, stream, probs_dev, n, total_tiles, out_kind,
                      epilogue);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
@@ -350,6 +536,9 @@ int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles
         if ((p.k & 15) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
         if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
           return FP8GMM_ERR_ALIGNMENT;
+        // the kernel addresses each operand through a buffer descriptor with 32-bit byte offsets
+        if ((uint64_t)p.m * (uint64_t)p.lda > 0xffffffffull || (uint64_t)p.n * (uint64_t)p.ldb > 0xffffffffull)
+          return FP8GMM_ERR_BAD_SHAPE;
       }
     }
     const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;

@@ -90,7 +90,8 @@ typedef struct fp8gmm_tensor_desc {
  * Both operands are K-contiguous ("TN"), the only layout the reference uses
  * (fp8_gmm/backend.py:25,57; csrc/fp8_gmm.h:7-11).  Pitches are in elements.
  * a, b must be 16-byte aligned and k, lda, ldb multiples of 16 (the same
- * divisibility cuBLASLt demands of the reference, grouped_linear.py:68).
+ * divisibility cuBLASLt demands of the reference, grouped_linear.py:68); one operand of one problem
+ * may span at most 4 GiB (m * lda, n * ldb < 2^32).
  * k == 0 is allowed and writes epilogue(0); m == 0 or n == 0 produce no work.
  *
  * Epilogue:  v = acc * (*a_scale_inv * *b_scale_inv)        (NULL scale = 1)
