@@ -168,6 +168,19 @@ __device__ __forceinline__ float gelu_tanh(float v) {
   return (0.5f * v) * (1.0f + t);
 }
 
+// tanh-GELU for the GEMM epilogue: same formula, but tanh through the hardware exp2 / rcp
+// approximations (about 1e-6 relative).  The GEMM accumulates in a different order than any CPU
+// check anyway, so nothing here has to be bit-reproducible; the dGELU kernel, which is compared
+// byte for byte, keeps det_tanh.
+__device__ __forceinline__ float gelu_tanh_fast(float v) {
+  const float v2 = v * v;
+  float u = (0.79788456f * v) * __builtin_fmaf(0.044715f, v2, 1.0f);
+  u = fminf(fmaxf(u, -10.f), 10.f);
+  const float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);  // exp(2u)
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+  return (0.5f * v) * (1.0f + t);
+}
+
 // Index of the last entry of a sorted device table whose key (read by `key(i)`) is <= x.
 // Uniform across the workgroup, so it compiles to scalar loads.
 template <typename KeyFn>

@@ -398,7 +398,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               v[q] = acc[i][j][g * 4 + q] * s;
-              r[q] = gelu ? gelu_tanh(v[q]) : v[q];
+              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
             }
             const int64_t off = (int64_t)m * ldc + n;
             if (vec && n + 3 < N) {
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               v[q] = acc[i][j][g * 4 + q] * s;
-              r[q] = gelu ? gelu_tanh(v[q]) : v[q];
+              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
               if (n + q < N) amax = amax_step(amax, r[q]);
             }
             uint32_t w;

@@ -22,7 +22,14 @@ import torch
 
 from .backend import fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
 from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
-from .utils import Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
+from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
+
+
+# Per-expert token counts are padded to this multiple in the TRANSPOSED operands of the weight-gradient
+# GEMMs (zeros along the contraction dimension, so results do not change).  The reference pads to 16,
+# what cuBLASLt needs (fp8_gmm/utils.py:57); here the natural unit is the 128 bytes of one K step of the
+# MFMA pipeline, which also keeps every row of those operands aligned to a cache line.
+MODULE_PAD_MULTIPLE = 128
 
 
 def row_slices(t, bounds):
@@ -58,7 +65,8 @@ class _GroupedLinear(torch.autograd.Function):
         wgrad_needed = is_grad_enabled and weight.requires_grad
         dgrad_needed = is_grad_enabled and input.requires_grad
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
-            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed,
+            pad_multiple=fp8_meta.get("pad_multiple", PAD_MULTIPLE),
         )
         if cumsums[-1] != input.size(0):
             raise RuntimeError("group_sizes must sum to the number of input rows")
@@ -182,8 +190,10 @@ class GroupedLinear(Fp8GroupedModuleBase):
     int64 tensor (or list) of rows per expert, in order; returns ``[tokens, out_features]`` bf16.
     """
 
-    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False):
+    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False,
+                 pad_multiple=MODULE_PAD_MULTIPLE):
         super().__init__()
+        self.fp8_meta["pad_multiple"] = pad_multiple
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.in_features = in_features
         self.out_features = out_features

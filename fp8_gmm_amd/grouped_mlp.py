@@ -28,8 +28,8 @@ from .backend import (
     multi_transpose,
 )
 from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
-from .grouped_linear import alloc_transposed, row_slices, transposed_views
-from .utils import Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
+from .grouped_linear import MODULE_PAD_MULTIPLE, alloc_transposed, row_slices, transposed_views
+from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
 _T = Fp8TensorType
 _M = MetaTensorType
@@ -44,7 +44,8 @@ class _GroupedMlp(torch.autograd.Function):
         # fc2's transposed weights feed the fc2 dgrad, which both the input and the fc1 weight gradients need
         dgrad_needed = is_grad_enabled and (input_requires_grad or weight_requires_grad)
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
-            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed,
+            pad_multiple=fp8_meta.get("pad_multiple", PAD_MULTIPLE),
         )
         if cumsums[-1] != input.size(0):
             raise RuntimeError("group_sizes must sum to the number of input rows")
@@ -227,8 +228,10 @@ class GroupedMlp(Fp8GroupedModuleBase):
     ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None)``.
     """
 
-    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda"):
+    def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
+                 pad_multiple=MODULE_PAD_MULTIPLE):
         super().__init__()
+        self.fp8_meta["pad_multiple"] = pad_multiple
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.num_groups = num_groups
         self.fc1_weight = torch.nn.Parameter(

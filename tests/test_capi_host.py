@@ -1,0 +1,135 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports every function the header
+declares, its structs have the documented layout, and the host-side planners validate and
+schedule correctly.  No kernel is launched here.
+"""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from fp8_gmm_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "fp8gmm.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fp8gmm_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_function():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared_functions()
+    assert len(names) >= 13
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/fp8gmm.h but not exported"
+    assert sorted(_lib.EXPORTS) == names, "the Python binding and the header list different functions"
+
+
+def test_struct_layouts_match_the_binding():
+    lib = _lib.load()
+    assert lib.fp8gmm_sizeof_tensor_desc() == _lib.TENSOR_DESC.itemsize == 64
+    assert lib.fp8gmm_sizeof_gemm_problem() == _lib.GEMM_PROBLEM.itemsize == 96
+    assert _lib.TENSOR_DESC.fields["rows"][1] == 48 and _lib.TENSOR_DESC.fields["block_begin"][1] == 60
+    assert _lib.GEMM_PROBLEM.fields["m"][1] == 64 and _lib.GEMM_PROBLEM.fields["tile_begin"][1] == 88
+    assert lib.fp8gmm_version() == 1
+    assert _lib.gemm_tile_shape() == (256, 256)
+    assert lib.fp8gmm_status_string(0) == b"ok"
+    assert b"NULL" in lib.fp8gmm_status_string(-1)
+
+
+def _desc(rows, cols, rows_padded=0, inp=0x1000, out=0x2000, out_t=0x3000, in2=0):
+    t = np.zeros(len(rows), dtype=_lib.TENSOR_DESC)
+    t["rows"], t["cols"], t["rows_padded"] = rows, cols, rows_padded
+    t["in"], t["out"], t["out_t"], t["in2"] = inp, out, out_t, in2
+    return t
+
+
+def test_plan_quantize_counts_16384_element_workgroups():
+    t = _desc([1, 1, 1, 0, 1], [16384, 16385, 1, 0, 3 * 16384], 0)
+    total = _lib.plan_multi_tensor(t, _lib.OP_QUANTIZE)
+    assert total == 1 + 2 + 1 + 0 + 3
+    assert t["block_begin"].tolist() == [0, 1, 3, 4, 4]
+
+
+def test_plan_pad_kernels_count_128x128_tiles_of_the_padded_extent():
+    t = _desc([137, 128, 0, 1], [256, 129, 64, 3221], [144, 128, 0, 16])
+    total = _lib.plan_multi_tensor(t, _lib.OP_PAD_CAST_TRANSPOSE)
+    assert t["block_begin"].tolist() == [0, 4, 6, 6]   # ceil(144/128)*ceil(256/128), 1*2, 0, 1*26
+    assert total == 4 + 2 + 0 + 26
+    # a transposed output narrower than the input is refused, like TORCH_CHECK(trans_cols >= num_rows)
+    bad = _desc([17], [8], [16])
+    with pytest.raises(_lib.Fp8GmmError):
+        _lib.plan_multi_tensor(bad, _lib.OP_PAD_TRANSPOSE)
+
+
+def test_plan_multi_tensor_error_codes():
+    lib = _lib.load()
+    total = ctypes.c_int(0)
+    t = _desc([4], [4], [16], inp=0)
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, _lib.OP_PAD_TRANSPOSE, ctypes.byref(total)) == -1
+    t = _desc([4], [4], [16], out_t=0)
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, _lib.OP_PAD_CAST_TRANSPOSE, ctypes.byref(total)) == -1
+    t = _desc([4], [4], [16])  # dgelu needs the second input
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, _lib.OP_PAD_CAST_TRANSPOSE_DGELU, ctypes.byref(total)) == -1
+    t = _desc([-1], [4], [16])
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, _lib.OP_QUANTIZE, ctypes.byref(total)) == -2
+    t = _desc([4], [4], [16])
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, 99, ctypes.byref(total)) == -6
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, -1, 0, ctypes.byref(total)) == -6
+    assert lib.fp8gmm_plan_multi_tensor(t.ctypes.data, 1, 0, None) == -1
+    assert lib.fp8gmm_plan_multi_tensor(None, 0, 0, ctypes.byref(total)) == 0 and total.value == 0
+
+
+def _prob(m, n, k, a=0x10000, b=0x20000, c=0x30000, lda=None, ldb=None, ldc=None):
+    t = np.zeros(len(m), dtype=_lib.GEMM_PROBLEM)
+    t["m"], t["n"], t["k"] = m, n, k
+    t["a"], t["b"], t["c"] = a, b, c
+    t["lda"] = k if lda is None else lda
+    t["ldb"] = k if ldb is None else ldb
+    t["ldc"] = n if ldc is None else ldc
+    return t
+
+
+def test_plan_grouped_gemm_tiles():
+    t = _prob([137, 0, 401, 256, 300], [512, 512, 512, 257, 64], [256, 256, 256, 0, 16])
+    total = _lib.plan_grouped_gemm(t)
+    assert t["tile_begin"].tolist() == [0, 2, 2, 6, 8]   # 1x2, 0, 2x2, 1x2, 2x1 tiles of 256 x 256
+    assert t["tiles_n"].tolist() == [2, 2, 2, 2, 1]
+    assert total == 10
+
+
+def test_plan_grouped_gemm_error_codes():
+    lib = _lib.load()
+    total = ctypes.c_int(0)
+
+    def rc(t):
+        return lib.fp8gmm_plan_grouped_gemm(t.ctypes.data, len(t), ctypes.byref(total))
+
+    assert rc(_prob([16], [16], [24])) == -4            # K not a multiple of 16
+    assert rc(_prob([16], [16], [32], a=0x10008)) == -4  # operand not 16-byte aligned
+    assert rc(_prob([16], [16], [32], lda=40)) == -4     # pitch not a multiple of 16
+    assert rc(_prob([16], [16], [32], lda=16)) == -2     # pitch smaller than k
+    assert rc(_prob([16], [16], [32], c=0)) == -1
+    assert rc(_prob([16], [16], [32], b=0)) == -1
+    assert rc(_prob([-1], [16], [32])) == -2
+    assert rc(_prob([70000], [16], [65536])) == -2      # operand larger than 4 GiB
+    assert rc(_prob([16], [16], [0], a=0, b=0)) == 0     # k == 0 never reads the operands
+    assert rc(_prob([0], [16], [32], a=0, b=0, c=0)) == 0 and total.value == 0
+
+
+def test_launch_entry_points_validate_before_touching_the_gpu():
+    lib = _lib.load()
+    assert lib.fp8gmm_multi_quantize(None, 0, 0, 0, None) == 0          # nothing to do
+    assert lib.fp8gmm_multi_quantize(None, 1, 1, 7, None) == -3         # unknown format
+    assert lib.fp8gmm_multi_quantize(None, 1, 1, 0, None) == -1         # table missing
+    assert lib.fp8gmm_multi_pad_cast_transpose(None, -1, 0, 0, None) == -6
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 1, 1, 2, 0, None) == -3  # e5m2 x e5m2
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 9, 0, None) == -3  # unknown output kind
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 8, None) == -6  # unknown epilogue flag
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 0, None) == -1
+    assert lib.fp8gmm_grouped_gemm(None, 0, 0, 0, 0, 2, 0, None) == 0

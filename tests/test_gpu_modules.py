@@ -205,3 +205,33 @@ def test_grouped_mlp_matches_bf16_autograd(dev):
     assert cos(xd.grad, xr.grad) > 0.99
     assert cos(module.fc1_weight.grad, w1r.grad) > 0.99
     assert cos(module.fc2_weight.grad, w2r.grad) > 0.99
+
+
+@pytest.mark.parametrize("kind", ["linear", "mlp"])
+def test_pad_multiple_does_not_change_results(dev, kind):
+    """Padding of the transposed wgrad operands only appends zeros along the contraction: the reference's
+    multiple (16) and the default here (128) must give bit-identical outputs and gradients."""
+    pkg = _pkg()
+    sizes, h, f = [137, 401, 0, 59, 403], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(3001)
+    x = randn_bf16((m, h), g).to(dev)
+    dy = randn_bf16((m, f if kind == "linear" else h), g, 1e-2).to(dev)
+    w1 = randn_bf16((e, f, h), g, 0.02).to(dev)
+    w2 = randn_bf16((e, h, f), g, 0.02).to(dev)
+    results = []
+    for pad in (16, 128):
+        if kind == "linear":
+            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad)
+            mod.weight_tensor.data.copy_(w1)
+        else:
+            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad)
+            mod.fc1_weight.data.copy_(w1)
+            mod.fc2_weight.data.copy_(w2)
+        xd = x.clone().requires_grad_()
+        with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=1)):
+            out = mod(xd, torch.tensor(sizes))
+        out.backward(dy)
+        results.append([out.detach(), xd.grad] + [p.grad for p in mod.parameters()])
+    for a, b in zip(*results):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))

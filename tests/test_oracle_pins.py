@@ -1,0 +1,281 @@
+"""Pins the CPU oracle to things that do not come from the oracle itself.
+
+The reference ships no golden vectors (its tests compare unseeded random tensors with torch ops
+at atol = rtol = 0.2), so every oracle function is pinned here against an independent source:
+PyTorch's own CPU fp8 / bf16 conversions, torch layout ops, double-precision closed forms, hand
+computed bytes, and algebraic invariants chosen so that a dropped term, a wrong sign or a
+transposed operand fails.
+"""
+import math
+
+import pytest
+import torch
+
+from helpers import REFERENCE_SHAPES, gen, randn_bf16, transpose_shapes
+from oracle import ref
+
+E4M3, E5M2 = torch.float8_e4m3fn, torch.float8_e5m2
+ALL_BF16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------------------------
+# fp32 -> fp8 (saturating RNE)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+@pytest.mark.parametrize("scale", [1.0, 0.5, 3.7, 448.0 / 3.1, 1e-3, 2.0**-10, 1234.5, -1.0, 57344.0 / 0.37, 1e-30])
+def test_cast_every_bf16_pattern_against_torch(dtype, scale):
+    """All 65 536 bf16 patterns times `scale`: clamp(+-max) then torch's own CPU cast."""
+    v = (ALL_BF16.float() * torch.tensor(scale, dtype=torch.float32)).contiguous()
+    mine = ref.f32_to_fp8(v, dtype).view(torch.uint8)
+    mx = ref.FP8_MAX[dtype]
+    theirs = v.clamp(-mx, mx).to(dtype).view(torch.uint8)
+    ok = ~torch.isnan(v)
+    assert torch.equal(mine[ok], theirs[ok])
+    assert set(mine[~ok].tolist()) <= {0x7F}, "every NaN becomes the canonical 0x7F"
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_cast_dense_fp32_against_torch(dtype):
+    g = gen(5)
+    v = torch.randn(2_000_000, generator=g) * torch.exp(torch.randn(2_000_000, generator=g) * 6)
+    mx = ref.FP8_MAX[dtype]
+    assert torch.equal(ref.f32_to_fp8(v, dtype).view(torch.uint8), v.clamp(-mx, mx).to(dtype).view(torch.uint8))
+
+
+HAND_CASES = [
+    # (format, value, expected byte) - worked out by hand from the format definitions
+    (E4M3, 0.0, 0x00), (E4M3, -0.0, 0x80),
+    (E4M3, 448.0, 0x7E), (E4M3, -448.0, 0xFE),            # max finite
+    (E4M3, 449.0, 0x7E), (E4M3, 464.0, 0x7E),              # above max: saturate (464 would tie to the NaN code)
+    (E4M3, 1e30, 0x7E), (E4M3, float("inf"), 0x7E), (E4M3, float("-inf"), 0xFE),
+    (E4M3, float("nan"), 0x7F),
+    (E4M3, 2.0**-9, 0x01),                                   # smallest subnormal
+    (E4M3, 2.0**-10, 0x00),                                  # exactly half of it: tie to even -> 0
+    (E4M3, 1.5 * 2.0**-9, 0x02),                             # tie between 1 and 2 quanta -> even (2)
+    (E4M3, 2.5 * 2.0**-9, 0x02),                             # tie between 2 and 3 -> even (2)
+    (E4M3, 2.0**-6, 0x08),                                   # smallest normal
+    (E4M3, 7.5 * 2.0**-9, 0x08),                             # subnormal that rounds up into the normal range
+    (E4M3, 1.0, 0x38), (E4M3, 1.0625, 0x38), (E4M3, 1.1875, 0x3A),  # ties to even in the normal range
+    (E4M3, 1.9375, 0x40),                                    # mantissa carry into the exponent
+    (E5M2, 57344.0, 0x7B), (E5M2, 60000.0, 0x7B), (E5M2, float("inf"), 0x7B), (E5M2, float("-inf"), 0xFB),
+    (E5M2, float("nan"), 0x7F),
+    (E5M2, 2.0**-16, 0x01), (E5M2, 2.0**-17, 0x00), (E5M2, 1.5 * 2.0**-16, 0x02),
+    (E5M2, 2.0**-14, 0x04), (E5M2, 1.0, 0x3C), (E5M2, 1.125, 0x3C), (E5M2, 1.375, 0x3E), (E5M2, -1.0, 0xBC),
+]
+
+
+@pytest.mark.parametrize("dtype,value,byte", HAND_CASES)
+def test_cast_hand_computed_bytes(dtype, value, byte):
+    got = ref.lib().orc_f32_to_fp8(value, ref.fmt_of(dtype))
+    assert got == byte, f"{value}: 0x{got:02x} != 0x{byte:02x}"
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_dequantise_all_codes_against_torch(dtype):
+    codes = torch.arange(256, dtype=torch.int32).to(torch.uint8).view(dtype)
+    mine, theirs = ref.fp8_to_f32(codes), codes.float()
+    ok = ~torch.isnan(theirs)
+    assert torch.equal(mine[ok].view(torch.int32), theirs[ok].view(torch.int32))
+    assert torch.isnan(mine[~ok]).all()
+    # round trip: every finite code survives cast(dequant(code))
+    finite = torch.isfinite(theirs)
+    back = ref.f32_to_fp8(theirs[finite].contiguous(), dtype).view(torch.uint8)
+    assert torch.equal(back, codes.view(torch.uint8)[finite])
+
+
+def test_bf16_rounding_against_torch():
+    g = gen(6)
+    v = torch.randn(1_000_000, generator=g) * torch.exp(torch.randn(1_000_000, generator=g) * 8)
+    v = torch.cat([v, torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1.00390625, 1.01171875, 3.3895e38])])
+    assert torch.equal(ref.f32_to_bf16(v).view(torch.int16), v.to(torch.bfloat16).view(torch.int16))
+
+
+# ---------------------------------------------------------------------------------------------
+# quantize / amax / layouts against torch ops (the closed forms of fp8_gmm/test.py:43-44,63-68,88-95)
+# ---------------------------------------------------------------------------------------------
+SHAPES = [s for s in REFERENCE_SHAPES if s[0] * s[1] <= 2_000_000] + [(17, 129), (1, 1)]
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_quantize_and_amax_against_torch(dtype):
+    g = gen(7)
+    mx = ref.FP8_MAX[dtype]
+    for shape in SHAPES:
+        x = randn_bf16(shape, g)
+        scale = torch.randn(1, generator=g)
+        out, amax = torch.empty(shape, dtype=dtype), torch.zeros(1)
+        ref.multi_quantize([x], [out], [scale], [amax])
+        expect = (x.float() * scale).clamp(-mx, mx).to(dtype)
+        assert torch.equal(out.view(torch.uint8), expect.view(torch.uint8))
+        assert amax.item() == x.float().abs().max().item()
+
+
+def test_amax_merges_with_previous_content_and_drops_nan():
+    x = torch.tensor([1.0, float("nan"), -3.0, 2.0], dtype=torch.bfloat16)
+    out = torch.empty(4, dtype=E4M3)
+    for prev, expect in [(0.0, 3.0), (2.5, 3.0), (7.0, 7.0)]:
+        amax = torch.tensor([prev])
+        ref.multi_quantize([x], [out], [torch.ones(1)], [amax])
+        assert amax.item() == expect
+    amax = torch.zeros(1)
+    ref.multi_quantize([torch.tensor([float("inf"), 1.0], dtype=torch.bfloat16)], [torch.empty(2, dtype=E4M3)],
+                       [torch.ones(1)], [amax])
+    assert math.isinf(amax.item())
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+@pytest.mark.parametrize("padded", [True, False])
+def test_transpose_layout_against_torch(dtype, padded):
+    g = gen(8)
+    for shape, tshape in zip(SHAPES, transpose_shapes(SHAPES, padded)):
+        x = randn_bf16(shape, g).to(dtype)
+        t = torch.full(tshape, 0x55, dtype=torch.uint8).view(dtype)
+        ref.multi_transpose([x], [t])
+        expect = torch.nn.functional.pad(x.view(torch.uint8).t(), (0, tshape[1] - shape[0]))
+        assert torch.equal(t.view(torch.uint8), expect)
+
+
+@pytest.mark.parametrize("dtype", [E4M3, E5M2])
+def test_cast_transpose_against_torch(dtype):
+    g = gen(9)
+    mx = ref.FP8_MAX[dtype]
+    for shape, tshape in zip(SHAPES, transpose_shapes(SHAPES, True)):
+        for scale_v in (1.7, -0.3):
+            x = randn_bf16(shape, g)
+            scale = torch.tensor([scale_v])
+            out = torch.empty(shape, dtype=dtype)
+            t = torch.full(tshape, 0x55, dtype=torch.uint8).view(dtype)
+            amax = torch.zeros(1)
+            ref.multi_cast_transpose([x], [out], [t], [scale], [amax])
+            y = (x.float() * scale).clamp(-mx, mx).to(dtype).view(torch.uint8)
+            pad_byte = 0x80 if scale_v < 0 else 0x00  # fp8(scale * 0): -0 for a negative scale
+            expect_t = torch.nn.functional.pad(y.t(), (0, tshape[1] - shape[0]), value=pad_byte)
+            assert torch.equal(out.view(torch.uint8), y)
+            assert torch.equal(t.view(torch.uint8), expect_t)
+            assert amax.item() == x.float().abs().max().item()
+
+
+def test_transpose_brute_force_tiny():
+    x = torch.arange(6, dtype=torch.uint8).reshape(2, 3).view(E4M3)
+    t = torch.full((3, 4), 0x55, dtype=torch.uint8).view(E4M3)
+    ref.multi_transpose([x], [t])
+    assert t.view(torch.uint8).tolist() == [[0, 3, 0, 0], [1, 4, 0, 0], [2, 5, 0, 0]]
+
+
+# ---------------------------------------------------------------------------------------------
+# tanh / GELU / dGELU against double-precision closed forms
+# ---------------------------------------------------------------------------------------------
+def test_tanh_error_bound():
+    u = torch.linspace(-12, 12, 1_000_001)
+    err = (ref.tanh(u).double() - torch.tanh(u.double())).abs().max().item()
+    assert err < 2e-7
+    special = ref.tanh(torch.tensor([0.0, -0.0, float("inf"), float("-inf"), 1e-20, -1e-20]))
+    assert special.tolist()[:4] == [0.0, -0.0, 1.0, -1.0] and abs(special[4]) < 1e-7
+    assert math.copysign(1.0, special[1].item()) == -1.0
+    assert torch.isnan(ref.tanh(torch.tensor([float("nan")]))).all()
+
+
+def test_dgelu_is_the_derivative_of_tanh_gelu():
+    """Closed form of fp8_gmm/test.py:32-34 in double, and a central difference of the GELU itself."""
+    c = torch.linspace(-8, 8, 400_001)
+    cd = c.double()
+    k = 0.79788456
+    th = torch.tanh(k * cd * (1 + 0.044715 * cd * cd))
+    closed = 0.5 * cd * ((1 - th * th) * (k + 0.1070322243 * cd * cd)) + 0.5 * (1 + th)
+    assert (ref.dgelu(c).double() - closed).abs().max().item() < 3e-6
+
+    def gelu64(x):
+        return 0.5 * x * (1 + torch.tanh(math.sqrt(2 / math.pi) * (x + 0.044715 * x**3)))
+
+    h = 1e-5
+    numeric = (gelu64(cd + h) - gelu64(cd - h)) / (2 * h)
+    assert (ref.dgelu(c).double() - numeric).abs().max().item() < 1e-5
+
+
+def test_gelu_matches_torch_tanh_gelu():
+    v = torch.linspace(-10, 10, 400_001)
+    mine = ref.gelu(v).double()
+    theirs = torch.nn.functional.gelu(v.double(), approximate="tanh")
+    assert (mine - theirs).abs().max().item() < 2e-6
+
+
+def test_dgelu_kernel_restatement():
+    """x = dy * dgelu(pre), amax over |x| of the unscaled product, pad byte from the scale sign."""
+    g = gen(10)
+    dy, pre = randn_bf16((37, 24), g), randn_bf16((37, 24), g, 2.0)
+    scale = torch.tensor([3.0])
+    out, t, amax = torch.empty(37, 24, dtype=E5M2), torch.empty(24, 48, dtype=E5M2), torch.zeros(1)
+    ref.multi_cast_transpose_dgelu([dy], [pre], [out], [t], [scale], [amax])
+    x = dy.float() * ref.dgelu(pre.float().contiguous())
+    assert torch.equal(out.view(torch.uint8), ref.f32_to_fp8((x * scale).contiguous(), E5M2).view(torch.uint8))
+    assert amax.item() == x.abs().max().item()
+    assert torch.equal(t.view(torch.uint8)[:, :37], out.view(torch.uint8).t())
+    assert not t.view(torch.uint8)[:, 37:].any()
+
+
+# ---------------------------------------------------------------------------------------------
+# GEMM
+# ---------------------------------------------------------------------------------------------
+def _q(x, dtype):
+    return ref.f32_to_fp8(x.float().contiguous(), dtype)
+
+
+def test_gemm_naive_against_torch_float64():
+    g = gen(11)
+    a, b = _q(randn_bf16((33, 48), g), E5M2), _q(randn_bf16((21, 48), g), E4M3)
+    expect = a.float().double() @ b.float().double().t()
+    assert torch.allclose(ref.gemm_acc_naive(a, b).double(), expect, rtol=1e-6, atol=1e-6)
+    assert torch.allclose(ref.gemm_acc(a, b).double(), expect, rtol=1e-5, atol=1e-5)
+    # a transposed operand or swapped roles would change the shape or the values
+    assert ref.gemm_acc_naive(a, b).shape == (33, 21)
+    assert not torch.allclose(ref.gemm_acc_naive(a, b)[:21, :21], ref.gemm_acc_naive(b, a[:21])[:21, :21].contiguous())
+
+
+def test_gemm_identity_and_power_of_two_exactness():
+    g = gen(12)
+    a = _q(randn_bf16((40, 64), g), E4M3)
+    eye = _q(torch.eye(64), E4M3)
+    assert torch.equal(ref.gemm_acc_naive(a, eye), ref.fp8_to_f32(a))
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
+    p = _q(vals[torch.randint(0, 8, (16, 32), generator=g)], E4M3)
+    q = _q(vals[torch.randint(0, 8, (8, 32), generator=g)], E4M3)
+    c = torch.empty(16, 8, dtype=torch.bfloat16)
+    ref.cublas_fp8_gemm(p, q, c, torch.tensor(0.5), torch.tensor(4.0), naive=True)
+    exact = (p.float() @ q.float().t()) * 2.0
+    assert torch.equal(c.float(), exact.to(torch.bfloat16).float())
+
+
+def test_grouped_gemm_is_the_per_expert_loop():
+    """fp8_gmm/test.py:209-214: expert i multiplies its row block with its own weight."""
+    g = gen(13)
+    sizes = [5, 0, 17, 3]
+    a, b = _q(randn_bf16((25, 32), g), E4M3), _q(randn_bf16((4, 16, 32), g), E4M3)
+    sa = [torch.tensor(0.5 + i) for i in range(4)]
+    sb = [torch.tensor(1.0 / (1 + i)) for i in range(4)]
+    c = ref.fp8_gmm(a, b, sizes, sa, sb)
+    start = 0
+    for i, s in enumerate(sizes):
+        expect = (a[start: start + s].float() @ b[i].float().t()) * (sa[i] * sb[i])
+        assert torch.equal(c[start: start + s].float(), expect.to(torch.bfloat16).float())
+        start += s
+
+
+def test_gelu_epilogue_definition():
+    g = gen(14)
+    a, b = _q(randn_bf16((9, 32), g), E4M3), _q(randn_bf16((7, 32), g), E4M3)
+    c, pre, amax = torch.empty(9, 7, dtype=E4M3), torch.empty(9, 7, dtype=torch.bfloat16), torch.zeros(1)
+    ref.cublas_fp8_gemm(a, b, c, torch.tensor(0.25), torch.tensor(2.0), pre, torch.tensor([3.0]), amax)
+    v = (a.float() @ b.float().t()) * 0.5
+    gl = ref.gelu(v.contiguous())
+    assert torch.equal(pre.float(), v.to(torch.bfloat16).float())
+    assert torch.equal(c.view(torch.uint8), ref.f32_to_fp8((gl * 3.0).contiguous(), E4M3).view(torch.uint8))
+    assert amax.item() == gl.abs().max().item()
+
+
+def test_scale_mul_is_left_to_right():
+    x = torch.tensor([1.0, -2.5, 3.1415], dtype=torch.bfloat16)
+    s1, s2 = torch.tensor([1e-20]), torch.tensor([1e20])
+    y = x.clone()
+    ref.multi_scale_mul([y], [s1], [s2])
+    expect = ((x.float() * s1) * s2).to(torch.bfloat16)
+    assert torch.equal(y.view(torch.int16), expect.view(torch.int16))
