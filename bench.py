@@ -62,6 +62,9 @@ def main():
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip per-kernel HIP events (pure wall time)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy (reads 256 MiB, writes 256 MiB) so that hardware "
+                         "byte counters collected around this command can be scaled against a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
@@ -100,6 +103,12 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     timing = None
     if args.no_kernel_events:
         t0 = time.perf_counter()
