@@ -86,6 +86,25 @@ __device__ __forceinline__ void global_store(void* p, T v) {
   *reinterpret_cast<__attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)) = v;
 }
 
+// Raw buffer descriptors: offsets past `bytes` read as zero and are dropped on store, so the fast paths
+// of the HBM-bound kernels need no per-lane branches and can issue all their loads back to back.
+constexpr uint32_t kOobOffset = 0xffffffffu;
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ u32x4 buf_load16(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, (int)off, 0, 0);
+}
+__device__ __forceinline__ u32x2 buf_load8(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+  return __builtin_amdgcn_raw_buffer_load_b64(r, (int)off, 0, 0);
+}
+__device__ __forceinline__ void buf_store16(u32x4 v, __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, 0);
+}
+__device__ __forceinline__ void buf_store8(u32x2 v, __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  __builtin_amdgcn_raw_buffer_store_b64(v, r, (int)off, 0, 0);
+}
+
 // max(acc, |x|) that never lets a NaN in (fmaxf semantics of the reference's amax).
 // A compare + select, not v_max_f32: in IEEE mode the hardware max returns a NaN when an
 // input is a signalling NaN (bf16 data can carry such patterns), which would erase `acc`.
@@ -119,7 +138,9 @@ __device__ __forceinline__ void block_amax_merge(float local, float* amax, float
     float m = stage[0];
 #pragma unroll
     for (int i = 1; i < NWAVES; ++i) m = fmaxf(m, stage[i]);
-    if (amax != nullptr && m > 0.f) atomic_max_nonneg(amax, m);
+    // amax only grows, so a value already at or above m (even a stale one) makes the atomic redundant;
+    // this keeps thousands of workgroups from queueing on one address.
+    if (amax != nullptr && m > 0.f && !(__builtin_nontemporal_load(amax) >= m)) atomic_max_nonneg(amax, m);
   }
 }
 

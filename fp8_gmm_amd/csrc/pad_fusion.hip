@@ -89,9 +89,70 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
   }
   const bool vec_t = (mpad % 16) == 0 && (reinterpret_cast<uintptr_t>(out_t) & 15) == 0;
 
+  // Descriptor path: every offset of the tensor fits 32 bits, so rows past m and columns past ncols become
+  // out-of-range buffer offsets (loads return zero = the padding value, stores are dropped) and all loads
+  // of the lane are issued back to back without a branch.
+  constexpr int kInBytes = OP == OP_TRANSPOSE ? 1 : 2;
+  const bool fast = vec_in && vec_t && (int64_t)m * ncols * kInBytes < (int64_t)0xffffffff &&
+                    (int64_t)ncols * mpad < (int64_t)0xffffffff;
+
   float mx = 0.f;
   uint32_t y[RPT][2];  // fp8 bytes of 8 rows x 8 columns; y[i][h] byte q = column 4 h + q of row i
 
+  if (fast) {
+    const uint32_t in_bytes = (uint32_t)((int64_t)m * ncols * kInBytes);
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(d.in, in_bytes);
+    uint32_t eoff[RPT];  // element offset of the lane's 8 columns in row i, or out of range
+#pragma unroll
+    for (int i = 0; i < RPT; ++i) {
+      const int row = r0 + RPT * rg + i;
+      eoff[i] = (row < m && col < ncols) ? (uint32_t)row * (uint32_t)ncols + (uint32_t)col : kOobOffset;
+    }
+    if constexpr (OP == OP_TRANSPOSE) {
+      u32x2 v[RPT];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) v[i] = buf_load8(rin, eoff[i]);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        y[i][0] = v[i].x;
+        y[i][1] = v[i].y;
+      }
+    } else {
+      u32x4 xa[RPT];
+      u32x4 ga[OP == OP_CAST_DGELU ? RPT : 1];
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) xa[i] = buf_load16(rin, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
+      if constexpr (OP == OP_CAST_DGELU) {
+        const __amdgpu_buffer_rsrc_t rpre = make_rsrc(d.in2, in_bytes);
+#pragma unroll
+        for (int i = 0; i < RPT; ++i) ga[i] = buf_load16(rpre, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
+      }
+      const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out != nullptr ? in_bytes / 2 : 0u);
+#pragma unroll
+      for (int i = 0; i < RPT; ++i) {
+        const uint32_t w[4] = {xa[i].x, xa[i].y, xa[i].z, xa[i].w};
+        float x[CPT];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          x[2 * q] = bf16_lo_to_f32(w[q]);
+          x[2 * q + 1] = bf16_hi_to_f32(w[q]);
+        }
+        if constexpr (OP == OP_CAST_DGELU) {
+          const uint32_t g[4] = {ga[i].x, ga[i].y, ga[i].z, ga[i].w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            x[2 * q] *= dgelu(bf16_lo_to_f32(g[q]));
+            x[2 * q + 1] *= dgelu(bf16_hi_to_f32(g[q]));
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < CPT; ++e) mx = amax_step(mx, x[e]);
+        y[i][0] = cvt4_fp8<FMT>(scale * x[0], scale * x[1], scale * x[2], scale * x[3]);
+        y[i][1] = cvt4_fp8<FMT>(scale * x[4], scale * x[5], scale * x[6], scale * x[7]);
+        buf_store8(u32x2{y[i][0], y[i][1]}, rout, eoff[i]);
+      }
+    }
+  } else {
 #pragma unroll
   for (int i = 0; i < RPT; ++i) {
     const int row = r0 + RPT * rg + i;
@@ -100,13 +161,9 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
     if constexpr (OP == OP_TRANSPOSE) {
       u32x2 v = {0u, 0u};
       if (row_ok) {
-        if (vec_in) {
-          if (col < ncols) v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(in8 + off));
-        } else {
 #pragma unroll
-          for (int e = 0; e < CPT; ++e)
-            if (col + e < ncols) v[e >> 2] |= (uint32_t)in8[off + e] << (8 * (e & 3));
-        }
+        for (int e = 0; e < CPT; ++e)
+          if (col + e < ncols) v[e >> 2] |= (uint32_t)in8[off + e] << (8 * (e & 3));
       }
       y[i][0] = v.x;
       y[i][1] = v.y;
@@ -115,28 +172,11 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
 #pragma unroll
       for (int e = 0; e < CPT; ++e) x[e] = 0.f;
       if (row_ok) {
-        if (vec_in) {
-          if (col < ncols) {
-            const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in16 + off));
-            x[0] = bf16_lo_to_f32(a.x); x[1] = bf16_hi_to_f32(a.x);
-            x[2] = bf16_lo_to_f32(a.y); x[3] = bf16_hi_to_f32(a.y);
-            x[4] = bf16_lo_to_f32(a.z); x[5] = bf16_hi_to_f32(a.z);
-            x[6] = bf16_lo_to_f32(a.w); x[7] = bf16_hi_to_f32(a.w);
-            if constexpr (OP == OP_CAST_DGELU) {
-              const u32x4 g = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(pre16 + off));
-              x[0] *= dgelu(bf16_lo_to_f32(g.x)); x[1] *= dgelu(bf16_hi_to_f32(g.x));
-              x[2] *= dgelu(bf16_lo_to_f32(g.y)); x[3] *= dgelu(bf16_hi_to_f32(g.y));
-              x[4] *= dgelu(bf16_lo_to_f32(g.z)); x[5] *= dgelu(bf16_hi_to_f32(g.z));
-              x[6] *= dgelu(bf16_lo_to_f32(g.w)); x[7] *= dgelu(bf16_hi_to_f32(g.w));
-            }
-          }
-        } else {
 #pragma unroll
-          for (int e = 0; e < CPT; ++e) {
-            if (col + e < ncols) {
-              x[e] = bf16_to_f32(in16[off + e]);
-              if constexpr (OP == OP_CAST_DGELU) x[e] *= dgelu(bf16_to_f32(pre16[off + e]));
-            }
+        for (int e = 0; e < CPT; ++e) {
+          if (col + e < ncols) {
+            x[e] = bf16_to_f32(in16[off + e]);
+            if constexpr (OP == OP_CAST_DGELU) x[e] *= dgelu(bf16_to_f32(pre16[off + e]));
           }
         }
       }
@@ -145,18 +185,12 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
       y[i][0] = cvt4_fp8<FMT>(scale * x[0], scale * x[1], scale * x[2], scale * x[3]);
       y[i][1] = cvt4_fp8<FMT>(scale * x[4], scale * x[5], scale * x[6], scale * x[7]);
       if (out != nullptr && row_ok) {
-        if (vec_in) {
-          if (col < ncols) {
-            const u32x2 o = {y[i][0], y[i][1]};
-            __builtin_nontemporal_store(o, reinterpret_cast<u32x2*>(out + off));
-          }
-        } else {
 #pragma unroll
-          for (int e = 0; e < CPT; ++e)
-            if (col + e < ncols) out[off + e] = (uint8_t)(y[i][e >> 2] >> (8 * (e & 3)));
-        }
+        for (int e = 0; e < CPT; ++e)
+          if (col + e < ncols) out[off + e] = (uint8_t)(y[i][e >> 2] >> (8 * (e & 3)));
       }
     }
+  }
   }
 
   // ---- 8 x 8 byte transpose in registers, then to the LDS tile ----
@@ -179,6 +213,7 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
   __syncthreads();
 
   // ---- LDS tile -> transposed output: 16 token rows of one column per lane and step ----
+  const __amdgpu_buffer_rsrc_t rt = make_rsrc(out_t, fast ? (uint32_t)((int64_t)ncols * mpad) : 0u);
 #pragma unroll
   for (int q = 0; q < (TN * TM / 16) / kPtThreads; ++q) {
     const int p = tid + kPtThreads * q;
@@ -190,10 +225,13 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
     if (f & 1) v = u32x4{v.z, v.w, v.x, v.y};   // odd swizzle: the two granules are swapped inside the slot
     const int gcol = c0 + j;
     const int grow = r0 + 16 * piece;
-    if (gcol < ncols && grow < mpad) {
+    const bool ok = gcol < ncols && grow < mpad;
+    if (fast) {
+      buf_store16(v, rt, ok ? (uint32_t)gcol * (uint32_t)mpad + (uint32_t)grow : kOobOffset);
+    } else if (ok) {
       uint8_t* dst = out_t + (int64_t)gcol * mpad + grow;
       if (vec_t) {
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(dst));
+        global_store(dst, v);
       } else {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll

@@ -4,8 +4,8 @@
 //
 // Replaces csrc/multi_pointwise.cu of the reference (multi_quantize_kernel :34-97,
 // multi_scale_mul_kernel :99-151).  HBM-bound: 2 B read + 1 B written per element
-// (quantize), 2 B + 2 B (scale_mul); every lane moves 32 bytes in and 16 bytes out per
-// step with 128-bit accesses, the wave reduces amax with cross-lane shuffles and the
+// (quantize), 2 B + 2 B (scale_mul); a wavefront reads 1 KB of contiguous bf16 per step
+// (one 128-bit load per lane, all steps issued before the first conversion), the wave reduces amax with cross-lane shuffles and the
 // workgroup issues a single integer atomic max.
 #include "device_utils.h"
 #include "tiling.h"
@@ -25,33 +25,55 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(const fp8gmm
   const uint16_t* __restrict__ in = static_cast<const uint16_t*>(d.in);
   uint8_t* __restrict__ out = static_cast<uint8_t*>(d.out);
   const float scale = d.scale ? *d.scale : 1.f;
-  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+                   numel * 2 < (int64_t)0xffffffff;
   float mx = 0.f;
 
+  if (vec) {
+    // fast path: all loads of the workgroup's 16384 elements are issued before the first conversion
+    const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, (uint32_t)(numel * 2));
+    const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, (uint32_t)numel);
+    u32x4 a[kPwSteps];
+    bool full[kPwSteps];
 #pragma unroll
-  for (int it = 0; it < kPwSteps; ++it) {
-    const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
-    if (vec && off + kPwVec <= numel) {
-      const u32x4 a = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + off));
-      const u32x4 b = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + off + 8));
-      const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-      uint32_t o[4];
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      full[it] = off + kPwVec <= numel;
+      a[it] = buf_load16(rin, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+    }
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      const uint32_t w[4] = {a[it].x, a[it].y, a[it].z, a[it].w};
+      uint32_t o[2];
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
         const float x0 = bf16_lo_to_f32(w[2 * q]), x1 = bf16_hi_to_f32(w[2 * q]);
         const float x2 = bf16_lo_to_f32(w[2 * q + 1]), x3 = bf16_hi_to_f32(w[2 * q + 1]);
         mx = amax_step(amax_step(mx, x0), x1);
         mx = amax_step(amax_step(mx, x2), x3);
         o[q] = cvt4_fp8<FMT>(x0 * scale, x1 * scale, x2 * scale, x3 * scale);
       }
-      const u32x4 ov = {o[0], o[1], o[2], o[3]};
-      __builtin_nontemporal_store(ov, reinterpret_cast<u32x4*>(out + off));
-    } else if (off < numel) {
-      const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
-      for (int j = 0; j < cnt; ++j) {
-        const float x = bf16_to_f32(in[off + j]);
-        mx = amax_step(mx, x);
-        out[off + j] = cvt1_fp8<FMT>(x * scale);
+      buf_store8(u32x2{o[0], o[1]}, rout, full[it] ? (uint32_t)off : kOobOffset);
+      if (!full[it] && off < numel) {  // the one partial group at the end of the tensor
+        for (int64_t j = off; j < numel; ++j) {
+          const float x = bf16_to_f32(in[j]);
+          mx = amax_step(mx, x);
+          out[j] = cvt1_fp8<FMT>(x * scale);
+        }
+      }
+    }
+  } else {
+#pragma unroll 1
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      if (off < numel) {
+        const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
+        for (int j = 0; j < cnt; ++j) {
+          const float x = bf16_to_f32(in[off + j]);
+          mx = amax_step(mx, x);
+          out[off + j] = cvt1_fp8<FMT>(x * scale);
+        }
       }
     }
   }
@@ -70,29 +92,42 @@ __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gm
   const float s1 = d.scale ? *d.scale : 1.f;
   const float* s2p = static_cast<const float*>(d.in2);
   const float s2 = s2p ? *s2p : 1.f;
-  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && numel * 2 < (int64_t)0xffffffff;
 
+  if (vec) {
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, (uint32_t)(numel * 2));
+    u32x4 a[kPwSteps];
+    bool full[kPwSteps];
 #pragma unroll
-  for (int it = 0; it < kPwSteps; ++it) {
-    const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
-    if (vec && off + kPwVec <= numel) {
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      full[it] = off + kPwVec <= numel;
+      a[it] = buf_load16(rx, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+    }
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        u32x4 a = *reinterpret_cast<const u32x4*>(x + off + 8 * h);
-        uint32_t w[4] = {a.x, a.y, a.z, a.w};
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      uint32_t w[4] = {a[it].x, a[it].y, a[it].z, a[it].w};
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          // left to right, as the reference: (x * s1) * s2
-          const float lo = bf16_lo_to_f32(w[q]) * s1 * s2;
-          const float hi = bf16_hi_to_f32(w[q]) * s1 * s2;
-          w[q] = pack_bf16x2(lo, hi);
-        }
-        const u32x4 o = {w[0], w[1], w[2], w[3]};
-        *reinterpret_cast<u32x4*>(x + off + 8 * h) = o;
+      for (int q = 0; q < 4; ++q) {
+        // left to right, as the reference: (x * s1) * s2
+        const float lo = bf16_lo_to_f32(w[q]) * s1 * s2;
+        const float hi = bf16_hi_to_f32(w[q]) * s1 * s2;
+        w[q] = pack_bf16x2(lo, hi);
       }
-    } else if (off < numel) {
-      const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
-      for (int j = 0; j < cnt; ++j) x[off + j] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(x[off + j]) * s1 * s2);
+      buf_store16(u32x4{w[0], w[1], w[2], w[3]}, rx, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+      if (!full[it] && off < numel) {
+        for (int64_t j = off; j < numel; ++j) x[j] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(x[j]) * s1 * s2);
+      }
+    }
+  } else {
+#pragma unroll 1
+    for (int it = 0; it < kPwSteps; ++it) {
+      const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
+      if (off < numel) {
+        const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
+        for (int j = 0; j < cnt; ++j) x[off + j] = (uint16_t)f32_to_bf16_bits(bf16_to_f32(x[off + j]) * s1 * s2);
+      }
     }
   }
 }

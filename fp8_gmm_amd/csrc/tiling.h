@@ -5,8 +5,8 @@ namespace fp8gmm {
 
 // ---- element-wise kernels (quantize, scale_mul) ----
 constexpr int kPwThreads = 256;                  // 4 wavefronts
-constexpr int kPwVec = 16;                       // elements per thread per step
-constexpr int kPwSteps = 4;                      // steps per workgroup
+constexpr int kPwVec = 8;                        // elements per thread per step (one 16-byte bf16 load)
+constexpr int kPwSteps = 8;                      // steps per workgroup
 constexpr int kPwBlockElems = kPwThreads * kPwVec * kPwSteps;  // 16384 elements per workgroup
 
 // ---- pad / cast / transpose kernels ----
