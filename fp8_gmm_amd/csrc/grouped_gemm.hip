@@ -282,8 +282,15 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 
     for (int kt = 0; kt < g.nk; ++kt) {
       const int h1 = ring_inc(hs), h2 = ring_inc(h1);
+      const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
+      const int free_hi = hs;                                         // will hold half-step + 5
+      // The pair for half-steps + 4 / + 5 is fetched in four quarters spread over both half-steps (token
+      // rows in the even one, weight rows in the odd one, one quarter every fourth MFMA).  Issued in one
+      // burst, the 64 KB of a pair keep the texture-address unit busy for about a thousand cycles and every
+      // wavefront queues behind it with its MFMAs.
       // ---- even half-step: its fragments are in fa0 / fb0.  The barrier proves that every wavefront has
-      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed.
+      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed
+      // (everything but the newest pair: 4 token-row + 4 weight-row loads).
       if (relaxed > 0) {
         FP8GMM_WAIT_VM_LGKM(kPairLoads + kFastStores);
         --relaxed;
@@ -292,54 +299,51 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       }
       __builtin_amdgcn_s_barrier();
       {
-        const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
-        const int free_hi = hs;                                         // will hold half-step + 5
         const uint8_t* qa = lds + h1 * HS + fa_off;
         const uint8_t* qb = lds + h1 * HS + fb_off;
         FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
         dma_part(free_lo, free_hi, 0);
         FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 1);
-        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 2);
-        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 3);
-        dma_advance();
-        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
         read_frag(fb1[0], qb);
         read_frag(fb1[1], qb + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_MF0(1, 1); FP8GMM_SB();
         read_frag(fa1[0], qa);
         read_frag(fa1[1], qa + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 1);
+        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
         read_frag(fa1[2], qa + 64 * HK);
         read_frag(fa1[3], qa + 96 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(3, 1); FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_MF0(3, 1); FP8GMM_SB();
       }
-      // ---- odd half-step: fragments in fa1 / fb1; fetch the next even step's fragments early so that
-      // they have arrived long before the next barrier asks for lgkmcnt(0).
+      // ---- odd half-step: fragments in fa1 / fb1.  Half-step + 2 sits in the low half of the pair whose
+      // weight rows were issued one half-step ago; only the 4 token-row loads of the newest pair may still
+      // be in flight.
       if (relaxed > 0) {
-        FP8GMM_WAIT_VM(kPairLoads + kFastStores);
+        FP8GMM_WAIT_VM(kPairLoads / 2 + kFastStores);
         --relaxed;
       } else {
-        FP8GMM_WAIT_VM(kPairLoads);
+        FP8GMM_WAIT_VM(kPairLoads / 2);
       }
       __builtin_amdgcn_s_barrier();
       {
         const uint8_t* qa = lds + h2 * HS + fa_off;
         const uint8_t* qb = lds + h2 * HS + fb_off;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 2);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
         read_frag(fb0[0], qb);
         read_frag(fb0[1], qb + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_MF1(1, 1); FP8GMM_SB();
         read_frag(fa0[0], qa);
         read_frag(fa0[1], qa + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 3);
+        dma_advance();
+        FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
         read_frag(fa0[2], qa + 64 * HK);
         read_frag(fa0[3], qa + 96 * HK);
-        FP8GMM_SB();
-        FP8GMM_MF1(1, 1); FP8GMM_MF1(2, 0); FP8GMM_MF1(2, 1); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1);
-        FP8GMM_SB();
+        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1); FP8GMM_SB();
       }
       hs = h2;
     }
