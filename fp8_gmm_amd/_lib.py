@@ -78,6 +78,8 @@ EXPORTS = (
     "fp8gmm_multi_pad_cast_transpose",
     "fp8gmm_multi_pad_cast_transpose_dgelu",
     "fp8gmm_grouped_gemm",
+    "fp8gmm_gemm_schedule",
+    "fp8gmm_gemm_fixup",
 )
 
 
@@ -130,6 +132,10 @@ def load():
     L.fp8gmm_multi_pad_cast_transpose_dgelu.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_grouped_gemm.restype = ci
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
+    L.fp8gmm_gemm_schedule.restype = ci
+    L.fp8gmm_gemm_schedule.argtypes = [vp, ci, ci, ci, ci, ci, vp, ci]
+    L.fp8gmm_gemm_fixup.restype = ci
+    L.fp8gmm_gemm_fixup.argtypes = [vp, ci, ci, ci, ci, ip, vp, ci]
     if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize:
         raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
     _lib = L
@@ -152,6 +158,29 @@ def plan_grouped_gemm(table):
     total = ctypes.c_int(0)
     check(load().fp8gmm_plan_grouped_gemm(table.ctypes.data, len(table), ctypes.byref(total)))
     return total.value
+
+
+def gemm_schedule(table, total_tiles, grid, stream_k, wg, max_items=4096):
+    """Items (tile, problem, m0, n0, k_begin, nk, slot) that workgroup `wg` of a `grid`-workgroup launch processes."""
+    buf = np.zeros((max_items, 7), dtype=np.int32)
+    n = load().fp8gmm_gemm_schedule(table.ctypes.data, len(table), total_tiles, grid, int(stream_k), wg,
+                                    buf.ctypes.data, max_items)
+    if n < 0:
+        check(n)
+    if n > max_items:
+        return gemm_schedule(table, total_tiles, grid, stream_k, wg, n)
+    return buf[:n]
+
+
+def gemm_fixup(table, total_tiles, grid, wg, max_slots=64):
+    """(tile, [slots in K order]) that fix-up workgroup `wg` completes; tile == -1: nothing to do."""
+    tile = ctypes.c_int(-1)
+    buf = np.zeros(max_slots, dtype=np.int32)
+    n = load().fp8gmm_gemm_fixup(table.ctypes.data, len(table), total_tiles, grid, wg, ctypes.byref(tile),
+                                 buf.ctypes.data, max_slots)
+    if n < 0:
+        check(n)
+    return tile.value, buf[:min(n, max_slots)].tolist()
 
 
 def gemm_tile_shape():

@@ -194,12 +194,10 @@ __device__ __forceinline__ float gelu_tanh(float v) {
 // check anyway, so nothing here has to be bit-reproducible; the dGELU kernel, which is compared
 // byte for byte, keeps det_tanh.
 __device__ __forceinline__ float gelu_tanh_fast(float v) {
-  const float v2 = v * v;
-  float u = (0.79788456f * v) * __builtin_fmaf(0.044715f, v2, 1.0f);
-  u = fminf(fmaxf(u, -10.f), 10.f);
-  const float e = __builtin_amdgcn_exp2f(u * 2.8853900817779268f);  // exp(2u)
-  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
-  return (0.5f * v) * (1.0f + t);
+  // 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)), u = 0.79788456 (v + 0.044715 v^3); constants carry 2 log2(e).
+  const float p = __builtin_fmaf(v * v, 0.10294324f, 2.3022082f);
+  const float e = __builtin_amdgcn_exp2f(-v * p);  // exp(-2u); inf for very negative v -> result -0
+  return v * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // Index of the last entry of a sorted device table whose key (read by `key(i)`) is <= x.

@@ -1,0 +1,224 @@
+// Work decomposition of the grouped GEMM: which (tile, K range) items a workgroup processes, in which
+// order, and which workgroup completes a tile that several workgroups shared along K.  Pure integer
+// arithmetic on the problem table, compiled for the device (the kernels) and for the host (the
+// introspection entry point the CPU tests use), so both see exactly the same schedule.
+#pragma once
+
+#include <stdint.h>
+
+#include "fp8gmm.h"
+#include "tiling.h"
+
+#if defined(__HIPCC__)
+#define FP8GMM_HD __host__ __device__ inline __attribute__((always_inline))
+#else
+#define FP8GMM_HD inline
+#endif
+
+namespace fp8gmm {
+
+constexpr int BM = kGemmTileM;  // 256
+constexpr int BN = kGemmTileN;  // 256
+constexpr int kNumXcd = 8;
+
+// ---- tail balancing (stream-K over the remainder of an XCD's tile range) ----
+// A range of n tiles on W workgroups takes ceil(n / W) rounds; when the last round is mostly empty the
+// remainder tiles (plus one full round when there are very few of them) are cut along K instead: the
+// region's K = 128 pair steps are dealt out in W equal contiguous pieces.  A piece that does not cover
+// a whole tile leaves its fp32 accumulators in a workspace slot; a second, small kernel adds the pieces
+// of such a tile in K order and runs the normal epilogue.  No workgroup ever waits for another one.
+constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many pair steps
+constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
+constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
+constexpr int kPartialBytes = BM * BN * 4;  // one slot: the 128 accumulators of the 512 lanes
+constexpr int kSlotsPerWg = 2;        // a piece that starts inside a tile, one that ends inside a tile
+
+struct Sched {
+  const fp8gmm_gemm_problem* probs;
+  int nprob, total_tiles;
+  int wgs;                     // workgroups per XCD
+  int range_begin, range_end;  // tiles of this XCD
+  int dp_rounds;               // workgroup j takes tiles range_begin + j + wgs * i, i < dp_rounds
+  int sk_begin;                // first tile of the stream-K region (== range_end: none)
+  int sk_wgs;                  // workgroups that take a piece of the region
+  int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (pair steps)
+};
+
+FP8GMM_HD int problem_end_tile(const Sched& s, int p) {
+  return (p + 1 < s.nprob) ? s.probs[p + 1].tile_begin : s.total_tiles;
+}
+// last problem whose first tile is <= tile
+FP8GMM_HD int problem_of_tile(const Sched& s, int tile) {
+  int lo = 0, hi = s.nprob - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (s.probs[mid].tile_begin <= tile) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+// A tile of problem p costs ceil(k / 128) pair steps (1 for k = 0: its epilogue still has to run).
+FP8GMM_HD int64_t tile_cost(const Sched& s, int p) {
+  const int c = (s.probs[p].k + 127) / 128;
+  return (int64_t)(c > 0 ? c : 1);
+}
+// cost of all tiles before `tile`
+FP8GMM_HD int64_t cost_before(const Sched& s, int tile) {
+  int64_t cum = 0;
+  for (int p = 0; p < s.nprob; ++p) {
+    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
+    if (tile <= t_begin) break;
+    cum += (int64_t)((tile < t_end ? tile : t_end) - t_begin) * tile_cost(s, p);
+  }
+  return cum;
+}
+// first tile whose preceding cost is >= c (total_tiles if there is none)
+FP8GMM_HD int first_tile_at_cost(const Sched& s, int64_t c) {
+  int64_t cum = 0;
+  for (int p = 0; p < s.nprob; ++p) {
+    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
+    const int64_t tc = tile_cost(s, p), n_t = t_end - t_begin;
+    if (cum + n_t * tc > c - tc) {  // some tile i of p has cum + i tc >= c
+      const int64_t i = c > cum ? (c - cum + tc - 1) / tc : 0;
+      if (i < n_t) return t_begin + (int)i;
+    }
+    cum += n_t * tc;
+  }
+  return s.total_tiles;
+}
+// the tile that holds cost offset c: cost_before(t) <= c < cost_before(t + 1)
+FP8GMM_HD int tile_holding_cost(const Sched& s, int64_t c) {
+  int64_t cum = 0;
+  for (int p = 0; p < s.nprob; ++p) {
+    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
+    const int64_t tc = tile_cost(s, p), n_t = t_end - t_begin;
+    if (c < cum + n_t * tc) return t_begin + (int)((c - cum) / tc);
+    cum += n_t * tc;
+  }
+  return s.total_tiles;
+}
+
+// Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal COST (k differs
+// per problem in the wgrad form), one per XCD, so that workgroups that share an L2 work on neighbouring
+// tiles; the workgroups of an XCD stride through the range, and share its remainder along K when that pays.
+FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob, int total_tiles,
+                                           int xcd, int wgs_per_xcd, bool sk_enable) {
+  s.probs = probs;
+  s.nprob = nprob;
+  s.total_tiles = total_tiles;
+  s.wgs = wgs_per_xcd;
+  const int64_t total_cost = cost_before(s, total_tiles);
+  const int64_t lo = (total_cost * xcd + kNumXcd - 1) / kNumXcd;
+  const int64_t hi = (total_cost * (xcd + 1) + kNumXcd - 1) / kNumXcd;
+  s.range_begin = first_tile_at_cost(s, lo);
+  s.range_end = first_tile_at_cost(s, hi);
+  const int n_x = s.range_end - s.range_begin;
+  const int W = wgs_per_xcd;
+  s.dp_rounds = (n_x + W - 1) / W;  // plain striding: the last round may be partial
+  s.sk_begin = s.range_end;
+  s.sk_wgs = 0;
+  s.sk_c0 = 0;
+  s.sk_cost = 0;
+  const int full = n_x / W, rem = n_x % W;
+  if (!sk_enable || rem == 0 || full > kSkMaxRounds) return;
+  // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves 4 %
+  if ((int64_t)(W - rem) * 25 < (int64_t)W * (full + 1)) return;
+  int n_sk = rem;
+  int rounds = full;
+  if (rem * 4 < W && full >= 1) {  // very few tiles: cut a full round with them, pieces of about a tile
+    n_sk += W;
+    rounds -= 1;
+  }
+  const int sk_begin = s.range_begin + rounds * W;
+  const int64_t c0 = cost_before(s, sk_begin);
+  const int64_t cost = cost_before(s, s.range_end) - c0;
+  int64_t w = W;
+  if (w > cost / kSkMinPairs) w = cost / kSkMinPairs;
+  if (w > (int64_t)n_sk * kSkMaxPieces) w = (int64_t)n_sk * kSkMaxPieces;
+  if (w <= n_sk) return;  // nothing to gain: at most one piece per tile
+  s.dp_rounds = rounds;
+  s.sk_begin = sk_begin;
+  s.sk_wgs = (int)w;
+  s.sk_c0 = c0;
+  s.sk_cost = cost;
+}
+
+// piece boundaries of the stream-K region, relative to sk_c0
+FP8GMM_HD int64_t sk_bound(const Sched& s, int j) { return s.sk_cost * j / s.sk_wgs; }
+
+struct Item {
+  int tile, prob, m0, n0;
+  int k_begin, nk;  // pair steps: first one, how many (0 for a problem without K)
+  int slot;         // workspace slot of a partial piece, -1: the piece is the whole tile
+};
+struct Cursor {
+  int dp_i;     // strided tiles already taken
+  int sk_tile;  // next tile of this workgroup's stream-K piece, -1: none left
+};
+
+FP8GMM_HD void cursor_init(const Sched& s, int j, Cursor& c) {
+  c.dp_i = 0;
+  c.sk_tile = -1;
+  if (j < s.sk_wgs && sk_bound(s, j) < sk_bound(s, j + 1)) c.sk_tile = tile_holding_cost(s, s.sk_c0 + sk_bound(s, j));
+}
+FP8GMM_HD bool cursor_valid(const Sched& s, int j, const Cursor& c) {
+  return (c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin) || c.sk_tile >= 0;
+}
+FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c) {
+  const bool dp = c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin;
+  Item it;
+  it.tile = dp ? s.range_begin + j + s.wgs * c.dp_i : c.sk_tile;
+  it.prob = problem_of_tile(s, it.tile);
+  const int local = it.tile - s.probs[it.prob].tile_begin;
+  const int tiles_m = (s.probs[it.prob].m + BM - 1) / BM;
+  it.m0 = (local % tiles_m) * BM;  // m fastest: neighbouring tiles share the weight slab
+  it.n0 = (local / tiles_m) * BN;
+  const int real_nk = (s.probs[it.prob].k + 127) / 128;  // a K tail is zero-filled
+  it.k_begin = 0;
+  it.nk = real_nk;
+  it.slot = -1;
+  if (!dp) {
+    const int64_t c_t = cost_before(s, it.tile) - s.sk_c0, k_t = tile_cost(s, it.prob);
+    const int64_t lo = sk_bound(s, j), hi = sk_bound(s, j + 1);
+    const int64_t p_lo = (lo > c_t ? lo : c_t) - c_t;
+    const int64_t p_hi = (hi < c_t + k_t ? hi : c_t + k_t) - c_t;
+    if (p_hi - p_lo < k_t) {  // only tiles with real K work are ever cut (k_t > 1)
+      it.k_begin = (int)p_lo;
+      it.nk = (int)(p_hi - p_lo);
+      it.slot = kSlotsPerWg * (xcd * s.wgs + j) + (p_lo == 0 ? 1 : 0);
+    }
+  }
+  return it;
+}
+FP8GMM_HD void cursor_advance(const Sched& s, int j, Cursor& c) {
+  if (c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin) {
+    ++c.dp_i;
+    return;
+  }
+  if (c.sk_tile < 0) return;
+  const int p = problem_of_tile(s, c.sk_tile);
+  const int64_t t_end_cost = cost_before(s, c.sk_tile) - s.sk_c0 + tile_cost(s, p);
+  c.sk_tile = (t_end_cost < sk_bound(s, j + 1) && c.sk_tile + 1 < s.range_end) ? c.sk_tile + 1 : -1;
+}
+
+
+
+// The tile that the workgroup of piece boundary j (1 <= j < sk_wgs) completes in the fix-up pass, or -1:
+// the FIRST boundary strictly inside a tile owns it.  `first_piece_wg` is the workgroup that holds the piece
+// from the tile's first pair step (slot kSlotsPerWg * wg + 1); the following pieces come from workgroups
+// j, j + 1, ... (slot kSlotsPerWg * wg) while their boundary lies inside the tile.
+FP8GMM_HD int fixup_tile(const Sched& s, int j, int* n_following) {
+  *n_following = 0;
+  if (j < 1 || j >= s.sk_wgs) return -1;
+  const int64_t b = sk_bound(s, j);
+  const int tile = tile_holding_cost(s, s.sk_c0 + b);
+  if (tile >= s.range_end) return -1;
+  const int64_t c_t = cost_before(s, tile) - s.sk_c0, k_t = tile_cost(s, problem_of_tile(s, tile));
+  if (b == c_t) return -1;                    // the boundary coincides with a tile boundary
+  if (sk_bound(s, j - 1) > c_t) return -1;    // an earlier boundary inside the same tile owns it
+  int n = 0;
+  for (int q = j; q < s.sk_wgs && sk_bound(s, q) < c_t + k_t; ++q) ++n;
+  *n_following = n;
+  return tile;
+}
+
+}  // namespace fp8gmm

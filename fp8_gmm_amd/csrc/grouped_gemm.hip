@@ -35,14 +35,18 @@
 //     fetched during the previous step) are issued first and the DMA issues / next-fragment
 //     LDS reads are interleaved between them (pinned with sched_barrier), so the MFMA pipe
 //     does not idle while the two wavefronts of a SIMD do their memory work.
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
+
 #include "device_utils.h"
+#include "gemm_schedule.h"
 #include "tiling.h"
 
 namespace fp8gmm {
 namespace {
 
-constexpr int BM = kGemmTileM;   // 256
-constexpr int BN = kGemmTileN;   // 256
 constexpr int HK = 64;           // bytes of K per half-slot / per MFMA
 constexpr int HS = (BM + BN) * HK;  // 32768 bytes per half-slot
 constexpr int RING = 5;
@@ -50,12 +54,12 @@ constexpr int NTHREADS = 512;
 constexpr int WM = 128, WN = 64;  // wavefront sub-tile
 constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
 constexpr int NT = WN / 32;       // 2 MFMA tiles along n per wave
-constexpr int kNumXcd = 8;
 constexpr int kPairLoads = 8;     // buffer_load ... lds instructions per wavefront per K = 128 pair
 constexpr int kFastStores = MT * NT * 2;  // 16-byte stores per wavefront in the interior bf16 epilogue
 constexpr int kRelaxedWaits = 3;  // barriers after such an epilogue that need not wait for its stores
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
 #define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
@@ -65,296 +69,22 @@ typedef unsigned u32pair __attribute__((ext_vector_type(2)));
 #define FP8GMM_DMA(lds_addr, voff, rsrc) \
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
 
-template <int A_FMT, int B_FMT>
-__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
-                                                                int nprob, int total_tiles, int out_kind,
-                                                                int epilogue) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wave_m = wave >> 2;  // 0..1
-  const int wave_n = wave & 3;   // 0..3
-  const int l32 = lane & 31;
-  const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
-
-  // DMA lane map: one wavefront instruction fills 16 rows x 64 B of a half-slot: lane -> row lane >> 2,
-  // slot chunk lane & 3.  With the swizzle (row >> 2) & 3 and row = 16 g + (lane >> 2) the GLOBAL chunk
-  // that has to land there is (lane & 3) ^ ((lane >> 4) & 3).
-  const int drow = lane >> 2;
-  const int dchunk = (lane & 3) ^ ((lane >> 4) & 3);
-  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 64 + 32 j + l32 (source 0)
-  const int fsw = (l32 >> 2) & 3;
-  const int fc0 = ((khalf * 2) ^ fsw) << 4;
-  const int fc1 = ((khalf * 2 + 1) ^ fsw) << 4;
-  const int fa_off = (wave_m * WM + l32) * HK;
-  const int fb_off = BM * HK + (wave_n * WN + l32) * HK;
-
-  // ---- this workgroup's tile sequence (uniform) ----
-  // Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal COST
-  // (a tile of problem p costs ceil(k_p / 128) pair steps; k differs per problem in the wgrad form),
-  // and the workgroups of an XCD stride through that XCD's range.
-  const int xcd = blockIdx.x % kNumXcd;
-  const int wg_in_xcd = blockIdx.x / kNumXcd;
-  const int wgs_per_xcd = gridDim.x / kNumXcd;  // the launcher keeps gridDim.x a multiple of 8
-  int range_begin = total_tiles, range_end = total_tiles;
-  {
-    auto tile_cost = [&](int p) {
-      const int c = (probs[p].k + 127) / 128;
-      return (int64_t)(c > 0 ? c : 1);
-    };
-    int64_t total_cost = 0;
-    for (int p = 0; p < nprob; ++p) {
-      const int t_end = (p + 1 < nprob) ? probs[p + 1].tile_begin : total_tiles;
-      total_cost += (int64_t)(t_end - probs[p].tile_begin) * tile_cost(p);
-    }
-    const int64_t lo = (total_cost * xcd + kNumXcd - 1) / kNumXcd;
-    const int64_t hi = (total_cost * (xcd + 1) + kNumXcd - 1) / kNumXcd;
-    // first tile whose preceding cost is >= lo (resp. hi)
-    int64_t cum = 0;
-    bool have_lo = false, have_hi = false;
-    for (int p = 0; p < nprob && !have_hi; ++p) {
-      const int t_begin = probs[p].tile_begin;
-      const int t_end = (p + 1 < nprob) ? probs[p + 1].tile_begin : total_tiles;
-      const int64_t c = tile_cost(p);
-      const int64_t n_t = t_end - t_begin;
-      if (!have_lo && cum + n_t * c > lo - c) {  // some tile i of p has cum + i c >= lo
-        const int64_t i = lo > cum ? (lo - cum + c - 1) / c : 0;
-        if (i < n_t) {
-          range_begin = t_begin + (int)i;
-          have_lo = true;
-        }
-      }
-      if (cum + n_t * c > hi - c) {
-        const int64_t i = hi > cum ? (hi - cum + c - 1) / c : 0;
-        if (i < n_t) {
-          range_end = t_begin + (int)i;
-          have_hi = true;
-        }
-      }
-      cum += n_t * c;
-    }
-    if (!have_lo) range_begin = total_tiles;
-  }
-  auto next_tile = [&](int t) { return t < range_end ? t : -1; };
-  struct Geo {
-    int prob, m0, n0, nk;
-  };
-  auto geo_of = [&](int tile) {
-    const int p = upper_slot(nprob, tile, [&](int i) { return probs[i].tile_begin; });
-    const int local = tile - probs[p].tile_begin;
-    const int tiles_m = (probs[p].m + BM - 1) / BM;
-    Geo g;
-    g.prob = p;
-    g.m0 = (local % tiles_m) * BM;  // m fastest: neighbouring tiles share the weight slab
-    g.n0 = (local / tiles_m) * BN;
-    g.nk = (probs[p].k + 127) / 128;  // K = 128 pairs; a K tail is zero-filled
-    return g;
-  };
-  const int t_stride = wgs_per_xcd;
-
-  int t_cp = next_tile(range_begin + wg_in_xcd);
-  if (t_cp < 0) return;
-
-  // ---- load side: runs two pairs ahead of the compute side, possibly in the next tile ----
-  int t_ld = t_cp;
-  int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
-  i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
-  uint32_t a_base[2], b_base[2];
-  uint32_t ok_mask = 0;  // bit part: rows of that part exist
-  auto load_setup = [&]() {
-    while (t_ld >= 0) {
-      const Geo g = geo_of(t_ld);
-      if (g.nk > 0) {
-        const fp8gmm_gemm_problem pr = probs[g.prob];
-        const uint64_t pa = (uint64_t)pr.a, pb = (uint64_t)pr.b;
-        const uint64_t sa = (uint64_t)pr.m * (uint64_t)pr.lda, sb = (uint64_t)pr.n * (uint64_t)pr.ldb;
-        rsrc_a[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pa);
-        rsrc_a[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pa >> 32));
-        rsrc_a[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sa > 0xffffffffull ? 0xffffffffull : sa));
-        rsrc_b[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pb);
-        rsrc_b[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pb >> 32));
-        rsrc_b[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sb > 0xffffffffull ? 0xffffffffull : sb));
-        ok_mask = 0;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int ar = g.m0 + (wave + 8 * j) * 16 + drow;
-          const int br = g.n0 + (wave + 8 * j) * 16 + drow;
-          if (ar < pr.m) ok_mask |= 1u << j;
-          if (br < pr.n) ok_mask |= 4u << j;
-          a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
-          b_base[j] = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
-        }
-        ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
-        ld_nk = g.nk;
-        ld_kt = 0;
-        return;
-      }
-      t_ld = next_tile(t_ld + t_stride);  // a tile without K work needs no loads
-    }
-  };
-  // One quarter of a pair: part 0, 1 = token row groups wave, wave + 8; part 2, 3 = weight row groups.
-  // Low 64-byte half into slot_lo, high half into slot_hi.  Past the end of the stream the loads are
-  // issued all the same with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
-  auto dma_part = [&](int slot_lo, int slot_hi, int part) {
-    const int j = part & 1;
-    const bool is_b = (part >> 1) != 0;
-    const int k0 = ld_kt * 128;
-    const bool rok = (t_ld >= 0) && ((ok_mask >> part) & 1);
-    const uint32_t base = is_b ? b_base[j] : a_base[j];
-    const uint32_t v_lo = (rok && k0 < ld_kmax) ? base + k0 : 0xffffffffu;
-    const uint32_t v_hi = (rok && k0 + 64 < ld_kmax) ? base + k0 + 64 : 0xffffffffu;
-    const uint32_t off = (is_b ? BM * HK : 0) + (wave + 8 * j) * 1024;
-    const uint32_t l_lo = __builtin_amdgcn_readfirstlane(lds_base + slot_lo * HS + off);
-    const uint32_t l_hi = __builtin_amdgcn_readfirstlane(lds_base + slot_hi * HS + off);
-    if (!is_b) {
-      FP8GMM_DMA(l_lo, v_lo, rsrc_a);
-      FP8GMM_DMA(l_hi, v_hi, rsrc_a);
-    } else {
-      FP8GMM_DMA(l_lo, v_lo, rsrc_b);
-      FP8GMM_DMA(l_hi, v_hi, rsrc_b);
-    }
-  };
-  auto dma_advance = [&]() {
-    if (t_ld < 0) return;
-    if (++ld_kt == ld_nk) {
-      t_ld = next_tile(t_ld + t_stride);
-      load_setup();
-    }
-  };
-  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
-
-  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: even / odd half-steps
-  auto read_frag = [&](i32x8& f, const uint8_t* base) {
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc0);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc1);
-    f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-  };
-
-  // ---- fill: pairs 0 and 1 of the stream into half-slots 0..3, first fragments into registers ----
-  load_setup();
-#pragma unroll
-  for (int part = 0; part < 4; ++part) dma_part(0, 1, part);
-  dma_advance();
-#pragma unroll
-  for (int part = 0; part < 4; ++part) dma_part(2, 3, part);
-  dma_advance();
-  FP8GMM_WAIT_VM(kPairLoads);
-  __builtin_amdgcn_s_barrier();
-  {
-    const uint8_t* sa = lds + fa_off;
-    const uint8_t* sb = lds + fb_off;
-    read_frag(fb0[0], sb);
-    read_frag(fb0[1], sb + 32 * HK);
-    read_frag(fa0[0], sa);
-    read_frag(fa0[1], sa + 32 * HK);
-    read_frag(fa0[2], sa + 64 * HK);
-    read_frag(fa0[3], sa + 96 * HK);
-  }
-  int hs = 0;  // half-slot of the current even half-step
-  // vmcnt counts loads and stores in issue order.  A barrier needs the pair before the newest one, so it
-  // normally waits for "all but the newest 8".  Right after an interior epilogue the newest operations
-  // also include that epilogue's kFastStores stores, which nothing in LDS depends on: for the next
-  // kRelaxedWaits barriers the needed pair is older than those stores, so they may stay in flight.
-  int relaxed = 0;
-
-// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
-#define FP8GMM_MF0(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
-#define FP8GMM_MF1(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
-
-  for (; t_cp >= 0; t_cp = next_tile(t_cp + t_stride)) {
-    const Geo g = geo_of(t_cp);
-    const fp8gmm_gemm_problem pr = probs[g.prob];
-    const int M = pr.m, N = pr.n;
-    const int m0 = g.m0, n0 = g.n0;
-
-    f32x16 acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    for (int kt = 0; kt < g.nk; ++kt) {
-      const int h1 = ring_inc(hs), h2 = ring_inc(h1);
-      const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
-      const int free_hi = hs;                                         // will hold half-step + 5
-      // The pair for half-steps + 4 / + 5 is fetched in four quarters spread over both half-steps (token
-      // rows in the even one, weight rows in the odd one, one quarter every fourth MFMA).  Issued in one
-      // burst, the 64 KB of a pair keep the texture-address unit busy for about a thousand cycles and every
-      // wavefront queues behind it with its MFMAs.
-      // ---- even half-step: its fragments are in fa0 / fb0.  The barrier proves that every wavefront has
-      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed
-      // (everything but the newest pair: 4 token-row + 4 weight-row loads).
-      if (relaxed > 0) {
-        FP8GMM_WAIT_VM_LGKM(kPairLoads + kFastStores);
-        --relaxed;
-      } else {
-        FP8GMM_WAIT_VM_LGKM(kPairLoads);
-      }
-      __builtin_amdgcn_s_barrier();
-      {
-        const uint8_t* qa = lds + h1 * HS + fa_off;
-        const uint8_t* qb = lds + h1 * HS + fb_off;
-        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 0);
-        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
-        read_frag(fb1[0], qb);
-        read_frag(fb1[1], qb + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_MF0(1, 1); FP8GMM_SB();
-        read_frag(fa1[0], qa);
-        read_frag(fa1[1], qa + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 1);
-        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
-        read_frag(fa1[2], qa + 64 * HK);
-        read_frag(fa1[3], qa + 96 * HK);
-        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_MF0(3, 1); FP8GMM_SB();
-      }
-      // ---- odd half-step: fragments in fa1 / fb1.  Half-step + 2 sits in the low half of the pair whose
-      // weight rows were issued one half-step ago; only the 4 token-row loads of the newest pair may still
-      // be in flight.
-      if (relaxed > 0) {
-        FP8GMM_WAIT_VM(kPairLoads / 2 + kFastStores);
-        --relaxed;
-      } else {
-        FP8GMM_WAIT_VM(kPairLoads / 2);
-      }
-      __builtin_amdgcn_s_barrier();
-      {
-        const uint8_t* qa = lds + h2 * HS + fa_off;
-        const uint8_t* qb = lds + h2 * HS + fb_off;
-        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 2);
-        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
-        read_frag(fb0[0], qb);
-        read_frag(fb0[1], qb + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_MF1(1, 1); FP8GMM_SB();
-        read_frag(fa0[0], qa);
-        read_frag(fa0[1], qa + 32 * HK);
-        FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 3);
-        dma_advance();
-        FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
-        read_frag(fa0[2], qa + 64 * HK);
-        read_frag(fa0[3], qa + 96 * HK);
-        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1); FP8GMM_SB();
-      }
-      hs = h2;
-    }
-    // ---- epilogue ----
+// Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
+// stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
+__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
+                                              int out_kind, int epilogue) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int l32 = lane & 31, khalf = lane >> 5;
+  const int M = pr.m, N = pr.n;
+  bool fast = false;
     const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
     const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
     const float s = sa_inv * sb_inv;
     const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
     const int64_t ldc = pr.ldc;
     float amax = 0.f;
-    relaxed = 0;
     const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
     if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
         ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
@@ -383,7 +113,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
           }
         }
       }
-      relaxed = kRelaxedWaits;
+      fast = true;
     } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
@@ -476,6 +206,273 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         if (lane == 0 && amax > 0.f) atomic_max_nonneg(pr.c_amax, amax);
       }
     }
+    return fast;
+}
+
+// Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
+// (r4 * 512 + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
+__device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* slot) {
+  float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = {acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        global_store(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4), v);
+      }
+}
+__device__ __forceinline__ void partial_add(f32x16 (&acc)[MT][NT], const uint8_t* slot) {
+  const float* base = reinterpret_cast<const float*>(slot) + threadIdx.x * 4;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 v = *reinterpret_cast<const float4*>(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4));
+        acc[i][j][4 * g + 0] += v.x;
+        acc[i][j][4 * g + 1] += v.y;
+        acc[i][j][4 * g + 2] += v.z;
+        acc[i][j][4 * g + 3] += v.w;
+      }
+}
+
+template <int A_FMT, int B_FMT>
+__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
+                                                                int nprob, int total_tiles, int out_kind,
+                                                                int epilogue, uint8_t* __restrict__ workspace) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_m = wave >> 2;  // 0..1
+  const int wave_n = wave & 3;   // 0..3
+  const int l32 = lane & 31;
+  const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  // DMA lane map: one wavefront instruction fills 16 rows x 64 B of a half-slot: lane -> row lane >> 2,
+  // slot chunk lane & 3.  With the swizzle (row >> 2) & 3 and row = 16 g + (lane >> 2) the GLOBAL chunk
+  // that has to land there is (lane & 3) ^ ((lane >> 4) & 3).
+  const int drow = lane >> 2;
+  const int dchunk = (lane & 3) ^ ((lane >> 4) & 3);
+  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 64 + 32 j + l32 (source 0)
+  const int fsw = (l32 >> 2) & 3;
+  const int fc0 = ((khalf * 2) ^ fsw) << 4;
+  const int fc1 = ((khalf * 2 + 1) ^ fsw) << 4;
+  const int fa_off = (wave_m * WM + l32) * HK;
+  const int fb_off = BM * HK + (wave_n * WN + l32) * HK;
+
+  // ---- this workgroup's item sequence (uniform): strided tiles of its XCD's range, then its piece of
+  // the range's stream-K region ----
+  const int xcd = blockIdx.x % kNumXcd;
+  const int wg_in_xcd = blockIdx.x / kNumXcd;
+  Sched sch;
+  sched_init(sch, probs, nprob, total_tiles, xcd, gridDim.x / kNumXcd, workspace != nullptr);  // gridDim.x % 8 == 0
+  Cursor c_cp, c_ld;
+  cursor_init(sch, wg_in_xcd, c_cp);
+  if (!cursor_valid(sch, wg_in_xcd, c_cp)) return;
+  c_ld = c_cp;
+
+  // ---- load side: runs two pairs ahead of the compute side, possibly in the next tile ----
+  bool ld_live = true;  // the load cursor still points at an item
+  int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
+  i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
+  uint32_t a_base[2], b_base[2];
+  uint32_t ok_mask = 0;  // bit part: rows of that part exist
+  auto load_setup = [&]() {
+    while ((ld_live = cursor_valid(sch, wg_in_xcd, c_ld))) {
+      const Item g = cursor_item(sch, xcd, wg_in_xcd, c_ld);
+      if (g.nk > 0) {
+        const fp8gmm_gemm_problem pr = probs[g.prob];
+        const uint64_t pa = (uint64_t)pr.a, pb = (uint64_t)pr.b;
+        const uint64_t sa = (uint64_t)pr.m * (uint64_t)pr.lda, sb = (uint64_t)pr.n * (uint64_t)pr.ldb;
+        rsrc_a[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pa);
+        rsrc_a[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pa >> 32));
+        rsrc_a[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sa > 0xffffffffull ? 0xffffffffull : sa));
+        rsrc_b[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pb);
+        rsrc_b[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pb >> 32));
+        rsrc_b[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sb > 0xffffffffull ? 0xffffffffull : sb));
+        ok_mask = 0;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int ar = g.m0 + (wave + 8 * j) * 16 + drow;
+          const int br = g.n0 + (wave + 8 * j) * 16 + drow;
+          if (ar < pr.m) ok_mask |= 1u << j;
+          if (br < pr.n) ok_mask |= 4u << j;
+          a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          b_base[j] = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
+        }
+        ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
+        ld_kt = g.k_begin;
+        ld_nk = g.k_begin + g.nk;
+        return;
+      }
+      cursor_advance(sch, wg_in_xcd, c_ld);  // an item without K work needs no loads
+    }
+  };
+  // One quarter of a pair: part 0, 1 = token row groups wave, wave + 8; part 2, 3 = weight row groups.
+  // Low 64-byte half into slot_lo, high half into slot_hi.  Past the end of the stream the loads are
+  // issued all the same with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
+  auto dma_part = [&](int slot_lo, int slot_hi, int part) {
+    const int j = part & 1;
+    const bool is_b = (part >> 1) != 0;
+    const int k0 = ld_kt * 128;
+    const bool rok = ld_live && ((ok_mask >> part) & 1);
+    const uint32_t base = is_b ? b_base[j] : a_base[j];
+    const uint32_t v_lo = (rok && k0 < ld_kmax) ? base + k0 : 0xffffffffu;
+    const uint32_t v_hi = (rok && k0 + 64 < ld_kmax) ? base + k0 + 64 : 0xffffffffu;
+    const uint32_t off = (is_b ? BM * HK : 0) + (wave + 8 * j) * 1024;
+    const uint32_t l_lo = __builtin_amdgcn_readfirstlane(lds_base + slot_lo * HS + off);
+    const uint32_t l_hi = __builtin_amdgcn_readfirstlane(lds_base + slot_hi * HS + off);
+    if (!is_b) {
+      FP8GMM_DMA(l_lo, v_lo, rsrc_a);
+      FP8GMM_DMA(l_hi, v_hi, rsrc_a);
+    } else {
+      FP8GMM_DMA(l_lo, v_lo, rsrc_b);
+      FP8GMM_DMA(l_hi, v_hi, rsrc_b);
+    }
+  };
+  auto dma_advance = [&]() {
+    if (!ld_live) return;
+    if (++ld_kt == ld_nk) {
+      cursor_advance(sch, wg_in_xcd, c_ld);
+      load_setup();
+    }
+  };
+  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
+
+  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: even / odd half-steps
+  auto read_frag = [&](i32x8& f, const uint8_t* base) {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc0);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc1);
+    f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+
+  // ---- fill: pairs 0 and 1 of the stream into half-slots 0..3, first fragments into registers ----
+  load_setup();
+#pragma unroll
+  for (int part = 0; part < 4; ++part) dma_part(0, 1, part);
+  dma_advance();
+#pragma unroll
+  for (int part = 0; part < 4; ++part) dma_part(2, 3, part);
+  dma_advance();
+  FP8GMM_WAIT_VM(kPairLoads);
+  __builtin_amdgcn_s_barrier();
+  {
+    const uint8_t* sa = lds + fa_off;
+    const uint8_t* sb = lds + fb_off;
+    read_frag(fb0[0], sb);
+    read_frag(fb0[1], sb + 32 * HK);
+    read_frag(fa0[0], sa);
+    read_frag(fa0[1], sa + 32 * HK);
+    read_frag(fa0[2], sa + 64 * HK);
+    read_frag(fa0[3], sa + 96 * HK);
+  }
+  int hs = 0;  // half-slot of the current even half-step
+  // vmcnt counts loads and stores in issue order.  A barrier needs the pair before the newest one, so it
+  // normally waits for "all but the newest 8".  Right after an interior epilogue the newest operations
+  // also include that epilogue's kFastStores stores, which nothing in LDS depends on: for the next
+  // kRelaxedWaits barriers the needed pair is older than those stores, so they may stay in flight.
+  int relaxed = 0;
+
+// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
+#define FP8GMM_MF0(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+#define FP8GMM_MF1(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+
+  for (; cursor_valid(sch, wg_in_xcd, c_cp); cursor_advance(sch, wg_in_xcd, c_cp)) {
+    const Item g = cursor_item(sch, xcd, wg_in_xcd, c_cp);
+    const fp8gmm_gemm_problem pr = probs[g.prob];
+    const int m0 = g.m0, n0 = g.n0;
+
+    f32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    for (int kt = 0; kt < g.nk; ++kt) {
+      const int h1 = ring_inc(hs), h2 = ring_inc(h1);
+      const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
+      const int free_hi = hs;                                         // will hold half-step + 5
+      // The pair for half-steps + 4 / + 5 is fetched in four quarters spread over both half-steps (token
+      // rows in the even one, weight rows in the odd one, one quarter every fourth MFMA).  Issued in one
+      // burst, the 64 KB of a pair keep the texture-address unit busy for about a thousand cycles and every
+      // wavefront queues behind it with its MFMAs.
+      // ---- even half-step: its fragments are in fa0 / fb0.  The barrier proves that every wavefront has
+      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed
+      // (everything but the newest pair: 4 token-row + 4 weight-row loads).
+      if (relaxed > 0) {
+        FP8GMM_WAIT_VM_LGKM(kPairLoads + kFastStores);
+        --relaxed;
+      } else {
+        FP8GMM_WAIT_VM_LGKM(kPairLoads);
+      }
+      __builtin_amdgcn_s_barrier();
+      {
+        const uint8_t* qa = lds + h1 * HS + fa_off;
+        const uint8_t* qb = lds + h1 * HS + fb_off;
+        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 0);
+        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
+        read_frag(fb1[0], qb);
+        read_frag(fb1[1], qb + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        read_frag(fa1[0], qa);
+        read_frag(fa1[1], qa + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 1);
+        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
+        read_frag(fa1[2], qa + 64 * HK);
+        read_frag(fa1[3], qa + 96 * HK);
+        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_MF0(3, 1); FP8GMM_SB();
+      }
+      // ---- odd half-step: fragments in fa1 / fb1.  Half-step + 2 sits in the low half of the pair whose
+      // weight rows were issued one half-step ago; only the 4 token-row loads of the newest pair may still
+      // be in flight.
+      if (relaxed > 0) {
+        FP8GMM_WAIT_VM(kPairLoads / 2 + kFastStores);
+        --relaxed;
+      } else {
+        FP8GMM_WAIT_VM(kPairLoads / 2);
+      }
+      __builtin_amdgcn_s_barrier();
+      {
+        const uint8_t* qa = lds + h2 * HS + fa_off;
+        const uint8_t* qb = lds + h2 * HS + fb_off;
+        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 2);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        read_frag(fb0[0], qb);
+        read_frag(fb0[1], qb + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_MF1(1, 1); FP8GMM_SB();
+        read_frag(fa0[0], qa);
+        read_frag(fa0[1], qa + 32 * HK);
+        FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
+        dma_part(free_lo, free_hi, 3);
+        dma_advance();
+        FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
+        read_frag(fa0[2], qa + 64 * HK);
+        read_frag(fa0[3], qa + 96 * HK);
+        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1); FP8GMM_SB();
+      }
+      hs = h2;
+    }
+    // ---- epilogue ----
+    if (g.slot >= 0) {
+      // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
+      partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
+      relaxed = 0;
+    } else {
+      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue) ? kRelaxedWaits : 0;
+    }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS
   FP8GMM_WAIT_VM(0);
@@ -483,6 +480,78 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 
 #undef FP8GMM_MF0
 #undef FP8GMM_MF1
+
+// Completes the tiles that the main kernel shared along K.  One workgroup per interior piece boundary of
+// every XCD's stream-K region; the FIRST boundary that falls strictly inside a tile owns that tile: it adds
+// the pieces in K order (workgroup j - 1 holds the piece from the tile's first pair step, workgroups j,
+// j + 1, ... the following ones) and runs the normal epilogue.
+__global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
+                                                                      int nprob, int total_tiles, int out_kind,
+                                                                      int epilogue,
+                                                                      const uint8_t* __restrict__ workspace,
+                                                                      int wgs_per_xcd) {
+  const int xcd = blockIdx.x % kNumXcd;
+  const int j = blockIdx.x / kNumXcd + 1;
+  Sched sch;
+  sched_init(sch, probs, nprob, total_tiles, xcd, wgs_per_xcd, true);
+  int n_following = 0;
+  const int tile = fixup_tile(sch, j, &n_following);
+  if (tile < 0) return;
+  const int prob = problem_of_tile(sch, tile);
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int jj = 0; jj < NT; ++jj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][jj][r] = 0.f;
+  partial_add(acc, workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + j - 1) + 1) * kPartialBytes);
+  for (int q = j; q < j + n_following; ++q)
+    partial_add(acc, workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + q)) * kPartialBytes);
+
+  const fp8gmm_gemm_problem pr = probs[prob];
+  const int local = tile - pr.tile_begin;
+  const int tiles_m = (pr.m + BM - 1) / BM;
+  tile_epilogue(acc, pr, (local % tiles_m) * BM, (local / tiles_m) * BN, out_kind, epilogue);
+}
+
+// Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)
+// and kept until the process ends.  Launches on one stream are ordered, so they can share it; a few
+// streams get a workspace each, further ones simply run without tail balancing.
+struct WorkspaceKey {
+  int device;
+  hipStream_t stream;
+  bool operator<(const WorkspaceKey& o) const {
+    return device != o.device ? device < o.device : reinterpret_cast<uintptr_t>(stream) < reinterpret_cast<uintptr_t>(o.stream);
+  }
+};
+constexpr size_t kMaxWorkspaces = 8;
+
+uint8_t* workspace_for(int device, hipStream_t stream, int grid) {
+  static std::mutex mu;
+  static std::map<WorkspaceKey, std::pair<uint8_t*, size_t>> cache;
+  const size_t bytes = (size_t)kSlotsPerWg * (size_t)grid * kPartialBytes;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find(WorkspaceKey{device, stream});
+  if (it != cache.end()) return it->second.second >= bytes ? it->second.first : nullptr;
+  if (cache.size() >= kMaxWorkspaces) return nullptr;
+  void* ptr = nullptr;
+  if (hipMalloc(&ptr, bytes) != hipSuccess) {
+    (void)hipGetLastError();  // e.g. under stream capture: run without tail balancing
+    return nullptr;
+  }
+  cache[WorkspaceKey{device, stream}] = {static_cast<uint8_t*>(ptr), bytes};
+  return static_cast<uint8_t*>(ptr);
+}
+
+bool stream_k_allowed() {
+  static const bool allowed = [] {
+    const char* e = getenv("FP8GMM_STREAMK");
+    return !(e != nullptr && e[0] == '0');
+  }();
+  return allowed;
+}
 
 template <int A_FMT, int B_FMT>
 int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
@@ -497,21 +566,34 @@ int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out
       return FP8GMM_ERR_LAUNCH;
     attr_set = true;
   }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
   if (num_cu == 0) {
-    int dev = 0;
     hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
-      return FP8GMM_ERR_NO_DEVICE;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
     num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
   // one workgroup per CU, a multiple of 8 so that every XCD gets the same number of workgroups
   int grid = (num_cu / kNumXcd) * kNumXcd;
   if (grid < kNumXcd) grid = kNumXcd;
-  const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
-  if (grid > needed) grid = needed;
+  // tail balancing can only pay when the launch has few rounds; it needs the whole grid even for few tiles
+  uint8_t* workspace = nullptr;
+  if (stream_k_allowed() && (int64_t)total_tiles <= (int64_t)kSkMaxRounds * grid && grid > kNumXcd)
+    workspace = workspace_for(dev, stream, grid);
+  if (workspace == nullptr) {
+    const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
+    if (grid > needed) grid = needed;
+  }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(NTHREADS), lds_bytes, stream, probs_dev, n, total_tiles, out_kind,
-                     epilogue);
-  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+                     epilogue, workspace);
+  if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
+  if (workspace != nullptr) {
+    const int wgs_per_xcd = grid / kNumXcd;
+    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(kNumXcd * (wgs_per_xcd - 1)), dim3(NTHREADS), 0, stream,
+                       probs_dev, n, total_tiles, out_kind, epilogue, workspace, wgs_per_xcd);
+    if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
+  }
+  return FP8GMM_OK;
 }
 
 }  // namespace

@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "../../include/fp8gmm.h"
+#include "gemm_schedule.h"
 #include "tiling.h"
 
 extern "C" {
@@ -66,6 +67,57 @@ int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* tota
   }
   *total_blocks = (int)blocks;
   return FP8GMM_OK;
+}
+
+int fp8gmm_gemm_schedule(const fp8gmm_gemm_problem* probs, int n, int total_tiles, int grid, int stream_k, int wg,
+                         int32_t* items, int max_items) {
+  using namespace fp8gmm;
+  if (n < 0 || total_tiles < 0 || grid <= 0 || (grid % kNumXcd) != 0 || wg < 0 || wg >= grid || max_items < 0)
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if ((n > 0 && probs == nullptr) || (max_items > 0 && items == nullptr)) return FP8GMM_ERR_NULL_POINTER;
+  if (n == 0 || total_tiles == 0) return 0;
+  const int xcd = wg % kNumXcd, j = wg / kNumXcd;
+  Sched s;
+  sched_init(s, probs, n, total_tiles, xcd, grid / kNumXcd, stream_k != 0);
+  Cursor c;
+  cursor_init(s, j, c);
+  int count = 0;
+  for (; cursor_valid(s, j, c); cursor_advance(s, j, c)) {
+    const Item it = cursor_item(s, xcd, j, c);
+    if (count < max_items) {
+      int32_t* r = items + 7 * count;
+      r[0] = it.tile; r[1] = it.prob; r[2] = it.m0; r[3] = it.n0; r[4] = it.k_begin; r[5] = it.nk; r[6] = it.slot;
+    }
+    ++count;
+  }
+  return count;
+}
+
+int fp8gmm_gemm_fixup(const fp8gmm_gemm_problem* probs, int n, int total_tiles, int grid, int wg, int32_t* tile,
+                      int32_t* slots, int max_slots) {
+  using namespace fp8gmm;
+  if (n < 0 || total_tiles < 0 || grid <= kNumXcd || (grid % kNumXcd) != 0 || wg < 0 || wg >= grid - kNumXcd ||
+      max_slots < 0)
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if (tile == nullptr || (n > 0 && probs == nullptr) || (max_slots > 0 && slots == nullptr))
+    return FP8GMM_ERR_NULL_POINTER;
+  *tile = -1;
+  if (n == 0 || total_tiles == 0) return 0;
+  const int xcd = wg % kNumXcd, j = wg / kNumXcd + 1, wgs = grid / kNumXcd;
+  Sched s;
+  sched_init(s, probs, n, total_tiles, xcd, wgs, true);
+  int n_following = 0;
+  const int t = fixup_tile(s, j, &n_following);
+  if (t < 0) return 0;
+  *tile = t;
+  int count = 0;
+  auto put = [&](int slot) {
+    if (count < max_slots) slots[count] = slot;
+    ++count;
+  };
+  put(kSlotsPerWg * (xcd * wgs + j - 1) + 1);
+  for (int q = j; q < j + n_following; ++q) put(kSlotsPerWg * (xcd * wgs + q));
+  return count;
 }
 
 }  // extern "C"

@@ -4,7 +4,10 @@
  * This is the boundary that replaces the reference's pybind11 module
  * `fp8_gmm_backend` (csrc/ops.cu:9-16).  Every function is `extern "C"`,
  * takes plain pointers and integers, returns an int status (0 = success,
- * negative = fp8gmm_status) and never throws, allocates, frees or synchronises.
+ * negative = fp8gmm_status) and never throws, frees or synchronises.  The only
+ * allocation is fp8gmm_grouped_gemm's tail-balancing workspace (128 MB, once per
+ * device and stream, for up to 8 streams; kept until the process ends; skipped,
+ * without error, when the allocation is refused or FP8GMM_STREAMK=0 is set).
  * All device work is enqueued on the HIP stream passed in (`hipStream_t`,
  * passed as `void*`; NULL = the default stream).
  *
@@ -163,6 +166,25 @@ int fp8gmm_multi_pad_cast_transpose_dgelu(const fp8gmm_tensor_desc* descs_dev, i
  */
 int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int a_fmt, int b_fmt,
                         int out_kind, int epilogue, void* stream);
+
+/* ---- schedule introspection (host only, no GPU needed) ------------------------------------ */
+/*
+ * The work items that workgroup `wg` of a grouped-GEMM launch with `grid` workgroups (a multiple of 8)
+ * processes, in order, for the HOST table `probs` (after fp8gmm_plan_grouped_gemm).  stream_k != 0:
+ * as in a launch that shares the tail tiles of each XCD's range along K.  Writes up to max_items records
+ * of 7 int32 - tile, problem, m0, n0, k_begin, nk, slot (k_begin / nk in steps of 128 bytes of K; slot = -1
+ * when the item is a whole tile, else the workspace slot that receives its partial sums) - and returns the
+ * number of items.  No counterpart in the reference (its CUTLASS scheduler is not observable); it lets the
+ * schedule be checked without a GPU.
+ */
+int fp8gmm_gemm_schedule(const fp8gmm_gemm_problem* probs, int n, int total_tiles, int grid, int stream_k, int wg,
+                         int32_t* items, int max_items);
+/*
+ * The tile that fix-up workgroup `wg` (0 <= wg < grid - 8) of such a launch completes (*tile, -1: none) and
+ * the workspace slots whose partial sums it adds, in K order (up to max_slots); returns their number.
+ */
+int fp8gmm_gemm_fixup(const fp8gmm_gemm_problem* probs, int n, int total_tiles, int grid, int wg, int32_t* tile,
+                      int32_t* slots, int max_slots);
 
 #ifdef __cplusplus
 }

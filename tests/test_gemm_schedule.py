@@ -1,0 +1,161 @@
+"""Work decomposition of the grouped GEMM, checked without a GPU through the library's introspection calls.
+
+What must hold for ANY problem list, grid and tail-balancing choice (the kernel relies on each of these):
+  * every (tile, K step) unit is processed exactly once; tiles without K work are visited exactly once;
+  * an item is either a whole tile (slot -1) or a proper part of one with a workspace slot that no other
+    item of the launch uses and that lies inside the kSlotsPerWg * grid slots of the workspace;
+  * every tile that was cut is completed by exactly one fix-up workgroup, which adds exactly the slots
+    written for that tile, in K order;
+  * workgroup wg works only on tiles of XCD range wg % 8, and the eight ranges tile the list in order.
+The expectations are stated from these properties, not recomputed with the scheduler's formulas.
+"""
+import numpy as np
+import pytest
+
+from fp8_gmm_amd import _lib
+
+TILE = 256
+
+
+def make_table(shapes):
+    """shapes: list of (m, n, k). Pointers are fake but non-null and aligned; nothing is dereferenced."""
+    t = np.zeros(len(shapes), dtype=_lib.GEMM_PROBLEM)
+    for i, (m, n, k) in enumerate(shapes):
+        t[i]["a"], t[i]["b"], t[i]["c"] = 0x10000, 0x20000, 0x30000
+        t[i]["m"], t[i]["n"], t[i]["k"] = m, n, k
+        t[i]["lda"] = t[i]["ldb"] = max(k, 16)
+        t[i]["ldc"] = max(n, 1)
+    total = _lib.plan_grouped_gemm(t)
+    return t, total
+
+
+def check_schedule(shapes, grid, stream_k):
+    table, total = make_table(shapes)
+    nk_of = [(k + 127) // 128 for (_, _, k) in shapes]
+    tiles_of = [((m + TILE - 1) // TILE) * ((n + TILE - 1) // TILE) for (m, n, _) in shapes]
+    assert total == sum(tiles_of)
+    tile_prob = np.repeat(np.arange(len(shapes)), tiles_of)
+
+    covered = [np.zeros(max(nk_of[p], 1), dtype=np.int32) for p in tile_prob]  # per tile, per K step
+    slots_written = {}  # slot -> (tile, k_begin, nk)
+    xcd_tiles = [set() for _ in range(8)]
+    n_partial_items = 0
+    for wg in range(grid):
+        items = _lib.gemm_schedule(table, total, grid, stream_k, wg)
+        for tile, prob, m0, n0, k_begin, nk, slot in items.tolist():
+            assert 0 <= tile < total and prob == tile_prob[tile]
+            m, n, _ = shapes[prob]
+            local = tile - int(table[prob]["tile_begin"])
+            tiles_m = (m + TILE - 1) // TILE
+            assert (m0, n0) == ((local % tiles_m) * TILE, (local // tiles_m) * TILE)
+            xcd_tiles[wg % 8].add(tile)
+            if nk_of[prob] == 0:
+                assert (k_begin, nk, slot) == (0, 0, -1)
+                covered[tile][0] += 1
+                continue
+            assert nk >= 1 and 0 <= k_begin and k_begin + nk <= nk_of[prob]
+            covered[tile][k_begin:k_begin + nk] += 1
+            if slot == -1:
+                assert (k_begin, nk) == (0, nk_of[prob])
+            else:
+                assert stream_k and nk < nk_of[prob]
+                assert 0 <= slot < 2 * grid and slot not in slots_written
+                slots_written[slot] = (tile, k_begin, nk)
+                n_partial_items += 1
+    for tile in range(total):
+        assert (covered[tile] == 1).all(), f"tile {tile} covered {covered[tile].tolist()}"
+    # XCD ranges are disjoint, contiguous and ordered
+    prev_end = 0
+    for x in range(8):
+        if xcd_tiles[x]:
+            lo, hi = min(xcd_tiles[x]), max(xcd_tiles[x])
+            assert lo == prev_end and xcd_tiles[x] == set(range(lo, hi + 1))
+            prev_end = hi + 1
+    assert prev_end == total
+
+    # fix-up: each cut tile exactly once, with exactly its slots in K order
+    cut_tiles = {}
+    for slot, (tile, k_begin, nk) in slots_written.items():
+        cut_tiles.setdefault(tile, []).append((k_begin, nk, slot))
+    done = set()
+    if stream_k and grid > 8:
+        for wg in range(grid - 8):
+            tile, slots = _lib.gemm_fixup(table, total, grid, wg)
+            if tile < 0:
+                assert slots == []
+                continue
+            assert tile in cut_tiles and tile not in done
+            done.add(tile)
+            pieces = sorted(cut_tiles[tile])
+            assert slots == [s for (_, _, s) in pieces]
+            # the pieces tile the K range of the tile without gaps
+            pos = 0
+            for k_begin, nk, _ in pieces:
+                assert k_begin == pos
+                pos += nk
+            assert pos == nk_of[tile_prob[tile]]
+    assert done == set(cut_tiles)
+    return n_partial_items
+
+
+MLP = [1439, 3146, 3993, 1820, 909, 3499, 669, 909]
+
+
+@pytest.mark.parametrize("grid", [256, 64, 8])
+@pytest.mark.parametrize("stream_k", [False, True])
+def test_config2_shapes(grid, stream_k):
+    fc1 = [(m, 14336, 4096) for m in MLP]
+    fc2 = [(m, 4096, 14336) for m in MLP]
+    wgrad = [(14336, 4096, (m + 127) // 128 * 128) for m in MLP]
+    check_schedule(fc1, grid, stream_k)
+    n_cut = check_schedule(fc2, grid, stream_k)
+    check_schedule(wgrad, grid, stream_k)
+    if stream_k and grid == 256:
+        # 1088 tiles on 256 workgroups: 4.25 rounds, so the tail must be shared along K
+        assert n_cut > 0
+
+
+def test_tail_balancing_is_off_when_it_cannot_pay():
+    # 28 full rounds: more than the limit, nothing may be cut
+    assert check_schedule([(14336, 4096, 2048)] * 8, 256, True) == 0
+    # an exact multiple of the grid: no remainder
+    assert check_schedule([(2048, 4096, 4096)] * 8, 256, True) == 0
+
+
+@pytest.mark.parametrize("shapes", [
+    [(1, 1, 16)],
+    [(256, 256, 128)],
+    [(256, 256, 4096)],                      # one tile, cut eight ways at most
+    [(300, 520, 1040)],
+    [(0, 128, 64), (128, 0, 64), (64, 64, 0), (100, 100, 4096)],   # empty problems, a problem without K
+    [(137, 64, 128), (401, 64, 128), (59, 64, 128), (403, 64, 128)],
+    [(2048, 4096, 14336)],
+    [(513, 777, 1616), (31, 2049, 48), (1025, 255, 8192)],
+])
+@pytest.mark.parametrize("grid", [256, 32, 8])
+def test_small_and_odd_shapes(shapes, grid):
+    check_schedule(shapes, grid, False)
+    check_schedule(shapes, grid, True)
+
+
+def test_random_problem_lists():
+    rng = np.random.default_rng(1234)
+    for _ in range(150):
+        e = int(rng.integers(1, 12))
+        shapes = []
+        for _ in range(e):
+            m = int(rng.choice([0, 1, 100, 256, 257, 700, 1500, 4000]))
+            n = int(rng.choice([0, 16, 256, 1000, 4096]))
+            k = int(rng.choice([0, 16, 128, 144, 1024, 4096, 14336]))
+            shapes.append((m, n, k))
+        grid = int(rng.choice([8, 16, 64, 256, 304]))
+        check_schedule(shapes, grid, bool(rng.integers(0, 2)))
+
+
+def test_argument_checks():
+    table, total = make_table([(256, 256, 128)])
+    buf = np.zeros((4, 7), dtype=np.int32)
+    L = _lib.load()
+    assert L.fp8gmm_gemm_schedule(table.ctypes.data, 1, total, 12, 1, 0, buf.ctypes.data, 4) < 0   # grid % 8 != 0
+    assert L.fp8gmm_gemm_schedule(table.ctypes.data, 1, total, 16, 1, 16, buf.ctypes.data, 4) < 0  # wg out of range
+    assert L.fp8gmm_gemm_schedule(None, 1, total, 16, 1, 0, buf.ctypes.data, 4) < 0

@@ -59,6 +59,66 @@ def test_power_of_two_operands_are_exact(dev, a_dtype, m, n, k):
     assert torch.equal(dc.cpu().view(torch.int16), c.view(torch.int16))
 
 
+@pytest.mark.parametrize("a_dtype", [E4M3, E5M2])
+@pytest.mark.parametrize("sizes,n,k", [([256], 256, 4096), ([700], 520, 2064), ([300, 0, 513, 90], 512, 7168)])
+def test_tiles_shared_along_k_are_exact(dev, a_dtype, sizes, n, k):
+    """Few tiles and a long K: the launch cuts tiles along K, leaves fp32 partial sums in its workspace and
+    completes them in the fix-up pass.  With operands from {0, +-0.25 .. +-2} every partial sum is exact, so
+    the result must still equal the exactly rounded oracle result bit for bit: a piece that is dropped,
+    added twice or taken from the wrong slot cannot pass.  The schedule introspection call proves that
+    this launch really does cut tiles."""
+    import numpy as np
+
+    from fp8_gmm_amd import _lib
+
+    backend = _backend()
+    table = np.zeros(len(sizes), dtype=_lib.GEMM_PROBLEM)
+    for i, m in enumerate(sizes):
+        table[i]["a"], table[i]["b"], table[i]["c"] = 0x1000, 0x1000, 0x1000
+        table[i]["m"], table[i]["n"], table[i]["k"] = m, n, k
+        table[i]["lda"] = table[i]["ldb"] = k
+        table[i]["ldc"] = n
+    total = _lib.plan_grouped_gemm(table)
+    grid = torch.cuda.get_device_properties(dev).multi_processor_count // 8 * 8
+    cut = sum(int((_lib.gemm_schedule(table, total, grid, True, wg)[:, 6] >= 0).sum()) for wg in range(grid))
+    assert cut > 0, "this shape was meant to exercise the shared-tile path"
+
+    g = gen(7 + n + k)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
+    m_total, e = sum(sizes), len(sizes)
+    a = _q(vals[torch.randint(0, 8, (m_total, k), generator=g)].to(torch.bfloat16), a_dtype)
+    b = _q(vals[torch.randint(0, 8, (e, n, k), generator=g)].to(torch.bfloat16), E4M3)
+    sa, sb = _scalars([0.5] * e), _scalars([2.0] * e)
+    c = torch.zeros(m_total, n, dtype=torch.bfloat16)
+    ref.fp8_gmm(a, b, sizes, sa, sb, c)  # the blocked oracle GEMM: with exact sums the order does not matter
+    gs = torch.tensor(sizes)
+    dsa, dsb = torch.tensor([0.5] * e, device=dev), torch.tensor([2.0] * e, device=dev)
+    dc = backend.fp8_gmm(a.to(dev), b.to(dev), gs, dsa, dsb, backward=(a_dtype == E5M2))
+    assert torch.equal(dc.cpu().view(torch.int16), c.view(torch.int16))
+    if a_dtype == E4M3:
+        # the fp8 + GELU + pre-activation + amax epilogue runs in the fix-up pass for the shared tiles
+        cg = torch.empty(m_total, n, dtype=E4M3, device=dev)
+        pre = torch.empty(m_total, n, dtype=torch.bfloat16, device=dev)
+        am = torch.zeros(e, device=dev)
+        cs = torch.tensor([0.25] * e, device=dev)
+        backend.fp8_gmm(a.to(dev), b.to(dev), gs, dsa, dsb, cg, E4M3, pre, cs, am)
+        assert torch.equal(pre.cpu().view(torch.int16), c.view(torch.int16))
+        # the kernel applies GELU to the fp32 value, before the bf16 rounding of the pre-activation copy
+        c32 = torch.zeros(m_total, n)
+        row = 0
+        for i, m in enumerate(sizes):
+            c32[row:row + m] = a[row:row + m].float() @ b[i].float().T
+            row += m
+        gelu = torch.nn.functional.gelu(c32, approximate="tanh")
+        want = ref.f32_to_fp8((gelu * 0.25).contiguous(), E4M3)
+        assert _fp8_code_distance(cg.cpu(), want).max() <= 1
+        row = 0
+        for i, m in enumerate(sizes):
+            if m:
+                assert torch.allclose(am[i].cpu(), gelu[row:row + m].abs().max(), rtol=1e-3)
+            row += m
+
+
 def test_identity_weights_reproduce_a(dev):
     backend = _backend()
     g = gen(7)
