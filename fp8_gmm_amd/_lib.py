@@ -59,7 +59,7 @@ GEMM_PROBLEM = np.dtype(
         ("ldb", "<i4"),
         ("ldc", "<i4"),
         ("tile_begin", "<i4"),
-        ("tiles_n", "<i4"),
+        ("cost_begin", "<i4"),
     ],
     align=False,
 )
@@ -78,6 +78,7 @@ EXPORTS = (
     "fp8gmm_multi_pad_cast_transpose",
     "fp8gmm_multi_pad_cast_transpose_dgelu",
     "fp8gmm_grouped_gemm",
+    "fp8gmm_delayed_scaling_update",
     "fp8gmm_gemm_schedule",
     "fp8gmm_gemm_fixup",
 )
@@ -132,6 +133,8 @@ def load():
     L.fp8gmm_multi_pad_cast_transpose_dgelu.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_grouped_gemm.restype = ci
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
+    L.fp8gmm_delayed_scaling_update.restype = ci
+    L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, vp]
     L.fp8gmm_gemm_schedule.restype = ci
     L.fp8gmm_gemm_schedule.argtypes = [vp, ci, ci, ci, ci, ci, vp, ci]
     L.fp8gmm_gemm_fixup.restype = ci

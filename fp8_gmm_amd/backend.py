@@ -348,6 +348,22 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device):
     _lib.check(rc)
 
 
+def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False):
+    """In-place delayed-scaling update of one direction in ONE kernel (the rule of
+    ``fp8.amax_and_scale_update``): ``amax_history`` [history, slots], ``scale`` / ``scale_inv`` [slots]."""
+    for t, what in ((amax_history, "amax_history"), (scale, "scale"), (scale_inv, "scale_inv")):
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            _fail(f"fp8_gmm_amd: {what} must be a contiguous fp32 tensor")
+    if amax_history.dim() != 2 or scale.numel() != amax_history.shape[1] or scale_inv.numel() != scale.numel():
+        _fail("fp8_gmm_amd: amax_history must be [history, slots] and scale / scale_inv [slots]")
+    dev = _device_of([amax_history, scale, scale_inv])
+    with torch.cuda.device(dev):
+        rc = _lib.load().fp8gmm_delayed_scaling_update(
+            amax_history.data_ptr(), scale.data_ptr(), scale_inv.data_ptr(), amax_history.shape[0],
+            amax_history.shape[1], float(fp8_max), int(margin), int(bool(most_recent)), _stream(dev))
+    _lib.check(rc)
+
+
 def _check_2d(t, what):
     if t.dim() != 2:
         _fail(f"fp8_gmm_amd: {what} must be 2-D")

@@ -42,6 +42,7 @@ struct Sched {
   int sk_begin;                // first tile of the stream-K region (== range_end: none)
   int sk_wgs;                  // workgroups that take a piece of the region
   int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (pair steps)
+  int64_t total_cost;          // cost of all tiles
 };
 
 FP8GMM_HD int problem_end_tile(const Sched& s, int p) {
@@ -61,40 +62,27 @@ FP8GMM_HD int64_t tile_cost(const Sched& s, int p) {
   const int c = (s.probs[p].k + 127) / 128;
   return (int64_t)(c > 0 ? c : 1);
 }
-// cost of all tiles before `tile`
+// cost of all tiles before `tile` (0 <= tile <= total_tiles); cost_begin is the plan's prefix sum
 FP8GMM_HD int64_t cost_before(const Sched& s, int tile) {
-  int64_t cum = 0;
-  for (int p = 0; p < s.nprob; ++p) {
-    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
-    if (tile <= t_begin) break;
-    cum += (int64_t)((tile < t_end ? tile : t_end) - t_begin) * tile_cost(s, p);
+  const int p = problem_of_tile(s, tile);
+  return (int64_t)s.probs[p].cost_begin + (int64_t)(tile - s.probs[p].tile_begin) * tile_cost(s, p);
+}
+// the tile that holds cost offset c: cost_before(t) <= c < cost_before(t + 1); total_tiles past the end
+FP8GMM_HD int tile_holding_cost(const Sched& s, int64_t c) {
+  if (c >= s.total_cost) return s.total_tiles;
+  int lo = 0, hi = s.nprob - 1;  // last problem whose prefix is <= c: it is not empty, as c < total_cost
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if ((int64_t)s.probs[mid].cost_begin <= c) lo = mid; else hi = mid - 1;
   }
-  return cum;
+  return s.probs[lo].tile_begin + (int)((c - s.probs[lo].cost_begin) / tile_cost(s, lo));
 }
 // first tile whose preceding cost is >= c (total_tiles if there is none)
 FP8GMM_HD int first_tile_at_cost(const Sched& s, int64_t c) {
-  int64_t cum = 0;
-  for (int p = 0; p < s.nprob; ++p) {
-    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
-    const int64_t tc = tile_cost(s, p), n_t = t_end - t_begin;
-    if (cum + n_t * tc > c - tc) {  // some tile i of p has cum + i tc >= c
-      const int64_t i = c > cum ? (c - cum + tc - 1) / tc : 0;
-      if (i < n_t) return t_begin + (int)i;
-    }
-    cum += n_t * tc;
-  }
-  return s.total_tiles;
-}
-// the tile that holds cost offset c: cost_before(t) <= c < cost_before(t + 1)
-FP8GMM_HD int tile_holding_cost(const Sched& s, int64_t c) {
-  int64_t cum = 0;
-  for (int p = 0; p < s.nprob; ++p) {
-    const int t_begin = s.probs[p].tile_begin, t_end = problem_end_tile(s, p);
-    const int64_t tc = tile_cost(s, p), n_t = t_end - t_begin;
-    if (c < cum + n_t * tc) return t_begin + (int)((c - cum) / tc);
-    cum += n_t * tc;
-  }
-  return s.total_tiles;
+  if (c <= 0) return 0;
+  const int t = tile_holding_cost(s, c);
+  if (t >= s.total_tiles) return s.total_tiles;
+  return cost_before(s, t) == c ? t : t + 1;
 }
 
 // Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal COST (k differs
@@ -106,7 +94,8 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   s.nprob = nprob;
   s.total_tiles = total_tiles;
   s.wgs = wgs_per_xcd;
-  const int64_t total_cost = cost_before(s, total_tiles);
+  s.total_cost = 0;
+  const int64_t total_cost = s.total_cost = cost_before(s, total_tiles);
   const int64_t lo = (total_cost * xcd + kNumXcd - 1) / kNumXcd;
   const int64_t hi = (total_cost * (xcd + 1) + kNumXcd - 1) / kNumXcd;
   s.range_begin = first_tile_at_cost(s, lo);

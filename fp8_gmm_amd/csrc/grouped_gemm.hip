@@ -609,7 +609,7 @@ void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n) {
 int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles) {
   if (n < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (total_tiles == nullptr || (n > 0 && probs == nullptr)) return FP8GMM_ERR_NULL_POINTER;
-  int64_t tiles = 0;
+  int64_t tiles = 0, cost = 0;
   for (int i = 0; i < n; ++i) {
     fp8gmm_gemm_problem& p = probs[i];
     if (p.m < 0 || p.n < 0 || p.k < 0) return FP8GMM_ERR_BAD_SHAPE;
@@ -630,9 +630,11 @@ int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles
     const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;
     const int64_t tn = (p.n + fp8gmm::BN - 1) / fp8gmm::BN;
     p.tile_begin = (int32_t)tiles;
-    p.tiles_n = (int32_t)tn;
+    p.cost_begin = (int32_t)cost;  // a tile costs ceil(k / 128) steps of the main loop (1 for k = 0)
+    const int64_t steps = (p.k + 127) / 128;
     tiles += tm * tn;
-    if (tiles > INT32_MAX / 16) return FP8GMM_ERR_BAD_SHAPE;
+    cost += tm * tn * (steps > 0 ? steps : 1);
+    if (tiles > INT32_MAX / 16 || cost > INT32_MAX / 2) return FP8GMM_ERR_BAD_SHAPE;
   }
   *total_tiles = (int)tiles;
   return FP8GMM_OK;

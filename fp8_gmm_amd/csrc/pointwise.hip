@@ -132,10 +132,56 @@ __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gm
   }
 }
 
+// Delayed-scaling update of one direction, one lane per scaling slot (columns of the [history, slots]
+// amax matrix are independent, rows of a column are walked by the lane that owns it):
+//   amax      = max over the history column (or its row 0)
+//   scale     = (1 / amax) * fp8_max * 2^-margin   where amax is finite and > 0, else unchanged
+//   scale_inv = 1 / scale
+//   history   : row i <- row i + 1, last row <- old row 0, then row 0 <- 0 (a history of one row is just cleared)
+// The factor is formed as reciprocal times fp8_max, which is what `fp8_max / amax` on a torch tensor
+// evaluates to; the two differ in the last bit for some inputs.
+__global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __restrict__ history,
+                                                                     float* __restrict__ scale,
+                                                                     float* __restrict__ scale_inv, int history_len,
+                                                                     int slots, float fp8_max, float margin_factor,
+                                                                     int most_recent) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= slots) return;
+  float* col = history + c;
+  const float first = col[0];
+  float amax = first;
+  if (!most_recent) {
+    // torch.max semantics: a NaN anywhere in the column wins
+    for (int i = 1; i < history_len; ++i) {
+      const float v = col[(size_t)i * slots];
+      amax = (v > amax || v != v) ? v : amax;
+    }
+  }
+  float sc = scale[c];
+  if (amax > 0.f && amax <= 3.4028234663852886e38f) sc = ((1.0f / amax) * fp8_max) * margin_factor;
+  scale[c] = sc;
+  scale_inv[c] = 1.0f / sc;
+  for (int i = 0; i + 1 < history_len; ++i) col[(size_t)i * slots] = col[(size_t)(i + 1) * slots];
+  if (history_len > 1) col[(size_t)(history_len - 1) * slots] = first;
+  col[0] = 0.f;
+}
+
 }  // namespace
 }  // namespace fp8gmm
 
 extern "C" {
+
+int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
+                                  float fp8_max, int margin, int most_recent, void* stream) {
+  if (history_len < 1 || slots < 0 || margin < -126 || margin > 126) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (slots == 0) return FP8GMM_OK;
+  if (amax_history == nullptr || scale == nullptr || scale_inv == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  const float margin_factor = __builtin_ldexpf(1.0f, -margin);
+  hipLaunchKernelGGL(fp8gmm::delayed_scaling_update_kernel, dim3((slots + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), amax_history, scale, scale_inv, history_len, slots, fp8_max,
+                     margin_factor, most_recent != 0);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
 
 int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
   if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;

@@ -117,12 +117,19 @@ class Fp8MetaTensors:
 
 
 def amax_and_scale_update(meta, fp8_max, fp8_recipe):
-    """Delayed-scaling update of one direction, in place (rule in the module docstring)."""
+    """Delayed-scaling update of one direction, in place (rule in the module docstring).
+
+    Scaling state that lives on the GPU is updated by one fused kernel
+    (``backend.delayed_scaling_update``); the torch statement of the rule below serves CPU tensors
+    (host-side tests of the bookkeeping) and is what the kernel is checked against bit for bit."""
     hist = meta.amax_history
-    if fp8_recipe.amax_compute_algo == "max":
-        amax = hist.max(dim=0).values
-    else:
-        amax = hist[0].clone()
+    most_recent = fp8_recipe.amax_compute_algo != "max"
+    if hist.is_cuda and float(fp8_recipe.margin) == int(fp8_recipe.margin):
+        from . import backend
+
+        backend.delayed_scaling_update(hist, meta.scale, meta.scale_inv, fp8_max, int(fp8_recipe.margin), most_recent)
+        return
+    amax = hist[0].clone() if most_recent else hist.max(dim=0).values
     sf = (fp8_max / amax) / (2.0 ** fp8_recipe.margin)
     ok = (amax > 0) & torch.isfinite(amax)
     meta.scale.copy_(torch.where(ok, sf, meta.scale))

@@ -118,7 +118,7 @@ typedef struct fp8gmm_gemm_problem {
   int32_t m, n, k;
   int32_t lda, ldb, ldc;
   int32_t tile_begin;        /* filled by fp8gmm_plan_grouped_gemm */
-  int32_t tiles_n;           /* filled by fp8gmm_plan_grouped_gemm */
+  int32_t cost_begin;        /* filled by fp8gmm_plan_grouped_gemm: K = 128 steps of all earlier tiles */
 } fp8gmm_gemm_problem;       /* 96 bytes */
 
 /* epilogue flags of fp8gmm_grouped_gemm */
@@ -138,7 +138,7 @@ void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n);
  * MultiPad* (csrc/multi_pointwise.cu:155-189,216-246; csrc/multi_pad_fusion.cu:442-488,505-559,587-644). */
 int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* total_blocks);
 
-/* Validates `probs[0..n)`, fills tile_begin / tiles_n, returns the tile count in *total_tiles.
+/* Validates `probs[0..n)`, fills tile_begin / cost_begin, returns the tile count in *total_tiles.
  * Replaces the host half of CutlassFp8GroupedGemm (csrc/fp8_gmm.cu:82-135). */
 int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles);
 
@@ -166,6 +166,17 @@ int fp8gmm_multi_pad_cast_transpose_dgelu(const fp8gmm_tensor_desc* descs_dev, i
  */
 int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int a_fmt, int b_fmt,
                         int out_kind, int epilogue, void* stream);
+
+/*
+ * Delayed-scaling update of one direction, in place, for `slots` scaling factors:
+ *   amax = max over the `history_len` rows of amax_history[history_len, slots] (most_recent != 0: row 0)
+ *   scale = (1 / amax) * fp8_max * 2^-margin where amax is finite and > 0, else unchanged;  scale_inv = 1 / scale
+ *   the history moves up by one row (the last row receives the old row 0) and row 0 is cleared.
+ * replaces the amax_and_scale_update of TransformerEngine's base module, which the reference's modules run
+ * through `self.prepare_forward(...)` (fp8_gmm/grouped_linear.py:206, fp8_gmm/grouped_mlp.py:349).
+ */
+int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
+                                  float fp8_max, int margin, int most_recent, void* stream);
 
 /* ---- schedule introspection (host only, no GPU needed) ------------------------------------ */
 /*

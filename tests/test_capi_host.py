@@ -99,7 +99,8 @@ def test_plan_grouped_gemm_tiles():
     t = _prob([137, 0, 401, 256, 300], [512, 512, 512, 257, 64], [256, 256, 256, 0, 16])
     total = _lib.plan_grouped_gemm(t)
     assert t["tile_begin"].tolist() == [0, 2, 2, 6, 8]   # 1x2, 0, 2x2, 1x2, 2x1 tiles of 256 x 256
-    assert t["tiles_n"].tolist() == [2, 2, 2, 2, 1]
+    # K = 128 steps of all earlier tiles: 2 tiles x 2 steps, none, 4 x 2, 2 tiles without K count 1 each
+    assert t["cost_begin"].tolist() == [0, 4, 4, 12, 14]
     assert total == 10
 
 

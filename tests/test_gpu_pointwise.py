@@ -285,3 +285,35 @@ def test_misaligned_views_take_the_scalar_path(dev):
     assert_bytes_equal(do, o, "cast")
     assert_bytes_equal(dt, t, "transpose")
     assert_scalar_bits_equal(da, a, "amax")
+
+
+@pytest.mark.parametrize("history_len,slots,margin,algo", [(1, 1, 0, "max"), (3, 4, 1, "max"), (16, 771, 0, "max"),
+                                                          (5, 384, 2, "most_recent"), (1024, 6, 0, "max")])
+def test_delayed_scaling_update_matches_the_torch_rule(dev, history_len, slots, margin, algo):
+    """The fused update kernel against the torch statement of the rule (fp8.amax_and_scale_update on CPU
+    tensors, itself checked against the oracle's Meta.update in the host tests): scale, scale_inv and the
+    rolled history bit for bit, including columns whose amax is 0, inf, NaN or denormal."""
+    from fp8_gmm_amd import fp8
+
+    g = gen(41 + history_len + slots)
+    hist = torch.rand(history_len, slots, generator=g) * 10.0 ** torch.randint(-6, 6, (1, slots), generator=g).float()
+    specials = [0.0, float("inf"), float("nan"), 1e-42, 3.0e38, 448.0, 1.0]
+    for j, v in enumerate(specials):
+        if j < slots:
+            hist[:, j] = 0.0 if v != v or v == float("inf") else v
+            hist[(j * 7) % history_len, j] = v
+    recipe = fp8.DelayedScaling(margin=margin, amax_history_len=history_len, amax_compute_algo=algo)
+    cpu = fp8.Fp8MetaTensors(slots, history_len, torch.device("cpu"))
+    gpu = fp8.Fp8MetaTensors(slots, history_len, dev)
+    start_scale = torch.rand(slots, generator=g) + 0.5
+    cpu.amax_history.copy_(hist), cpu.scale.copy_(start_scale)
+    gpu.amax_history.copy_(hist), gpu.scale.copy_(start_scale)
+    for step in range(3):
+        fp8.amax_and_scale_update(cpu, 448.0, recipe)
+        fp8.amax_and_scale_update(gpu, 448.0, recipe)
+        for name in ("scale", "scale_inv", "amax_history"):
+            a, b = getattr(gpu, name).cpu(), getattr(cpu, name)
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), f"{name} differs at step {step}"
+        bump = torch.rand(slots, generator=g) * 3.0
+        cpu.amax_history[0] += bump
+        gpu.amax_history[0] += bump.to(dev)
