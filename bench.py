@@ -54,6 +54,13 @@ def splits(kind, experts, tokens, seed):
     return [int(v) for v in rng.multinomial(tokens, p)]
 
 
+# HBM bytes per grouped-GEMM launch (reads + writes), from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs whose
+# summary is profiles/config2_mlp_step_hbm_traffic.md (counter units calibrated against a 256 MiB copy:
+# 2 KiB per FETCH_SIZE unit, 1 KiB per WRITE_SIZE unit).  Counters cannot be read from inside this process,
+# so the figure is carried here; the algorithmic bytes of one launch are 1.09 GB.
+GEMM_HBM_TRAFFIC_BYTES = {"config2": 3.20e9}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -137,7 +144,7 @@ def main():
                                  "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4)}
                 roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
                             "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),
-                            "traffic": None}
+                            "traffic": GEMM_HBM_TRAFFIC_BYTES.get(args.workload)}
             else:
                 gbs = d["work"] / (d["ms"] * 1e-3) / 1e9
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
