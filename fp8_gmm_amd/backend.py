@@ -139,6 +139,10 @@ def _scalar_ptrs(scalars, n, what):
     """Device addresses of n fp32 scalars given as a list of 0-d / 1-element tensors, a 1-D tensor, or None."""
     if scalars is None:
         return np.zeros(n, dtype=np.uint64)
+    if isinstance(scalars, np.ndarray):  # device addresses already (Fp8MetaWrapper.get_meta_pointers)
+        if scalars.dtype != np.uint64 or scalars.shape != (n,):
+            _fail(f"fp8_gmm_amd: expected {n} device addresses for {what}")
+        return scalars
     if isinstance(scalars, torch.Tensor):
         if scalars.dtype != torch.float32 or scalars.numel() != n or not scalars.is_contiguous():
             _fail(f"fp8_gmm_amd: {what} must be {n} contiguous fp32 values")
@@ -179,20 +183,147 @@ def _launch_multi(op, table, out_fmt, device):
     _lib.check(rc)
 
 
-def _check_lists(n, **lists):
-    for name, lst in lists.items():
-        if len(lst) != n:
-            _fail(f"fp8_gmm_amd: {name} has {len(lst)} entries, expected {n}")
+class TensorBatch:
+    """n row-major 2-D tensors of one dtype on one device, held as arrays (address, rows, columns, row
+    pitch in elements) instead of n tensor objects.
+
+    The reference's entry points take Python lists of per-expert tensor views; with a hundred experts
+    creating and inspecting those views costs more host time than the kernels run.  The modules
+    therefore describe "rows bounds[i]:bounds[i+1] of this tensor", "slice i of this stack" or "block i
+    of this buffer seen transposed" with array arithmetic on one base address.  Every entry point that
+    takes a list of tensors also takes a TensorBatch."""
+
+    __slots__ = ("ptr", "rows", "cols", "pitch", "dtype", "device", "_keep")
+
+    def __init__(self, ptr, rows, cols, pitch, dtype, device, keep=()):
+        n = len(ptr)
+        self.ptr = np.asarray(ptr, dtype=np.uint64)
+        self.rows = np.broadcast_to(np.asarray(rows, dtype=np.int64), (n,))
+        self.cols = np.broadcast_to(np.asarray(cols, dtype=np.int64), (n,))
+        self.pitch = np.broadcast_to(np.asarray(pitch, dtype=np.int64), (n,))
+        self.dtype = dtype
+        self.device = device
+        self._keep = tuple(keep)  # the tensors whose memory is described stay alive with the batch
+
+    def __len__(self):
+        return len(self.ptr)
+
+    @property
+    def contiguous(self):
+        return bool(np.all((self.pitch == self.cols) | (self.rows <= 1) | (self.cols == 0)))
+
+    @staticmethod
+    def rows_of(t, bounds):
+        """Row blocks bounds[i]:bounds[i+1] of a contiguous 2-D tensor."""
+        if t.dim() != 2 or not t.is_contiguous():
+            _fail("fp8_gmm_amd: row blocks need a contiguous 2-D tensor")
+        b = np.asarray(bounds, dtype=np.int64)
+        cols = t.shape[1]
+        ptr = np.uint64(t.data_ptr()) + (b[:-1] * (cols * t.element_size())).astype(np.uint64)
+        return TensorBatch(ptr, np.diff(b), cols, cols, t.dtype, t.device, (t,))
+
+    @staticmethod
+    def stack_of(t):
+        """The slices t[i] of a contiguous [n, rows, cols] tensor."""
+        if t.dim() != 3 or not t.is_contiguous():
+            _fail("fp8_gmm_amd: a stack needs a contiguous 3-D tensor")
+        n, r, c = t.shape
+        ptr = np.uint64(t.data_ptr()) + np.arange(n, dtype=np.uint64) * np.uint64(r * c * t.element_size())
+        return TensorBatch(ptr, r, c, c, t.dtype, t.device, (t,))
+
+    @staticmethod
+    def transposed_blocks_of(flat, bounds):
+        """Block i = rows bounds[i]:bounds[i+1] of the contiguous buffer flat[sum, features], reinterpreted as
+        the [features, bounds[i+1] - bounds[i]] transpose that the pad/transpose kernels write."""
+        if flat.dim() != 2 or not flat.is_contiguous():
+            _fail("fp8_gmm_amd: transposed blocks need a contiguous 2-D buffer")
+        b = np.asarray(bounds, dtype=np.int64)
+        feat = flat.shape[1]
+        ptr = np.uint64(flat.data_ptr()) + (b[:-1] * (feat * flat.element_size())).astype(np.uint64)
+        width = np.diff(b)
+        return TensorBatch(ptr, feat, width, width, flat.dtype, flat.device, (flat,))
+
+    @staticmethod
+    def concat(batches):
+        batches = [b for b in batches if b is not None and len(b)]
+        if not batches:
+            return None
+        first = batches[0]
+        for b in batches[1:]:
+            if b.dtype != first.dtype:
+                _fail("fp8_gmm_amd: all tensors of one argument must share a dtype")
+            if b.device != first.device:
+                _fail("fp8_gmm_amd: all tensors of one call must live on the same device")
+        keep = tuple(t for b in batches for t in b._keep)
+        return TensorBatch(np.concatenate([b.ptr for b in batches]), np.concatenate([b.rows for b in batches]),
+                           np.concatenate([b.cols for b in batches]), np.concatenate([b.pitch for b in batches]),
+                           first.dtype, first.device, keep)
+
+    def __add__(self, other):
+        return TensorBatch.concat([self, other])
 
 
-def _common_fp8_dtype(outputs):
-    dt = outputs[0].dtype
+def _as_batch(tensors, what, flatten=False):
+    """A list of tensors (the reference's calling convention) as a TensorBatch.  flatten: any contiguous
+    shape, seen as one row of numel elements; otherwise 2-D with a contiguous last dimension."""
+    if isinstance(tensors, TensorBatch):
+        return tensors
+    tensors = list(tensors)
+    n = len(tensors)
+    dev = _device_of(tensors)
+    ptr = np.zeros(n, dtype=np.uint64)
+    rows = np.zeros(n, dtype=np.int64)
+    cols = np.zeros(n, dtype=np.int64)
+    pitch = np.zeros(n, dtype=np.int64)
+    dtype = tensors[0].dtype if n else None
+    for i, t in enumerate(tensors):
+        if t.dtype != dtype:
+            _fail(f"fp8_gmm_amd: all {what} of one call must share one dtype")
+        ptr[i] = t.data_ptr()
+        if flatten:
+            if not t.is_contiguous():
+                _fail(f"fp8_gmm_amd: {what} must be contiguous")
+            numel = t.numel()
+            rows[i], cols[i], pitch[i] = (1 if numel else 0), numel, numel
+        else:
+            if t.dim() != 2:
+                _fail(f"fp8_gmm_amd: {what} must be 2-D")
+            r, c = t.shape
+            if c > 1 and t.stride(1) != 1:
+                _fail(f"fp8_gmm_amd: {what} must have a contiguous last dimension")
+            rows[i], cols[i] = r, c
+            pitch[i] = t.stride(0) if (r > 1 and c > 0 and not t.is_contiguous()) else c
+    return TensorBatch(ptr, rows, cols, pitch, dtype, dev, tensors)
+
+
+def _same_device(*batches):
+    dev = None
+    for b in batches:
+        if b is None:
+            continue
+        if b.device is None or b.device.type != "cuda":
+            _fail("fp8_gmm_amd: expected GPU tensors (the HIP path has no CPU fallback)")
+        if dev is None:
+            dev = b.device
+        elif b.device != dev:
+            _fail("fp8_gmm_amd: all tensors of one call must live on the same device")
+    return dev
+
+
+def _fp8_dtype_of(*batches):
+    dt = batches[0].dtype
     if dt not in _FP8_DTYPES:
         _fail("fp8_gmm_amd: outputs must be float8_e4m3fn or float8_e5m2")
-    for o in outputs:
-        if o.dtype != dt:
+    for b in batches[1:]:
+        if b.dtype != dt:
             _fail("fp8_gmm_amd: all fp8 outputs of one call must share one fp8 dtype")
     return dt
+
+
+def _check_counts(n, **args):
+    for name, a in args.items():
+        if len(a) != n:
+            _fail(f"fp8_gmm_amd: {name} has {len(a)} entries, expected {n}")
 
 
 # ------------------------------------------------------------------------------------------------
@@ -203,24 +334,23 @@ def multi_quantize(inputs, outputs, scales, amaxes):
     n = len(inputs)
     if n == 0:
         return
-    _check_lists(n, outputs=outputs, scales=scales, amaxes=amaxes)
-    dev = _device_of(list(inputs) + list(outputs))
-    dt = _common_fp8_dtype(outputs)
+    _check_counts(n, outputs=outputs, scales=scales, amaxes=amaxes)
+    x, o = _as_batch(inputs, "multi_quantize inputs", flatten=True), _as_batch(outputs, "outputs", flatten=True)
+    dev = _same_device(x, o)
+    dt = _fp8_dtype_of(o)
+    if x.dtype != torch.bfloat16:
+        _fail("fp8_gmm_amd: multi_quantize inputs must be bfloat16")
+    if not (x.contiguous and o.contiguous):
+        _fail("fp8_gmm_amd: multi_quantize needs contiguous tensors")
+    numel = x.rows * x.cols
+    if np.any(numel != o.rows * o.cols):
+        _fail("fp8_gmm_amd: multi_quantize input / output shapes differ")
+    if np.any(numel >= 2**31):
+        _fail("fp8_gmm_amd: tensors of 2^31 or more elements are not supported")
     table = np.zeros(n, dtype=TENSOR_DESC)
-    for i, (x, o) in enumerate(zip(inputs, outputs)):
-        if x.dtype != torch.bfloat16:
-            _fail("fp8_gmm_amd: multi_quantize inputs must be bfloat16")
-        if x.shape != o.shape:
-            _fail("fp8_gmm_amd: multi_quantize input / output shapes differ")
-        if not (x.is_contiguous() and o.is_contiguous()):
-            _fail("fp8_gmm_amd: multi_quantize needs contiguous tensors")
-        table["in"][i] = x.data_ptr()
-        table["out"][i] = o.data_ptr()
-        numel = x.numel()
-        if numel >= 2**31:
-            _fail("fp8_gmm_amd: tensors of 2^31 or more elements are not supported")
-        table["rows"][i] = 1 if numel else 0
-        table["cols"][i] = numel
+    table["in"], table["out"] = x.ptr, o.ptr
+    table["rows"] = (numel > 0).astype(np.int32)
+    table["cols"] = numel
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
     _launch_multi(_lib.OP_QUANTIZE, table, _FMT[dt], dev)
@@ -231,34 +361,33 @@ def multi_scale_mul(inputs, scales_1, scales_2):
     n = len(inputs)
     if n == 0:
         return
-    _check_lists(n, scales_1=scales_1, scales_2=scales_2)
-    dev = _device_of(inputs)
+    _check_counts(n, scales_1=scales_1, scales_2=scales_2)
+    x = _as_batch(inputs, "multi_scale_mul inputs", flatten=True)
+    dev = _same_device(x)
+    if x.dtype != torch.bfloat16:
+        _fail("fp8_gmm_amd: multi_scale_mul inputs must be bfloat16")
+    if not x.contiguous:
+        _fail("fp8_gmm_amd: multi_scale_mul needs contiguous tensors")
+    numel = x.rows * x.cols
     table = np.zeros(n, dtype=TENSOR_DESC)
-    for i, x in enumerate(inputs):
-        if x.dtype != torch.bfloat16:
-            _fail("fp8_gmm_amd: multi_scale_mul inputs must be bfloat16")
-        if not x.is_contiguous():
-            _fail("fp8_gmm_amd: multi_scale_mul needs contiguous tensors")
-        table["in"][i] = x.data_ptr()
-        numel = x.numel()
-        table["rows"][i] = 1 if numel else 0
-        table["cols"][i] = numel
+    table["in"] = x.ptr
+    table["rows"] = (numel > 0).astype(np.int32)
+    table["cols"] = numel
     table["scale"] = _scalar_ptrs(scales_1, n, "scales_1")
     table["in2"] = _scalar_ptrs(scales_2, n, "scales_2")
     _launch_multi(_lib.OP_SCALE_MUL, table, _lib.E4M3, dev)
 
 
-def _fill_transpose_shapes(table, i, x, t):
-    if x.dim() != 2 or t.dim() != 2:
-        _fail("fp8_gmm_amd: transposes work on 2-D tensors")
-    m, ncols = x.shape
-    if t.shape[0] != ncols or t.shape[1] < m:
+def _fill_transpose_shapes(table, x, t):
+    if np.any(t.rows != x.cols) or np.any(t.cols < x.rows):
         _fail("fp8_gmm_amd: transposed output must be [cols, M] with M >= rows")
-    if not (x.is_contiguous() and t.is_contiguous()):
+    if not (x.contiguous and t.contiguous):
         _fail("fp8_gmm_amd: transposes need contiguous tensors")
-    table["rows"][i] = m
-    table["cols"][i] = ncols
-    table["rows_padded"][i] = t.shape[1]
+    if np.any(x.rows >= 2**31) or np.any(x.cols >= 2**31) or np.any(t.cols >= 2**31):
+        _fail("fp8_gmm_amd: tensor extents of 2^31 or more are not supported")
+    table["rows"] = x.rows
+    table["cols"] = x.cols
+    table["rows_padded"] = t.cols
 
 
 def multi_transpose(inputs, outputs):
@@ -266,15 +395,14 @@ def multi_transpose(inputs, outputs):
     n = len(inputs)
     if n == 0:
         return
-    _check_lists(n, outputs=outputs)
-    dev = _device_of(list(inputs) + list(outputs))
+    _check_counts(n, outputs=outputs)
+    x, t = _as_batch(inputs, "multi_transpose inputs"), _as_batch(outputs, "multi_transpose outputs")
+    dev = _same_device(x, t)
+    if x.dtype not in _FP8_DTYPES or x.dtype != t.dtype:
+        _fail("fp8_gmm_amd: multi_transpose needs fp8 inputs and outputs of the same dtype")
     table = np.zeros(n, dtype=TENSOR_DESC)
-    for i, (x, t) in enumerate(zip(inputs, outputs)):
-        if x.dtype not in _FP8_DTYPES or x.dtype != t.dtype:
-            _fail("fp8_gmm_amd: multi_transpose needs fp8 inputs and outputs of the same dtype")
-        _fill_transpose_shapes(table, i, x, t)
-        table["in"][i] = x.data_ptr()
-        table["out_t"][i] = t.data_ptr()
+    _fill_transpose_shapes(table, x, t)
+    table["in"], table["out_t"] = x.ptr, t.ptr
     _launch_multi(_lib.OP_PAD_TRANSPOSE, table, _lib.E4M3, dev)
 
 
@@ -283,19 +411,19 @@ def multi_cast_transpose(inputs, outputs, trans_outputs, scales, amaxes):
     n = len(inputs)
     if n == 0:
         return
-    _check_lists(n, outputs=outputs, trans_outputs=trans_outputs, scales=scales, amaxes=amaxes)
-    dev = _device_of(list(inputs) + list(outputs) + list(trans_outputs))
-    dt = _common_fp8_dtype(list(outputs) + list(trans_outputs))
+    _check_counts(n, outputs=outputs, trans_outputs=trans_outputs, scales=scales, amaxes=amaxes)
+    x = _as_batch(inputs, "multi_cast_transpose inputs")
+    o = _as_batch(outputs, "multi_cast_transpose outputs")
+    t = _as_batch(trans_outputs, "multi_cast_transpose transposed outputs")
+    dev = _same_device(x, o, t)
+    dt = _fp8_dtype_of(o, t)
+    if x.dtype != torch.bfloat16:
+        _fail("fp8_gmm_amd: multi_cast_transpose inputs must be bfloat16")
+    if np.any(x.rows != o.rows) or np.any(x.cols != o.cols) or not o.contiguous:
+        _fail("fp8_gmm_amd: multi_cast_transpose input / output shapes differ or output not contiguous")
     table = np.zeros(n, dtype=TENSOR_DESC)
-    for i, (x, o, t) in enumerate(zip(inputs, outputs, trans_outputs)):
-        if x.dtype != torch.bfloat16:
-            _fail("fp8_gmm_amd: multi_cast_transpose inputs must be bfloat16")
-        if x.shape != o.shape or not o.is_contiguous():
-            _fail("fp8_gmm_amd: multi_cast_transpose input / output shapes differ or output not contiguous")
-        _fill_transpose_shapes(table, i, x, t)
-        table["in"][i] = x.data_ptr()
-        table["out"][i] = o.data_ptr()
-        table["out_t"][i] = t.data_ptr()
+    _fill_transpose_shapes(table, x, t)
+    table["in"], table["out"], table["out_t"] = x.ptr, o.ptr, t.ptr
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
     _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE, table, _FMT[dt], dev)
@@ -306,21 +434,22 @@ def multi_cast_transpose_dgelu(inputs, gelu_inputs, outputs, trans_outputs, scal
     n = len(inputs)
     if n == 0:
         return
-    _check_lists(n, gelu_inputs=gelu_inputs, outputs=outputs, trans_outputs=trans_outputs, scales=scales,
-                 amaxes=amaxes)
-    dev = _device_of(list(inputs) + list(gelu_inputs) + list(outputs) + list(trans_outputs))
-    dt = _common_fp8_dtype(list(outputs) + list(trans_outputs))
+    _check_counts(n, gelu_inputs=gelu_inputs, outputs=outputs, trans_outputs=trans_outputs, scales=scales,
+                  amaxes=amaxes)
+    x = _as_batch(inputs, "multi_cast_transpose_dgelu inputs")
+    g = _as_batch(gelu_inputs, "multi_cast_transpose_dgelu gelu inputs")
+    o = _as_batch(outputs, "multi_cast_transpose_dgelu outputs")
+    t = _as_batch(trans_outputs, "multi_cast_transpose_dgelu transposed outputs")
+    dev = _same_device(x, g, o, t)
+    dt = _fp8_dtype_of(o, t)
+    if x.dtype != torch.bfloat16 or g.dtype != torch.bfloat16:
+        _fail("fp8_gmm_amd: multi_cast_transpose_dgelu inputs must be bfloat16")
+    same = np.all(x.rows == o.rows) and np.all(x.cols == o.cols) and np.all(x.rows == g.rows) and np.all(x.cols == g.cols)
+    if not same or not (o.contiguous and g.contiguous):
+        _fail("fp8_gmm_amd: multi_cast_transpose_dgelu shapes differ or tensors not contiguous")
     table = np.zeros(n, dtype=TENSOR_DESC)
-    for i, (x, g, o, t) in enumerate(zip(inputs, gelu_inputs, outputs, trans_outputs)):
-        if x.dtype != torch.bfloat16 or g.dtype != torch.bfloat16:
-            _fail("fp8_gmm_amd: multi_cast_transpose_dgelu inputs must be bfloat16")
-        if x.shape != o.shape or x.shape != g.shape or not (o.is_contiguous() and g.is_contiguous()):
-            _fail("fp8_gmm_amd: multi_cast_transpose_dgelu shapes differ or tensors not contiguous")
-        _fill_transpose_shapes(table, i, x, t)
-        table["in"][i] = x.data_ptr()
-        table["in2"][i] = g.data_ptr()
-        table["out"][i] = o.data_ptr()
-        table["out_t"][i] = t.data_ptr()
+    _fill_transpose_shapes(table, x, t)
+    table["in"], table["in2"], table["out"], table["out_t"] = x.ptr, g.ptr, o.ptr, t.ptr
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
     _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE_DGELU, table, _FMT[dt], dev)
@@ -364,14 +493,6 @@ def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, mo
     _lib.check(rc)
 
 
-def _check_2d(t, what):
-    if t.dim() != 2:
-        _fail(f"fp8_gmm_amd: {what} must be 2-D")
-    if t.stride(1) != 1 and t.shape[1] > 1:
-        _fail(f"fp8_gmm_amd: {what} must have a contiguous last dimension")
-    return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], 1)
-
-
 def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_outs=None, c_scales=None,
                  c_amaxes=None):
     """c_list[i][m, n] = epilogue(a_list[i][m, k] . b_list[i][n, k]^T) for all i in ONE launch.
@@ -379,39 +500,37 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
     The list form of ``cublas_fp8_gemm``: the reference issues these as a Python loop of
     cuBLASLt calls (wgrad, grouped_linear.py:173-182; grouped_mlp.py:234-242,313-322).
     k may differ per entry and may be 0 (the output is then the epilogue of zero).
+    Lists of tensors or TensorBatches.
     """
     n = len(a_list)
     if n == 0:
         return
-    _check_lists(n, b_list=b_list, c_list=c_list)
-    dev = _device_of(list(a_list) + list(b_list) + list(c_list))
-    a_dt, b_dt, c_dt = a_list[0].dtype, b_list[0].dtype, c_list[0].dtype
-    fp8_out = c_dt in _FP8_DTYPES
+    _check_counts(n, b_list=b_list, c_list=c_list)
+    a, b, c = _as_batch(a_list, "a"), _as_batch(b_list, "b"), _as_batch(c_list, "c")
+    aux = None if pre_gelu_outs is None else _as_batch(pre_gelu_outs, "pre_gelu_outs")
+    dev = _same_device(a, b, c, aux)
+    fp8_out = c.dtype in _FP8_DTYPES
     if fp8_out and c_scales is None:
         _fail("fp8_gmm_amd: an fp8 GEMM output needs c_scales")
+    if np.any(a.cols != b.cols) or np.any(c.rows != a.rows) or np.any(c.cols != b.rows):
+        _fail("fp8_gmm_amd: GEMM shapes do not match: a [m, k], b [n, k], c [m, n]")
     table = np.zeros(n, dtype=GEMM_PROBLEM)
-    for i, (a, b, c) in enumerate(zip(a_list, b_list, c_list)):
-        if a.dtype != a_dt or b.dtype != b_dt or c.dtype != c_dt:
-            _fail("fp8_gmm_amd: all problems of one grouped GEMM must share dtypes")
-        lda, ldb, ldc = _check_2d(a, "a"), _check_2d(b, "b"), _check_2d(c, "c")
-        m, k = a.shape
-        nn, kb = b.shape
-        if k != kb or tuple(c.shape) != (m, nn):
-            _fail("fp8_gmm_amd: GEMM shapes do not match: a [m, k], b [n, k], c [m, n]")
-        table["a"][i], table["b"][i], table["c"][i] = a.data_ptr(), b.data_ptr(), c.data_ptr()
-        table["m"][i], table["n"][i], table["k"][i] = m, nn, k
-        table["lda"][i], table["ldb"][i], table["ldc"][i] = max(lda, k), max(ldb, k), max(ldc, nn)
-        if pre_gelu_outs is not None:
-            aux = pre_gelu_outs[i]
-            if aux.dtype != torch.bfloat16 or tuple(aux.shape) != (m, nn) or _check_2d(aux, "pre_gelu_out") != ldc:
-                _fail("fp8_gmm_amd: pre_gelu_out must be bf16 [m, n] with the row pitch of c")
-            table["aux"][i] = aux.data_ptr()
+    table["a"], table["b"], table["c"] = a.ptr, b.ptr, c.ptr
+    table["m"], table["n"], table["k"] = a.rows, b.rows, a.cols
+    table["lda"] = np.maximum(a.pitch, a.cols)
+    table["ldb"] = np.maximum(b.pitch, b.cols)
+    table["ldc"] = np.maximum(c.pitch, c.cols)
+    if aux is not None:
+        if len(aux) != n or aux.dtype != torch.bfloat16 or np.any(aux.rows != c.rows) or np.any(aux.cols != c.cols) \
+                or np.any(np.maximum(aux.pitch, aux.cols) != table["ldc"]):
+            _fail("fp8_gmm_amd: pre_gelu_out must be bf16 [m, n] with the row pitch of c")
+        table["aux"] = aux.ptr
     table["a_scale_inv"] = _scalar_ptrs(a_scale_invs, n, "a_scale_invs")
     table["b_scale_inv"] = _scalar_ptrs(b_scale_invs, n, "b_scale_invs")
     if fp8_out:
         table["c_scale"] = _scalar_ptrs(c_scales, n, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, n, "c_amaxes")
-    _launch_gemm(table, a_dt, b_dt, c_dt, pre_gelu_outs is not None, dev)
+    _launch_gemm(table, a.dtype, b.dtype, c.dtype, aux is not None, dev)
 
 
 def cublas_fp8_gemm(a, b, c, a_scale_inv, b_scale_inv, pre_gelu_out=None, c_scale=None, c_amax=None, backward=False):
@@ -502,6 +621,5 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
         table["c_amax"] = _scalar_ptrs(c_amaxes, e, "c_amaxes")
     _launch_gemm(table, a.dtype, b.dtype, c.dtype, pre_gelu_out is not None, dev)
     if cutlass:
-        c_groups = [c[starts[i]: starts[i + 1]] for i in range(e)]
-        multi_scale_mul(c_groups, a_scale_invs, b_scale_invs)
+        multi_scale_mul(TensorBatch.rows_of(c, starts), a_scale_invs, b_scale_invs)
     return c

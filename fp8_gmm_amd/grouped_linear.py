@@ -18,9 +18,10 @@ the two-rounding data flow of the reference's CUTLASS path, see ``backend.fp8_gm
 """
 import math
 
+import numpy as np
 import torch
 
-from .backend import fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
+from .backend import TensorBatch, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
 from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
@@ -33,27 +34,22 @@ MODULE_PAD_MULTIPLE = 128
 
 
 def row_slices(t, bounds):
-    """Per-expert row blocks of a token-major tensor."""
-    return [t[bounds[i]: bounds[i + 1]] for i in range(len(bounds) - 1)]
+    """Per-expert row blocks of a token-major tensor (described by arrays: no per-expert tensor objects)."""
+    return TensorBatch.rows_of(t, bounds)
 
 
 def transposed_views(flat, bounds):
-    """Per-expert ``[features, tokens_i]`` views of a flat ``[sum(tokens_i), features]`` buffer.
+    """Per-expert ``[features, tokens_i]`` blocks of a flat ``[sum(tokens_i), features]`` buffer.
 
     Expert i owns the contiguous block of rows ``bounds[i]:bounds[i+1]``; the block is
     reinterpreted as the transpose ``[features, bounds[i+1]-bounds[i]]``
     (reference grouped_linear.py:36-52).
     """
-    feat = flat.shape[1]
-    views = []
-    for i in range(len(bounds) - 1):
-        rows = bounds[i + 1] - bounds[i]
-        views.append(flat[bounds[i]: bounds[i + 1]].view(feat, rows) if rows > 0 else flat.new_empty((feat, 0)))
-    return views
+    return TensorBatch.transposed_blocks_of(flat, bounds)
 
 
 def alloc_transposed(features, padded, bounds, padded_bounds, dtype, device):
-    """Buffer + per-expert views for the transposed copy of a ``[tokens, features]`` operand."""
+    """Buffer + per-expert blocks for the transposed copy of a ``[tokens, features]`` operand."""
     b = padded_bounds if padded else bounds
     flat = torch.empty(b[-1], features, dtype=dtype, device=device)
     return flat, transposed_views(flat, b)
@@ -80,49 +76,45 @@ class _GroupedLinear(torch.autograd.Function):
 
         input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
         input_t_fp8 = None
-        x_scales = meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kScale)
-        x_amaxes = meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kAmax)
+        x_scales = meta.get_meta_pointers(Fp8TensorType.kInputGroup1, MetaTensorType.kScale)
+        x_amaxes = meta.get_meta_pointers(Fp8TensorType.kInputGroup1, MetaTensorType.kAmax)
         if wgrad_needed:
             input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums,
                                                       fp8_dtype, dev)
-            with_t[0].extend(row_slices(input, cumsums))
-            with_t[1].extend(row_slices(input_fp8, cumsums))
-            with_t[2].extend(x_t_views)
-            with_t[3].extend(x_scales)
-            with_t[4].extend(x_amaxes)
+            for lst, item in zip(with_t, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_t_views,
+                                          x_scales, x_amaxes)):
+                lst.append(item)
         else:
-            plain[0].extend(row_slices(input, cumsums))
-            plain[1].extend(row_slices(input_fp8, cumsums))
-            plain[2].extend(x_scales)
-            plain[3].extend(x_amaxes)
+            for lst, item in zip(plain, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_scales,
+                                         x_amaxes)):
+                lst.append(item)
 
         weight_fp8 = torch.empty(weight.shape, dtype=fp8_dtype, device=weight.device)
         weight_t_fp8 = None
-        w_scales = meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kScale)
-        w_amaxes = meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kAmax)
+        w_scales = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kScale)
+        w_amaxes = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kAmax)
         if dgrad_needed:
             weight_t_fp8 = torch.empty(num_groups, weight.size(2), weight.size(1), dtype=fp8_dtype,
                                        device=weight.device)
-            with_t[0].extend(weight.unbind(0))
-            with_t[1].extend(weight_fp8.unbind(0))
-            with_t[2].extend(weight_t_fp8.unbind(0))
-            with_t[3].extend(w_scales)
-            with_t[4].extend(w_amaxes)
+            for lst, item in zip(with_t, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8),
+                                          TensorBatch.stack_of(weight_t_fp8), w_scales, w_amaxes)):
+                lst.append(item)
         else:
-            plain[0].extend(weight.unbind(0))
-            plain[1].extend(weight_fp8.unbind(0))
-            plain[2].extend(w_scales)
-            plain[3].extend(w_amaxes)
+            for lst, item in zip(plain, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8), w_scales,
+                                         w_amaxes)):
+                lst.append(item)
 
         if plain[0]:
-            multi_quantize(*plain)
+            multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
+                           np.concatenate(plain[3]))
         if with_t[0]:
-            multi_cast_transpose(*with_t)
+            multi_cast_transpose(TensorBatch.concat(with_t[0]), TensorBatch.concat(with_t[1]),
+                                 TensorBatch.concat(with_t[2]), np.concatenate(with_t[3]), np.concatenate(with_t[4]))
 
         out = fp8_gmm(
             input_fp8, weight_fp8, group_sizes,
-            meta.get_meta_tensors(Fp8TensorType.kInputGroup1, MetaTensorType.kScaleInv),
-            meta.get_meta_tensors(Fp8TensorType.kWeightGroup1, MetaTensorType.kScaleInv),
+            meta.get_meta_pointers(Fp8TensorType.kInputGroup1, MetaTensorType.kScaleInv),
+            meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kScaleInv),
             backward=False, cutlass=cutlass,
         )
 
@@ -151,9 +143,9 @@ class _GroupedLinear(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         dev = grad_out.device
 
-        g_scales = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScale)
-        g_amaxes = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kAmax)
-        g_scale_invs = meta.get_meta_tensors(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScaleInv)
+        g_scales = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScale)
+        g_amaxes = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kAmax)
+        g_scale_invs = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScaleInv)
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
         g_t_views = None
         if ctx.weight_requires_grad:
@@ -168,7 +160,7 @@ class _GroupedLinear(torch.autograd.Function):
         if ctx.input_requires_grad:
             grad_input = fp8_gmm(
                 grad_out_fp8, weight_t_fp8, ctx.group_sizes, g_scale_invs,
-                meta.get_meta_tensors(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
+                meta.get_meta_pointers(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
                 backward=True, cutlass=ctx.cutlass,
             )
 
@@ -177,8 +169,8 @@ class _GroupedLinear(torch.autograd.Function):
             grad_weight = torch.empty(ctx.weight_shape, dtype=torch.bfloat16, device=dev)
             x_t_views = transposed_views(input_t_fp8, padded_cumsums if padded else cumsums)
             grouped_gemm(
-                g_t_views, x_t_views, list(grad_weight.unbind(0)), g_scale_invs,
-                meta.get_meta_tensors(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv),
+                g_t_views, x_t_views, TensorBatch.stack_of(grad_weight), g_scale_invs,
+                meta.get_meta_pointers(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv),
             )
         return grad_input, grad_weight, None, None, None, None
 

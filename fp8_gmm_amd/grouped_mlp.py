@@ -17,9 +17,11 @@ Experts with zero tokens are allowed; each wgrad is one grouped launch.
 """
 import math
 
+import numpy as np
 import torch
 
 from .backend import (
+    TensorBatch,
     fp8_gmm,
     grouped_gemm,
     multi_cast_transpose,
@@ -59,67 +61,64 @@ class _GroupedMlp(torch.autograd.Function):
 
         input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
         input_t_fp8 = None
-        x_scales = meta.get_meta_tensors(_T.kInputGroup1, _M.kScale)
-        x_amaxes = meta.get_meta_tensors(_T.kInputGroup1, _M.kAmax)
+        x_scales = meta.get_meta_pointers(_T.kInputGroup1, _M.kScale)
+        x_amaxes = meta.get_meta_pointers(_T.kInputGroup1, _M.kAmax)
         if wgrad_needed:
             input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums, fp8_dtype, dev)
-            with_t[0].extend(row_slices(input, cumsums))
-            with_t[1].extend(row_slices(input_fp8, cumsums))
-            with_t[2].extend(x_t_views)
-            with_t[3].extend(x_scales)
-            with_t[4].extend(x_amaxes)
+            for lst, item in zip(with_t, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_t_views,
+                                          x_scales, x_amaxes)):
+                lst.append(item)
         else:
-            plain[0].extend(row_slices(input, cumsums))
-            plain[1].extend(row_slices(input_fp8, cumsums))
-            plain[2].extend(x_scales)
-            plain[3].extend(x_amaxes)
+            for lst, item in zip(plain, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_scales,
+                                         x_amaxes)):
+                lst.append(item)
 
         fc1_weight_fp8 = torch.empty(fc1_weight.shape, dtype=fp8_dtype, device=dev)
         fc2_weight_fp8 = torch.empty(fc2_weight.shape, dtype=fp8_dtype, device=dev)
         fc1_weight_t_fp8 = fc2_weight_t_fp8 = None
-        w_scales = meta.get_meta_tensors(_T.kWeightGroup1, _M.kScale) + meta.get_meta_tensors(_T.kWeightGroup2, _M.kScale)
-        w_amaxes = meta.get_meta_tensors(_T.kWeightGroup1, _M.kAmax) + meta.get_meta_tensors(_T.kWeightGroup2, _M.kAmax)
-        w_in = list(fc1_weight.unbind(0)) + list(fc2_weight.unbind(0))
-        w_out = list(fc1_weight_fp8.unbind(0)) + list(fc2_weight_fp8.unbind(0))
+        w_scales = np.concatenate([meta.get_meta_pointers(_T.kWeightGroup1, _M.kScale),
+                                   meta.get_meta_pointers(_T.kWeightGroup2, _M.kScale)])
+        w_amaxes = np.concatenate([meta.get_meta_pointers(_T.kWeightGroup1, _M.kAmax),
+                                   meta.get_meta_pointers(_T.kWeightGroup2, _M.kAmax)])
+        w_in = TensorBatch.stack_of(fc1_weight) + TensorBatch.stack_of(fc2_weight)
+        w_out = TensorBatch.stack_of(fc1_weight_fp8) + TensorBatch.stack_of(fc2_weight_fp8)
         if dgrad_needed:
             fc1_weight_t_fp8 = torch.empty(num_groups, fc1_weight.size(2), fc1_weight.size(1), dtype=fp8_dtype,
                                            device=dev)
             fc2_weight_t_fp8 = torch.empty(num_groups, fc2_weight.size(2), fc2_weight.size(1), dtype=fp8_dtype,
                                            device=dev)
-            with_t[0].extend(w_in)
-            with_t[1].extend(w_out)
-            with_t[2].extend(list(fc1_weight_t_fp8.unbind(0)) + list(fc2_weight_t_fp8.unbind(0)))
-            with_t[3].extend(w_scales)
-            with_t[4].extend(w_amaxes)
+            w_t = TensorBatch.stack_of(fc1_weight_t_fp8) + TensorBatch.stack_of(fc2_weight_t_fp8)
+            for lst, item in zip(with_t, (w_in, w_out, w_t, w_scales, w_amaxes)):
+                lst.append(item)
         else:
-            plain[0].extend(w_in)
-            plain[1].extend(w_out)
-            plain[2].extend(w_scales)
-            plain[3].extend(w_amaxes)
+            for lst, item in zip(plain, (w_in, w_out, w_scales, w_amaxes)):
+                lst.append(item)
 
         if plain[0]:
-            multi_quantize(*plain)
+            multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
+                           np.concatenate(plain[3]))
         if with_t[0]:
-            multi_cast_transpose(*with_t)
+            multi_cast_transpose(TensorBatch.concat(with_t[0]), TensorBatch.concat(with_t[1]),
+                                 TensorBatch.concat(with_t[2]), np.concatenate(with_t[3]), np.concatenate(with_t[4]))
 
         pre_gelu_out = torch.empty(tokens, ffn, dtype=torch.bfloat16, device=dev)
         gelu_out_fp8 = torch.empty(tokens, ffn, dtype=fp8_dtype, device=dev)
         # fc1: GELU-aux epilogue, fp8 output scaled for fc2 (slot InputGroup2)
         fp8_gmm(
             input_fp8, fc1_weight_fp8, group_sizes,
-            meta.get_meta_tensors(_T.kInputGroup1, _M.kScaleInv),
-            meta.get_meta_tensors(_T.kWeightGroup1, _M.kScaleInv),
+            meta.get_meta_pointers(_T.kInputGroup1, _M.kScaleInv),
+            meta.get_meta_pointers(_T.kWeightGroup1, _M.kScaleInv),
             c=gelu_out_fp8, pre_gelu_out=pre_gelu_out,
-            c_scales=meta.get_meta_tensors(_T.kInputGroup2, _M.kScale),
-            c_amaxes=meta.get_meta_tensors(_T.kInputGroup2, _M.kAmax),
+            c_scales=meta.get_meta_pointers(_T.kInputGroup2, _M.kScale),
+            c_amaxes=meta.get_meta_pointers(_T.kInputGroup2, _M.kAmax),
             backward=False, cutlass=False,
         )
         if not is_grad_enabled:
             pre_gelu_out = None
         out = fp8_gmm(
             gelu_out_fp8, fc2_weight_fp8, group_sizes,
-            meta.get_meta_tensors(_T.kInputGroup2, _M.kScaleInv),
-            meta.get_meta_tensors(_T.kWeightGroup2, _M.kScaleInv),
+            meta.get_meta_pointers(_T.kInputGroup2, _M.kScaleInv),
+            meta.get_meta_pointers(_T.kWeightGroup2, _M.kScaleInv),
             backward=False, cutlass=False,
         )
         if not wgrad_needed:
@@ -156,9 +155,9 @@ class _GroupedMlp(torch.autograd.Function):
         dev = grad_out.device
         wgrad = ctx.weight_requires_grad
 
-        g1_scales = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kScale)
-        g1_amaxes = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kAmax)
-        g1_scale_invs = meta.get_meta_tensors(_T.kGradOutputGroup1, _M.kScaleInv)
+        g1_scales = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kScale)
+        g1_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kAmax)
+        g1_scale_invs = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kScaleInv)
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
 
         grad_fc2_weight = None
@@ -172,8 +171,8 @@ class _GroupedMlp(torch.autograd.Function):
             # fc2 wgrad: dW2[i][H, F] = dY_i^T[H, Mpad] . gelu_i^T[F, Mpad]^T
             grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev)
             grouped_gemm(
-                g_t_views, gelu_t_views, list(grad_fc2_weight.unbind(0)), g1_scale_invs,
-                meta.get_meta_tensors(_T.kForwardInputGroup2, _M.kScaleInv),
+                g_t_views, gelu_t_views, TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs,
+                meta.get_meta_pointers(_T.kForwardInputGroup2, _M.kScaleInv),
             )
         else:
             multi_quantize(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g1_scales, g1_amaxes)
@@ -181,7 +180,7 @@ class _GroupedMlp(torch.autograd.Function):
         # fc2 dgrad: d(gelu_out)[tokens, F]
         grad_gelu_out = fp8_gmm(
             grad_out_fp8, fc2_weight_t_fp8, ctx.group_sizes, g1_scale_invs,
-            meta.get_meta_tensors(_T.kForwardWeightGroup2, _M.kScaleInv),
+            meta.get_meta_pointers(_T.kForwardWeightGroup2, _M.kScaleInv),
             backward=True, cutlass=False,
         )
 
@@ -191,17 +190,17 @@ class _GroupedMlp(torch.autograd.Function):
         multi_cast_transpose_dgelu(
             row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums), row_slices(grad_pre_fp8, cumsums),
             grad_pre_t_views,
-            meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kScale),
-            meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kAmax),
+            meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale),
+            meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax),
         )
-        g2_scale_invs = meta.get_meta_tensors(_T.kGradOutputGroup2, _M.kScaleInv)
+        g2_scale_invs = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScaleInv)
 
         grad_input = None
         handle = None
         if ctx.input_requires_grad:
             grad_input = fp8_gmm(
                 grad_pre_fp8, fc1_weight_t_fp8, ctx.group_sizes, g2_scale_invs,
-                meta.get_meta_tensors(_T.kForwardWeightGroup1, _M.kScaleInv),
+                meta.get_meta_pointers(_T.kForwardWeightGroup1, _M.kScaleInv),
                 backward=True, cutlass=False,
             )
             if ctx.has_tp:
@@ -214,8 +213,8 @@ class _GroupedMlp(torch.autograd.Function):
             # fc1 wgrad: dW1[i][F, H] = d(pre)_i^T[F, Mpad] . X_i^T[H, Mpad]^T
             grad_fc1_weight = torch.empty(ctx.fc1_weight_shape, dtype=torch.bfloat16, device=dev)
             grouped_gemm(
-                grad_pre_t_views, transposed_views(input_t_fp8, t_bounds), list(grad_fc1_weight.unbind(0)),
-                g2_scale_invs, meta.get_meta_tensors(_T.kForwardInputGroup1, _M.kScaleInv),
+                grad_pre_t_views, transposed_views(input_t_fp8, t_bounds), TensorBatch.stack_of(grad_fc1_weight),
+                g2_scale_invs, meta.get_meta_pointers(_T.kForwardInputGroup1, _M.kScaleInv),
             )
         if handle is not None:
             handle.wait()

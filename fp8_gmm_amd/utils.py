@@ -7,6 +7,7 @@ maps :26-45, ``cumsum_group_sizes`` :48-62, ``Fp8MetaWrapper`` :65-103); the
 """
 from enum import IntEnum
 
+import numpy as np
 import torch
 
 PAD_MULTIPLE = 16  # the transposed (wgrad) operands pad each expert's tokens to this (reference utils.py:57)
@@ -140,8 +141,8 @@ class Fp8MetaWrapper:
         return [flat[first + i * stride] for i in range(self._num_groups)]
 
     def get_meta_pointers(self, fp8_tensor_type, meta_tensor_type):
-        """Device addresses of the same E slots, without creating E tensor views."""
+        """Device addresses of the same E slots as a uint64 array, without creating E tensor views
+        (every backend entry point takes such an array wherever it takes a list of scalars)."""
         flat, first, stride = self._select(fp8_tensor_type, meta_tensor_type)
         base = flat.data_ptr() + first * flat.element_size()
-        step = stride * flat.element_size()
-        return [base + i * step for i in range(self._num_groups)]
+        return np.uint64(base) + np.arange(self._num_groups, dtype=np.uint64) * np.uint64(stride * flat.element_size())

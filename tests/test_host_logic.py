@@ -86,7 +86,7 @@ def test_meta_wrapper_slot_arithmetic(e):
         # views, not copies: the kernels write amax in place; and the pointer form addresses the same slots
         views = w.get_meta_tensors(ttype, MetaTensorType.kAmax)
         ptrs = w.get_meta_pointers(ttype, MetaTensorType.kAmax)
-        assert [v.data_ptr() for v in views] == ptrs
+        assert [v.data_ptr() for v in views] == [int(p) for p in ptrs]
         assert views[0].data_ptr() == meta.amax_history.data_ptr() + 4 * slots[0]
 
 
@@ -177,3 +177,36 @@ def test_prepare_forward_allocates_three_and_two_slots_per_gemm():
         with m2.prepare_forward(x, None, num_gemms=6):
             pass
     assert m2.fp8_meta["scaling_fwd"].scale.eq(3).all()
+
+
+def test_tensor_batch_describes_the_same_memory_as_views():
+    """TensorBatch (array form of "per-expert views") must address exactly what the tensor views address."""
+    from fp8_gmm_amd.backend import TensorBatch
+
+    x = torch.zeros(10, 6, dtype=torch.bfloat16)
+    bounds = [0, 3, 3, 7, 10]
+    b = TensorBatch.rows_of(x, bounds)
+    views = [x[bounds[i]: bounds[i + 1]] for i in range(4)]
+    assert [int(p) for p in b.ptr] == [x.data_ptr() + bounds[i] * 6 * 2 for i in range(4)]
+    assert b.rows.tolist() == [v.shape[0] for v in views] and b.cols.tolist() == [6] * 4 and b.contiguous
+    assert [int(p) for p, v in zip(b.ptr, views) if v.numel()] == [v.data_ptr() for v in views if v.numel()]
+
+    w = torch.zeros(3, 4, 5, dtype=torch.float8_e4m3fn)
+    s = TensorBatch.stack_of(w)
+    assert [int(p) for p in s.ptr] == [v.data_ptr() for v in w.unbind(0)]
+    assert (s.rows.tolist(), s.cols.tolist()) == ([4] * 3, [5] * 3)
+
+    flat = torch.zeros(12, 6, dtype=torch.float8_e4m3fn)
+    pb = [0, 4, 4, 8, 12]
+    t = TensorBatch.transposed_blocks_of(flat, pb)
+    for i in range(4):
+        rows = pb[i + 1] - pb[i]
+        if rows:
+            v = flat[pb[i]: pb[i + 1]].view(6, rows)  # the reference's reinterpretation (grouped_linear.py:36-52)
+            assert int(t.ptr[i]) == v.data_ptr() and (int(t.rows[i]), int(t.cols[i])) == tuple(v.shape)
+    both = b + TensorBatch.rows_of(x, [0, 10])
+    assert len(both) == 5 and both.rows.tolist() == [3, 0, 4, 3, 10]
+    with pytest.raises(RuntimeError):
+        TensorBatch.concat([b, s])  # dtypes differ
+    with pytest.raises(RuntimeError):
+        TensorBatch.rows_of(x.t(), [0, 1])  # not contiguous
