@@ -37,6 +37,8 @@ TENSOR_DESC = np.dtype(
         ("cols", "<i4"),
         ("rows_padded", "<i4"),
         ("block_begin", "<i4"),
+        ("amax_partial", "<u4"),   # scratch of the kernels (zeroed by the plan)
+        ("reserved", "<u4", (15,)),  # pads the descriptor to one 128-byte cache line
     ],
     align=False,
 )

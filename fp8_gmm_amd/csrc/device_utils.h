@@ -126,9 +126,10 @@ __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
   atomicMax(reinterpret_cast<int*>(addr), __float_as_int(v));
 }
 
-// Block-wide amax merge for blocks of NWAVES waves. `stage` is NWAVES floats of LDS.
+// Block-wide amax merge for blocks of NWAVES waves. `stage` is NWAVES floats of LDS.  `target` is the
+// tensor's own partial-amax word (fp8gmm_tensor_desc::amax_partial), not the caller's amax slot.
 template <int NWAVES>
-__device__ __forceinline__ void block_amax_merge(float local, float* amax, float* stage) {
+__device__ __forceinline__ void block_amax_merge(float local, uint32_t* target, float* stage) {
   float w = wave_max(local);
   const int lane = threadIdx.x % kWaveSize;
   const int wave = threadIdx.x / kWaveSize;
@@ -138,10 +139,20 @@ __device__ __forceinline__ void block_amax_merge(float local, float* amax, float
     float m = stage[0];
 #pragma unroll
     for (int i = 1; i < NWAVES; ++i) m = fmaxf(m, stage[i]);
-    // amax only grows, so a value already at or above m (even a stale one) makes the atomic redundant;
-    // this keeps thousands of workgroups from queueing on one address.
-    if (amax != nullptr && m > 0.f && !(__builtin_nontemporal_load(amax) >= m)) atomic_max_nonneg(amax, m);
+    // amax only grows, so a value already at or above m (even a stale one) makes the atomic redundant
+    float* t = reinterpret_cast<float*>(target);
+    if (target != nullptr && m > 0.f && !(__builtin_nontemporal_load(t) >= m)) atomic_max_nonneg(t, m);
   }
+}
+
+// Second pass of the calls that record amax: one lane per tensor merges the tensor's partial into the
+// caller's slot.  n atomics in total, against one per workgroup of the main kernel.
+[[maybe_unused]] static __global__ __launch_bounds__(256) void amax_merge_kernel(const fp8gmm_tensor_desc* __restrict__ descs, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float p = __builtin_bit_cast(float, descs[i].amax_partial);
+  float* amax = descs[i].amax;
+  if (amax != nullptr && p > 0.f) atomic_max_nonneg(amax, p);
 }
 
 // tanh from a fixed sequence of IEEE single-precision operations (mul, add, fma,

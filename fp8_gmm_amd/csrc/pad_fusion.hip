@@ -51,7 +51,7 @@ __device__ __forceinline__ void transpose4x4(uint32_t a, uint32_t b, uint32_t c,
 }
 
 template <int OP, int FMT>
-__global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tensor_desc* __restrict__ descs, int n) {
+__global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(fp8gmm_tensor_desc* __restrict__ descs, int n) {
   __shared__ __attribute__((aligned(16))) uint8_t tl[TN * TM];
   __shared__ float stage[kPtThreads / kWaveSize];
 
@@ -241,15 +241,17 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(const fp8gmm_tens
     }
   }
 
-  if constexpr (OP != OP_TRANSPOSE) block_amax_merge<kPtThreads / kWaveSize>(mx, d.amax, stage);
+  if constexpr (OP != OP_TRANSPOSE)
+    block_amax_merge<kPtThreads / kWaveSize>(mx, d.amax != nullptr ? &descs[t].amax_partial : nullptr, stage);
 }
 
 template <int OP>
-int launch_fmt(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, hipStream_t s) {
+int launch_fmt(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, hipStream_t s) {
   if (out_fmt == FP8GMM_E4M3)
     hipLaunchKernelGGL((multi_pad_kernel<OP, FP8GMM_E4M3>), dim3(total_blocks), dim3(kPtThreads), 0, s, descs_dev, n);
   else
     hipLaunchKernelGGL((multi_pad_kernel<OP, FP8GMM_E5M2>), dim3(total_blocks), dim3(kPtThreads), 0, s, descs_dev, n);
+  if (OP != OP_TRANSPOSE) hipLaunchKernelGGL(amax_merge_kernel, dim3((n + 255) / 256), dim3(256), 0, s, descs_dev, n);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
@@ -275,11 +277,11 @@ int fp8gmm_multi_pad_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int t
   const int rc = fp8gmm::check_args(descs_dev, n, total_blocks, FP8GMM_E4M3, &nothing);
   if (rc != FP8GMM_OK || nothing) return rc;
   // a pure byte shuffle: the fp8 flavour does not matter
-  return fp8gmm::launch_fmt<fp8gmm::OP_TRANSPOSE>(descs_dev, n, total_blocks, FP8GMM_E4M3,
-                                                  static_cast<hipStream_t>(stream));
+  return fp8gmm::launch_fmt<fp8gmm::OP_TRANSPOSE>(const_cast<fp8gmm_tensor_desc*>(descs_dev), n, total_blocks,
+                                                  FP8GMM_E4M3, static_cast<hipStream_t>(stream));
 }
 
-int fp8gmm_multi_pad_cast_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+int fp8gmm_multi_pad_cast_transpose(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
                                     void* stream) {
   bool nothing;
   const int rc = fp8gmm::check_args(descs_dev, n, total_blocks, out_fmt, &nothing);
@@ -287,7 +289,7 @@ int fp8gmm_multi_pad_cast_transpose(const fp8gmm_tensor_desc* descs_dev, int n, 
   return fp8gmm::launch_fmt<fp8gmm::OP_CAST>(descs_dev, n, total_blocks, out_fmt, static_cast<hipStream_t>(stream));
 }
 
-int fp8gmm_multi_pad_cast_transpose_dgelu(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+int fp8gmm_multi_pad_cast_transpose_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
                                           void* stream) {
   bool nothing;
   const int rc = fp8gmm::check_args(descs_dev, n, total_blocks, out_fmt, &nothing);

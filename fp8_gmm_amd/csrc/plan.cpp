@@ -62,6 +62,7 @@ int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* tota
       nb = tr * tc;
     }
     d.block_begin = (int32_t)blocks;
+    d.amax_partial = 0;
     blocks += nb;
     if (blocks > INT32_MAX / 2) return FP8GMM_ERR_BAD_SHAPE;
   }

@@ -14,8 +14,7 @@ namespace fp8gmm {
 namespace {
 
 template <int FMT>
-__global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(const fp8gmm_tensor_desc* __restrict__ descs,
-                                                                    int n) {
+__global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tensor_desc* __restrict__ descs, int n) {
   __shared__ float stage[kPwThreads / kWaveSize];
   const int bid = blockIdx.x;
   const int t = upper_slot(n, bid, [&](int i) { return descs[i].block_begin; });
@@ -77,7 +76,7 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(const fp8gmm
       }
     }
   }
-  block_amax_merge<kPwThreads / kWaveSize>(mx, d.amax, stage);
+  block_amax_merge<kPwThreads / kWaveSize>(mx, d.amax != nullptr ? &descs[t].amax_partial : nullptr, stage);
 }
 
 __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gmm_tensor_desc* __restrict__ descs,
@@ -183,7 +182,7 @@ int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scal
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
-int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+int fp8gmm_multi_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
   if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_fmt != FP8GMM_E4M3 && out_fmt != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
   if (n == 0 || total_blocks == 0) return FP8GMM_OK;
@@ -195,6 +194,7 @@ int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_
   else
     hipLaunchKernelGGL(fp8gmm::multi_quantize_kernel<FP8GMM_E5M2>, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0, s,
                        descs_dev, n);
+  hipLaunchKernelGGL(fp8gmm::amax_merge_kernel, dim3((n + 255) / 256), dim3(256), 0, s, descs_dev, n);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 

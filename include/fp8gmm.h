@@ -65,7 +65,12 @@ typedef enum fp8gmm_status {
  * `scale` NULL means 1.0 (reference csrc/multi_pointwise.cu:51); `amax` NULL
  * means "do not record" (csrc/multi_pad_fusion.cu:290).  `amax` is merged with
  * its previous content by an integer atomic max and must hold a non-negative
- * value on entry (csrc/utils.cuh:183-185).  For quantize / scale_mul, `cols`
+ * value on entry (csrc/utils.cuh:183-185).  The workgroups of a tensor first
+ * reduce into the descriptor's own `amax_partial` (one cache line per tensor:
+ * the amax slots of the reference's layout sit a few bytes apart, and thousands
+ * of atomics on one line serialise); a second, tiny launch of the same call
+ * merges the partials into the slots.  The device table is therefore WRITTEN by
+ * the calls that record amax and has to be uploaded afresh for every call.  For quantize / scale_mul, `cols`
  * may carry the whole element count with rows = 1.
  */
 typedef struct fp8gmm_tensor_desc {
@@ -79,7 +84,9 @@ typedef struct fp8gmm_tensor_desc {
   int32_t cols;
   int32_t rows_padded;  /* second dimension of out_t, >= rows; ignored by ops without out_t */
   int32_t block_begin;  /* filled by fp8gmm_plan_*: first workgroup of this tensor */
-} fp8gmm_tensor_desc;   /* 64 bytes */
+  uint32_t amax_partial; /* scratch of the kernels, zeroed by fp8gmm_plan_*: running max|x| of this tensor */
+  uint32_t reserved[15]; /* pads the descriptor to one 128-byte cache line */
+} fp8gmm_tensor_desc;   /* 128 bytes */
 
 /* which multi-tensor kernel a plan is for */
 #define FP8GMM_OP_QUANTIZE 0
@@ -144,16 +151,16 @@ int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles
 
 /* ---- launches (descs_dev / probs_dev: DEVICE copies of planned tables) ------------------- */
 /* replaces MultiQuantize, csrc/multi_pointwise.cu:155 (pybind name multi_quantize, csrc/ops.cu:11) */
-int fp8gmm_multi_quantize(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream);
+int fp8gmm_multi_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream);
 /* replaces MultiScaleMul, csrc/multi_pointwise.cu:216 (multi_scale_mul, csrc/ops.cu:12) */
 int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream);
 /* replaces MultiPadTranspose, csrc/multi_pad_fusion.cu:442 (multi_pad_transpose, csrc/ops.cu:13) */
 int fp8gmm_multi_pad_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream);
 /* replaces MultiPadCastTranspose, csrc/multi_pad_fusion.cu:505 (multi_pad_cast_transpose, csrc/ops.cu:14) */
-int fp8gmm_multi_pad_cast_transpose(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+int fp8gmm_multi_pad_cast_transpose(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
                                     void* stream);
 /* replaces MultiPadCastTransposeDgelu, csrc/multi_pad_fusion.cu:587 (multi_pad_cast_transpose_dgelu, csrc/ops.cu:15) */
-int fp8gmm_multi_pad_cast_transpose_dgelu(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
+int fp8gmm_multi_pad_cast_transpose_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
                                           void* stream);
 
 /*

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_function():
 
 def test_struct_layouts_match_the_binding():
     lib = _lib.load()
-    assert lib.fp8gmm_sizeof_tensor_desc() == _lib.TENSOR_DESC.itemsize == 64
+    assert lib.fp8gmm_sizeof_tensor_desc() == _lib.TENSOR_DESC.itemsize == 128  # one cache line per tensor
     assert lib.fp8gmm_sizeof_gemm_problem() == _lib.GEMM_PROBLEM.itemsize == 96
     assert _lib.TENSOR_DESC.fields["rows"][1] == 48 and _lib.TENSOR_DESC.fields["block_begin"][1] == 60
     assert _lib.GEMM_PROBLEM.fields["m"][1] == 64 and _lib.GEMM_PROBLEM.fields["tile_begin"][1] == 88
