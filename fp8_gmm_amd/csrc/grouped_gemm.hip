@@ -203,7 +203,10 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       }
       if (pr.c_amax != nullptr) {
         amax = wave_max(amax);
-        if (lane == 0 && amax > 0.f) atomic_max_nonneg(pr.c_amax, amax);
+        // amax only grows: once the slot holds a value at or above this wavefront's, the atomic is redundant
+        // (the slots of all experts share a cache line, and atomics on one line serialise)
+        if (lane == 0 && amax > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= amax))
+          atomic_max_nonneg(pr.c_amax, amax);
       }
     }
     return fast;
