@@ -302,3 +302,31 @@ def test_argument_errors_raise(dev):
     with pytest.raises(RuntimeError):  # CPU tensors: no fallback
         backend.multi_quantize([torch.zeros(8, dtype=torch.bfloat16)], [torch.zeros(8, dtype=E4M3)], [torch.ones(1)],
                                [torch.zeros(1)])
+
+
+def test_shared_tiles_on_concurrent_streams(dev):
+    """Launches that cut tiles along K keep their partial sums in a workspace owned by (device, stream): GEMMs
+    running at the same time on different streams must not see each other's partial sums, and streams beyond
+    the number of workspaces the library keeps simply run without tail balancing.  Exact data, so any
+    cross-talk shows up as a bit difference."""
+    backend = _backend()
+    m, n, k = 300, 512, 8192
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
+    streams = [torch.cuda.Stream(device=dev) for _ in range(10)]
+    ops, wants, outs = [], [], []
+    for i in range(len(streams)):
+        g = gen(500 + i)
+        a = _q(vals[torch.randint(0, 8, (m, k), generator=g)].to(torch.bfloat16), E4M3).to(dev)
+        b = _q(vals[torch.randint(0, 8, (1, n, k), generator=g)].to(torch.bfloat16), E4M3).to(dev)
+        ops.append((a, b))
+        wants.append((a.float() @ b[0].float().t()).to(torch.bfloat16))
+    one = torch.ones(1, device=dev)
+    torch.cuda.synchronize()
+    for rep in range(3):
+        outs = []
+        for s, (a, b) in zip(streams, ops):
+            with torch.cuda.stream(s):
+                outs.append(backend.fp8_gmm(a, b, torch.tensor([m]), one, one))
+        torch.cuda.synchronize()
+        for i, (c, want) in enumerate(zip(outs, wants)):
+            assert torch.equal(c.view(torch.int16), want.view(torch.int16)), f"stream {i}, repetition {rep}"
