@@ -31,6 +31,7 @@ constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
 constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
 constexpr int kPartialBytes = BM * BN * 4;  // one slot: the 128 accumulators of the 512 lanes
+constexpr int kTileOverhead = 4;      // fixed cost of a tile (epilogue, switch) in K = 128 steps, measured
 constexpr int kSlotsPerWg = 2;        // a piece that starts inside a tile, one that ends inside a tile
 
 struct Sched {
@@ -62,32 +63,40 @@ FP8GMM_HD int64_t tile_cost(const Sched& s, int p) {
   const int c = (s.probs[p].k + 127) / 128;
   return (int64_t)(c > 0 ? c : 1);
 }
-// cost of all tiles before `tile` (0 <= tile <= total_tiles); cost_begin is the plan's prefix sum
-FP8GMM_HD int64_t cost_before(const Sched& s, int tile) {
+// Work before `tile` (0 <= tile <= total_tiles) when every tile counts its K steps plus `ov` steps of fixed
+// overhead; cost_begin is the plan's prefix sum of the K steps alone.  ov = 0 is the unit in which tiles are
+// cut along K; ov = kTileOverhead is the weight that balances the XCD ranges.
+FP8GMM_HD int64_t work_before(const Sched& s, int tile, int ov) {
   const int p = problem_of_tile(s, tile);
-  return (int64_t)s.probs[p].cost_begin + (int64_t)(tile - s.probs[p].tile_begin) * tile_cost(s, p);
+  return (int64_t)s.probs[p].cost_begin + (int64_t)ov * s.probs[p].tile_begin +
+         (int64_t)(tile - s.probs[p].tile_begin) * (tile_cost(s, p) + ov);
 }
-// the tile that holds cost offset c: cost_before(t) <= c < cost_before(t + 1); total_tiles past the end
-FP8GMM_HD int tile_holding_cost(const Sched& s, int64_t c) {
-  if (c >= s.total_cost) return s.total_tiles;
-  int lo = 0, hi = s.nprob - 1;  // last problem whose prefix is <= c: it is not empty, as c < total_cost
+FP8GMM_HD int64_t cost_before(const Sched& s, int tile) { return work_before(s, tile, 0); }
+// the tile that holds work offset c: work_before(t) <= c < work_before(t + 1); total_tiles past the end
+FP8GMM_HD int tile_holding_work(const Sched& s, int64_t c, int ov) {
+  if (c >= s.total_cost + (int64_t)ov * s.total_tiles) return s.total_tiles;
+  int lo = 0, hi = s.nprob - 1;  // last problem whose prefix is <= c: it is not empty, as c < the total
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
-    if ((int64_t)s.probs[mid].cost_begin <= c) lo = mid; else hi = mid - 1;
+    if ((int64_t)s.probs[mid].cost_begin + (int64_t)ov * s.probs[mid].tile_begin <= c) lo = mid; else hi = mid - 1;
   }
-  return s.probs[lo].tile_begin + (int)((c - s.probs[lo].cost_begin) / tile_cost(s, lo));
+  const int64_t before = (int64_t)s.probs[lo].cost_begin + (int64_t)ov * s.probs[lo].tile_begin;
+  return s.probs[lo].tile_begin + (int)((c - before) / (tile_cost(s, lo) + ov));
 }
-// first tile whose preceding cost is >= c (total_tiles if there is none)
-FP8GMM_HD int first_tile_at_cost(const Sched& s, int64_t c) {
+FP8GMM_HD int tile_holding_cost(const Sched& s, int64_t c) { return tile_holding_work(s, c, 0); }
+// first tile whose preceding work is >= c (total_tiles if there is none)
+FP8GMM_HD int first_tile_at_work(const Sched& s, int64_t c, int ov) {
   if (c <= 0) return 0;
-  const int t = tile_holding_cost(s, c);
+  const int t = tile_holding_work(s, c, ov);
   if (t >= s.total_tiles) return s.total_tiles;
-  return cost_before(s, t) == c ? t : t + 1;
+  return work_before(s, t, ov) == c ? t : t + 1;
 }
 
-// Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal COST (k differs
-// per problem in the wgrad form), one per XCD, so that workgroups that share an L2 work on neighbouring
-// tiles; the workgroups of an XCD stride through the range, and share its remainder along K when that pays.
+// Workgroup i runs on XCD i % 8.  The tile list is cut into 8 contiguous ranges of equal WORK, one per XCD,
+// so that workgroups that share an L2 work on neighbouring tiles; the workgroups of an XCD stride through the
+// range, and share its remainder along K when that pays.  k differs per problem in the wgrad form, and a
+// tile costs its K steps plus a fixed part (epilogue, tile switch) worth about kTileOverhead steps: balancing
+// K steps alone left the XCDs that hold the short-K problems 17 % more work than the others.
 FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob, int total_tiles,
                                            int xcd, int wgs_per_xcd, bool sk_enable) {
   s.probs = probs;
@@ -95,11 +104,12 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   s.total_tiles = total_tiles;
   s.wgs = wgs_per_xcd;
   s.total_cost = 0;
-  const int64_t total_cost = s.total_cost = cost_before(s, total_tiles);
-  const int64_t lo = (total_cost * xcd + kNumXcd - 1) / kNumXcd;
-  const int64_t hi = (total_cost * (xcd + 1) + kNumXcd - 1) / kNumXcd;
-  s.range_begin = first_tile_at_cost(s, lo);
-  s.range_end = first_tile_at_cost(s, hi);
+  s.total_cost = cost_before(s, total_tiles);
+  const int64_t total_work = s.total_cost + (int64_t)kTileOverhead * total_tiles;
+  const int64_t lo = (total_work * xcd + kNumXcd - 1) / kNumXcd;
+  const int64_t hi = (total_work * (xcd + 1) + kNumXcd - 1) / kNumXcd;
+  s.range_begin = first_tile_at_work(s, lo, kTileOverhead);
+  s.range_end = first_tile_at_work(s, hi, kTileOverhead);
   const int n_x = s.range_end - s.range_begin;
   const int W = wgs_per_xcd;
   s.dp_rounds = (n_x + W - 1) / W;  // plain striding: the last round may be partial
@@ -134,6 +144,20 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
 // piece boundaries of the stream-K region, relative to sk_c0
 FP8GMM_HD int64_t sk_bound(const Sched& s, int j) { return s.sk_cost * j / s.sk_wgs; }
 
+// Tile `local` of a problem with tiles_m x tiles_n tiles -> its row / column block.  The m index runs fastest
+// inside groups of kRasterRows m-tiles: 32 consecutive tiles (one round of an XCD's workgroups) then form an
+// 8 x 4 block that needs 12 operand slabs, whatever the shape of the problem (a 56 x 16 weight-gradient
+// problem walked with m fastest over all 56 rows would need 33).
+constexpr int kRasterRows = 8;
+FP8GMM_HD void tile_origin(int m, int n, int local, int* m0, int* n0) {
+  const int tiles_m = (m + BM - 1) / BM, tiles_n = (n + BN - 1) / BN;
+  const int group = local / (kRasterRows * tiles_n);
+  const int within = local - group * (kRasterRows * tiles_n);
+  const int rows = tiles_m - group * kRasterRows < kRasterRows ? tiles_m - group * kRasterRows : kRasterRows;
+  *m0 = (group * kRasterRows + within % rows) * BM;
+  *n0 = (within / rows) * BN;
+}
+
 struct Item {
   int tile, prob, m0, n0;
   int k_begin, nk;  // pair steps: first one, how many (0 for a problem without K)
@@ -157,10 +181,7 @@ FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c) {
   Item it;
   it.tile = dp ? s.range_begin + j + s.wgs * c.dp_i : c.sk_tile;
   it.prob = problem_of_tile(s, it.tile);
-  const int local = it.tile - s.probs[it.prob].tile_begin;
-  const int tiles_m = (s.probs[it.prob].m + BM - 1) / BM;
-  it.m0 = (local % tiles_m) * BM;  // m fastest: neighbouring tiles share the weight slab
-  it.n0 = (local / tiles_m) * BN;
+  tile_origin(s.probs[it.prob].m, s.probs[it.prob].n, it.tile - s.probs[it.prob].tile_begin, &it.m0, &it.n0);
   const int real_nk = (s.probs[it.prob].k + 127) / 128;  // a K tail is zero-filled
   it.k_begin = 0;
   it.nk = real_nk;

@@ -10,8 +10,8 @@
 //   * the output of every problem is cut into 256 x 256 tiles; all tiles of all problems form
 //     one list walked by a persistent grid (one workgroup per CU).  The list is split into 8
 //     contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so that workgroups that
-//     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest, so
-//     neighbouring tiles share the weight slab.
+//     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest within
+//     groups of 8 rows of tiles, so one round of an XCD's 32 workgroups is an 8 x 4 block of tiles.
 //   * a workgroup is 8 wavefronts (2 along m x 4 along n); a wavefront owns a 128 x 64
 //     sub-tile = 4 x 2 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4 (128 accumulator registers).
 //     The weight operand is MFMA source 0 and the token operand source 1: every lane then
@@ -514,9 +514,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8g
     partial_add(acc, workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + q)) * kPartialBytes);
 
   const fp8gmm_gemm_problem pr = probs[prob];
-  const int local = tile - pr.tile_begin;
-  const int tiles_m = (pr.m + BM - 1) / BM;
-  tile_epilogue(acc, pr, (local % tiles_m) * BM, (local / tiles_m) * BN, out_kind, epilogue);
+  int m0, n0;
+  tile_origin(pr.m, pr.n, tile - pr.tile_begin, &m0, &n0);
+  tile_epilogue(acc, pr, m0, n0, out_kind, epilogue);
 }
 
 // Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)

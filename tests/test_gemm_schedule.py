@@ -6,7 +6,9 @@ What must hold for ANY problem list, grid and tail-balancing choice (the kernel 
     item of the launch uses and that lies inside the kSlotsPerWg * grid slots of the workspace;
   * every tile that was cut is completed by exactly one fix-up workgroup, which adds exactly the slots
     written for that tile, in K order;
-  * workgroup wg works only on tiles of XCD range wg % 8, and the eight ranges tile the list in order.
+  * workgroup wg works only on tiles of XCD range wg % 8, and the eight ranges tile the list in order;
+  * the tiles of a problem map one-to-one onto the 256 x 256 blocks of its output, and 32 consecutive tiles of
+    a large problem form a compact block (at most 12 distinct row / column blocks), not a strip.
 The expectations are stated from these properties, not recomputed with the scheduler's formulas.
 """
 import numpy as np
@@ -40,14 +42,15 @@ def check_schedule(shapes, grid, stream_k):
     slots_written = {}  # slot -> (tile, k_begin, nk)
     xcd_tiles = [set() for _ in range(8)]
     n_partial_items = 0
+    origin_of = {}
     for wg in range(grid):
         items = _lib.gemm_schedule(table, total, grid, stream_k, wg)
         for tile, prob, m0, n0, k_begin, nk, slot in items.tolist():
             assert 0 <= tile < total and prob == tile_prob[tile]
             m, n, _ = shapes[prob]
-            local = tile - int(table[prob]["tile_begin"])
-            tiles_m = (m + TILE - 1) // TILE
-            assert (m0, n0) == ((local % tiles_m) * TILE, (local // tiles_m) * TILE)
+            assert m0 % TILE == 0 and n0 % TILE == 0 and 0 <= m0 < m and 0 <= n0 < n
+            origin_of.setdefault(tile, (prob, m0, n0))
+            assert origin_of[tile] == (prob, m0, n0)   # every piece of a tile agrees on where the tile is
             xcd_tiles[wg % 8].add(tile)
             if nk_of[prob] == 0:
                 assert (k_begin, nk, slot) == (0, 0, -1)
@@ -64,6 +67,11 @@ def check_schedule(shapes, grid, stream_k):
                 n_partial_items += 1
     for tile in range(total):
         assert (covered[tile] == 1).all(), f"tile {tile} covered {covered[tile].tolist()}"
+    # the tiles of a problem cover every 256 x 256 block of its output exactly once
+    for p, (m, n, _) in enumerate(shapes):
+        blocks = sorted((m0, n0) for (pp, m0, n0) in origin_of.values() if pp == p)
+        want = sorted((i * TILE, j * TILE) for i in range((m + TILE - 1) // TILE) for j in range((n + TILE - 1) // TILE))
+        assert blocks == want, f"problem {p}"
     # XCD ranges are disjoint, contiguous and ordered
     prev_end = 0
     for x in range(8):
@@ -159,3 +167,18 @@ def test_argument_checks():
     assert L.fp8gmm_gemm_schedule(table.ctypes.data, 1, total, 12, 1, 0, buf.ctypes.data, 4) < 0   # grid % 8 != 0
     assert L.fp8gmm_gemm_schedule(table.ctypes.data, 1, total, 16, 1, 16, buf.ctypes.data, 4) < 0  # wg out of range
     assert L.fp8gmm_gemm_schedule(None, 1, total, 16, 1, 0, buf.ctypes.data, 4) < 0
+
+
+def test_consecutive_tiles_form_compact_blocks():
+    """One round of an XCD is 32 consecutive tiles: they must touch few distinct operand slabs (8 row blocks +
+    4 column blocks), also for weight-gradient shapes with many more row blocks than column blocks."""
+    for shape in [(14336, 4096, 2048), (4096, 14336, 2048), (2048, 14336, 4096)]:
+        table, total = make_table([shape])
+        tiles = {}
+        for wg in range(256):
+            for tile, _, m0, n0, *_ in _lib.gemm_schedule(table, total, 256, False, wg).tolist():
+                tiles[tile] = (m0, n0)
+        for start in range(0, total - 31, 32):
+            rows = {tiles[t][0] for t in range(start, start + 32)}
+            cols = {tiles[t][1] for t in range(start, start + 32)}
+            assert len(rows) + len(cols) <= 12, (shape, start, len(rows), len(cols))
