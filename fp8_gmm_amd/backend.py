@@ -10,6 +10,9 @@ descriptor table, has the C library plan it, uploads it through pinned memory on
 the current stream and enqueues ONE kernel.  Nothing here computes on the CPU and
 there is no fallback: without the HIP library the import fails.
 """
+import contextlib
+import threading
+
 import numpy as np
 import torch
 
@@ -131,6 +134,74 @@ def _upload(table, device):
     return pinned.to(device, non_blocking=True)
 
 
+# A launch needs its table in device memory, and every upload is a small copy kernel with a dispatch gap on
+# either side (about 20 us per launch on an otherwise busy GPU).  Inside ``batched_uploads()`` the entry
+# points only plan and queue their launch; at the end of the block all queued tables travel in ONE copy
+# and the kernels are launched back to back, in the order they were queued.
+_pending = threading.local()
+
+
+@contextlib.contextmanager
+def batched_uploads():
+    """Queue the launches issued inside the block and upload all their tables with one copy at its end.
+
+    Only for sequences made of this module's entry points: anything else that consumes their results
+    (a torch op, a collective) has to come after the block, because the kernels are not enqueued before
+    the block ends.  Nested blocks join the outermost one.  If the block raises, nothing is launched."""
+    if getattr(_pending, "items", None) is not None:
+        yield
+        return
+    _pending.items = []
+    try:
+        yield
+        items = _pending.items
+    finally:
+        _pending.items = None
+    _flush(items)
+
+
+def flush_uploads():
+    """Upload and launch what has been queued so far (for a consumer inside the block that is not one of this
+    module's entry points, e.g. a collective on a result); queueing goes on afterwards."""
+    items = getattr(_pending, "items", None)
+    if items:
+        _pending.items = []
+        _flush(items)
+
+
+def _submit(table, device, launch, keep):
+    """Run ``launch(device address of table)`` now, or queue it when inside ``batched_uploads()``.
+
+    ``keep`` holds every tensor the table points into.  A queued table is only raw addresses: without the
+    references the caller's temporaries would be freed before the launch, and the allocator could hand
+    their memory to someone else - to the uploaded tables themselves, for one."""
+    items = getattr(_pending, "items", None)
+    if items is not None:
+        items.append((table, device, launch, keep))
+        return
+    dev_table = _upload(table, device)
+    launch(dev_table.data_ptr())
+
+
+def _flush(items):
+    by_device = {}
+    for it in items:
+        by_device.setdefault(it[1], []).append(it)
+    for device, group in by_device.items():
+        offsets, total = [], 0
+        for table, _, _, _ in group:
+            offsets.append(total)
+            total += (table.nbytes + 127) // 128 * 128   # every table on its own cache lines
+        pinned = torch.empty(total, dtype=torch.uint8, pin_memory=True)
+        host = pinned.numpy()
+        for (table, _, _, _), off in zip(group, offsets):
+            host[off: off + table.nbytes] = table.view(np.uint8).reshape(-1)
+        dev_tables = pinned.to(device, non_blocking=True)
+        base = dev_tables.data_ptr()
+        for (_, _, launch, _), off in zip(group, offsets):
+            launch(base + off)
+
+
 def _stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -160,27 +231,30 @@ def _scalar_ptrs(scalars, n, what):
     return out
 
 
-def _launch_multi(op, table, out_fmt, device):
+def _launch_multi(op, table, out_fmt, device, keep):
     """Plan, upload and launch one multi-tensor kernel over `table`."""
     total = _lib.plan_multi_tensor(table, op)
     if total == 0:
         return
     L = _lib.load()
-    dev_table = _upload(table, device)
     n = len(table)
-    with torch.cuda.device(device), _timed(_OP_NAMES[op], lambda: _algorithmic_bytes(op, table)):
-        s = _stream(device)
-        if op == _lib.OP_QUANTIZE:
-            rc = L.fp8gmm_multi_quantize(dev_table.data_ptr(), n, total, out_fmt, s)
-        elif op == _lib.OP_SCALE_MUL:
-            rc = L.fp8gmm_multi_scale_mul(dev_table.data_ptr(), n, total, s)
-        elif op == _lib.OP_PAD_TRANSPOSE:
-            rc = L.fp8gmm_multi_pad_transpose(dev_table.data_ptr(), n, total, s)
-        elif op == _lib.OP_PAD_CAST_TRANSPOSE:
-            rc = L.fp8gmm_multi_pad_cast_transpose(dev_table.data_ptr(), n, total, out_fmt, s)
-        else:
-            rc = L.fp8gmm_multi_pad_cast_transpose_dgelu(dev_table.data_ptr(), n, total, out_fmt, s)
-    _lib.check(rc)
+
+    def launch(dev_ptr):
+        with torch.cuda.device(device), _timed(_OP_NAMES[op], lambda: _algorithmic_bytes(op, table)):
+            s = _stream(device)
+            if op == _lib.OP_QUANTIZE:
+                rc = L.fp8gmm_multi_quantize(dev_ptr, n, total, out_fmt, s)
+            elif op == _lib.OP_SCALE_MUL:
+                rc = L.fp8gmm_multi_scale_mul(dev_ptr, n, total, s)
+            elif op == _lib.OP_PAD_TRANSPOSE:
+                rc = L.fp8gmm_multi_pad_transpose(dev_ptr, n, total, s)
+            elif op == _lib.OP_PAD_CAST_TRANSPOSE:
+                rc = L.fp8gmm_multi_pad_cast_transpose(dev_ptr, n, total, out_fmt, s)
+            else:
+                rc = L.fp8gmm_multi_pad_cast_transpose_dgelu(dev_ptr, n, total, out_fmt, s)
+        _lib.check(rc)
+
+    _submit(table, device, launch, keep)
 
 
 class TensorBatch:
@@ -353,7 +427,7 @@ def multi_quantize(inputs, outputs, scales, amaxes):
     table["cols"] = numel
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
-    _launch_multi(_lib.OP_QUANTIZE, table, _FMT[dt], dev)
+    _launch_multi(_lib.OP_QUANTIZE, table, _FMT[dt], dev, (x, o, scales, amaxes))
 
 
 def multi_scale_mul(inputs, scales_1, scales_2):
@@ -375,7 +449,7 @@ def multi_scale_mul(inputs, scales_1, scales_2):
     table["cols"] = numel
     table["scale"] = _scalar_ptrs(scales_1, n, "scales_1")
     table["in2"] = _scalar_ptrs(scales_2, n, "scales_2")
-    _launch_multi(_lib.OP_SCALE_MUL, table, _lib.E4M3, dev)
+    _launch_multi(_lib.OP_SCALE_MUL, table, _lib.E4M3, dev, (x, scales_1, scales_2))
 
 
 def _fill_transpose_shapes(table, x, t):
@@ -403,7 +477,7 @@ def multi_transpose(inputs, outputs):
     table = np.zeros(n, dtype=TENSOR_DESC)
     _fill_transpose_shapes(table, x, t)
     table["in"], table["out_t"] = x.ptr, t.ptr
-    _launch_multi(_lib.OP_PAD_TRANSPOSE, table, _lib.E4M3, dev)
+    _launch_multi(_lib.OP_PAD_TRANSPOSE, table, _lib.E4M3, dev, (x, t))
 
 
 def multi_cast_transpose(inputs, outputs, trans_outputs, scales, amaxes):
@@ -426,7 +500,7 @@ def multi_cast_transpose(inputs, outputs, trans_outputs, scales, amaxes):
     table["in"], table["out"], table["out_t"] = x.ptr, o.ptr, t.ptr
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
-    _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE, table, _FMT[dt], dev)
+    _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE, table, _FMT[dt], dev, (x, o, t, scales, amaxes))
 
 
 def multi_cast_transpose_dgelu(inputs, gelu_inputs, outputs, trans_outputs, scales, amaxes):
@@ -452,13 +526,13 @@ def multi_cast_transpose_dgelu(inputs, gelu_inputs, outputs, trans_outputs, scal
     table["in"], table["in2"], table["out"], table["out_t"] = x.ptr, g.ptr, o.ptr, t.ptr
     table["scale"] = _scalar_ptrs(scales, n, "scales")
     table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
-    _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE_DGELU, table, _FMT[dt], dev)
+    _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE_DGELU, table, _FMT[dt], dev, (x, g, o, t, scales, amaxes))
 
 
 # ------------------------------------------------------------------------------------------------
 # GEMMs
 # ------------------------------------------------------------------------------------------------
-def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device):
+def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep):
     if a_dtype not in _FP8_DTYPES or b_dtype not in _FP8_DTYPES:
         _fail("fp8_gmm_amd: GEMM operands must be fp8")
     if a_dtype == torch.float8_e5m2 and b_dtype == torch.float8_e5m2:
@@ -468,13 +542,15 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device):
     total = _lib.plan_grouped_gemm(table)
     if total == 0:
         return
-    dev_table = _upload(table, device)
-    with torch.cuda.device(device), _timed("grouped_gemm", lambda: _algorithmic_flops(table)):
-        rc = _lib.load().fp8gmm_grouped_gemm(
-            dev_table.data_ptr(), len(table), total, _FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype],
-            _lib.EPI_GELU if gelu else 0, _stream(device),
-        )
-    _lib.check(rc)
+    n = len(table)
+    fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], _lib.EPI_GELU if gelu else 0)
+
+    def launch(dev_ptr):
+        with torch.cuda.device(device), _timed("grouped_gemm", lambda: _algorithmic_flops(table)):
+            rc = _lib.load().fp8gmm_grouped_gemm(dev_ptr, n, total, *fmts, _stream(device))
+        _lib.check(rc)
+
+    _submit(table, device, launch, keep)
 
 
 def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False):
@@ -530,7 +606,8 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
     if fp8_out:
         table["c_scale"] = _scalar_ptrs(c_scales, n, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, n, "c_amaxes")
-    _launch_gemm(table, a.dtype, b.dtype, c.dtype, aux is not None, dev)
+    _launch_gemm(table, a.dtype, b.dtype, c.dtype, aux is not None, dev,
+                 (a, b, c, aux, a_scale_invs, b_scale_invs, c_scales, c_amaxes))
 
 
 def cublas_fp8_gemm(a, b, c, a_scale_inv, b_scale_inv, pre_gelu_out=None, c_scale=None, c_amax=None, backward=False):
@@ -619,7 +696,8 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     if fp8_out:
         table["c_scale"] = _scalar_ptrs(c_scales, e, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, e, "c_amaxes")
-    _launch_gemm(table, a.dtype, b.dtype, c.dtype, pre_gelu_out is not None, dev)
+    _launch_gemm(table, a.dtype, b.dtype, c.dtype, pre_gelu_out is not None, dev,
+                 (a, b, c, pre_gelu_out, a_scale_invs, b_scale_invs, c_scales, c_amaxes))
     if cutlass:
         multi_scale_mul(TensorBatch.rows_of(c, starts), a_scale_invs, b_scale_invs)
     return c

@@ -21,7 +21,7 @@ import math
 import numpy as np
 import torch
 
-from .backend import TensorBatch, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
+from .backend import TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
 from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
@@ -56,8 +56,19 @@ def alloc_transposed(features, padded, bounds, padded_bounds, dtype, device):
 
 
 class _GroupedLinear(torch.autograd.Function):
+    # Each pass queues its launches and uploads all their tables with one copy (backend.batched_uploads).
     @staticmethod
-    def forward(ctx, input, weight, group_sizes, fp8_meta, is_grad_enabled, cutlass):
+    def forward(ctx, *args):
+        with batched_uploads():
+            return _GroupedLinear._forward(ctx, *args)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        with batched_uploads():
+            return _GroupedLinear._backward(ctx, grad_out)
+
+    @staticmethod
+    def _forward(ctx, input, weight, group_sizes, fp8_meta, is_grad_enabled, cutlass):
         wgrad_needed = is_grad_enabled and weight.requires_grad
         dgrad_needed = is_grad_enabled and input.requires_grad
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
@@ -135,7 +146,7 @@ class _GroupedLinear(torch.autograd.Function):
         return out
 
     @staticmethod
-    def backward(ctx, grad_out):
+    def _backward(ctx, grad_out):
         input_t_fp8, weight_t_fp8 = ctx.saved_tensors
         meta = ctx.meta
         cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded

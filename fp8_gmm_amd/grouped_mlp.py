@@ -22,6 +22,8 @@ import torch
 
 from .backend import (
     TensorBatch,
+    batched_uploads,
+    flush_uploads,
     fp8_gmm,
     grouped_gemm,
     multi_cast_transpose,
@@ -38,8 +40,19 @@ _M = MetaTensorType
 
 
 class _GroupedMlp(torch.autograd.Function):
+    # Each pass queues its launches and uploads all their tables with one copy (backend.batched_uploads).
     @staticmethod
-    def forward(ctx, input, fc1_weight, fc2_weight, group_sizes, fp8_meta, is_grad_enabled, has_tp, tp_group):
+    def forward(ctx, *args):
+        with batched_uploads():
+            return _GroupedMlp._forward(ctx, *args)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        with batched_uploads():
+            return _GroupedMlp._backward(ctx, grad_out)
+
+    @staticmethod
+    def _forward(ctx, input, fc1_weight, fc2_weight, group_sizes, fp8_meta, is_grad_enabled, has_tp, tp_group):
         input_requires_grad = input.requires_grad
         weight_requires_grad = fc1_weight.requires_grad
         wgrad_needed = is_grad_enabled and weight_requires_grad
@@ -145,7 +158,7 @@ class _GroupedMlp(torch.autograd.Function):
         return out
 
     @staticmethod
-    def backward(ctx, grad_out):
+    def _backward(ctx, grad_out):
         input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
         meta = ctx.meta
         cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
@@ -204,6 +217,7 @@ class _GroupedMlp(torch.autograd.Function):
                 backward=True, cutlass=False,
             )
             if ctx.has_tp:
+                flush_uploads()  # the collective must see grad_input
                 handle = torch.distributed.all_reduce(
                     grad_input, op=torch.distributed.ReduceOp.SUM, group=ctx.tp_group, async_op=True
                 )

@@ -330,3 +330,57 @@ def test_shared_tiles_on_concurrent_streams(dev):
         torch.cuda.synchronize()
         for i, (c, want) in enumerate(zip(outs, wants)):
             assert torch.equal(c.view(torch.int16), want.view(torch.int16)), f"stream {i}, repetition {rep}"
+
+
+def test_batched_uploads_runs_the_queued_launches_in_order(dev):
+    """Inside backend.batched_uploads() launches are queued and their tables travel in one copy; a chain
+    (GEMM -> in-place scale_mul on its result -> quantize of that) must give the same bytes as the immediate
+    calls, nothing may run before the block ends, and a block that raises launches nothing."""
+    backend = _backend()
+    g = gen(77)
+    sizes = [100, 0, 300]
+    m, k, n = sum(sizes), 128, 96
+    a = _q(randn_bf16((m, k), g), E4M3).to(dev)
+    b = _q(randn_bf16((len(sizes), n, k), g), E4M3).to(dev)
+    sa = torch.tensor([0.5, 2.0, 1.5], device=dev)
+    sb = torch.tensor([1.0, 0.25, 3.0], device=dev)
+    one = torch.ones(1, device=dev)
+
+    def chain(c, q, amax):
+        backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, c, cutlass=True)   # GEMM + multi_scale_mul
+        backend.multi_quantize([c], [q], [one], [amax])
+
+    c0 = torch.zeros(m, n, dtype=torch.bfloat16, device=dev)
+    q0 = torch.zeros(m, n, dtype=torch.uint8, device=dev).view(E4M3)
+    am0 = torch.zeros(1, device=dev)
+    chain(c0, q0, am0)
+    c1, q1, am1 = torch.zeros_like(c0), torch.zeros(m, n, dtype=torch.uint8, device=dev).view(E4M3), torch.zeros(1, device=dev)
+    with backend.batched_uploads():
+        chain(c1, q1, am1)
+        torch.cuda.synchronize()
+        assert not c1.any() and am1.item() == 0.0, "queued launches ran before the end of the block"
+    assert torch.equal(c1.view(torch.int16), c0.view(torch.int16))
+    assert torch.equal(q1.view(torch.uint8), q0.view(torch.uint8)) and am1.item() == am0.item()
+    # a queued launch keeps the tensors it addresses alive: the caller's temporary may go out of scope, and the
+    # allocator may hand its memory to the next allocation, before the kernel has even been enqueued
+    src = randn_bf16((512, 256), g).to(dev)
+    want = torch.empty(512, 256, dtype=torch.uint8, device=dev).view(E4M3)
+    backend.multi_quantize([src], [want], [one], [torch.zeros(1, device=dev)])
+    got = torch.empty_like(want)
+    with backend.batched_uploads():
+        def queue_with_temporary():
+            tmp = src.clone()
+            backend.multi_quantize([tmp], [got], [one], [torch.zeros(1, device=dev)])
+        queue_with_temporary()
+        junk = [torch.full((512, 256), 7.0, dtype=torch.bfloat16, device=dev) for _ in range(4)]
+    assert torch.equal(got.view(torch.uint8), want.view(torch.uint8)) and len(junk) == 4
+    c2 = torch.zeros_like(c0)
+    with pytest.raises(ZeroDivisionError):
+        with backend.batched_uploads():
+            backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, c2)
+            1 / 0
+    torch.cuda.synchronize()
+    assert not c2.any()
+    backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, c2)   # and the queue is usable again, immediately
+    torch.cuda.synchronize()
+    assert c2.any()
