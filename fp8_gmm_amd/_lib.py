@@ -23,8 +23,9 @@ OP_SCALE_MUL = 1
 OP_PAD_TRANSPOSE = 2
 OP_PAD_CAST_TRANSPOSE = 3
 OP_PAD_CAST_TRANSPOSE_DGELU = 4
+OP_CAST_DGELU = 5
 
-# struct fp8gmm_tensor_desc (64 bytes)
+# struct fp8gmm_tensor_desc (128 bytes)
 TENSOR_DESC = np.dtype(
     [
         ("in", "<u8"),
@@ -79,6 +80,7 @@ EXPORTS = (
     "fp8gmm_multi_pad_transpose",
     "fp8gmm_multi_pad_cast_transpose",
     "fp8gmm_multi_pad_cast_transpose_dgelu",
+    "fp8gmm_multi_cast_dgelu",
     "fp8gmm_grouped_gemm",
     "fp8gmm_delayed_scaling_update",
     "fp8gmm_gemm_schedule",
@@ -133,10 +135,12 @@ def load():
     L.fp8gmm_multi_pad_cast_transpose.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_multi_pad_cast_transpose_dgelu.restype = ci
     L.fp8gmm_multi_pad_cast_transpose_dgelu.argtypes = [vp, ci, ci, ci, vp]
+    L.fp8gmm_multi_cast_dgelu.restype = ci
+    L.fp8gmm_multi_cast_dgelu.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_grouped_gemm.restype = ci
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
     L.fp8gmm_delayed_scaling_update.restype = ci
-    L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, vp]
+    L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_gemm_schedule.restype = ci
     L.fp8gmm_gemm_schedule.argtypes = [vp, ci, ci, ci, ci, ci, vp, ci]
     L.fp8gmm_gemm_fixup.restype = ci

@@ -91,6 +91,7 @@ _OP_NAMES = {
     _lib.OP_PAD_TRANSPOSE: "multi_pad_transpose",
     _lib.OP_PAD_CAST_TRANSPOSE: "multi_pad_cast_transpose",
     _lib.OP_PAD_CAST_TRANSPOSE_DGELU: "multi_pad_cast_transpose_dgelu",
+    _lib.OP_CAST_DGELU: "multi_cast_dgelu",
 }
 
 
@@ -103,6 +104,8 @@ def _algorithmic_bytes(op, table):
         return int((rows * cols * 3).sum())
     if op == _lib.OP_SCALE_MUL:
         return int((rows * cols * 4).sum())
+    if op == _lib.OP_CAST_DGELU:
+        return int((rows * cols * 5).sum())
     has_out = (table["out"] != 0).astype(np.int64)
     in_bytes = {_lib.OP_PAD_TRANSPOSE: 1, _lib.OP_PAD_CAST_TRANSPOSE: 2, _lib.OP_PAD_CAST_TRANSPOSE_DGELU: 4}[op]
     return int((cols * (rows * in_bytes + rows * has_out + rpad)).sum())
@@ -250,6 +253,8 @@ def _launch_multi(op, table, out_fmt, device, keep):
                 rc = L.fp8gmm_multi_pad_transpose(dev_ptr, n, total, s)
             elif op == _lib.OP_PAD_CAST_TRANSPOSE:
                 rc = L.fp8gmm_multi_pad_cast_transpose(dev_ptr, n, total, out_fmt, s)
+            elif op == _lib.OP_CAST_DGELU:
+                rc = L.fp8gmm_multi_cast_dgelu(dev_ptr, n, total, out_fmt, s)
             else:
                 rc = L.fp8gmm_multi_pad_cast_transpose_dgelu(dev_ptr, n, total, out_fmt, s)
         _lib.check(rc)
@@ -529,6 +534,39 @@ def multi_cast_transpose_dgelu(inputs, gelu_inputs, outputs, trans_outputs, scal
     _launch_multi(_lib.OP_PAD_CAST_TRANSPOSE_DGELU, table, _FMT[dt], dev, (x, g, o, t, scales, amaxes))
 
 
+def multi_cast_dgelu(inputs, gelu_inputs, outputs, scales, amaxes):
+    """outputs[i] = fp8(x * scales[i]) with x = inputs[i] * dgelu(gelu_inputs[i]); amaxes[i] = max(amaxes[i], max|x|).
+
+    ``multi_cast_transpose_dgelu`` without the transposed copy, for a backward pass that needs no weight
+    gradient.  The reference has no such kernel and notes the gap (fp8_gmm/grouped_mlp.py:252-253); the
+    bytes and amax are those of ``multi_cast_transpose_dgelu``'s ``outputs``."""
+    n = len(inputs)
+    if n == 0:
+        return
+    _check_counts(n, gelu_inputs=gelu_inputs, outputs=outputs, scales=scales, amaxes=amaxes)
+    x = _as_batch(inputs, "multi_cast_dgelu inputs", flatten=True)
+    g = _as_batch(gelu_inputs, "multi_cast_dgelu gelu inputs", flatten=True)
+    o = _as_batch(outputs, "multi_cast_dgelu outputs", flatten=True)
+    dev = _same_device(x, g, o)
+    dt = _fp8_dtype_of(o)
+    if x.dtype != torch.bfloat16 or g.dtype != torch.bfloat16:
+        _fail("fp8_gmm_amd: multi_cast_dgelu inputs must be bfloat16")
+    if not (x.contiguous and g.contiguous and o.contiguous):
+        _fail("fp8_gmm_amd: multi_cast_dgelu needs contiguous tensors")
+    numel = x.rows * x.cols
+    if np.any(numel != o.rows * o.cols) or np.any(numel != g.rows * g.cols):
+        _fail("fp8_gmm_amd: multi_cast_dgelu input / gelu input / output shapes differ")
+    if np.any(numel >= 2**31):
+        _fail("fp8_gmm_amd: tensors of 2^31 or more elements are not supported")
+    table = np.zeros(n, dtype=TENSOR_DESC)
+    table["in"], table["in2"], table["out"] = x.ptr, g.ptr, o.ptr
+    table["rows"] = (numel > 0).astype(np.int32)
+    table["cols"] = numel
+    table["scale"] = _scalar_ptrs(scales, n, "scales")
+    table["amax"] = _scalar_ptrs(amaxes, n, "amaxes")
+    _launch_multi(_lib.OP_CAST_DGELU, table, _FMT[dt], dev, (x, g, o, scales, amaxes))
+
+
 # ------------------------------------------------------------------------------------------------
 # GEMMs
 # ------------------------------------------------------------------------------------------------
@@ -553,9 +591,11 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep):
     _submit(table, device, launch, keep)
 
 
-def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False):
+def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False, keep_scale_inv=None):
     """In-place delayed-scaling update of one direction in ONE kernel (the rule of
-    ``fp8.amax_and_scale_update``): ``amax_history`` [history, slots], ``scale`` / ``scale_inv`` [slots]."""
+    ``fp8.amax_and_scale_update``): ``amax_history`` [history, slots], ``scale`` / ``scale_inv`` [slots].
+    ``keep_scale_inv=(period, phase)`` leaves ``scale_inv[slot]`` untouched where ``slot % period == phase``."""
+    period, phase = keep_scale_inv if keep_scale_inv is not None else (0, 0)
     for t, what in ((amax_history, "amax_history"), (scale, "scale"), (scale_inv, "scale_inv")):
         if t.dtype != torch.float32 or not t.is_contiguous():
             _fail(f"fp8_gmm_amd: {what} must be a contiguous fp32 tensor")
@@ -565,7 +605,8 @@ def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, mo
     with torch.cuda.device(dev):
         rc = _lib.load().fp8gmm_delayed_scaling_update(
             amax_history.data_ptr(), scale.data_ptr(), scale_inv.data_ptr(), amax_history.shape[0],
-            amax_history.shape[1], float(fp8_max), int(margin), int(bool(most_recent)), _stream(dev))
+            amax_history.shape[1], float(fp8_max), int(margin), int(bool(most_recent)), int(period), int(phase),
+            _stream(dev))
     _lib.check(rc)
 
 

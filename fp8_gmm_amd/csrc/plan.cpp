@@ -34,7 +34,7 @@ size_t fp8gmm_sizeof_gemm_problem(void) { return sizeof(fp8gmm_gemm_problem); }
 
 int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* total_blocks) {
   if (n < 0) return FP8GMM_ERR_BAD_ARGUMENT;
-  if (op < FP8GMM_OP_QUANTIZE || op > FP8GMM_OP_PAD_CAST_TRANSPOSE_DGELU) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (op < FP8GMM_OP_QUANTIZE || op > FP8GMM_OP_CAST_DGELU) return FP8GMM_ERR_BAD_ARGUMENT;
   if (total_blocks == nullptr || (n > 0 && descs == nullptr)) return FP8GMM_ERR_NULL_POINTER;
   int64_t blocks = 0;
   for (int i = 0; i < n; ++i) {
@@ -42,10 +42,11 @@ int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* tota
     if (d.rows < 0 || d.cols < 0) return FP8GMM_ERR_BAD_SHAPE;
     const int64_t numel = (int64_t)d.rows * d.cols;
     int64_t nb = 0;
-    if (op == FP8GMM_OP_QUANTIZE || op == FP8GMM_OP_SCALE_MUL) {
+    if (op == FP8GMM_OP_QUANTIZE || op == FP8GMM_OP_SCALE_MUL || op == FP8GMM_OP_CAST_DGELU) {
       if (numel > 0) {
         if (d.in == nullptr) return FP8GMM_ERR_NULL_POINTER;
-        if (op == FP8GMM_OP_QUANTIZE && d.out == nullptr) return FP8GMM_ERR_NULL_POINTER;
+        if (op != FP8GMM_OP_SCALE_MUL && d.out == nullptr) return FP8GMM_ERR_NULL_POINTER;
+        if (op == FP8GMM_OP_CAST_DGELU && d.in2 == nullptr) return FP8GMM_ERR_NULL_POINTER;
       }
       nb = (numel + fp8gmm::kPwBlockElems - 1) / fp8gmm::kPwBlockElems;
     } else {

@@ -13,7 +13,9 @@
 namespace fp8gmm {
 namespace {
 
-template <int FMT>
+// DGELU: the value cast is x = in * dgelu(in2) (in = gradient of the GELU output, in2 = pre-GELU activation),
+// the same product, in the same order, as the transposing kernel forms.
+template <int FMT, bool DGELU>
 __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tensor_desc* __restrict__ descs, int n) {
   __shared__ float stage[kPwThreads / kWaveSize];
   const int bid = blockIdx.x;
@@ -22,23 +24,33 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tenso
   const int64_t numel = (int64_t)d.rows * d.cols;
   const int64_t base = (int64_t)(bid - d.block_begin) * kPwBlockElems;
   const uint16_t* __restrict__ in = static_cast<const uint16_t*>(d.in);
+  const uint16_t* __restrict__ pre = static_cast<const uint16_t*>(d.in2);
   uint8_t* __restrict__ out = static_cast<uint8_t*>(d.out);
   const float scale = d.scale ? *d.scale : 1.f;
-  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0 &&
+  const bool vec = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out) |
+                     (DGELU ? reinterpret_cast<uintptr_t>(pre) : 0)) & 15) == 0 &&
                    numel * 2 < (int64_t)0xffffffff;
   float mx = 0.f;
+  auto value = [&](int64_t j) {
+    float x = bf16_to_f32(in[j]);
+    if constexpr (DGELU) x *= dgelu(bf16_to_f32(pre[j]));
+    return x;
+  };
 
   if (vec) {
     // fast path: all loads of the workgroup's 16384 elements are issued before the first conversion
     const __amdgpu_buffer_rsrc_t rin = make_rsrc(in, (uint32_t)(numel * 2));
     const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, (uint32_t)numel);
+    const __amdgpu_buffer_rsrc_t rpre = make_rsrc(DGELU ? pre : in, (uint32_t)(numel * 2));
     u32x4 a[kPwSteps];
+    u32x4 g[DGELU ? kPwSteps : 1];
     bool full[kPwSteps];
 #pragma unroll
     for (int it = 0; it < kPwSteps; ++it) {
       const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
       full[it] = off + kPwVec <= numel;
       a[it] = buf_load16(rin, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+      if constexpr (DGELU) g[it] = buf_load16(rpre, full[it] ? (uint32_t)(off * 2) : kOobOffset);
     }
 #pragma unroll
     for (int it = 0; it < kPwSteps; ++it) {
@@ -47,8 +59,15 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tenso
       uint32_t o[2];
 #pragma unroll
       for (int q = 0; q < 2; ++q) {
-        const float x0 = bf16_lo_to_f32(w[2 * q]), x1 = bf16_hi_to_f32(w[2 * q]);
-        const float x2 = bf16_lo_to_f32(w[2 * q + 1]), x3 = bf16_hi_to_f32(w[2 * q + 1]);
+        float x0 = bf16_lo_to_f32(w[2 * q]), x1 = bf16_hi_to_f32(w[2 * q]);
+        float x2 = bf16_lo_to_f32(w[2 * q + 1]), x3 = bf16_hi_to_f32(w[2 * q + 1]);
+        if constexpr (DGELU) {
+          const uint32_t p[4] = {g[it].x, g[it].y, g[it].z, g[it].w};
+          x0 *= dgelu(bf16_lo_to_f32(p[2 * q]));
+          x1 *= dgelu(bf16_hi_to_f32(p[2 * q]));
+          x2 *= dgelu(bf16_lo_to_f32(p[2 * q + 1]));
+          x3 *= dgelu(bf16_hi_to_f32(p[2 * q + 1]));
+        }
         mx = amax_step(amax_step(mx, x0), x1);
         mx = amax_step(amax_step(mx, x2), x3);
         o[q] = cvt4_fp8<FMT>(x0 * scale, x1 * scale, x2 * scale, x3 * scale);
@@ -56,7 +75,7 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tenso
       buf_store8(u32x2{o[0], o[1]}, rout, full[it] ? (uint32_t)off : kOobOffset);
       if (!full[it] && off < numel) {  // the one partial group at the end of the tensor
         for (int64_t j = off; j < numel; ++j) {
-          const float x = bf16_to_f32(in[j]);
+          const float x = value(j);
           mx = amax_step(mx, x);
           out[j] = cvt1_fp8<FMT>(x * scale);
         }
@@ -69,7 +88,7 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tenso
       if (off < numel) {
         const int cnt = (numel - off < kPwVec) ? (int)(numel - off) : kPwVec;
         for (int j = 0; j < cnt; ++j) {
-          const float x = bf16_to_f32(in[off + j]);
+          const float x = value(off + j);
           mx = amax_step(mx, x);
           out[off + j] = cvt1_fp8<FMT>(x * scale);
         }
@@ -135,7 +154,8 @@ __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gm
 // amax matrix are independent, rows of a column are walked by the lane that owns it):
 //   amax      = max over the history column (or its row 0)
 //   scale     = (1 / amax) * fp8_max * 2^-margin   where amax is finite and > 0, else unchanged
-//   scale_inv = 1 / scale
+//   scale_inv = 1 / scale, except in slots with slot % keep_period == keep_phase (keep_period > 0): those
+//               keep their value, for tensors whose fp8 copy from an earlier pass is still in use
 //   history   : row i <- row i + 1, last row <- old row 0, then row 0 <- 0 (a history of one row is just cleared)
 // The factor is formed as reciprocal times fp8_max, which is what `fp8_max / amax` on a torch tensor
 // evaluates to; the two differ in the last bit for some inputs.
@@ -143,7 +163,8 @@ __global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __re
                                                                      float* __restrict__ scale,
                                                                      float* __restrict__ scale_inv, int history_len,
                                                                      int slots, float fp8_max, float margin_factor,
-                                                                     int most_recent) {
+                                                                     int most_recent, int keep_period,
+                                                                     int keep_phase) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= slots) return;
   float* col = history + c;
@@ -159,7 +180,7 @@ __global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __re
   float sc = scale[c];
   if (amax > 0.f && amax <= 3.4028234663852886e38f) sc = ((1.0f / amax) * fp8_max) * margin_factor;
   scale[c] = sc;
-  scale_inv[c] = 1.0f / sc;
+  if (!(keep_period > 0 && c % keep_period == keep_phase)) scale_inv[c] = 1.0f / sc;
   for (int i = 0; i + 1 < history_len; ++i) col[(size_t)i * slots] = col[(size_t)(i + 1) * slots];
   if (history_len > 1) col[(size_t)(history_len - 1) * slots] = first;
   col[0] = 0.f;
@@ -168,34 +189,48 @@ __global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __re
 }  // namespace
 }  // namespace fp8gmm
 
-extern "C" {
-
-int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
-                                  float fp8_max, int margin, int most_recent, void* stream) {
-  if (history_len < 1 || slots < 0 || margin < -126 || margin > 126) return FP8GMM_ERR_BAD_ARGUMENT;
-  if (slots == 0) return FP8GMM_OK;
-  if (amax_history == nullptr || scale == nullptr || scale_inv == nullptr) return FP8GMM_ERR_NULL_POINTER;
-  const float margin_factor = __builtin_ldexpf(1.0f, -margin);
-  hipLaunchKernelGGL(fp8gmm::delayed_scaling_update_kernel, dim3((slots + 255) / 256), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), amax_history, scale, scale_inv, history_len, slots, fp8_max,
-                     margin_factor, most_recent != 0);
-  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
-}
-
-int fp8gmm_multi_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+namespace {
+template <bool DGELU>
+int launch_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
   if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_fmt != FP8GMM_E4M3 && out_fmt != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
   if (n == 0 || total_blocks == 0) return FP8GMM_OK;
   if (descs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (out_fmt == FP8GMM_E4M3)
-    hipLaunchKernelGGL(fp8gmm::multi_quantize_kernel<FP8GMM_E4M3>, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0, s,
-                       descs_dev, n);
+    hipLaunchKernelGGL((fp8gmm::multi_quantize_kernel<FP8GMM_E4M3, DGELU>), dim3(total_blocks),
+                       dim3(fp8gmm::kPwThreads), 0, s, descs_dev, n);
   else
-    hipLaunchKernelGGL(fp8gmm::multi_quantize_kernel<FP8GMM_E5M2>, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0, s,
-                       descs_dev, n);
+    hipLaunchKernelGGL((fp8gmm::multi_quantize_kernel<FP8GMM_E5M2, DGELU>), dim3(total_blocks),
+                       dim3(fp8gmm::kPwThreads), 0, s, descs_dev, n);
   hipLaunchKernelGGL(fp8gmm::amax_merge_kernel, dim3((n + 255) / 256), dim3(256), 0, s, descs_dev, n);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+}  // namespace
+
+extern "C" {
+
+int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
+                                  float fp8_max, int margin, int most_recent, int keep_period, int keep_phase,
+                                  void* stream) {
+  if (history_len < 1 || slots < 0 || margin < -126 || margin > 126) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (keep_period < 0 || (keep_period > 0 && (keep_phase < 0 || keep_phase >= keep_period)))
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if (slots == 0) return FP8GMM_OK;
+  if (amax_history == nullptr || scale == nullptr || scale_inv == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  const float margin_factor = __builtin_ldexpf(1.0f, -margin);
+  hipLaunchKernelGGL(fp8gmm::delayed_scaling_update_kernel, dim3((slots + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), amax_history, scale, scale_inv, history_len, slots, fp8_max,
+                     margin_factor, most_recent != 0, keep_period, keep_phase);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_multi_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+  return launch_quantize<false>(descs_dev, n, total_blocks, out_fmt, stream);
+}
+
+int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+  return launch_quantize<true>(descs_dev, n, total_blocks, out_fmt, stream);
 }
 
 int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, void* stream) {

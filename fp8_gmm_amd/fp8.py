@@ -18,6 +18,11 @@ meaning, sized for what the grouped modules use:
       amax_history = roll(amax_history, -1, dim=0);  amax_history[0] = 0
   fp8_max is 448 for e4m3 and 57344 for e5m2.  HYBRID means e4m3 for forward tensors
   and e5m2 for gradients.
+* FP8 weight caching (``forward(..., is_first_microbatch=True / False)``, TransformerEngine's convention, which
+  the reference stubs out at grouped_linear.py:200-202 and grouped_mlp.py:343-345): the first micro-batch of a
+  step casts the weights into buffers the module keeps, the later ones reuse them and skip the cast.  On those
+  later passes the update leaves the weights' ``scale_inv`` alone (the cached bytes were cast with it) and their
+  amax slots receive nothing.  ``None`` (the default, and all the reference supports) casts on every pass.
 * Both directions are updated.  (The reference never enters TransformerEngine's
   backward context, so its gradient scales stay at their initial value of 1; updating
   them is a deliberate difference - e5m2 gradients need real scales.)
@@ -116,8 +121,9 @@ class Fp8MetaTensors:
         self.amax_history.copy_(state["amax_history"])
 
 
-def amax_and_scale_update(meta, fp8_max, fp8_recipe):
+def amax_and_scale_update(meta, fp8_max, fp8_recipe, keep_scale_inv=None):
     """Delayed-scaling update of one direction, in place (rule in the module docstring).
+    ``keep_scale_inv=(period, phase)``: ``scale_inv`` of the slots with ``slot % period == phase`` is not touched.
 
     Scaling state that lives on the GPU is updated by one fused kernel
     (``backend.delayed_scaling_update``); the torch statement of the rule below serves CPU tensors
@@ -127,16 +133,46 @@ def amax_and_scale_update(meta, fp8_max, fp8_recipe):
     if hist.is_cuda and float(fp8_recipe.margin) == int(fp8_recipe.margin):
         from . import backend
 
-        backend.delayed_scaling_update(hist, meta.scale, meta.scale_inv, fp8_max, int(fp8_recipe.margin), most_recent)
+        backend.delayed_scaling_update(hist, meta.scale, meta.scale_inv, fp8_max, int(fp8_recipe.margin), most_recent,
+                                       keep_scale_inv)
         return
     amax = hist[0].clone() if most_recent else hist.max(dim=0).values
     sf = (fp8_max / amax) / (2.0 ** fp8_recipe.margin)
     ok = (amax > 0) & torch.isfinite(amax)
     meta.scale.copy_(torch.where(ok, sf, meta.scale))
-    meta.scale_inv.copy_(1.0 / meta.scale)
+    new_inv = 1.0 / meta.scale
+    if keep_scale_inv is not None:
+        kept = torch.arange(meta.scale.numel(), device=meta.scale.device) % keep_scale_inv[0] == keep_scale_inv[1]
+        new_inv = torch.where(kept, meta.scale_inv, new_inv)
+    meta.scale_inv.copy_(new_inv)
     if hist.shape[0] > 1:
         hist.copy_(torch.roll(hist, -1, 0))
     hist[0].zero_()
+
+
+class Fp8WeightCache:
+    """fp8 copies (row-major and transposed) of one ``[E, N, K]`` weight stack, kept across micro-batches."""
+
+    def __init__(self):
+        self.fp8 = None      # [E, N, K]
+        self.fp8_t = None    # [E, K, N]
+        self.valid = False   # fp8 holds a cast of the weights
+        self.valid_t = False  # fp8_t does too
+
+    def buffers(self, weight, dtype):
+        if self.fp8 is None or self.fp8.shape != weight.shape or self.fp8.dtype != dtype \
+                or self.fp8.device != weight.device:
+            e, n, k = weight.shape
+            self.fp8 = torch.empty(e, n, k, dtype=dtype, device=weight.device)
+            self.fp8_t = torch.empty(e, k, n, dtype=dtype, device=weight.device)
+            self.valid = self.valid_t = False
+        return self.fp8, self.fp8_t
+
+    def require(self, transposed):
+        if not self.valid or (transposed and not self.valid_t):
+            raise RuntimeError(
+                "is_first_microbatch=False, but no earlier pass with is_first_microbatch=True has cast the "
+                "weights" + (" with their transposes (it ran without gradients)" if self.valid else ""))
 
 
 class Fp8GroupedModuleBase(torch.nn.Module):
@@ -144,11 +180,17 @@ class Fp8GroupedModuleBase(torch.nn.Module):
 
     FWD_SLOTS_PER_GEMM = 3
     BWD_SLOTS_PER_GEMM = 2
+    WEIGHT_SLOT = 1  # position of a GEMM's weight among its forward slots (input, weight, output)
 
     def __init__(self):
         super().__init__()
         self.fp8_meta = {}
         self._fp8_steps = 0
+        self._weight_caches = []  # Fp8WeightCache objects of the subclass; dropped whenever the scales are replaced
+
+    def _invalidate_weight_caches(self):
+        for cache in self._weight_caches:
+            cache.valid = cache.valid_t = False
 
     def _init_fp8_meta(self, fp8_recipe, num_gemms, device):
         meta = self.fp8_meta
@@ -167,6 +209,7 @@ class Fp8GroupedModuleBase(torch.nn.Module):
         meta["fp8_max_fwd"] = FP8_MAX[get_fp8_te_dtype(fp8_recipe, True)]
         meta["fp8_max_bwd"] = FP8_MAX[get_fp8_te_dtype(fp8_recipe, False)]
         self._fp8_steps = 0
+        self._invalidate_weight_caches()
 
     @contextlib.contextmanager
     def prepare_forward(self, inp, is_first_microbatch, num_gemms=1):
@@ -174,16 +217,19 @@ class Fp8GroupedModuleBase(torch.nn.Module):
 
         Outside ``fp8_autocast`` the default recipe is used (the modules are FP8-only).
         In training mode every pass after the first starts with the delayed-scaling
-        update of both directions, every ``recipe.interval`` passes.
+        update of both directions, every ``recipe.interval`` passes.  ``is_first_microbatch=False``
+        (cached fp8 weights are reused) keeps the weights' ``scale_inv`` out of that update.
         """
-        assert is_first_microbatch is None, "FP8 weight caching across micro-batches is not implemented"
+        update_weights = is_first_microbatch is None or bool(is_first_microbatch)
         fp8_recipe = current_recipe() or self.fp8_meta.get("recipe") or DelayedScaling()
         self._init_fp8_meta(fp8_recipe, num_gemms, inp.device)
         self._apply_pending_state()
         if self.training and torch.is_grad_enabled():
             if self._fp8_steps > 0 and self._fp8_steps % fp8_recipe.interval == 0:
                 with torch.no_grad():
-                    amax_and_scale_update(self.fp8_meta["scaling_fwd"], self.fp8_meta["fp8_max_fwd"], fp8_recipe)
+                    amax_and_scale_update(
+                        self.fp8_meta["scaling_fwd"], self.fp8_meta["fp8_max_fwd"], fp8_recipe,
+                        None if update_weights else (self.FWD_SLOTS_PER_GEMM, self.WEIGHT_SLOT))
                     amax_and_scale_update(self.fp8_meta["scaling_bwd"], self.fp8_meta["fp8_max_bwd"], fp8_recipe)
             self._fp8_steps += 1
         yield
@@ -218,3 +264,4 @@ class Fp8GroupedModuleBase(torch.nn.Module):
         fwd.load_state(state["scaling_fwd"])
         bwd.load_state(state["scaling_bwd"])
         self._fp8_steps = state["steps"]
+        self._invalidate_weight_caches()

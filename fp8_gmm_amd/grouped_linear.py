@@ -22,7 +22,7 @@ import numpy as np
 import torch
 
 from .backend import TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
-from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
+from .fp8 import Fp8GroupedModuleBase, Fp8WeightCache, get_fp8_te_dtype
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
 
@@ -55,6 +55,38 @@ def alloc_transposed(features, padded, bounds, padded_bounds, dtype, device):
     return flat, transposed_views(flat, b)
 
 
+def stage_weight_cast(weight, fp8_dtype, transpose_needed, is_grad_enabled, cache, update, scales, amaxes, plain,
+                      with_t):
+    """Chooses where the fp8 copies of a ``[E, N, K]`` weight stack live and appends their cast to the pending
+    cast lists (``plain``: cast only, ``with_t``: cast + transpose).  Returns ``(weight_fp8, weight_t_fp8)``.
+
+    Without a cache the copies are temporaries of this pass and the transposed one exists only when this pass
+    needs it (reference grouped_linear.py:64-85).  With a cache (fp8.Fp8WeightCache) they are the module's
+    buffers: a refreshing pass casts into them - with the transpose whenever gradients are enabled, since later
+    micro-batches may need it - and a reusing pass appends nothing."""
+    e, n, k = weight.shape
+    if cache is None:
+        weight_fp8 = torch.empty(weight.shape, dtype=fp8_dtype, device=weight.device)
+        weight_t_fp8 = torch.empty(e, k, n, dtype=fp8_dtype, device=weight.device) if transpose_needed else None
+        cast_t = transpose_needed
+    else:
+        weight_fp8, weight_t_fp8 = cache.buffers(weight, fp8_dtype)
+        if not update:
+            cache.require(transpose_needed)
+            return weight_fp8, (weight_t_fp8 if transpose_needed else None)
+        cast_t = is_grad_enabled
+        cache.valid, cache.valid_t = True, cast_t
+    if cast_t:
+        for lst, item in zip(with_t, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8),
+                                      TensorBatch.stack_of(weight_t_fp8), scales, amaxes)):
+            lst.append(item)
+    else:
+        for lst, item in zip(plain, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8), scales,
+                                     amaxes)):
+            lst.append(item)
+    return weight_fp8, (weight_t_fp8 if transpose_needed else None)
+
+
 class _GroupedLinear(torch.autograd.Function):
     # Each pass queues its launches and uploads all their tables with one copy (backend.batched_uploads).
     @staticmethod
@@ -68,7 +100,10 @@ class _GroupedLinear(torch.autograd.Function):
             return _GroupedLinear._backward(ctx, grad_out)
 
     @staticmethod
-    def _forward(ctx, input, weight, group_sizes, fp8_meta, is_grad_enabled, cutlass):
+    def _forward(ctx, input, weight, group_sizes, fp8_meta, is_grad_enabled, cutlass, weight_cache=None,
+                 update_fp8_weights=True):
+        """The reference's argument list (grouped_linear.py:13) plus, as TransformerEngine's own linear layers
+        have them, the cache of fp8 weights and whether this pass refreshes it."""
         wgrad_needed = is_grad_enabled and weight.requires_grad
         dgrad_needed = is_grad_enabled and input.requires_grad
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
@@ -100,20 +135,10 @@ class _GroupedLinear(torch.autograd.Function):
                                          x_amaxes)):
                 lst.append(item)
 
-        weight_fp8 = torch.empty(weight.shape, dtype=fp8_dtype, device=weight.device)
-        weight_t_fp8 = None
         w_scales = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kScale)
         w_amaxes = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kAmax)
-        if dgrad_needed:
-            weight_t_fp8 = torch.empty(num_groups, weight.size(2), weight.size(1), dtype=fp8_dtype,
-                                       device=weight.device)
-            for lst, item in zip(with_t, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8),
-                                          TensorBatch.stack_of(weight_t_fp8), w_scales, w_amaxes)):
-                lst.append(item)
-        else:
-            for lst, item in zip(plain, (TensorBatch.stack_of(weight), TensorBatch.stack_of(weight_fp8), w_scales,
-                                         w_amaxes)):
-                lst.append(item)
+        weight_fp8, weight_t_fp8 = stage_weight_cast(weight, fp8_dtype, dgrad_needed, is_grad_enabled, weight_cache,
+                                                     update_fp8_weights, w_scales, w_amaxes, plain, with_t)
 
         if plain[0]:
             multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
@@ -183,7 +208,7 @@ class _GroupedLinear(torch.autograd.Function):
                 g_t_views, x_t_views, TensorBatch.stack_of(grad_weight), g_scale_invs,
                 meta.get_meta_pointers(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv),
             )
-        return grad_input, grad_weight, None, None, None, None
+        return grad_input, grad_weight, None, None, None, None, None, None
 
 
 class GroupedLinear(Fp8GroupedModuleBase):
@@ -191,6 +216,8 @@ class GroupedLinear(Fp8GroupedModuleBase):
 
     ``forward(input[tokens, in_features], group_sizes[E])`` where ``group_sizes`` is a CPU
     int64 tensor (or list) of rows per expert, in order; returns ``[tokens, out_features]`` bf16.
+    ``is_first_microbatch``: None casts the weights to fp8 on every pass; True casts them into buffers the
+    module keeps; False reuses those buffers (gradient accumulation over micro-batches of one optimizer step).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False,
@@ -207,15 +234,24 @@ class GroupedLinear(Fp8GroupedModuleBase):
         )
         bound = math.sqrt(1.0 / in_features)
         torch.nn.init.uniform_(self.weight_tensor.data, -bound, bound)
+        self._weight_cache = Fp8WeightCache()
+        self._weight_caches.append(self._weight_cache)
 
     def get_fp8_weights_scratchpad(self, is_first_microbatch):
-        assert is_first_microbatch is None
-        return [None, None]
+        """``[weight_fp8, weight_t_fp8]``: the buffers that keep the fp8 weights across micro-batches, or Nones
+        when ``is_first_microbatch`` is None and every pass casts into temporaries (all the reference
+        supports, grouped_linear.py:200-202)."""
+        if is_first_microbatch is None:
+            return [None, None]
+        dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
+        return list(self._weight_cache.buffers(self.weight_tensor, dtype))
 
     def forward(self, input, group_sizes, is_first_microbatch=None):
         with self.prepare_forward(input, is_first_microbatch, self.num_groups):
             grad = torch.is_grad_enabled()
             args = (input, self.weight_tensor, group_sizes, self.fp8_meta, grad, self.cutlass)
+            if is_first_microbatch is not None:
+                args += (self._weight_cache, bool(is_first_microbatch))
             if grad:
                 return _GroupedLinear.apply(*args)
             return _GroupedLinear.forward(None, *args)

@@ -27,12 +27,13 @@ from .backend import (
     fp8_gmm,
     grouped_gemm,
     multi_cast_transpose,
+    multi_cast_dgelu,
     multi_cast_transpose_dgelu,
     multi_quantize,
     multi_transpose,
 )
-from .fp8 import Fp8GroupedModuleBase, get_fp8_te_dtype
-from .grouped_linear import MODULE_PAD_MULTIPLE, alloc_transposed, row_slices, transposed_views
+from .fp8 import Fp8GroupedModuleBase, Fp8WeightCache, get_fp8_te_dtype
+from .grouped_linear import MODULE_PAD_MULTIPLE, alloc_transposed, row_slices, stage_weight_cast, transposed_views
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
 _T = Fp8TensorType
@@ -52,7 +53,8 @@ class _GroupedMlp(torch.autograd.Function):
             return _GroupedMlp._backward(ctx, grad_out)
 
     @staticmethod
-    def _forward(ctx, input, fc1_weight, fc2_weight, group_sizes, fp8_meta, is_grad_enabled, has_tp, tp_group):
+    def _forward(ctx, input, fc1_weight, fc2_weight, group_sizes, fp8_meta, is_grad_enabled, has_tp, tp_group,
+                 weight_caches=(None, None), update_fp8_weights=True):
         input_requires_grad = input.requires_grad
         weight_requires_grad = fc1_weight.requires_grad
         wgrad_needed = is_grad_enabled and weight_requires_grad
@@ -86,26 +88,14 @@ class _GroupedMlp(torch.autograd.Function):
                                          x_amaxes)):
                 lst.append(item)
 
-        fc1_weight_fp8 = torch.empty(fc1_weight.shape, dtype=fp8_dtype, device=dev)
-        fc2_weight_fp8 = torch.empty(fc2_weight.shape, dtype=fp8_dtype, device=dev)
-        fc1_weight_t_fp8 = fc2_weight_t_fp8 = None
-        w_scales = np.concatenate([meta.get_meta_pointers(_T.kWeightGroup1, _M.kScale),
-                                   meta.get_meta_pointers(_T.kWeightGroup2, _M.kScale)])
-        w_amaxes = np.concatenate([meta.get_meta_pointers(_T.kWeightGroup1, _M.kAmax),
-                                   meta.get_meta_pointers(_T.kWeightGroup2, _M.kAmax)])
-        w_in = TensorBatch.stack_of(fc1_weight) + TensorBatch.stack_of(fc2_weight)
-        w_out = TensorBatch.stack_of(fc1_weight_fp8) + TensorBatch.stack_of(fc2_weight_fp8)
-        if dgrad_needed:
-            fc1_weight_t_fp8 = torch.empty(num_groups, fc1_weight.size(2), fc1_weight.size(1), dtype=fp8_dtype,
-                                           device=dev)
-            fc2_weight_t_fp8 = torch.empty(num_groups, fc2_weight.size(2), fc2_weight.size(1), dtype=fp8_dtype,
-                                           device=dev)
-            w_t = TensorBatch.stack_of(fc1_weight_t_fp8) + TensorBatch.stack_of(fc2_weight_t_fp8)
-            for lst, item in zip(with_t, (w_in, w_out, w_t, w_scales, w_amaxes)):
-                lst.append(item)
-        else:
-            for lst, item in zip(plain, (w_in, w_out, w_scales, w_amaxes)):
-                lst.append(item)
+        fc1_weight_fp8, fc1_weight_t_fp8 = stage_weight_cast(
+            fc1_weight, fp8_dtype, dgrad_needed, is_grad_enabled, weight_caches[0], update_fp8_weights,
+            meta.get_meta_pointers(_T.kWeightGroup1, _M.kScale), meta.get_meta_pointers(_T.kWeightGroup1, _M.kAmax),
+            plain, with_t)
+        fc2_weight_fp8, fc2_weight_t_fp8 = stage_weight_cast(
+            fc2_weight, fp8_dtype, dgrad_needed, is_grad_enabled, weight_caches[1], update_fp8_weights,
+            meta.get_meta_pointers(_T.kWeightGroup2, _M.kScale), meta.get_meta_pointers(_T.kWeightGroup2, _M.kAmax),
+            plain, with_t)
 
         if plain[0]:
             multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
@@ -197,15 +187,21 @@ class _GroupedMlp(torch.autograd.Function):
             backward=True, cutlass=False,
         )
 
-        # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8 (+ padded transpose for fc1 wgrad)
+        # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8; the padded transpose only feeds fc1 wgrad
+        # (the reference always transposes and notes the missing cast-only kernel, grouped_mlp.py:252-253)
         grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
-        _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums, grad_dtype, dev)
-        multi_cast_transpose_dgelu(
-            row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums), row_slices(grad_pre_fp8, cumsums),
-            grad_pre_t_views,
-            meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale),
-            meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax),
-        )
+        g2_scales = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale)
+        g2_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax)
+        if wgrad:
+            _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
+                                                   dev)
+            multi_cast_transpose_dgelu(
+                row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums),
+                row_slices(grad_pre_fp8, cumsums), grad_pre_t_views, g2_scales, g2_amaxes,
+            )
+        else:
+            multi_cast_dgelu(row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums),
+                             row_slices(grad_pre_fp8, cumsums), g2_scales, g2_amaxes)
         g2_scale_invs = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScaleInv)
 
         grad_input = None
@@ -232,13 +228,15 @@ class _GroupedMlp(torch.autograd.Function):
             )
         if handle is not None:
             handle.wait()
-        return grad_input, grad_fc1_weight, grad_fc2_weight, None, None, None, None, None
+        return grad_input, grad_fc1_weight, grad_fc2_weight, None, None, None, None, None, None, None
 
 
 class GroupedMlp(Fp8GroupedModuleBase):
     """E expert MLPs ``in_features -> out_features -> in_features`` with tanh-GELU, no biases.
 
-    ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None)``.
+    ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None, is_first_microbatch=None)``;
+    ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
+    the module's fp8 weight buffers).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
@@ -256,15 +254,23 @@ class GroupedMlp(Fp8GroupedModuleBase):
         b1, b2 = math.sqrt(1.0 / in_features), math.sqrt(1.0 / out_features)
         torch.nn.init.uniform_(self.fc1_weight.data, -b1, b1)
         torch.nn.init.uniform_(self.fc2_weight.data, -b2, b2)
+        self._weight_caches.extend([Fp8WeightCache(), Fp8WeightCache()])
 
     def get_fp8_weights_scratchpad(self, is_first_microbatch):
-        assert is_first_microbatch is None
-        return [None, None, None, None]
+        """``[fc1_weight_fp8, fc1_weight_t_fp8, fc2_weight_fp8, fc2_weight_t_fp8]`` kept across micro-batches, or
+        Nones when ``is_first_microbatch`` is None (all the reference supports, grouped_mlp.py:343-345)."""
+        if is_first_microbatch is None:
+            return [None, None, None, None]
+        dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
+        return list(self._weight_caches[0].buffers(self.fc1_weight, dtype)) + \
+            list(self._weight_caches[1].buffers(self.fc2_weight, dtype))
 
     def forward(self, input, group_sizes, has_tp=False, tp_group=None, is_first_microbatch=None):
         with self.prepare_forward(input, is_first_microbatch, self.num_groups * 2):
             grad = torch.is_grad_enabled()
             args = (input, self.fc1_weight, self.fc2_weight, group_sizes, self.fp8_meta, grad, has_tp, tp_group)
+            if is_first_microbatch is not None:
+                args += (tuple(self._weight_caches), bool(is_first_microbatch))
             if grad:
                 return _GroupedMlp.apply(*args)
             return _GroupedMlp.forward(None, *args)

@@ -61,6 +61,7 @@ typedef enum fp8gmm_status {
  *  multi_pad_transpose             fp8        -          -               fp8 [cols, rows_padded]     -
  *  multi_pad_cast_transpose        bf16       -          fp8 (or NULL)   fp8 [cols, rows_padded]     read / max-merged
  *  multi_pad_cast_transpose_dgelu  bf16 dy    bf16 pre   fp8 (or NULL)   fp8 [cols, rows_padded]     read / max-merged
+ *  multi_cast_dgelu                bf16 dy    bf16 pre   fp8 same shape  -                           read / max-merged
  *
  * `scale` NULL means 1.0 (reference csrc/multi_pointwise.cu:51); `amax` NULL
  * means "do not record" (csrc/multi_pad_fusion.cu:290).  `amax` is merged with
@@ -94,6 +95,7 @@ typedef struct fp8gmm_tensor_desc {
 #define FP8GMM_OP_PAD_TRANSPOSE 2
 #define FP8GMM_OP_PAD_CAST_TRANSPOSE 3
 #define FP8GMM_OP_PAD_CAST_TRANSPOSE_DGELU 4
+#define FP8GMM_OP_CAST_DGELU 5
 
 /*
  * One GEMM of a grouped launch:  c[m, n] = epilogue( a[m, k] . b[n, k]^T ).
@@ -163,6 +165,11 @@ int fp8gmm_multi_pad_cast_transpose(fp8gmm_tensor_desc* descs_dev, int n, int to
 int fp8gmm_multi_pad_cast_transpose_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt,
                                           void* stream);
 
+/* x = dy * dgelu(pre) cast to fp8 WITHOUT the transposed copy: the kernel the reference says it lacks
+ * ("Maybe need a new kernel for cast_dgelu only when weight requires no grad", fp8_gmm/grouped_mlp.py:252-253).
+ * Same values and bytes as the `out` of fp8gmm_multi_pad_cast_transpose_dgelu. */
+int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream);
+
 /*
  * One persistent launch over all tiles of all problems.
  * replaces Fp8GroupedGemm, csrc/fp8_gmm.cu:163 (pybind name fp8_gmm, csrc/ops.cu:10) and the
@@ -178,12 +185,15 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:
  *   amax = max over the `history_len` rows of amax_history[history_len, slots] (most_recent != 0: row 0)
  *   scale = (1 / amax) * fp8_max * 2^-margin where amax is finite and > 0, else unchanged;  scale_inv = 1 / scale
+ *   keep_period > 0: scale_inv of the slots with slot % keep_period == keep_phase is left as it is (the weights'
+ *   slots while fp8 weights cast in an earlier micro-batch are reused: they must keep the factor they were cast with)
  *   the history moves up by one row (the last row receives the old row 0) and row 0 is cleared.
  * replaces the amax_and_scale_update of TransformerEngine's base module, which the reference's modules run
  * through `self.prepare_forward(...)` (fp8_gmm/grouped_linear.py:206, fp8_gmm/grouped_mlp.py:349).
  */
 int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
-                                  float fp8_max, int margin, int most_recent, void* stream);
+                                  float fp8_max, int margin, int most_recent, int keep_period, int keep_phase,
+                                  void* stream);
 
 /* ---- schedule introspection (host only, no GPU needed) ------------------------------------ */
 /*

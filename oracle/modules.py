@@ -28,13 +28,17 @@ class Meta:
         self.scale_inv = torch.ones(slots, dtype=torch.float32)
         self.amax_history = torch.zeros(history_len, slots, dtype=torch.float32)
 
-    def update(self, fp8_max, margin=0, algo="max"):
+    def update(self, fp8_max, margin=0, algo="max", keep_scale_inv=()):
+        """keep_scale_inv: slots whose scale_inv stays as it is (weights whose cached fp8 copy is reused)."""
         hist = self.amax_history
         amax = hist.max(dim=0).values if algo == "max" else hist[0].clone()
         sf = (fp8_max / amax) / (2.0 ** margin)
         ok = (amax > 0) & torch.isfinite(amax)
         self.scale = torch.where(ok, sf, self.scale).to(torch.float32)
+        old_inv = self.scale_inv
         self.scale_inv = (1.0 / self.scale).to(torch.float32)
+        for slot in keep_scale_inv:
+            self.scale_inv[slot] = old_inv[slot]
         if hist.shape[0] > 1:
             self.amax_history = torch.roll(hist, -1, 0)
         self.amax_history[0].zero_()
@@ -91,18 +95,20 @@ def _wgrad(g_ts, x_ts, g_inv, x_inv):
     return torch.stack(outs)
 
 
-def grouped_linear_step(x, w, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2):
+def grouped_linear_step(x, w, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2,
+                        cached=None):
     """One forward + backward of GroupedLinear with the scales currently in ``fwd`` / ``bwd``.
 
     Records amaxes into the metas (history row 0), returns out, grad_input, grad_weight and the fp8
-    intermediates.  x [M, K] bf16, w [E, N, K] bf16, dy [M, N] bf16.
+    intermediates.  x [M, K] bf16, w [E, N, K] bf16, dy [M, N] bf16.  ``cached``: the result of an earlier
+    step whose fp8 weights are reused instead of casting ``w`` (a micro-batch after the first).
     """
     e = len(sizes)
     xs = [3 * i for i in range(e)]
     ws = [3 * i + 1 for i in range(e)]
     gs = [2 * i for i in range(e)]
     x_fp8, x_ts = _cast_rows(x, sizes, xs, fwd, fwd_dtype)
-    w_fp8, w_t_fp8 = _cast_weights(w, ws, fwd, fwd_dtype)
+    w_fp8, w_t_fp8 = (cached["w_fp8"], cached["w_t_fp8"]) if cached else _cast_weights(w, ws, fwd, fwd_dtype)
     out = _gmm_bf16(x_fp8, w_fp8, sizes, [fwd.scale_inv[s] for s in xs], [fwd.scale_inv[s] for s in ws])
     fwd_inv = fwd.scale_inv.clone()  # the copy the backward pass dequantises with (utils.py:77-78)
     dy_fp8, dy_ts = _cast_rows(dy, sizes, gs, bwd, bwd_dtype)
@@ -113,8 +119,10 @@ def grouped_linear_step(x, w, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn
                 w_t_fp8=w_t_fp8, dy_fp8=dy_fp8, dy_ts=dy_ts)
 
 
-def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2):
-    """One forward + backward of GroupedMlp. x [M, H], w1 [E, F, H], w2 [E, H, F], dy [M, H]."""
+def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2,
+                     cached=None):
+    """One forward + backward of GroupedMlp. x [M, H], w1 [E, F, H], w2 [E, H, F], dy [M, H].
+    ``cached``: the result of an earlier step whose fp8 weights are reused."""
     e = len(sizes)
     b = _bounds(sizes)
     x1 = [3 * i for i in range(e)]
@@ -126,8 +134,11 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
     m, ffn = x.shape[0], w1.shape[1]
 
     x_fp8, x_ts = _cast_rows(x, sizes, x1, fwd, fwd_dtype)
-    w1_fp8, w1_t = _cast_weights(w1, w1s, fwd, fwd_dtype)
-    w2_fp8, w2_t = _cast_weights(w2, w2s, fwd, fwd_dtype)
+    if cached:
+        w1_fp8, w1_t, w2_fp8, w2_t = (cached[k] for k in ("w1_fp8", "w1_t_fp8", "w2_fp8", "w2_t_fp8"))
+    else:
+        w1_fp8, w1_t = _cast_weights(w1, w1s, fwd, fwd_dtype)
+        w2_fp8, w2_t = _cast_weights(w2, w2s, fwd, fwd_dtype)
     pre = torch.zeros(m, ffn, dtype=torch.bfloat16)
     gelu_fp8 = torch.zeros(m, ffn, dtype=fwd_dtype)
     ref.fp8_gmm(x_fp8, w1_fp8, sizes, [fwd.scale_inv[s] for s in x1], [fwd.scale_inv[s] for s in w1s], gelu_fp8,
@@ -160,4 +171,4 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
     grad_input = _gmm_bf16(dpre_fp8, w1_t, sizes, g2_inv, [fwd_inv[s] for s in w1s])
     grad_w1 = _wgrad(dpre_ts, x_ts, g2_inv, [fwd_inv[s] for s in x1])
     return dict(out=out, grad_input=grad_input, grad_w1=grad_w1, grad_w2=grad_w2, pre=pre, gelu_fp8=gelu_fp8,
-                grad_gelu=grad_gelu, dpre_fp8=dpre_fp8)
+                grad_gelu=grad_gelu, dpre_fp8=dpre_fp8, w1_fp8=w1_fp8, w1_t_fp8=w1_t, w2_fp8=w2_fp8, w2_t_fp8=w2_t)

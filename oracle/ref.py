@@ -199,6 +199,15 @@ def multi_cast_transpose_dgelu(inputs, gelu_inputs, outputs, trans_outputs, scal
         )
 
 
+def multi_cast_dgelu(inputs, gelu_inputs, outputs, scales, amaxes):
+    """x = dy * dgelu(pre) cast to fp8, no transposed copy.  The reference has no such kernel and says so
+    (fp8_gmm/grouped_mlp.py:252-253); it is defined as the row-major output of multi_cast_transpose_dgelu."""
+    for x, g, o, s, a in zip(inputs, gelu_inputs, outputs, scales, amaxes):
+        rows = x.reshape(-1, x.shape[-1]) if x.dim() > 0 and x.numel() > 0 else x.reshape(0, 1)
+        t = torch.empty(rows.shape[1], rows.shape[0], dtype=o.dtype)
+        multi_cast_transpose_dgelu([rows], [g.reshape(rows.shape)], [o.reshape(rows.shape)], [t], [s], [a])
+
+
 def gemm_acc_naive(a, b):
     """acc[m, n] = sum_k a[m, k] b[n, k] on dequantised fp8, double accumulation in C (small sizes)."""
     _cpu_contig(a)

@@ -235,3 +235,141 @@ def test_pad_multiple_does_not_change_results(dev, kind):
         results.append([out.detach(), xd.grad] + [p.grad for p in mod.parameters()])
     for a, b in zip(*results):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+
+
+def test_grouped_linear_reuses_cached_fp8_weights(dev):
+    """is_first_microbatch: True casts the weights into the module's buffers, False reuses them.  The weights
+    are CHANGED between the two micro-batches, so only a pass that really reuses the cached bytes (and their
+    scale_inv) can match the oracle, which is handed the first pass's fp8 weights; a later True picks up the
+    new weights."""
+    pkg = _pkg()
+    sizes, k, n = [137, 401, 59, 403], 256, 512
+    e, m, hist = len(sizes), sum(sizes), 2
+    g = gen(3001)
+    w = randn_bf16((e, n, k), g, 0.02)
+    w_changed = (w.float() * 1.5 + 0.01).to(torch.bfloat16)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
+    fwd, bwd = orc.Meta(3 * e, hist), orc.Meta(2 * e, hist)
+    weight_slots = [3 * i + 1 for i in range(e)]
+    plan = [(True, w), (True, w), (False, w_changed), (False, w_changed), (True, w_changed)]
+    cached = None
+    for step, (first, w_now) in enumerate(plan):
+        x = randn_bf16((m, k), g)
+        dy = randn_bf16((m, n), g, 1e-2)
+        if step > 0:
+            fwd.update(448.0, keep_scale_inv=() if first else weight_slots)
+            bwd.update(57344.0)
+        o = orc.grouped_linear_step(x, w_now, sizes, dy, fwd, bwd, cached=None if first else cached)
+        if first:
+            cached = o
+        module.weight_tensor.data.copy_(w_now)
+        xd = x.to(dev).requires_grad_()
+        module.weight_tensor.grad = None
+        with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
+            out = module(xd, torch.tensor(sizes), is_first_microbatch=first)
+        out.backward(dy.to(dev))
+        gm = module.fp8_meta
+        assert_scalar_bits_equal(gm["scaling_fwd"].scale, fwd.scale, f"step {step} fwd scale")
+        assert_scalar_bits_equal(gm["scaling_fwd"].scale_inv, fwd.scale_inv, f"step {step} fwd scale_inv")
+        assert_scalar_bits_equal(gm["scaling_fwd"].amax_history, fwd.amax_history, f"step {step} fwd amax history")
+        assert_scalar_bits_equal(gm["scaling_bwd"].amax_history, bwd.amax_history, f"step {step} bwd amax history")
+        if not first:   # nothing was cast: the weights' amax slots received nothing
+            assert not gm["scaling_fwd"].amax_history[0][weight_slots].any()
+        w_fp8, w_t_fp8 = module.get_fp8_weights_scratchpad(first)
+        assert torch.equal(w_fp8.cpu().view(torch.uint8), cached["w_fp8"].view(torch.uint8)), f"step {step}"
+        assert torch.equal(w_t_fp8.cpu().view(torch.uint8), cached["w_t_fp8"].view(torch.uint8)), f"step {step}"
+        assert_gemm_close(out, o["out"].float(), 1e-2, f"step {step} out")
+        assert_gemm_close(xd.grad, o["grad_input"].float(), 1e-2, f"step {step} grad_input")
+        assert_gemm_close(module.weight_tensor.grad, o["grad_weight"].float(), 1e-2, f"step {step} grad_weight")
+    assert module.get_fp8_weights_scratchpad(None) == [None, None]
+
+
+def test_cached_weights_need_a_first_microbatch(dev):
+    pkg = _pkg()
+    module = pkg.GroupedLinear(64, 64, 2, torch.bfloat16, device=dev)
+    x = torch.zeros(32, 64, dtype=torch.bfloat16, device=dev, requires_grad=True)
+    with pytest.raises(RuntimeError, match="is_first_microbatch=False"):
+        module(x, [16, 16], is_first_microbatch=False)
+    with torch.no_grad():
+        module(x, [16, 16], is_first_microbatch=True)      # casts without the transposes
+        module(x, [16, 16], is_first_microbatch=False)     # enough for another pass without gradients
+    with pytest.raises(RuntimeError, match="transposes"):
+        module(x, [16, 16], is_first_microbatch=False)     # but not for one that needs dgrad
+
+
+@pytest.mark.parametrize("frozen", [False, True], ids=["trainable", "frozen-weights"])
+def test_grouped_mlp_cached_weights_equal_recast_weights(dev, frozen):
+    """Once the weights' scales have settled (constant weights), reusing the cached fp8 weights must give the
+    same bits as casting them again: module A runs True, True, False, False, module B casts on every pass.
+    With frozen weights the backward pass takes the cast-only dGELU kernel and skips the weight gradients."""
+    pkg = _pkg()
+    sizes, h, f = [137, 0, 401, 59, 403], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(3002)
+    w1 = randn_bf16((e, f, h), g, 0.02).to(dev)
+    w2 = randn_bf16((e, h, f), g, 0.02).to(dev)
+    mods = []
+    for _ in range(2):
+        mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+        mod.fc1_weight.data.copy_(w1)
+        mod.fc2_weight.data.copy_(w2)
+        if frozen:
+            mod.fc1_weight.requires_grad_(False)
+            mod.fc2_weight.requires_grad_(False)
+        mods.append(mod)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=4)
+    gs = torch.tensor(sizes)
+    weight_slots = [3 * i + 1 for i in range(2 * e)]
+    for step, first in enumerate([True, True, False, False]):
+        x = randn_bf16((m, h), g).to(dev)
+        dy = randn_bf16((m, h), g, 1e-2).to(dev)
+        res = []
+        for mod, flag in zip(mods, (first, None)):
+            xd = x.clone().requires_grad_()
+            mod.zero_grad()
+            with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
+                out = mod(xd, gs, is_first_microbatch=flag)
+            out.backward(dy)
+            res.append((out, xd.grad, mod.fc1_weight.grad, mod.fc2_weight.grad))
+        for name, a, b in zip(("out", "grad_input", "grad_fc1", "grad_fc2"), *res):
+            if a is None:
+                assert b is None and frozen
+                continue
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}: {name} differs"
+        fa, fb = mods[0].fp8_meta["scaling_fwd"], mods[1].fp8_meta["scaling_fwd"]
+        assert torch.equal(fa.scale, fb.scale) and torch.equal(fa.scale_inv, fb.scale_inv), f"step {step}"
+        if first:
+            assert torch.equal(fa.amax_history, fb.amax_history)
+        else:
+            assert not fa.amax_history[0][weight_slots].any() and fb.amax_history[0][weight_slots].all()
+        assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
+
+
+def test_grouped_mlp_frozen_weights_against_the_oracle(dev):
+    """No weight gradients: padded transposes are skipped and d(pre-GELU) goes through the cast-only dGELU
+    kernel; output and grad_input must still be the oracle's."""
+    pkg = _pkg()
+    sizes, h, f = MLP_CASES["small"]
+    e, m = len(sizes), sum(sizes)
+    g = gen(3003)
+    w1 = randn_bf16((e, f, h), g, 0.02)
+    w2 = randn_bf16((e, h, f), g, 0.02)
+    x = randn_bf16((m, h), g)
+    dy = randn_bf16((m, h), g, 1e-2)
+    module = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+    module.fc1_weight.data.copy_(w1)
+    module.fc2_weight.data.copy_(w2)
+    module.fc1_weight.requires_grad_(False)
+    module.fc2_weight.requires_grad_(False)
+    fwd, bwd = orc.Meta(3 * 2 * e, 1), orc.Meta(2 * 2 * e, 1)
+    o = orc.grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd)
+    xd = x.to(dev).requires_grad_()
+    with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=1)):
+        out = module(xd, torch.tensor(sizes))
+    out.backward(dy.to(dev))
+    assert module.fc1_weight.grad is None and module.fc2_weight.grad is None
+    assert_close_multistage(out, o["out"], 5e-3, "out")
+    assert_close_multistage(xd.grad, o["grad_input"], 1e-2, "grad_input")
+    _check_amax(module.fp8_meta["scaling_bwd"], bwd, [2 * i for i in range(e)], [2 * (e + i) for i in range(e)],
+                "frozen bwd")

@@ -190,6 +190,47 @@ def test_dgelu_every_bf16_pattern(dev):
     assert_scalar_bits_equal(da, a, "dgelu amax")
 
 
+@pytest.mark.parametrize("dtype", FP8_DTYPES)
+def test_multi_cast_dgelu_without_transpose(dev, dtype):
+    """The cast-only dGELU kernel writes exactly the row-major bytes and amax of the transposing one; checked
+    against the oracle and against the transposing kernel itself, on aligned, odd, tiny and multi-block shapes
+    and on every bf16 pre-activation pattern."""
+    backend = _backend()
+    g = gen(15)
+    shapes = SMALL_SHAPES + [(300, 517), (1, 70001), (0, 16)]
+    ins = [randn_bf16(s, g) for s in shapes] + [torch.ones(256, 256, dtype=torch.bfloat16)]
+    pres = [randn_bf16(s, g, std=2.0) for s in shapes] + [ALL_BF16.reshape(256, 256).clone()]
+    shapes = shapes + [(256, 256)]
+    scales = _scales(len(shapes), g)
+    outs = [torch.empty(s, dtype=dtype) for s in shapes]
+    amaxes = [torch.zeros(1) for _ in shapes]
+    ref.multi_cast_dgelu(ins, pres, outs, scales, amaxes)
+    d_outs = [torch.full(s, 0x55, dtype=torch.uint8, device=dev).view(dtype) for s in shapes]
+    d_amaxes = [torch.zeros(1, device=dev) for _ in shapes]
+    backend.multi_cast_dgelu(_to_dev(ins, dev), _to_dev(pres, dev), d_outs, _to_dev(scales, dev), d_amaxes)
+    t_outs = [torch.empty(s, dtype=dtype, device=dev) for s in shapes]
+    t_touts = [torch.empty(s[1], s[0], dtype=dtype, device=dev) for s in shapes]
+    t_amaxes = [torch.zeros(1, device=dev) for _ in shapes]
+    backend.multi_cast_transpose_dgelu(_to_dev(ins, dev), _to_dev(pres, dev), t_outs, t_touts, _to_dev(scales, dev),
+                                       t_amaxes)
+    for i, s in enumerate(shapes):
+        assert_bytes_equal(d_outs[i], outs[i], f"cast {s}")
+        assert_scalar_bits_equal(d_amaxes[i], amaxes[i], f"amax {s}")
+        assert torch.equal(d_outs[i].view(torch.uint8), t_outs[i].view(torch.uint8)), f"kernels disagree on {s}"
+        assert_scalar_bits_equal(d_amaxes[i], t_amaxes[i].cpu(), f"kernels disagree on amax {s}")
+    # misaligned views take the per-element path: same bytes
+    base_x = randn_bf16((1, 4099), g).to(dev)
+    base_p = randn_bf16((1, 4099), g).to(dev)
+    xo, po = base_x[:, 1:], base_p[:, 1:]
+    o_view = torch.empty(1, 4099, dtype=dtype, device=dev)[:, 1:]
+    am = torch.zeros(1, device=dev)
+    backend.multi_cast_dgelu([xo], [po], [o_view], [scales[0].to(dev)], [am])
+    want, want_amax = torch.empty(1, 4098, dtype=dtype), torch.zeros(1)
+    ref.multi_cast_dgelu([xo.cpu().contiguous()], [po.cpu().contiguous()], [want], [scales[0]], [want_amax])
+    assert_bytes_equal(o_view, want, "misaligned cast")
+    assert_scalar_bits_equal(am, want_amax, "misaligned amax")
+
+
 def test_pad_multiple_128_with_outliers(dev):
     """The bandwidth configuration in small: ragged [M_i, 512] tensors, pad to 128, +-200 outliers."""
     backend = _backend()

@@ -165,9 +165,6 @@ def test_prepare_forward_allocates_three_and_two_slots_per_gemm():
     assert m.fp8_meta["scaling_bwd"].scale.shape == (12,)
     assert m.fp8_meta["scaling_fwd"].amax_history.shape == (7, 18)
     assert m.fp8_meta["scaling_fwd"].scale.eq(1).all() and m.fp8_meta["scaling_bwd"].scale_inv.eq(1).all()
-    with pytest.raises(AssertionError):
-        with m.prepare_forward(x, True, num_gemms=6):
-            pass
     # scaling state round-trips through extra_state
     m.fp8_meta["scaling_fwd"].scale.fill_(3.0)
     state = m.get_extra_state()
@@ -177,6 +174,57 @@ def test_prepare_forward_allocates_three_and_two_slots_per_gemm():
         with m2.prepare_forward(x, None, num_gemms=6):
             pass
     assert m2.fp8_meta["scaling_fwd"].scale.eq(3).all()
+
+
+def test_reusing_cached_weights_keeps_their_scale_inv():
+    """is_first_microbatch=False: the update still moves every scale, but the weights' scale_inv (slot 1 of
+    each GEMM's three forward slots) stays what the cached fp8 weights were cast with; True / None update all."""
+    m = fp8.Fp8GroupedModuleBase()
+    x = torch.zeros(4, 8)
+    rec = fp8.DelayedScaling(amax_history_len=1)
+    weight_slots = torch.tensor([1, 4])
+    other_slots = torch.tensor([0, 2, 3, 5])
+
+    def step(first, amax):
+        with fp8.fp8_autocast(fp8_recipe=rec), m.prepare_forward(x, first, num_gemms=2):
+            pass
+        m.fp8_meta["scaling_fwd"].amax_history[0] = amax   # what the kernels of the pass would record
+        m.fp8_meta["scaling_bwd"].amax_history[0] = 1.0
+
+    step(True, 2.0)                       # first pass: no update yet, scales 1
+    step(False, 4.0)                      # update from amax 2: scale 224, weights keep scale_inv 1
+    fwd = m.fp8_meta["scaling_fwd"]
+    assert fwd.scale.eq(224.0).all()
+    assert fwd.scale_inv[weight_slots].eq(1.0).all() and fwd.scale_inv[other_slots].eq(1 / 224.0).all()
+    assert m.fp8_meta["scaling_bwd"].scale_inv.eq(1 / 57344.0).all()   # the gradient direction has no weights
+    step(True, 8.0)                       # update from amax 4: everything follows
+    assert fwd.scale.eq(112.0).all() and fwd.scale_inv.eq(1 / 112.0).all()
+    step(None, 8.0)
+    assert fwd.scale.eq(56.0).all() and fwd.scale_inv.eq(1 / 56.0).all()
+
+
+def test_weight_cache_bookkeeping():
+    cache = fp8.Fp8WeightCache()
+    w = torch.zeros(3, 4, 5, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="is_first_microbatch=False"):
+        cache.require(False)
+    a, a_t = cache.buffers(w, torch.float8_e4m3fn)
+    assert a.shape == (3, 4, 5) and a_t.shape == (3, 5, 4) and a.dtype == a_t.dtype == torch.float8_e4m3fn
+    b, b_t = cache.buffers(w, torch.float8_e4m3fn)
+    assert b is a and b_t is a_t                        # kept, not reallocated
+    cache.valid = True
+    cache.require(False)
+    with pytest.raises(RuntimeError, match="transposes"):
+        cache.require(True)
+    c, _ = cache.buffers(torch.zeros(3, 4, 6, dtype=torch.bfloat16), torch.float8_e4m3fn)
+    assert c is not a and not cache.valid               # a new shape drops the old contents
+    # a module drops its caches when the scaling state is replaced
+    m = fp8.Fp8GroupedModuleBase()
+    m._weight_caches.append(cache)
+    cache.valid = cache.valid_t = True
+    with fp8.fp8_autocast(fp8_recipe=fp8.DelayedScaling(amax_history_len=3)), m.prepare_forward(w, None, 2):
+        pass
+    assert not cache.valid and not cache.valid_t
 
 
 def test_tensor_batch_describes_the_same_memory_as_views():
