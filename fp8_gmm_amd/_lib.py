@@ -83,6 +83,12 @@ EXPORTS = (
     "fp8gmm_multi_cast_dgelu",
     "fp8gmm_grouped_gemm",
     "fp8gmm_delayed_scaling_update",
+    "fp8gmm_route_workspace_bytes",
+    "fp8gmm_route_sort",
+    "fp8gmm_route_invert",
+    "fp8gmm_moe_gather",
+    "fp8gmm_moe_scatter",
+    "fp8gmm_moe_scatter_wgrad",
     "fp8gmm_gemm_schedule",
     "fp8gmm_gemm_fixup",
 )
@@ -141,6 +147,18 @@ def load():
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
+    L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t
+    L.fp8gmm_route_workspace_bytes.argtypes = [ci, ci]
+    L.fp8gmm_route_sort.restype = ci
+    L.fp8gmm_route_sort.argtypes = [vp, ci, ci, vp, vp, vp, vp, vp, vp, vp]
+    L.fp8gmm_route_invert.restype = ci
+    L.fp8gmm_route_invert.argtypes = [vp, ci, vp, vp]
+    L.fp8gmm_moe_gather.restype = ci
+    L.fp8gmm_moe_gather.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
+    L.fp8gmm_moe_scatter.restype = ci
+    L.fp8gmm_moe_scatter.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
+    L.fp8gmm_moe_scatter_wgrad.restype = ci
+    L.fp8gmm_moe_scatter_wgrad.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     L.fp8gmm_gemm_schedule.restype = ci
     L.fp8gmm_gemm_schedule.argtypes = [vp, ci, ci, ci, ci, ci, vp, ci]
     L.fp8gmm_gemm_fixup.restype = ci

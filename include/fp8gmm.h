@@ -195,6 +195,48 @@ int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scal
                                   float fp8_max, int margin, int most_recent, int keep_period, int keep_phase,
                                   void* stream);
 
+/* ---- token routing around the expert layers ----------------------------------------------- */
+/*
+ * The reference's example MoE layers (fp8_gmm/example.py:15-32,50-59,86-94,113-119) take these steps from the
+ * megablocks package, which is not part of the reference tree (no version is pinned anywhere in it); the
+ * functions below implement the published meaning of megablocks.ops.sort / histogram / inclusive_cumsum /
+ * gather / scatter for int32 expert ids and bf16 rows.
+ *
+ * fp8gmm_route_sort: stable sort of `expert_of[0..n)` (values in [0, num_experts), num_experts <= 4096; values
+ * outside are clamped into the range) by expert.  Every output may be NULL:
+ *   bin_ids[p]  expert of sorted position p            (ops.sort, first result)
+ *   indices[p]  original position of sorted position p (ops.sort, second result)
+ *   inverse[i]  sorted position of original position i (the inverse permutation)
+ *   tokens_per_expert[e]  entries of expert e          (ops.histogram)
+ *   bins[e]     end of expert e in sorted order        (ops.inclusive_cumsum of the histogram)
+ * replaces indices_and_bins, fp8_gmm/example.py:26-32.  `workspace`: fp8gmm_route_workspace_bytes(n, num_experts)
+ * bytes of device memory, contents irrelevant.
+ */
+size_t fp8gmm_route_workspace_bytes(int n, int num_experts);
+int fp8gmm_route_sort(const int32_t* expert_of, int n, int num_experts, int32_t* bin_ids, int32_t* indices,
+                      int32_t* inverse, int32_t* tokens_per_expert, int32_t* bins, void* workspace, void* stream);
+/* inverse[indices[i]] = i for a permutation `indices` of 0..n-1 (entries outside that range are skipped) */
+int fp8gmm_route_invert(const int32_t* indices, int n, int32_t* inverse, void* stream);
+/*
+ * out[i, :] = bf16(w_i * x[indices[i] / top_k, :]) for i in [0, rows_out), w_i = weights[indices[i]] or 1 when
+ * weights == NULL (then rows are copied unchanged).  x: bf16 [rows_out / top_k, hidden], out: bf16 [rows_out, hidden].
+ * replaces ops.gather (fp8_gmm/example.py:52,88,115) and, with weights, the backward pass of ops.scatter.
+ */
+int fp8gmm_moe_gather(const void* x, const int32_t* indices, const float* weights, void* out, int rows_out,
+                      int hidden, int top_k, void* stream);
+/*
+ * out[t, :] = bf16(sum_k w[t * top_k + k] * x[inverse[t * top_k + k], :]) for t in [0, tokens): fp32 sum over
+ * k = 0 .. top_k - 1 in that order, each product rounded to fp32 before it is added; w = 1 when weights == NULL.
+ * x: bf16 [tokens * top_k, hidden] in sorted order, out: bf16 [tokens, hidden].
+ * replaces ops.scatter (fp8_gmm/example.py:59,94,119) and, without weights, the backward pass of ops.gather.
+ */
+int fp8gmm_moe_scatter(const void* x, const int32_t* inverse, const float* weights, void* out, int tokens, int hidden,
+                       int top_k, void* stream);
+/* grad_w[indices[i]] = < x[i, :], grad_out[indices[i] / top_k, :] > in fp32: gradient of ops.scatter with respect
+ * to its weights.  x: bf16 [rows, hidden] (sorted order), grad_out: bf16 [rows / top_k, hidden], grad_w: fp32 [rows]. */
+int fp8gmm_moe_scatter_wgrad(const void* x, const void* grad_out, const int32_t* indices, float* grad_w, int rows,
+                             int hidden, int top_k, void* stream);
+
 /* ---- schedule introspection (host only, no GPU needed) ------------------------------------ */
 /*
  * The work items that workgroup `wg` of a grouped-GEMM launch with `grid` workgroups (a multiple of 8)

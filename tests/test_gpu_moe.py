@@ -1,0 +1,201 @@
+"""Token routing on the GPU (sort / histogram / gather / scatter and their gradients) against the CPU oracle,
+and the routed example layers end to end.  Integer results and copied rows are compared bit for bit; scatter's
+bf16 output too (the kernel and the oracle follow the same fp32 sequence); only the per-row dot products of
+scatter's weight gradient, whose summation order differs, get a tolerance (1e-5 relative to the row norms)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _ops():
+    from fp8_gmm_amd import moe_ops
+
+    return moe_ops
+
+
+def _ids(n, e, seed, kind="uniform"):
+    rng = np.random.default_rng(seed)
+    if kind == "zipf":
+        p = 1.0 / np.arange(1, e + 1) ** 1.1
+        return rng.choice(e, size=n, p=p / p.sum())
+    if kind == "one":
+        return np.full(n, e - 1)
+    return rng.integers(0, e, size=n)
+
+
+ROUTE_CASES = [(1, 1, "uniform"), (63, 4, "uniform"), (64, 2, "uniform"), (1000, 4, "uniform"), (1025, 7, "zipf"),
+               (32768, 8, "uniform"), (24576, 64, "zipf"), (65536, 128, "uniform"), (70000, 4096, "uniform"),
+               (5000, 16, "one"), (0, 8, "uniform")]
+
+
+@pytest.mark.parametrize("n,e,kind", ROUTE_CASES)
+def test_sort_histogram_and_bins(dev, n, e, kind):
+    ops = _ops()
+    ids = _ids(n, e, 100 + n, kind)
+    x = torch.tensor(ids, dtype=torch.int32, device=dev)
+    want_indices, want_bin_ids, want_bins, want_counts = orc.indices_and_bins(ids, e)
+    indices, bin_ids, bins, counts = ops.indices_and_bins(x, max(int(np.ceil(np.log2(e))), 1), e)
+    assert indices.dtype == bin_ids.dtype == bins.dtype == counts.dtype == torch.int32
+    assert indices.cpu().tolist() == want_indices.tolist()
+    assert bin_ids.cpu().tolist() == want_bin_ids.tolist()
+    assert counts.cpu().tolist() == want_counts.tolist()
+    assert bins.cpu().tolist() == want_bins.tolist()
+    # the single operators give the same answers
+    end_bit = max(int(np.ceil(np.log2(e))), 1)
+    s_ids, s_idx = ops.sort(x, end_bit)
+    assert torch.equal(s_ids, bin_ids) and torch.equal(s_idx, indices)
+    assert torch.equal(ops.histogram(x, e), counts)
+    assert torch.equal(ops.inclusive_cumsum(counts, 0), bins)
+    _, _, inverse, _, _ = ops.route(x, e, want_inverse=True)
+    assert inverse.cpu().tolist() == orc.invert(want_indices).tolist()
+
+
+def test_out_of_range_ids_are_clamped(dev):
+    ops = _ops()
+    x = torch.tensor([5, -3, 2, 9, 0], dtype=torch.int32, device=dev)
+    bin_ids, indices = ops.sort(x, 2)          # ids below 4
+    assert bin_ids.cpu().tolist() == [0, 0, 2, 3, 3] and indices.cpu().tolist() == [1, 4, 2, 0, 3]
+    with pytest.raises(RuntimeError):
+        ops.histogram(x, 5000)
+    with pytest.raises(RuntimeError):
+        ops.sort(x.long())
+
+
+ROW_CASES = [(1, 1, 8, 1), (37, 2, 256, 4), (128, 2, 4096, 8), (50, 1, 520, 3), (64, 8, 768, 16), (33, 3, 100, 5),
+             (16, 2, 6, 2), (0, 2, 64, 4)]
+
+
+@pytest.mark.parametrize("tokens,top_k,hidden,e", ROW_CASES)
+def test_gather_scatter_and_their_gradients(dev, tokens, top_k, hidden, e):
+    ops = _ops()
+    g = torch.Generator().manual_seed(7 + tokens)
+    ids = _ids(tokens * top_k, e, 200 + tokens)
+    indices_cpu = orc.sort(ids)[1]
+    indices = torch.tensor(indices_cpu, dtype=torch.int32, device=dev)
+    x = torch.randn(tokens, hidden, generator=g).to(torch.bfloat16)
+    y = torch.randn(tokens * top_k, hidden, generator=g).to(torch.bfloat16)
+    w = torch.rand(tokens * top_k, generator=g)
+    grad_rows = torch.randn(tokens * top_k, hidden, generator=g).to(torch.bfloat16)
+    grad_tok = torch.randn(tokens, hidden, generator=g).to(torch.bfloat16)
+
+    xd = x.to(dev).requires_grad_()
+    got = ops.gather(xd, indices, None, None, top_k)
+    assert torch.equal(got.cpu().view(torch.int16), orc.gather(x, indices_cpu, top_k).view(torch.int16))
+    got.backward(grad_rows.to(dev))
+    assert torch.equal(xd.grad.cpu().view(torch.int16),
+                       orc.gather_backward(grad_rows, indices_cpu, top_k).view(torch.int16))
+
+    for weights in (w, None):
+        yd = y.to(dev).requires_grad_()
+        wd = weights.to(dev).requires_grad_() if weights is not None else None
+        out = ops.scatter(yd, indices, None, wd, None, top_k)
+        assert torch.equal(out.cpu().view(torch.int16), orc.scatter(y, indices_cpu, top_k, weights).view(torch.int16))
+        out.backward(grad_tok.to(dev))
+        want_gx, want_gw = orc.scatter_backward(grad_tok, y, indices_cpu, top_k, weights)
+        assert torch.equal(yd.grad.cpu().view(torch.int16), want_gx.view(torch.int16))
+        if weights is not None and tokens:
+            idx = torch.as_tensor(indices_cpu.astype(np.int64))
+            bound = torch.zeros(tokens * top_k)
+            bound[idx] = y.float().norm(dim=1) * grad_tok.float()[idx // top_k].norm(dim=1)
+            assert ((wd.grad.cpu() - want_gw).abs() <= 1e-5 * bound + 1e-30).all()
+
+
+def test_bad_arguments_are_rejected(dev):
+    ops = _ops()
+    x = torch.zeros(4, 8, dtype=torch.bfloat16, device=dev)
+    idx = torch.arange(8, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError):
+        ops.gather(x.float(), idx, None, None, 2)
+    with pytest.raises(RuntimeError):
+        ops.gather(x, idx[:5], None, None, 2)
+    with pytest.raises(RuntimeError):
+        ops.scatter(x, idx[:4], None, torch.ones(3, device=dev), None, 2)
+    with pytest.raises(RuntimeError):
+        ops.gather(x.cpu(), idx.cpu(), None, None, 2)
+
+
+@pytest.mark.parametrize("kind", ["mlp", "linear"])
+def test_routed_layer_forward_against_the_oracle_composition(dev, kind):
+    """Fp8MlpModule / Fp8LinearModule: with the layer's own routing decisions (read back from the GPU) the output
+    must be scatter(experts(gather(x))) as the CPU oracle computes it."""
+    import fp8_gmm_amd as pkg
+    from fp8_gmm_amd import moe
+    from helpers import assert_close_multistage
+    from oracle import modules as orc_mod
+
+    tokens, h, f, e, top_k = 96, 128, 256, 5, 2
+    torch.manual_seed(11)
+    layer = (moe.Fp8MlpModule if kind == "mlp" else moe.Fp8LinearModule)(h, f, e, top_k, device=dev)
+    x = torch.randn(tokens, h).to(torch.bfloat16)
+    with torch.no_grad(), pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=1)):
+        out = layer(x.to(dev))
+        weights0, selected = layer.gating_network(x.to(dev)), None
+        weights0, selected = pkg.moe_ops.topk(weights0, top_k)
+    ids = selected.flatten().cpu().numpy()
+    w = weights0.flatten().cpu()
+    indices, _, _, counts = orc.indices_and_bins(ids, e)
+    sizes = counts.tolist()
+    xs = orc.gather(x, indices, top_k)
+    if kind == "mlp":
+        fwd, bwd = orc_mod.Meta(3 * 2 * e, 1), orc_mod.Meta(2 * 2 * e, 1)
+        y = orc_mod.grouped_mlp_step(xs, layer.grouped_mlp.fc1_weight.detach().cpu(),
+                                     layer.grouped_mlp.fc2_weight.detach().cpu(), sizes,
+                                     torch.zeros(tokens * top_k, h, dtype=torch.bfloat16), fwd, bwd)["out"]
+    else:
+        zeros = torch.zeros(tokens * top_k, f, dtype=torch.bfloat16)
+        fwd, bwd = orc_mod.Meta(3 * e, 1), orc_mod.Meta(2 * e, 1)
+        mid = orc_mod.grouped_linear_step(xs, layer.grouped_linear1.weight_tensor.detach().cpu(), sizes, zeros, fwd,
+                                          bwd)["out"]
+        mid = torch.nn.functional.gelu(mid.float()).to(torch.bfloat16)
+        fwd, bwd = orc_mod.Meta(3 * e, 1), orc_mod.Meta(2 * e, 1)
+        y = orc_mod.grouped_linear_step(mid, layer.grouped_linear2.weight_tensor.detach().cpu(), sizes,
+                                        torch.zeros(tokens * top_k, h, dtype=torch.bfloat16), fwd, bwd)["out"]
+    want = orc.scatter(y, indices, top_k, w)
+    assert_close_multistage(out, want, 1e-2, f"{kind} layer output")
+
+
+def test_routed_mlp_layer_trains_like_a_dense_fp32_model(dev):
+    """Forward + backward of Fp8MlpModule against an fp32 autograd model of the same routed layer (same routing
+    decisions): cosine similarity of the output and of every gradient, gating weights included."""
+    import fp8_gmm_amd as pkg
+    from fp8_gmm_amd import moe
+
+    tokens, h, f, e, top_k = 512, 256, 512, 8, 2
+    torch.manual_seed(12)
+    layer = moe.Fp8MlpModule(h, f, e, top_k, device=dev)
+    x = torch.randn(tokens, h, device=dev).to(torch.bfloat16)
+    dy = torch.randn(tokens, h, device=dev).to(torch.bfloat16)
+    for _ in range(2):   # the second pass runs with real scales
+        xd = x.clone().requires_grad_()
+        layer.zero_grad()
+        with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=2)):
+            out = layer(xd)
+        out.backward(dy)
+
+    xr = x.float().requires_grad_()
+    gate = layer.gating_network.weight.detach().float().requires_grad_()
+    w1 = layer.grouped_mlp.fc1_weight.detach().float().requires_grad_()
+    w2 = layer.grouped_mlp.fc2_weight.detach().float().requires_grad_()
+    logits = layer.gating_network(x).float()                  # the layer's own bf16 logits decide the routing
+    _, selected = pkg.moe_ops.topk(logits, top_k)
+    probs = torch.softmax(xr @ gate.t(), dim=1)
+    ref = torch.zeros(tokens, h, device=dev)
+    for k in range(top_k):
+        ek = selected[:, k]
+        hidden = torch.nn.functional.gelu(torch.einsum("th,tfh->tf", xr, w1[ek]), approximate="tanh")
+        ref = ref + probs.gather(1, ek[:, None]) * torch.einsum("tf,thf->th", hidden, w2[ek])
+    ref.backward(dy.float())
+
+    def cos(a, b):
+        a, b = a.detach().float().flatten(), b.detach().float().flatten()
+        return (torch.dot(a, b) / (a.norm() * b.norm())).item()
+
+    assert cos(out, ref) > 0.995
+    assert cos(xd.grad, xr.grad) > 0.99
+    assert cos(layer.grouped_mlp.fc1_weight.grad, w1.grad) > 0.99
+    assert cos(layer.grouped_mlp.fc2_weight.grad, w2.grad) > 0.99
+    assert cos(layer.gating_network.weight.grad, gate.grad) > 0.98
