@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|example]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -39,6 +39,9 @@ WORKLOADS = {
     "config2": ("mlp", 8, 4096, 14336, 16384, "dirichlet"),
     "config3": ("linear", 64, 2048, 1408, 24576, "zipf"),
     "config4": ("mlp", 128, 2048, 768, 65536, "uniform"),
+    # the reference's own benchmark recipe (fp8_gmm/example.py:133): a routed layer, 16384 tokens, top-2 of 16
+    # experts, router + gather + GroupedMlp + weighted scatter; `tokens` counts rows after routing
+    "example": ("routed_mlp", 16, 4096, 6400, 32768, "router"),
 }
 
 
@@ -82,11 +85,17 @@ def main():
     from fp8_gmm_amd.backend import kernel_timing
 
     kind, experts, hidden, ffn, tokens, splitter = WORKLOADS[args.workload]
-    idx = int(args.workload[-1])
-    sizes = splits(splitter, experts, tokens, 1000 + idx)
+    idx = int(args.workload[-1]) if args.workload[-1].isdigit() else 9
+    sizes = splits(splitter, experts, tokens, 1000 + idx) if splitter != "router" else None
     dev = torch.device("cuda:0")
     torch.manual_seed(1000 + idx)
-    if kind == "mlp":
+    top_k = 2
+    if kind == "routed_mlp":
+        from fp8_gmm_amd.moe import Fp8MlpModule
+
+        module = Fp8MlpModule(hidden, ffn, experts, top_k, device=dev)
+        out_features, gemms = hidden, 6
+    elif kind == "mlp":
         module = pkg.GroupedMlp(hidden, ffn, experts, torch.bfloat16, device=dev)
         module.fc1_weight.data.normal_(0, 0.02)
         module.fc2_weight.data.normal_(0, 0.02)
@@ -95,9 +104,10 @@ def main():
         module = pkg.GroupedLinear(hidden, ffn, experts, torch.bfloat16, device=dev)
         module.weight_tensor.data.normal_(0, 0.02)
         out_features, gemms = ffn, 3
-    x = torch.randn(tokens, hidden, device=dev, dtype=torch.bfloat16).requires_grad_()
-    dy = (torch.randn(tokens, out_features, device=dev) * 1e-2).to(torch.bfloat16)
-    gs = torch.tensor(sizes, dtype=torch.int64)
+    in_rows = tokens // top_k if kind == "routed_mlp" else tokens
+    x = torch.randn(in_rows, hidden, device=dev, dtype=torch.bfloat16).requires_grad_()
+    dy = (torch.randn(in_rows, out_features, device=dev) * 1e-2).to(torch.bfloat16)
+    gs = torch.tensor(sizes, dtype=torch.int64) if sizes is not None else None
     fp8_recipe = pkg.DelayedScaling(amax_history_len=16)
     flops_per_gemm = 2.0 * tokens * hidden * ffn
     flops_per_step = gemms * flops_per_gemm
@@ -106,7 +116,7 @@ def main():
         module.zero_grad(set_to_none=True)
         x.grad = None
         with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
-            out = module(x, gs, is_first_microbatch=first)
+            out = module(x) if gs is None else module(x, gs, is_first_microbatch=first)
         out.backward(dy)
 
     for _ in range(args.warmup):
@@ -154,17 +164,19 @@ def main():
 
     # Not the headline: the same step as a micro-batch after the first of an optimizer step, reusing the fp8
     # weights cast by the first (is_first_microbatch=False), which the reference stubs out.
-    step(True)
-    step(False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
+    also = None
+    if gs is not None:
+        step(True)
         step(False)
-    torch.cuda.synchronize()
-    cached_ms = (time.perf_counter() - t0) / args.steps * 1e3
-    also = {"later_microbatch_with_cached_fp8_weights": {
-        "ms_per_step": round(cached_ms, 4), "value": round(flops_per_step / (cached_ms * 1e-3) / 1e12, 2),
-        "unit": "TFLOP/s"}}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step(False)
+        torch.cuda.synchronize()
+        cached_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        also = {"later_microbatch_with_cached_fp8_weights": {
+            "ms_per_step": round(cached_ms, 4), "value": round(flops_per_step / (cached_ms * 1e-3) / 1e12, 2),
+            "unit": "TFLOP/s"}}
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -178,6 +190,7 @@ def main():
                "sample": f"all {sample_tokens} tokens through one expert, {hidden}->{ffn} MLP fwd+bwd (6 GEMMs, "
                          f"{fl / 1e9:.0f} GFLOP) incl. weight quantisation, {secs:.1f} s"}
 
+    names = {"mlp": "GroupedMlp", "linear": "GroupedLinear", "routed_mlp": "Fp8MlpModule (router, gather, GroupedMlp, scatter)"}
     line = {
         "metric": "FP8 grouped-GEMM TFLOP/s fwd+bwd, % of MI355X FP8 MFMA peak, E=8 MoE MLP",
         "value": round(value, 2),
@@ -192,9 +205,10 @@ def main():
         "vs_baseline": None,
         "dtype": "fp8",
         "data": "synthetic",
-        "config": {"workload": f"{args.workload}: Grouped{'Mlp' if kind == 'mlp' else 'Linear'} fwd+bwd, E={experts}, "
+        "config": {"workload": f"{args.workload}: {names[kind]} fwd+bwd, E={experts}, "
                                f"hidden={hidden}, ffn={ffn}, tokens={tokens}, split={splitter}",
-                   "group_sizes": sizes if experts <= 16 else f"{experts} experts, min {min(sizes)} max {max(sizes)}",
+                   "group_sizes": "decided by the router" if sizes is None else
+                                  sizes if experts <= 16 else f"{experts} experts, min {min(sizes)} max {max(sizes)}",
                    "gemm_flops_per_step": flops_per_step},
         "roofline": roofline,
         "cpu_baseline": cpu,

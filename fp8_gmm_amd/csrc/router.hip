@@ -199,22 +199,24 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_kernel(const uint1
   uint16_t* dst = out + (size_t)t * hidden;
   if (vec) {
     const __amdgpu_buffer_rsrc_t rd = make_rsrc(dst, (uint32_t)hidden * 2u);
-    for (int c0 = 0; c0 < hidden; c0 += 64 * 8 * 2) {
-      float acc[2][8];
+    constexpr int kU = 4;  // 16-byte loads in flight per lane and source row
+    for (int c0 = 0; c0 < hidden; c0 += 64 * 8 * kU) {
+      float acc[kU][8];
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+      for (int u = 0; u < kU; ++u)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[u][j] = 0.f;
+#pragma unroll 2
       for (int k = 0; k < top_k; ++k) {
         const int32_t p = inverse[(size_t)t * top_k + k];
         const bool ok = (uint32_t)p < (uint32_t)rows;
         const float w = weights != nullptr ? weights[(size_t)t * top_k + k] : 1.0f;
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(x + (size_t)(ok ? p : 0) * hidden, ok ? (uint32_t)hidden * 2u : 0u);
-        u32x4 v[2];
+        u32x4 v[kU];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) v[u] = buf_load16(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+        for (int u = 0; u < kU; ++u) v[u] = buf_load16(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < kU; ++u) {
           const uint32_t q[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_kernel(const uint1
         }
       }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < kU; ++u) {
         const u32x4 o = {pack_bf16x2(acc[u][0], acc[u][1]), pack_bf16x2(acc[u][2], acc[u][3]),
                          pack_bf16x2(acc[u][4], acc[u][5]), pack_bf16x2(acc[u][6], acc[u][7])};
         buf_store16(o, rd, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);

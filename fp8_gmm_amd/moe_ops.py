@@ -19,7 +19,7 @@ are clamped into the range instead of being undefined.
 import torch
 
 from . import _lib
-from .backend import _fail, _stream
+from .backend import _fail, _stream, _timed
 
 MAX_EXPERTS = 4096  # size of the on-chip expert table of the sort kernels
 
@@ -123,7 +123,7 @@ def _gather_rows(x, indices, weights, top_k):
     """out[i] = weights[indices[i]] * x[indices[i] // top_k]"""
     rows, hidden = x.shape[0] * top_k, x.shape[1]
     out = torch.empty(rows, hidden, dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with torch.cuda.device(x.device), _timed("moe_gather", lambda: 4 * rows * hidden):
         rc = _lib.load().fp8gmm_moe_gather(x.data_ptr(), indices.data_ptr(),
                                            weights.data_ptr() if weights is not None else None, out.data_ptr(),
                                            rows, hidden, top_k, _stream(x.device))
@@ -135,7 +135,7 @@ def _scatter_rows(x, inverse, weights, top_k):
     """out[t] = sum_k weights[t * top_k + k] * x[inverse[t * top_k + k]]"""
     tokens, hidden = x.shape[0] // top_k, x.shape[1]
     out = torch.empty(tokens, hidden, dtype=x.dtype, device=x.device)
-    with torch.cuda.device(x.device):
+    with torch.cuda.device(x.device), _timed("moe_scatter", lambda: 2 * (x.shape[0] + tokens) * hidden):
         rc = _lib.load().fp8gmm_moe_scatter(x.data_ptr(), inverse.data_ptr(),
                                             weights.data_ptr() if weights is not None else None, out.data_ptr(),
                                             tokens, hidden, top_k, _stream(x.device))
