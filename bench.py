@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|example]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -66,12 +66,82 @@ def splits(kind, experts, tokens, seed):
 GEMM_HBM_TRAFFIC_BYTES = {"config2": 2.42e9}
 
 
+def bench_cast_pad(args):
+    """config5: the bandwidth-bound path alone - ONE multi-tensor cast + transpose + amax + pad-to-128 launch over
+    8 bf16 activation tensors [M_i, 4096], M_i uniform in [1, 8191], N(0, 1) values with 0.1 % outliers at +-200."""
+    import fp8_gmm_amd as pkg  # noqa: F401  (loads the library)
+    from fp8_gmm_amd import backend
+    from fp8_gmm_amd.backend import kernel_timing
+
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(1005)
+    rows = [int(v) for v in rng.integers(1, 8192, size=8)]
+    cols, pad = 4096, 128
+    torch.manual_seed(1005)
+    ins, outs, touts, scales = [], [], [], []
+    for m in rows:
+        x = torch.randn(m, cols, device=dev)
+        hit = torch.rand(m, cols, device=dev) < 1e-3
+        sign = torch.where(torch.rand(m, cols, device=dev) < 0.5, -200.0, 200.0)
+        x = torch.where(hit, sign, x).to(torch.bfloat16)
+        ins.append(x)
+        outs.append(torch.empty(m, cols, dtype=torch.float8_e4m3fn, device=dev))
+        touts.append(torch.empty(cols, (m + pad - 1) // pad * pad, dtype=torch.float8_e4m3fn, device=dev))
+        scales.append((448.0 / x.float().abs().max()).reshape(1))
+    amaxes = torch.zeros(len(rows), device=dev)
+    nbytes = sum(cols * (3 * m + (m + pad - 1) // pad * pad) for m in rows)
+
+    def step():
+        backend.multi_cast_transpose(ins, outs, touts, scales, amaxes)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    with kernel_timing() as timing:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    d = timing.summary()["multi_pad_cast_transpose"]
+    ach = d["work"] / (d["ms"] * 1e-3) / 1e9
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import ref
+
+        m = 2048
+        x = ins[0][: min(m, rows[0])].cpu().contiguous() if rows[0] >= m else torch.randn(m, cols).to(torch.bfloat16)
+        m = x.shape[0]
+        o = torch.empty(m, cols, dtype=torch.float8_e4m3fn)
+        t = torch.empty(cols, (m + pad - 1) // pad * pad, dtype=torch.float8_e4m3fn)
+        a = torch.zeros(1)
+        reps, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < 10.0:
+            ref.multi_cast_transpose([x], [o], [t], [scales[0].cpu()], [a])
+            reps += 1
+        secs = time.perf_counter() - t0
+        cpu = {"value": round(reps * cols * (3 * m + t.shape[1]) / secs / 1e9, 3), "unit": "GB/s", "cores": 1,
+               "kind": "port", "sample": f"{reps} casts of one [{m}, {cols}] tensor by the scalar C oracle, {secs:.1f} s"}
+    print(json.dumps({
+        "metric": "cast + transpose + amax + pad GB/s, % of MI355X HBM bandwidth (8 activation tensors)",
+        "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16->fp8", "data": "synthetic",
+        "config": {"workload": "config5: multi_cast_transpose over 8 x [M_i, 4096] bf16, pad 128, e4m3, "
+                               "0.1 % outliers at +-200", "rows": rows, "bytes_per_step": nbytes},
+        "roofline": {"kernel": "multi_pad_kernel<cast+transpose>", "bound": "hbm", "achieved": round(ach, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": cpu,
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip per-kernel HIP events (pure wall time)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -80,6 +150,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+    if args.workload == "config5":
+        return bench_cast_pad(args)
 
     import fp8_gmm_amd as pkg
     from fp8_gmm_amd.backend import kernel_timing

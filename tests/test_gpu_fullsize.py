@@ -156,3 +156,39 @@ def test_grouped_mlp_full_size_step(dev):
         assert cos(module.fc1_weight.grad[i], w1.grad) > 0.99, f"expert {i} fc1 grad"
         assert cos(module.fc2_weight.grad[i], w2.grad) > 0.99, f"expert {i} fc2 grad"
     assert torch.isfinite(out.float()).all() and torch.isfinite(module.fc1_weight.grad.float()).all()
+
+
+def test_cast_pad_bandwidth_configuration_full_size(dev):
+    """Config 5 at its real size: 8 tensors [M_i, 4096], M_i in [1, 8191], pad to 128, +-200 outliers, e4m3 with
+    scale 448 / amax.  Size-independent checks: transposed copy = transpose + zero padding, amax = max|x| (the
+    outliers), nothing saturates wrongly (dequantised outliers are exactly +-448 / scale), sampled rows equal
+    the oracle's bytes."""
+    import numpy as np
+
+    backend = _backend()
+    rng = np.random.default_rng(1005)
+    rows = [int(v) for v in rng.integers(1, 8192, size=8)] + [1, 127, 129]
+    cols, pad = 4096, 128
+    g = torch.Generator(device=dev).manual_seed(1005)
+    ins, outs, touts, scales = [], [], [], []
+    for m in rows:
+        x = torch.randn(m, cols, generator=g, device=dev)
+        hit = torch.rand(m, cols, generator=g, device=dev) < 1e-3
+        x = torch.where(hit, torch.where(torch.rand(m, cols, generator=g, device=dev) < 0.5, -200.0, 200.0), x)
+        x[0, 0] = 200.0
+        ins.append(x.to(torch.bfloat16))
+        outs.append(torch.full((m, cols), 0x55, dtype=torch.uint8, device=dev).view(E4M3))
+        touts.append(torch.full((cols, (m + pad - 1) // pad * pad), 0x55, dtype=torch.uint8, device=dev).view(E4M3))
+        scales.append((448.0 / ins[-1].float().abs().max()).reshape(1))
+    amaxes = torch.zeros(len(rows), device=dev)
+    backend.multi_cast_transpose(ins, outs, touts, scales, amaxes)
+    for i, m in enumerate(rows):
+        o8, t8 = outs[i].view(torch.uint8), touts[i].view(torch.uint8)
+        assert torch.equal(t8[:, :m], o8.t()), f"tensor {i}"
+        if t8.shape[1] > m:
+            assert int(t8[:, m:].max()) == 0, f"tensor {i}: padding"
+        assert amaxes[i].item() == 200.0
+        assert outs[i][0, 0].float().item() == 448.0       # the outlier lands exactly on the largest finite value
+        for r in (0, m // 2, m - 1):
+            want = ref.f32_to_fp8((ins[i][r: r + 1].float().cpu() * scales[i].item()).contiguous(), E4M3)
+            assert_bytes_equal(outs[i][r: r + 1], want, f"tensor {i} row {r}")
