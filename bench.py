@@ -66,6 +66,61 @@ def splits(kind, experts, tokens, seed):
 GEMM_HBM_TRAFFIC_BYTES = {"config2": 2.42e9}
 
 
+def sample_shader_clock(work):
+    """Runs work() while a thread reads, about once per millisecond, the current shader clock (MHz, pp_dpm_sclk)
+    and board power (W, hwmon power1_input) that the driver publishes in sysfs.  Returns (clock samples, power
+    samples, power cap in W or None), keeping only what was read while the GPU was out of its idle state; empty
+    lists where the nodes cannot be read."""
+    import glob
+    import re
+    import threading
+
+    clk_nodes = glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")
+    pwr_nodes = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+    cap_nodes = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap")
+    clocks, watts, stop = [], [], threading.Event()
+
+    def read(node):
+        try:
+            with open(node) as f:
+                return f.read()
+        except OSError:
+            return ""
+
+    def reader():
+        while not stop.is_set():
+            busy = False
+            for node in clk_nodes:
+                m = re.search(r"(\d+)\s*Mhz\s*\*", read(node), re.IGNORECASE)
+                if m and int(m.group(1)) >= 400:
+                    clocks.append(int(m.group(1)))
+                    busy = True
+            if busy:
+                for node in pwr_nodes:
+                    txt = read(node).strip()
+                    if txt.isdigit():
+                        watts.append(int(txt) / 1e6)
+            time.sleep(0.001)
+
+    cap = None
+    for node in cap_nodes:
+        txt = read(node).strip()
+        if txt.isdigit():
+            cap = int(txt) / 1e6
+    if not clk_nodes:
+        return [], [], cap
+    torch.cuda.synchronize()
+    t = threading.Thread(target=reader, daemon=True)
+    t.start()
+    try:
+        work()
+        torch.cuda.synchronize()
+    finally:
+        stop.set()
+        t.join()
+    return clocks, watts, cap
+
+
 def bench_cast_pad(args):
     """config5: the bandwidth-bound path alone - ONE multi-tensor cast + transpose + amax + pad-to-128 launch over
     8 bf16 activation tensors [M_i, 4096], M_i uniform in [1, 8191], N(0, 1) values with 0.1 % outliers at +-200."""
@@ -234,6 +289,43 @@ def main():
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
                                  "GBps": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
 
+    # Shader clock under this workload, from the driver's sysfs node (what rocm-smi --showclocks prints), sampled
+    # by a thread during a separate pass of 40 steps.  The 5.0 PFLOP/s MFMA peak assumes the 2.4 GHz maximum:
+    # 256 CUs x 8192 flop per clock.
+    clock = None
+    mhz, watts, cap = sample_shader_clock(lambda: [step() for _ in range(40)])
+    if mhz and roofline is not None:
+        mean = sum(mhz) / len(mhz)
+        clock = {"driver_reported": {"shader_mhz_mean": round(mean, 1), "shader_mhz_min": min(mhz),
+                                     "shader_mhz_max": max(mhz), "samples": len(mhz),
+                                     "board_power_w_mean": round(sum(watts) / len(watts), 1) if watts else None,
+                                     "board_power_w_max": max(watts) if watts else None, "board_power_cap_w": cap,
+                                     "source": "pp_dpm_sclk and hwmon power1_input (sysfs), 1 ms period, over 40 "
+                                               "extra steps"}}
+    # ... and the clock the GEMM launches really ran at: cycles / time counted inside a measurement build of the
+    # kernel by the first workgroup of every XCD (fp8gmm_gemm_clock_probe), over 5 more steps
+    if roofline is not None:
+        from fp8_gmm_amd import _lib
+
+        counters = torch.zeros(32, dtype=torch.int64, device=dev)
+        _lib.check(_lib.load().fp8gmm_gemm_clock_probe(counters.data_ptr()))
+        try:
+            for _ in range(5):
+                step()
+            torch.cuda.synchronize()
+        finally:
+            _lib.check(_lib.load().fp8gmm_gemm_clock_probe(None))
+        c = counters.cpu().reshape(8, 4).to(torch.float64)
+        if (c[:, 3] > 0).all():
+            per_xcd = (c[:, 2] / c[:, 3] * 100.0).tolist()
+            eff = sum(per_xcd) / len(per_xcd)
+            peak_at_clock = 256 * 8192 * eff * 1e6 / 1e12
+            clock = dict(clock or {})
+            clock["counted_in_gemm_kernel"] = {
+                "shader_mhz_mean": round(eff, 1), "per_xcd": [round(v, 1) for v in per_xcd],
+                "mfma_peak_at_that_clock_tflops": round(peak_at_clock, 1),
+                "gemm_frac_of_peak_at_that_clock": round(roofline["achieved"] / peak_at_clock, 4)}
+
     # Not the headline: the same step as a micro-batch after the first of an optimizer step, reusing the fp8
     # weights cast by the first (is_first_microbatch=False), which the reference stubs out.
     also = None
@@ -285,6 +377,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "kernels": kernels,
+        "clock": clock,
         "also": also,
     }
     print(json.dumps(line))

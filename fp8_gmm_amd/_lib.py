@@ -83,6 +83,7 @@ EXPORTS = (
     "fp8gmm_multi_cast_dgelu",
     "fp8gmm_grouped_gemm",
     "fp8gmm_delayed_scaling_update",
+    "fp8gmm_gemm_clock_probe",
     "fp8gmm_route_workspace_bytes",
     "fp8gmm_route_sort",
     "fp8gmm_route_invert",
@@ -145,6 +146,8 @@ def load():
     L.fp8gmm_multi_cast_dgelu.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_grouped_gemm.restype = ci
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
+    L.fp8gmm_gemm_clock_probe.restype = ci
+    L.fp8gmm_gemm_clock_probe.argtypes = [vp]
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t

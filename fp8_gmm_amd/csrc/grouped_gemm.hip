@@ -35,6 +35,7 @@
 //     fetched during the previous step) are issued first and the DMA issues / next-fragment
 //     LDS reads are interleaved between them (pinned with sched_barrier), so the MFMA pipe
 //     does not idle while the two wavefronts of a SIMD do their memory work.
+#include <atomic>
 #include <cstdlib>
 #include <map>
 #include <mutex>
@@ -242,12 +243,40 @@ __device__ __forceinline__ void partial_add(f32x16 (&acc)[MT][NT], const uint8_t
       }
 }
 
-template <int A_FMT, int B_FMT>
+// Measurement hook (fp8gmm_gemm_clock_probe): 8 x 4 uint64 of device memory, or null.
+__device__ uint64_t* volatile d_clock_probe = nullptr;
+
+// PROBE: measurement build of the same kernel.  The first workgroup of every XCD writes its shader-cycle counter
+// and the constant 100 MHz counter when it starts and adds the differences to two running totals when it ends,
+// so that the caller can derive the clock the launches really ran at (the counters of different compute units are
+// not comparable, hence the same workgroup takes both readings).  The production build (PROBE = false) contains none of it.
+template <bool PROBE>
+__device__ __forceinline__ void clock_probe_mark(int which) {
+  if constexpr (PROBE) {
+    if (blockIdx.x < kNumXcd && threadIdx.x == 0) {
+      volatile uint64_t* const p = d_clock_probe;
+      if (p != nullptr) {
+        volatile uint64_t* const q = p + 4 * blockIdx.x;
+        const uint64_t cycles = (uint64_t)clock64(), ticks = (uint64_t)wall_clock64();
+        if (which == 0) {
+          q[0] = cycles;
+          q[1] = ticks;
+        } else {  // totals over all launches since the counters were cleared
+          q[2] += cycles - q[0];
+          q[3] += ticks - q[1];
+        }
+      }
+    }
+  }
+}
+
+template <int A_FMT, int B_FMT, bool PROBE>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
                                                                 int nprob, int total_tiles, int out_kind,
                                                                 int epilogue, uint8_t* __restrict__ workspace) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
+  clock_probe_mark<PROBE>(0);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -479,6 +508,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS
   FP8GMM_WAIT_VM(0);
+  clock_probe_mark<PROBE>(1);
 }
 
 #undef FP8GMM_MF0
@@ -556,13 +586,15 @@ bool stream_k_allowed() {
   return allowed;
 }
 
-template <int A_FMT, int B_FMT>
-int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
-           hipStream_t stream) {
+std::atomic<bool> g_clock_probe_on{false};
+
+template <int A_FMT, int B_FMT, bool PROBE>
+int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
+                   hipStream_t stream) {
   static int num_cu = 0;
   static bool attr_set = false;
   const size_t lds_bytes = (size_t)RING * HS;
-  auto kernel = grouped_gemm_kernel<A_FMT, B_FMT>;
+  auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE>;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -599,6 +631,14 @@ int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out
   return FP8GMM_OK;
 }
 
+template <int A_FMT, int B_FMT>
+int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
+           hipStream_t stream) {
+  if (g_clock_probe_on.load(std::memory_order_relaxed))
+    return launch_variant<A_FMT, B_FMT, true>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
+  return launch_variant<A_FMT, B_FMT, false>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
+}
+
 }  // namespace
 }  // namespace fp8gmm
 
@@ -607,6 +647,14 @@ extern "C" {
 void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n) {
   if (tile_m) *tile_m = fp8gmm::BM;
   if (tile_n) *tile_n = fp8gmm::BN;
+}
+
+int fp8gmm_gemm_clock_probe(uint64_t* dev_counters) {
+  // synchronous copy into the device-side pointer of the current device
+  if (hipMemcpyToSymbol(HIP_SYMBOL(fp8gmm::d_clock_probe), &dev_counters, sizeof(dev_counters)) != hipSuccess)
+    return FP8GMM_ERR_LAUNCH;
+  fp8gmm::g_clock_probe_on.store(dev_counters != nullptr, std::memory_order_relaxed);
+  return FP8GMM_OK;
 }
 
 int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles) {

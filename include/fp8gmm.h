@@ -182,6 +182,16 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
                         int out_kind, int epilogue, void* stream);
 
 /*
+ * Measurement hook, no counterpart in the reference.  While `dev_counters` (device memory, 8 x 4 uint64, one
+ * group of four per XCD) is set, fp8gmm_grouped_gemm launches a measurement build of its kernel in which the
+ * first workgroup of every XCD writes {shader-cycle counter, 100 MHz counter} when it starts ([0], [1]) and adds
+ * the elapsed cycles and ticks to [2], [3] when it ends (clear them first): [2] / [3] * 100 MHz is the clock the
+ * launches really ran at, which the clock the driver reports overstates while the chip is power-limited.  NULL (the default) restores the normal kernel.
+ * Applies to the current device; the call synchronises.  bench.py reports the figure.
+ */
+int fp8gmm_gemm_clock_probe(uint64_t* dev_counters);
+
+/*
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:
  *   amax = max over the `history_len` rows of amax_history[history_len, slots] (most_recent != 0: row 0)
  *   scale = (1 / amax) * fp8_max * 2^-margin where amax is finite and > 0, else unchanged;  scale_inv = 1 / scale

@@ -384,3 +384,36 @@ def test_batched_uploads_runs_the_queued_launches_in_order(dev):
     backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, c2)   # and the queue is usable again, immediately
     torch.cuda.synchronize()
     assert c2.any()
+
+
+def test_clock_probe_build_gives_the_same_results_and_a_plausible_clock(dev):
+    """The measurement build of the GEMM kernel (fp8gmm_gemm_clock_probe) must compute exactly what the normal
+    build computes, and its counters must describe a shader clock inside the chip's range."""
+    from fp8_gmm_amd import _lib
+
+    backend = _backend()
+    g = torch.Generator(device=dev).manual_seed(77)
+    sizes = [700, 0, 1300, 48]
+    k, n = 2048, 1536
+    a = torch.randn(sum(sizes), k, generator=g, device=dev).to(E4M3)
+    b = torch.randn(len(sizes), n, k, generator=g, device=dev).to(E4M3)
+    sa = torch.full((len(sizes),), 0.5, device=dev)
+    sb = torch.full((len(sizes),), 0.25, device=dev)
+    want = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
+    counters = torch.zeros(32, dtype=torch.int64, device=dev)
+    L = _lib.load()
+    _lib.check(L.fp8gmm_gemm_clock_probe(counters.data_ptr()))
+    try:
+        got = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
+        got2 = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
+        torch.cuda.synchronize()
+    finally:
+        _lib.check(L.fp8gmm_gemm_clock_probe(None))
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
+    c = counters.cpu().reshape(8, 4).double()
+    assert (c[:, 3] > 0).all(), "every XCD's first workgroup must have reported"
+    mhz = c[:, 2] / c[:, 3] * 100.0
+    assert ((mhz > 300) & (mhz < 2600)).all(), mhz.tolist()
+    after = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)     # back on the normal build
+    assert torch.equal(after.view(torch.int16), want.view(torch.int16))
