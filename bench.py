@@ -199,6 +199,9 @@ def main():
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip per-kernel HIP events (pure wall time)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the extra passes after the timed region (clock / power sampling, cached-weights "
+                         "step): what a profiler should see")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy (reads 256 MiB, writes 256 MiB) so that hardware "
                          "byte counters collected around this command can be scaled against a known transfer")
@@ -293,7 +296,8 @@ def main():
     # by a thread during a separate pass of 40 steps.  The 5.0 PFLOP/s MFMA peak assumes the 2.4 GHz maximum:
     # 256 CUs x 8192 flop per clock.
     clock = None
-    mhz, watts, cap = sample_shader_clock(lambda: [step() for _ in range(40)])
+    mhz, watts, cap = ([], [], None) if args.headline_only else sample_shader_clock(
+        lambda: [step() for _ in range(40)])
     if mhz and roofline is not None:
         mean = sum(mhz) / len(mhz)
         clock = {"driver_reported": {"shader_mhz_mean": round(mean, 1), "shader_mhz_min": min(mhz),
@@ -304,7 +308,7 @@ def main():
                                                "extra steps"}}
     # ... and the clock the GEMM launches really ran at: cycles / time counted inside a measurement build of the
     # kernel by the first workgroup of every XCD (fp8gmm_gemm_clock_probe), over 5 more steps
-    if roofline is not None:
+    if roofline is not None and not args.headline_only:
         from fp8_gmm_amd import _lib
 
         counters = torch.zeros(32, dtype=torch.int64, device=dev)
@@ -329,7 +333,7 @@ def main():
     # Not the headline: the same step as a micro-batch after the first of an optimizer step, reusing the fp8
     # weights cast by the first (is_first_microbatch=False), which the reference stubs out.
     also = None
-    if gs is not None:
+    if gs is not None and not args.headline_only:
         step(True)
         step(False)
         torch.cuda.synchronize()
