@@ -417,3 +417,50 @@ def test_clock_probe_build_gives_the_same_results_and_a_plausible_clock(dev):
     assert ((mhz > 300) & (mhz < 2600)).all(), mhz.tolist()
     after = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)     # back on the normal build
     assert torch.equal(after.view(torch.int16), want.view(torch.int16))
+
+
+def test_random_problem_lists_are_exact(dev):
+    """Sixty random grouped problems (ragged and empty experts, K and N that are not tile multiples, both operand
+    formats, the stacked and the list calling form).  Operands come from {0, +-0.25 .. +-2} and the scales are
+    powers of two, so every fp32 partial sum is exact in any order: the result must equal torch's fp32 matmul of
+    the dequantised operands bit for bit, whatever tiles, K pieces and fix-ups the schedule chose."""
+    import numpy as np
+
+    backend = _backend()
+    rng = np.random.default_rng(4242)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    g = torch.Generator(device=dev).manual_seed(4242)
+
+    def exact(shape, dtype):
+        return vals[torch.randint(0, 8, shape, generator=g, device=dev)].to(dtype)
+
+    for trial in range(60):
+        e = int(rng.integers(1, 9))
+        a_dtype = E5M2 if rng.integers(0, 2) else E4M3
+        if trial % 2 == 0:   # fp8_gmm form: one N and K, ragged rows
+            sizes = [int(rng.choice([0, 1, 15, 100, 256, 257, 700, 1500])) for _ in range(e)]
+            n = int(rng.choice([16, 48, 256, 272, 1000, 1536]))
+            k = int(rng.choice([16, 64, 128, 144, 1024, 2064, 4096]))
+            a = exact((sum(sizes), k), a_dtype)
+            b = exact((e, n, k), E4M3)
+            sa = torch.full((e,), 0.5, device=dev)
+            sb = torch.full((e,), 2.0, device=dev)
+            c = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, backward=(a_dtype == E5M2))
+            row = 0
+            for i, s in enumerate(sizes):
+                want = (a[row: row + s].float() @ b[i].float().t()).to(torch.bfloat16)
+                assert torch.equal(c[row: row + s].view(torch.int16), want.view(torch.int16)), \
+                    f"trial {trial} expert {i}: sizes {sizes} n {n} k {k} {a_dtype}"
+                row += s
+        else:                # list form: every problem has its own m, n, k (the weight-gradient shape)
+            shapes = [(int(rng.choice([1, 64, 300, 768])), int(rng.choice([16, 256, 520])),
+                       int(rng.choice([0, 16, 128, 400, 1152, 4096]))) for _ in range(e)]
+            a_list = [exact((m, k), a_dtype) for m, n, k in shapes]
+            b_list = [exact((n, k), E4M3) for m, n, k in shapes]
+            c_list = [torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev) for m, n, k in shapes]
+            ones = torch.ones(e, device=dev)
+            backend.grouped_gemm(a_list, b_list, c_list, ones, ones)
+            for i, (m, n, k) in enumerate(shapes):
+                want = (a_list[i].float() @ b_list[i].float().t()).to(torch.bfloat16)
+                assert torch.equal(c_list[i].view(torch.int16), want.view(torch.int16)), \
+                    f"trial {trial} problem {i}: shapes {shapes} {a_dtype}"
