@@ -17,6 +17,7 @@ E4M3 = 0
 E5M2 = 1
 OUT_BF16 = 2
 EPI_GELU = 1
+GEMM_B_KMAJOR = 2
 
 OP_QUANTIZE = 0
 OP_SCALE_MUL = 1
@@ -75,6 +76,7 @@ EXPORTS = (
     "fp8gmm_gemm_tile_shape",
     "fp8gmm_plan_multi_tensor",
     "fp8gmm_plan_grouped_gemm",
+    "fp8gmm_plan_grouped_gemm_layout",
     "fp8gmm_multi_quantize",
     "fp8gmm_multi_scale_mul",
     "fp8gmm_multi_pad_transpose",
@@ -132,6 +134,8 @@ def load():
     L.fp8gmm_plan_multi_tensor.argtypes = [vp, ci, ci, ip]
     L.fp8gmm_plan_grouped_gemm.restype = ci
     L.fp8gmm_plan_grouped_gemm.argtypes = [vp, ci, ip]
+    L.fp8gmm_plan_grouped_gemm_layout.restype = ci
+    L.fp8gmm_plan_grouped_gemm_layout.argtypes = [vp, ci, ci, ip]
     L.fp8gmm_multi_quantize.restype = ci
     L.fp8gmm_multi_quantize.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_multi_scale_mul.restype = ci
@@ -184,9 +188,9 @@ def plan_multi_tensor(table, op):
     return total.value
 
 
-def plan_grouped_gemm(table):
+def plan_grouped_gemm(table, layout=0):
     total = ctypes.c_int(0)
-    check(load().fp8gmm_plan_grouped_gemm(table.ctypes.data, len(table), ctypes.byref(total)))
+    check(load().fp8gmm_plan_grouped_gemm_layout(table.ctypes.data, len(table), layout, ctypes.byref(total)))
     return total.value
 
 

@@ -570,18 +570,21 @@ def multi_cast_dgelu(inputs, gelu_inputs, outputs, scales, amaxes):
 # ------------------------------------------------------------------------------------------------
 # GEMMs
 # ------------------------------------------------------------------------------------------------
-def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep):
+def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=False):
     if a_dtype not in _FP8_DTYPES or b_dtype not in _FP8_DTYPES:
         _fail("fp8_gmm_amd: GEMM operands must be fp8")
     if a_dtype == torch.float8_e5m2 and b_dtype == torch.float8_e5m2:
         _fail("fp8_gmm_amd: e5m2 x e5m2 GEMMs are not supported")
     if c_dtype not in _OUT_KIND:
         _fail("fp8_gmm_amd: GEMM output must be bfloat16 or fp8")
-    total = _lib.plan_grouped_gemm(table)
+    if b_kmajor and b_dtype != torch.float8_e4m3fn:
+        _fail("fp8_gmm_amd: a contraction-major b must be float8_e4m3fn")
+    layout = _lib.GEMM_B_KMAJOR if b_kmajor else 0
+    total = _lib.plan_grouped_gemm(table, layout)
     if total == 0:
         return
     n = len(table)
-    fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], _lib.EPI_GELU if gelu else 0)
+    fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], (_lib.EPI_GELU if gelu else 0) | layout)
 
     def launch(dev_ptr):
         with torch.cuda.device(device), _timed("grouped_gemm", lambda: _algorithmic_flops(table)):
@@ -678,7 +681,7 @@ def _group_sizes_list(group_sizes):
 
 
 def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch.bfloat16, pre_gelu_out=None,
-            c_scales=None, c_amaxes=None, backward=False, cutlass=False):
+            c_scales=None, c_amaxes=None, backward=False, cutlass=False, b_transposed=False):
     """Grouped GEMM over row slices of ``a``: expert i multiplies rows
     ``[sum(group_sizes[:i]), sum(group_sizes[:i+1]))`` of ``a[tokens, k]`` with ``b[i][n, k]^T``.
 
@@ -687,6 +690,10 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     followed by ``multi_scale_mul`` (two roundings); the default applies the scales to
     the fp32 accumulator in the GEMM epilogue (one rounding), like its cuBLASLt path.
     Experts with zero rows are allowed.
+
+    ``b_transposed=True`` (not in the reference): ``b`` is ``[experts, k, n]`` and expert i multiplies with
+    ``b[i]`` as it stands.  That is a forward weight stack used by the data-gradient GEMM without the transposed
+    copy the reference casts for it (grouped_linear.py:69-74,163); same results, bit for bit.
     """
     sizes = _group_sizes_list(group_sizes)
     e = len(sizes)
@@ -695,11 +702,11 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     if not (a.is_contiguous() and b.is_contiguous()):
         _fail("fp8_gmm_amd: fp8_gmm expects contiguous a and b")
     tokens, k = a.shape
-    if b.shape[0] != e or b.shape[2] != k:
-        _fail("fp8_gmm_amd: b must be [len(group_sizes), n, k] with k == a.shape[1]")
+    if b.shape[0] != e or b.shape[1 if b_transposed else 2] != k:
+        _fail("fp8_gmm_amd: b must be [len(group_sizes), n, k] with k == a.shape[1] ([.., k, n] when b_transposed)")
     if any(g < 0 for g in sizes) or sum(sizes) != tokens:
         _fail("fp8_gmm_amd: group_sizes must be non-negative and sum to a.shape[0]")
-    nn = b.shape[1]
+    nn = b.shape[2 if b_transposed else 1]
     if c is None:
         c = torch.empty(tokens, nn, device=a.device, dtype=c_dtype)
     if tuple(c.shape) != (tokens, nn) or not c.is_contiguous():
@@ -729,7 +736,7 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     table["n"] = nn
     table["k"] = k
     table["lda"] = k
-    table["ldb"] = k
+    table["ldb"] = nn if b_transposed else k
     table["ldc"] = nn
     if not cutlass:
         table["a_scale_inv"] = _scalar_ptrs(a_scale_invs, e, "a_scale_invs")
@@ -738,7 +745,7 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
         table["c_scale"] = _scalar_ptrs(c_scales, e, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, e, "c_amaxes")
     _launch_gemm(table, a.dtype, b.dtype, c.dtype, pre_gelu_out is not None, dev,
-                 (a, b, c, pre_gelu_out, a_scale_invs, b_scale_invs, c_scales, c_amaxes))
+                 (a, b, c, pre_gelu_out, a_scale_invs, b_scale_invs, c_scales, c_amaxes), b_kmajor=b_transposed)
     if cutlass:
         multi_scale_mul(TensorBatch.rows_of(c, starts), a_scale_invs, b_scale_invs)
     return c

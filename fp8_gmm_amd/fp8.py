@@ -159,13 +159,16 @@ class Fp8WeightCache:
         self.valid = False   # fp8 holds a cast of the weights
         self.valid_t = False  # fp8_t does too
 
-    def buffers(self, weight, dtype):
+    def buffers(self, weight, dtype, with_transpose=True):
         if self.fp8 is None or self.fp8.shape != weight.shape or self.fp8.dtype != dtype \
                 or self.fp8.device != weight.device:
-            e, n, k = weight.shape
-            self.fp8 = torch.empty(e, n, k, dtype=dtype, device=weight.device)
-            self.fp8_t = torch.empty(e, k, n, dtype=dtype, device=weight.device)
+            self.fp8 = torch.empty(weight.shape, dtype=dtype, device=weight.device)
+            self.fp8_t = None
             self.valid = self.valid_t = False
+        if with_transpose and self.fp8_t is None:
+            e, n, k = weight.shape
+            self.fp8_t = torch.empty(e, k, n, dtype=dtype, device=weight.device)
+            self.valid_t = False
         return self.fp8, self.fp8_t
 
     def require(self, transposed):

@@ -88,12 +88,14 @@ class _GroupedMlp(torch.autograd.Function):
                                          x_amaxes)):
                 lst.append(item)
 
+        transposed_weights = bool(fp8_meta.get("transposed_weights", False))
+        need_t, cache_t = dgrad_needed and transposed_weights, is_grad_enabled and transposed_weights
         fc1_weight_fp8, fc1_weight_t_fp8 = stage_weight_cast(
-            fc1_weight, fp8_dtype, dgrad_needed, is_grad_enabled, weight_caches[0], update_fp8_weights,
+            fc1_weight, fp8_dtype, need_t, cache_t, weight_caches[0], update_fp8_weights,
             meta.get_meta_pointers(_T.kWeightGroup1, _M.kScale), meta.get_meta_pointers(_T.kWeightGroup1, _M.kAmax),
             plain, with_t)
         fc2_weight_fp8, fc2_weight_t_fp8 = stage_weight_cast(
-            fc2_weight, fp8_dtype, dgrad_needed, is_grad_enabled, weight_caches[1], update_fp8_weights,
+            fc2_weight, fp8_dtype, need_t, cache_t, weight_caches[1], update_fp8_weights,
             meta.get_meta_pointers(_T.kWeightGroup2, _M.kScale), meta.get_meta_pointers(_T.kWeightGroup2, _M.kAmax),
             plain, with_t)
 
@@ -128,7 +130,13 @@ class _GroupedMlp(torch.autograd.Function):
             gelu_out_fp8 = None
 
         if is_grad_enabled:
-            ctx.save_for_backward(input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8, pre_gelu_out, gelu_out_fp8)
+            if transposed_weights:
+                w1_dgrad, w2_dgrad = fc1_weight_t_fp8, fc2_weight_t_fp8
+            else:  # the data-gradient GEMMs read the row-major copies in place
+                w1_dgrad = fc1_weight_fp8 if (dgrad_needed and input_requires_grad) else None
+                w2_dgrad = fc2_weight_fp8 if dgrad_needed else None
+            ctx.save_for_backward(input_t_fp8, w1_dgrad, w2_dgrad, pre_gelu_out, gelu_out_fp8)
+            ctx.transposed_weights = transposed_weights
             ctx.group_sizes = group_sizes
             meta.set_forward_scale_inv_cloned()
             ctx.meta = meta
@@ -149,7 +157,8 @@ class _GroupedMlp(torch.autograd.Function):
 
     @staticmethod
     def _backward(ctx, grad_out):
-        input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
+        input_t_fp8, fc1_weight_dgrad, fc2_weight_dgrad, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
+        b_transposed = not ctx.transposed_weights
         meta = ctx.meta
         cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
         t_bounds = padded_cumsums if padded else cumsums
@@ -182,9 +191,9 @@ class _GroupedMlp(torch.autograd.Function):
 
         # fc2 dgrad: d(gelu_out)[tokens, F]
         grad_gelu_out = fp8_gmm(
-            grad_out_fp8, fc2_weight_t_fp8, ctx.group_sizes, g1_scale_invs,
+            grad_out_fp8, fc2_weight_dgrad, ctx.group_sizes, g1_scale_invs,
             meta.get_meta_pointers(_T.kForwardWeightGroup2, _M.kScaleInv),
-            backward=True, cutlass=False,
+            backward=True, cutlass=False, b_transposed=b_transposed,
         )
 
         # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8; the padded transpose only feeds fc1 wgrad
@@ -208,9 +217,9 @@ class _GroupedMlp(torch.autograd.Function):
         handle = None
         if ctx.input_requires_grad:
             grad_input = fp8_gmm(
-                grad_pre_fp8, fc1_weight_t_fp8, ctx.group_sizes, g2_scale_invs,
+                grad_pre_fp8, fc1_weight_dgrad, ctx.group_sizes, g2_scale_invs,
                 meta.get_meta_pointers(_T.kForwardWeightGroup1, _M.kScaleInv),
-                backward=True, cutlass=False,
+                backward=True, cutlass=False, b_transposed=b_transposed,
             )
             if ctx.has_tp:
                 flush_uploads()  # the collective must see grad_input
@@ -235,14 +244,15 @@ class GroupedMlp(Fp8GroupedModuleBase):
     """E expert MLPs ``in_features -> out_features -> in_features`` with tanh-GELU, no biases.
 
     ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None, is_first_microbatch=None)``;
-    ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
+    ``transposed_weights`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
     the module's fp8 weight buffers).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
-                 pad_multiple=MODULE_PAD_MULTIPLE):
+                 pad_multiple=MODULE_PAD_MULTIPLE, transposed_weights=False):
         super().__init__()
         self.fp8_meta["pad_multiple"] = pad_multiple
+        self.fp8_meta["transposed_weights"] = transposed_weights
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.num_groups = num_groups
         self.fc1_weight = torch.nn.Parameter(
@@ -262,8 +272,9 @@ class GroupedMlp(Fp8GroupedModuleBase):
         if is_first_microbatch is None:
             return [None, None, None, None]
         dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
-        return list(self._weight_caches[0].buffers(self.fc1_weight, dtype)) + \
-            list(self._weight_caches[1].buffers(self.fc2_weight, dtype))
+        tw = self.fp8_meta["transposed_weights"]
+        return list(self._weight_caches[0].buffers(self.fc1_weight, dtype, tw)) + \
+            list(self._weight_caches[1].buffers(self.fc2_weight, dtype, tw))
 
     def forward(self, input, group_sizes, has_tp=False, tp_group=None, is_first_microbatch=None):
         with self.prepare_forward(input, is_first_microbatch, self.num_groups * 2):

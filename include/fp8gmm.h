@@ -130,8 +130,14 @@ typedef struct fp8gmm_gemm_problem {
   int32_t cost_begin;        /* filled by fp8gmm_plan_grouped_gemm: K = 128 steps of all earlier tiles */
 } fp8gmm_gemm_problem;       /* 96 bytes */
 
-/* epilogue flags of fp8gmm_grouped_gemm */
+/* flags of fp8gmm_grouped_gemm (its `epilogue` argument) */
 #define FP8GMM_EPI_GELU 1
+/* b is stored contraction-major: b[k, n] with n contiguous and ldb >= n its row pitch, i.e.
+ * c[m, n] = epilogue( a[m, k] . b[k, n] ).  This is a forward weight [N_fwd = k, K_fwd = n] as the data-gradient
+ * GEMM needs it, read in place: the reference casts a transposed copy of every weight for that GEMM instead
+ * (fp8_gmm/grouped_linear.py:69-74,163).  b must be e4m3, n a multiple of 16, k * ldb < 2^32.  Plan such tables
+ * with fp8gmm_plan_grouped_gemm_layout(..., FP8GMM_GEMM_B_KMAJOR, ...). */
+#define FP8GMM_GEMM_B_KMAJOR 2
 
 /* ---- library info ------------------------------------------------------------------------- */
 int fp8gmm_version(void);
@@ -150,6 +156,8 @@ int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* tota
 /* Validates `probs[0..n)`, fills tile_begin / cost_begin, returns the tile count in *total_tiles.
  * Replaces the host half of CutlassFp8GroupedGemm (csrc/fp8_gmm.cu:82-135). */
 int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles);
+/* The same for a launch with layout flags (0 or FP8GMM_GEMM_B_KMAJOR): only the checks on b differ. */
+int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layout, int* total_tiles);
 
 /* ---- launches (descs_dev / probs_dev: DEVICE copies of planned tables) ------------------- */
 /* replaces MultiQuantize, csrc/multi_pointwise.cu:155 (pybind name multi_quantize, csrc/ops.cu:11) */

@@ -464,3 +464,45 @@ def test_random_problem_lists_are_exact(dev):
                 want = (a_list[i].float() @ b_list[i].float().t()).to(torch.bfloat16)
                 assert torch.equal(c_list[i].view(torch.int16), want.view(torch.int16)), \
                     f"trial {trial} problem {i}: shapes {shapes} {a_dtype}"
+
+
+@pytest.mark.parametrize("a_dtype", [E4M3, E5M2])
+def test_contraction_major_b_gives_the_same_bits(dev, a_dtype):
+    """fp8_gmm(..., b_transposed=True) reads b[i] as [k, n] in place: for every shape it must return exactly what
+    the row-major path returns for b[i].t().contiguous() (same schedule, same MFMA order), random data included;
+    and exact data must equal the fp32 matmul."""
+    import numpy as np
+
+    backend = _backend()
+    rng = np.random.default_rng(99)
+    g = torch.Generator(device=dev).manual_seed(99)
+    cases = [([256], 256, 128), ([300, 0, 513, 90], 512, 1040), ([1, 15], 16, 16), ([700], 272, 2064),
+             ([137, 401, 59, 403], 256, 512), ([2048, 100], 4096, 1408), ([64], 1536, 80)]
+    for sizes, n, k in cases:
+        e = len(sizes)
+        a = torch.randn(sum(sizes), k, generator=g, device=dev).to(a_dtype)
+        b_kn = torch.randn(e, k, n, generator=g, device=dev).to(E4M3)           # contraction-major
+        b_nk = b_kn.transpose(1, 2).contiguous()
+        sa = torch.rand(e, generator=g, device=dev) + 0.5
+        sb = torch.rand(e, generator=g, device=dev) + 0.5
+        want = backend.fp8_gmm(a, b_nk, torch.tensor(sizes), sa, sb, backward=True)
+        got = backend.fp8_gmm(a, b_kn, torch.tensor(sizes), sa, sb, backward=True, b_transposed=True)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"sizes {sizes} n {n} k {k}"
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    for trial in range(10):
+        e = int(rng.integers(1, 6))
+        sizes = [int(rng.choice([0, 1, 100, 256, 700])) for _ in range(e)]
+        n = int(rng.choice([16, 48, 256, 1008]))
+        k = int(rng.choice([16, 144, 1024, 4096]))
+        a = vals[torch.randint(0, 8, (sum(sizes), k), generator=g, device=dev)].to(a_dtype)
+        b = vals[torch.randint(0, 8, (e, k, n), generator=g, device=dev)].to(E4M3)
+        ones = torch.ones(e, device=dev)
+        c = backend.fp8_gmm(a, b, torch.tensor(sizes), ones, ones, backward=True, b_transposed=True)
+        row = 0
+        for i, s in enumerate(sizes):
+            want = (a[row: row + s].float() @ b[i].float()).to(torch.bfloat16)
+            assert torch.equal(c[row: row + s].view(torch.int16), want.view(torch.int16)), f"{sizes} {n} {k} expert {i}"
+            row += s
+    with pytest.raises(RuntimeError):   # n must be a multiple of 16 in this layout
+        backend.fp8_gmm(torch.zeros(4, 16, device=dev).to(a_dtype), torch.zeros(1, 16, 8, device=dev).to(E4M3),
+                        [4], None, None, b_transposed=True)

@@ -237,7 +237,8 @@ def test_pad_multiple_does_not_change_results(dev, kind):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
-def test_grouped_linear_reuses_cached_fp8_weights(dev):
+@pytest.mark.parametrize("transposed_weights", [False, True], ids=["in-place-dgrad", "reference-layout"])
+def test_grouped_linear_reuses_cached_fp8_weights(dev, transposed_weights):
     """is_first_microbatch: True casts the weights into the module's buffers, False reuses them.  The weights
     are CHANGED between the two micro-batches, so only a pass that really reuses the cached bytes (and their
     scale_inv) can match the oracle, which is handed the first pass's fp8 weights; a later True picks up the
@@ -248,7 +249,7 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev):
     g = gen(3001)
     w = randn_bf16((e, n, k), g, 0.02)
     w_changed = (w.float() * 1.5 + 0.01).to(torch.bfloat16)
-    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev, transposed_weights=transposed_weights)
     fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
     fwd, bwd = orc.Meta(3 * e, hist), orc.Meta(2 * e, hist)
     weight_slots = [3 * i + 1 for i in range(e)]
@@ -278,7 +279,10 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev):
             assert not gm["scaling_fwd"].amax_history[0][weight_slots].any()
         w_fp8, w_t_fp8 = module.get_fp8_weights_scratchpad(first)
         assert torch.equal(w_fp8.cpu().view(torch.uint8), cached["w_fp8"].view(torch.uint8)), f"step {step}"
-        assert torch.equal(w_t_fp8.cpu().view(torch.uint8), cached["w_t_fp8"].view(torch.uint8)), f"step {step}"
+        if transposed_weights:
+            assert torch.equal(w_t_fp8.cpu().view(torch.uint8), cached["w_t_fp8"].view(torch.uint8)), f"step {step}"
+        else:
+            assert w_t_fp8 is None   # the data-gradient GEMM reads w_fp8 in place
         assert_gemm_close(out, o["out"].float(), 1e-2, f"step {step} out")
         assert_gemm_close(xd.grad, o["grad_input"].float(), 1e-2, f"step {step} grad_input")
         assert_gemm_close(module.weight_tensor.grad, o["grad_weight"].float(), 1e-2, f"step {step} grad_weight")
@@ -287,7 +291,7 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev):
 
 def test_cached_weights_need_a_first_microbatch(dev):
     pkg = _pkg()
-    module = pkg.GroupedLinear(64, 64, 2, torch.bfloat16, device=dev)
+    module = pkg.GroupedLinear(64, 64, 2, torch.bfloat16, device=dev, transposed_weights=True)
     x = torch.zeros(32, 64, dtype=torch.bfloat16, device=dev, requires_grad=True)
     with pytest.raises(RuntimeError, match="is_first_microbatch=False"):
         module(x, [16, 16], is_first_microbatch=False)
@@ -373,3 +377,38 @@ def test_grouped_mlp_frozen_weights_against_the_oracle(dev):
     assert_close_multistage(xd.grad, o["grad_input"], 1e-2, "grad_input")
     _check_amax(module.fp8_meta["scaling_bwd"], bwd, [2 * i for i in range(e)], [2 * (e + i) for i in range(e)],
                 "frozen bwd")
+
+
+@pytest.mark.parametrize("kind", ["linear", "mlp"])
+def test_in_place_dgrad_equals_the_reference_layout(dev, kind):
+    """By default no transposed fp8 weights are cast and the data-gradient GEMMs read the row-major copies in
+    place; with transposed_weights=True the reference's [E, K, N] copies are cast and used.  Same bits either way,
+    over three steps of delayed scaling."""
+    pkg = _pkg()
+    sizes, h, f = [137, 0, 401, 59, 403], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(3004)
+    mods = []
+    for tw in (False, True):
+        if kind == "linear":
+            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, transposed_weights=tw)
+        else:
+            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, transposed_weights=tw)
+        mods.append(mod)
+    mods[1].load_state_dict(mods[0].state_dict())
+    out_cols = f if kind == "linear" else h
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=2)
+    for step in range(3):
+        x = randn_bf16((m, h), g).to(dev)
+        dy = randn_bf16((m, out_cols), g, 1e-2).to(dev)
+        res = []
+        for mod in mods:
+            xd = x.clone().requires_grad_()
+            mod.zero_grad()
+            with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
+                out = mod(xd, torch.tensor(sizes))
+            out.backward(dy)
+            res.append([out, xd.grad] + [p.grad for p in mod.parameters()])
+        for a, b in zip(*res):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}"
+        assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
