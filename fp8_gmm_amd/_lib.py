@@ -18,6 +18,7 @@ E5M2 = 1
 OUT_BF16 = 2
 EPI_GELU = 1
 GEMM_B_KMAJOR = 2
+GEMM_A_KMAJOR = 4
 
 OP_QUANTIZE = 0
 OP_SCALE_MUL = 1

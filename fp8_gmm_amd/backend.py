@@ -570,7 +570,7 @@ def multi_cast_dgelu(inputs, gelu_inputs, outputs, scales, amaxes):
 # ------------------------------------------------------------------------------------------------
 # GEMMs
 # ------------------------------------------------------------------------------------------------
-def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=False):
+def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=False, a_kmajor=False):
     if a_dtype not in _FP8_DTYPES or b_dtype not in _FP8_DTYPES:
         _fail("fp8_gmm_amd: GEMM operands must be fp8")
     if a_dtype == torch.float8_e5m2 and b_dtype == torch.float8_e5m2:
@@ -579,7 +579,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         _fail("fp8_gmm_amd: GEMM output must be bfloat16 or fp8")
     if b_kmajor and b_dtype != torch.float8_e4m3fn:
         _fail("fp8_gmm_amd: a contraction-major b must be float8_e4m3fn")
-    layout = _lib.GEMM_B_KMAJOR if b_kmajor else 0
+    layout = (_lib.GEMM_B_KMAJOR if b_kmajor else 0) | (_lib.GEMM_A_KMAJOR if a_kmajor else 0)
     total = _lib.plan_grouped_gemm(table, layout)
     if total == 0:
         return
@@ -614,13 +614,18 @@ def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, mo
 
 
 def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_outs=None, c_scales=None,
-                 c_amaxes=None):
+                 c_amaxes=None, transposed=False):
     """c_list[i][m, n] = epilogue(a_list[i][m, k] . b_list[i][n, k]^T) for all i in ONE launch.
 
     The list form of ``cublas_fp8_gemm``: the reference issues these as a Python loop of
     cuBLASLt calls (wgrad, grouped_linear.py:173-182; grouped_mlp.py:234-242,313-322).
     k may differ per entry and may be 0 (the output is then the epilogue of zero).
     Lists of tensors or TensorBatches.
+
+    ``transposed=True`` (not in the reference): the operands are given contraction-major, ``a_list[i][k, m]`` and
+    ``b_list[i][k, n]``, and ``c = a^T . b``.  That is the weight gradient ``dW = dY^T . X`` on the row-major
+    gradient and activation slices of an expert, with no padded transposed copies; k (the expert's row count) may be
+    any number, m and n must be multiples of 16.
     """
     n = len(a_list)
     if n == 0:
@@ -632,11 +637,16 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
     fp8_out = c.dtype in _FP8_DTYPES
     if fp8_out and c_scales is None:
         _fail("fp8_gmm_amd: an fp8 GEMM output needs c_scales")
-    if np.any(a.cols != b.cols) or np.any(c.rows != a.rows) or np.any(c.cols != b.rows):
-        _fail("fp8_gmm_amd: GEMM shapes do not match: a [m, k], b [n, k], c [m, n]")
     table = np.zeros(n, dtype=GEMM_PROBLEM)
     table["a"], table["b"], table["c"] = a.ptr, b.ptr, c.ptr
-    table["m"], table["n"], table["k"] = a.rows, b.rows, a.cols
+    if transposed:
+        if np.any(a.rows != b.rows) or np.any(c.rows != a.cols) or np.any(c.cols != b.cols):
+            _fail("fp8_gmm_amd: GEMM shapes do not match: a [k, m], b [k, n], c [m, n]")
+        table["m"], table["n"], table["k"] = a.cols, b.cols, a.rows
+    else:
+        if np.any(a.cols != b.cols) or np.any(c.rows != a.rows) or np.any(c.cols != b.rows):
+            _fail("fp8_gmm_amd: GEMM shapes do not match: a [m, k], b [n, k], c [m, n]")
+        table["m"], table["n"], table["k"] = a.rows, b.rows, a.cols
     table["lda"] = np.maximum(a.pitch, a.cols)
     table["ldb"] = np.maximum(b.pitch, b.cols)
     table["ldc"] = np.maximum(c.pitch, c.cols)
@@ -651,7 +661,8 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
         table["c_scale"] = _scalar_ptrs(c_scales, n, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, n, "c_amaxes")
     _launch_gemm(table, a.dtype, b.dtype, c.dtype, aux is not None, dev,
-                 (a, b, c, aux, a_scale_invs, b_scale_invs, c_scales, c_amaxes))
+                 (a, b, c, aux, a_scale_invs, b_scale_invs, c_scales, c_amaxes), b_kmajor=transposed,
+                 a_kmajor=transposed)
 
 
 def cublas_fp8_gemm(a, b, c, a_scale_inv, b_scale_inv, pre_gelu_out=None, c_scale=None, c_amax=None, backward=False):

@@ -276,7 +276,10 @@ __device__ __forceinline__ void clock_probe_mark(int which) {
 // gathered with four transposing reads (ds_read_b64_tr_b8: in a group of 16 lanes, lane 8 h + i receives byte i
 // of the 8 bytes addressed by lanes 2 b + h, b = 0..7).  Everything else - schedule, MFMA order, epilogue -
 // is shared, so both layouts produce the same bits.
-template <int A_FMT, int B_FMT, bool PROBE, bool B_TR>
+// A_TR: the same for operand a (a[k][m], pitch lda): with both, c = a^T . b contracts over the rows of two
+// row-major matrices, which is the weight-gradient GEMM on the un-transposed activations and gradients; rows
+// past k read as zeros, so the contraction length needs no padding.
+template <int A_FMT, int B_FMT, bool PROBE, bool A_TR, bool B_TR>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
                                                                 int nprob, int total_tiles, int out_kind,
                                                                 int epilogue, uint8_t* __restrict__ workspace) {
@@ -308,6 +311,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   const int fbt_row = BM * HK + (32 * khalf + tr_b) * 256 + 8 * tr_h;
   const int fbt_off0 = fbt_row + (((wave_n * 4 + tr_g) ^ (2 * tr_b)) << 4);
   const int fbt_off1 = fbt_row + (((wave_n * 4 + 2 + tr_g) ^ (2 * tr_b)) << 4);
+  // A_TR: logical chunk wave_m * 8 + 2 i + g of the token half of the half-slot
+  const int fat_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
+  int fat_off[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) fat_off[i] = fat_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
 
   // ---- this workgroup's item sequence (uniform): strided tiles of its XCD's range, then its piece of
   // the range's stream-K region ----
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   // ---- load side: runs two pairs ahead of the compute side, possibly in the next tile ----
   bool ld_live = true;  // the load cursor still points at an item
   int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
-  [[maybe_unused]] int ld_ldb = 0, ld_bkmax = 0;  // B_TR only
+  [[maybe_unused]] int ld_lda = 0, ld_ldb = 0, ld_trkmax = 0;  // contraction-major operands only
   i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
   uint32_t a_base[2], b_base[2];
   uint32_t ok_mask = 0;  // bit part: rows of that part exist
@@ -333,7 +341,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       if (g.nk > 0) {
         const fp8gmm_gemm_problem pr = probs[g.prob];
         const uint64_t pa = (uint64_t)pr.a, pb = (uint64_t)pr.b;
-        const uint64_t sa = (uint64_t)pr.m * (uint64_t)pr.lda;
+        const uint64_t sa = (uint64_t)(A_TR ? pr.k : pr.m) * (uint64_t)pr.lda;
         const uint64_t sb = (uint64_t)(B_TR ? pr.k : pr.n) * (uint64_t)pr.ldb;  // rows of b times its pitch
         rsrc_a[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pa);
         rsrc_a[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pa >> 32));
@@ -346,24 +354,30 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         for (int j = 0; j < 2; ++j) {
           const int ar = g.m0 + (wave + 8 * j) * 16 + drow;
           const int br = g.n0 + (wave + 8 * j) * 16 + drow;
-          if (ar < pr.m) ok_mask |= 1u << j;
-          a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          // contraction-major operand: one instruction fills 4 contraction rows x 256 B: lane -> row
+          // (wave + 8 j) * 4 + lane / 16 of the half-slot, physical chunk lane % 16, which must receive
+          // global chunk p ^ 2 (row mod 8)
+          const int krow = (wave + 8 * j) * 4 + (lane >> 4);
+          const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
+          if constexpr (!A_TR) {
+            if (ar < pr.m) ok_mask |= 1u << j;
+            a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          } else {
+            if (g.m0 + tr_col < pr.m) ok_mask |= 1u << j;
+            a_base[j] = (uint32_t)krow * (uint32_t)pr.lda + (uint32_t)(g.m0 + tr_col);
+          }
           if constexpr (!B_TR) {
             if (br < pr.n) ok_mask |= 4u << j;
             b_base[j] = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
           } else {
-            // one instruction fills 4 contraction rows x 256 B: lane -> row (wave + 8 j) * 4 + lane / 16 of
-            // the half-slot, physical chunk lane % 16, which must receive global chunk p ^ 2 (row mod 8)
-            const int krow = (wave + 8 * j) * 4 + (lane >> 4);
-            const int gcol = g.n0 + (((lane & 15) ^ (2 * (krow & 7))) << 4);
-            if (gcol < pr.n) ok_mask |= 4u << j;
-            b_base[j] = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)gcol;
+            if (g.n0 + tr_col < pr.n) ok_mask |= 4u << j;
+            b_base[j] = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)(g.n0 + tr_col);
           }
         }
-        if constexpr (B_TR) {
-          ld_ldb = pr.ldb;
-          ld_bkmax = pr.k - (wave * 4 + (lane >> 4));  // row k0 + krow of part j exists iff k0 + 32 j < ld_bkmax
-        }
+        if constexpr (A_TR) ld_lda = pr.lda;
+        if constexpr (B_TR) ld_ldb = pr.ldb;
+        // row k0 + krow of part j of a contraction-major operand exists iff k0 + 32 j < ld_trkmax
+        if constexpr (A_TR || B_TR) ld_trkmax = pr.k - (wave * 4 + (lane >> 4));
         ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
         ld_kt = g.k_begin;
         ld_nk = g.k_begin + g.nk;
@@ -382,10 +396,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     const bool rok = ld_live && ((ok_mask >> part) & 1);
     const uint32_t base = is_b ? b_base[j] : a_base[j];
     uint32_t v_lo, v_hi;
-    if (B_TR && is_b) {
-      const uint32_t row0 = (uint32_t)k0 * (uint32_t)ld_ldb;  // k * ldb < 2^32 is checked when the table is planned
-      v_lo = (rok && k0 + 32 * j < ld_bkmax) ? base + row0 : 0xffffffffu;
-      v_hi = (rok && k0 + 64 + 32 * j < ld_bkmax) ? base + row0 + 64u * (uint32_t)ld_ldb : 0xffffffffu;
+    if (is_b ? B_TR : A_TR) {
+      const uint32_t ld = (uint32_t)(is_b ? ld_ldb : ld_lda);
+      const uint32_t row0 = (uint32_t)k0 * ld;  // k * pitch < 2^32 is checked when the table is planned
+      v_lo = (rok && k0 + 32 * j < ld_trkmax) ? base + row0 : 0xffffffffu;
+      v_hi = (rok && k0 + 64 + 32 * j < ld_trkmax) ? base + row0 + 64u * ld : 0xffffffffu;
     } else {
       v_lo = (rok && k0 < ld_kmax) ? base + k0 : 0xffffffffu;
       v_hi = (rok && k0 + 64 < ld_kmax) ? base + k0 + 64 : 0xffffffffu;
@@ -419,17 +434,26 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 
   typedef int i32x2 __attribute__((ext_vector_type(2)));
   typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
-  // weight fragment j of the half-slot at `slot`: rows = weight rows in the row-major layout, else gathered
+  auto read_frag_tr = [&](i32x8& f, uint32_t a) {  // 4 x 8 contraction rows of the lane's column
+    const i32x2 t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a));
+    const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 2048));
+    const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 4096));
+    const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
+    f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
+  };
+  // weight fragment j / token fragment i of the half-slot at `slot`
   auto read_frag_b = [&](i32x8& f, const uint8_t* slot, int j) {
     if constexpr (!B_TR) {
       read_frag(f, slot + fb_off + j * 32 * HK);
     } else {
-      const uint32_t a = (uint32_t)(uintptr_t)slot + (j == 0 ? fbt_off0 : fbt_off1);
-      const i32x2 t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a));
-      const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 2048));
-      const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 4096));
-      const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
-      f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
+      read_frag_tr(f, (uint32_t)(uintptr_t)slot + (j == 0 ? fbt_off0 : fbt_off1));
+    }
+  };
+  auto read_frag_a = [&](i32x8& f, const uint8_t* slot, int i) {
+    if constexpr (!A_TR) {
+      read_frag(f, slot + fa_off + i * 32 * HK);
+    } else {
+      read_frag_tr(f, (uint32_t)(uintptr_t)slot + fat_off[i]);
     }
   };
 
@@ -444,13 +468,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   FP8GMM_WAIT_VM(kPairLoads);
   __builtin_amdgcn_s_barrier();
   {
-    const uint8_t* sa = lds + fa_off;
     read_frag_b(fb0[0], lds, 0);
     read_frag_b(fb0[1], lds, 1);
-    read_frag(fa0[0], sa);
-    read_frag(fa0[1], sa + 32 * HK);
-    read_frag(fa0[2], sa + 64 * HK);
-    read_frag(fa0[3], sa + 96 * HK);
+    read_frag_a(fa0[0], lds, 0);
+    read_frag_a(fa0[1], lds, 1);
+    read_frag_a(fa0[2], lds, 2);
+    read_frag_a(fa0[3], lds, 3);
   }
   int hs = 0;  // half-slot of the current even half-step
   // vmcnt counts loads and stores in issue order.  A barrier needs the pair before the newest one, so it
@@ -497,7 +520,6 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       }
       __builtin_amdgcn_s_barrier();
       {
-        const uint8_t* qa = lds + h1 * HS + fa_off;
         const uint8_t* qb = lds + h1 * HS;
         FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
         dma_part(free_lo, free_hi, 0);
@@ -505,13 +527,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         read_frag_b(fb1[0], qb, 0);
         read_frag_b(fb1[1], qb, 1);
         FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_MF0(1, 1); FP8GMM_SB();
-        read_frag(fa1[0], qa);
-        read_frag(fa1[1], qa + 32 * HK);
+        read_frag_a(fa1[0], qb, 0);
+        read_frag_a(fa1[1], qb, 1);
         FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
         dma_part(free_lo, free_hi, 1);
         FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
-        read_frag(fa1[2], qa + 64 * HK);
-        read_frag(fa1[3], qa + 96 * HK);
+        read_frag_a(fa1[2], qb, 2);
+        read_frag_a(fa1[3], qb, 3);
         FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_MF0(3, 1); FP8GMM_SB();
       }
       // ---- odd half-step: fragments in fa1 / fb1.  Half-step + 2 sits in the low half of the pair whose
@@ -525,7 +547,6 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       }
       __builtin_amdgcn_s_barrier();
       {
-        const uint8_t* qa = lds + h2 * HS + fa_off;
         const uint8_t* qb = lds + h2 * HS;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
         dma_part(free_lo, free_hi, 2);
@@ -533,14 +554,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         read_frag_b(fb0[0], qb, 0);
         read_frag_b(fb0[1], qb, 1);
         FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_MF1(1, 1); FP8GMM_SB();
-        read_frag(fa0[0], qa);
-        read_frag(fa0[1], qa + 32 * HK);
+        read_frag_a(fa0[0], qb, 0);
+        read_frag_a(fa0[1], qb, 1);
         FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
         dma_part(free_lo, free_hi, 3);
         dma_advance();
         FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
-        read_frag(fa0[2], qa + 64 * HK);
-        read_frag(fa0[3], qa + 96 * HK);
+        read_frag_a(fa0[2], qb, 2);
+        read_frag_a(fa0[3], qb, 3);
         FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1); FP8GMM_SB();
       }
       hs = h2;
@@ -636,13 +657,13 @@ bool stream_k_allowed() {
 
 std::atomic<bool> g_clock_probe_on{false};
 
-template <int A_FMT, int B_FMT, bool PROBE, bool B_TR>
+template <int A_FMT, int B_FMT, bool PROBE, bool A_TR, bool B_TR>
 int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
                    hipStream_t stream) {
   static int num_cu = 0;
   static bool attr_set = false;
   const size_t lds_bytes = (size_t)RING * HS;
-  auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE, B_TR>;
+  auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE, A_TR, B_TR>;
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
@@ -679,12 +700,14 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles,
   return FP8GMM_OK;
 }
 
-template <int A_FMT, int B_FMT, bool B_TR>
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
 int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
            hipStream_t stream) {
-  if (g_clock_probe_on.load(std::memory_order_relaxed))
-    return launch_variant<A_FMT, B_FMT, true, B_TR>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
-  return launch_variant<A_FMT, B_FMT, false, B_TR>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
+  if constexpr (!A_TR && !B_TR) {  // the measurement build exists for the row-major layout only
+    if (g_clock_probe_on.load(std::memory_order_relaxed))
+      return launch_variant<A_FMT, B_FMT, true, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
+  }
+  return launch_variant<A_FMT, B_FMT, false, A_TR, B_TR>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
 }
 
 }  // namespace
@@ -710,28 +733,30 @@ int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles
 }
 
 int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layout, int* total_tiles) {
-  if (n < 0 || (layout & ~FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (n < 0 || (layout & ~(FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR))) return FP8GMM_ERR_BAD_ARGUMENT;
+  const bool a_kmajor = (layout & FP8GMM_GEMM_A_KMAJOR) != 0;
   const bool b_kmajor = (layout & FP8GMM_GEMM_B_KMAJOR) != 0;
+  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;  // not a combination the path uses
   if (total_tiles == nullptr || (n > 0 && probs == nullptr)) return FP8GMM_ERR_NULL_POINTER;
   int64_t tiles = 0, cost = 0;
   for (int i = 0; i < n; ++i) {
     fp8gmm_gemm_problem& p = probs[i];
     if (p.m < 0 || p.n < 0 || p.k < 0) return FP8GMM_ERR_BAD_SHAPE;
-    if (p.lda < p.k || p.ldb < (b_kmajor ? p.n : p.k) || p.ldc < p.n) return FP8GMM_ERR_BAD_SHAPE;
+    if (p.lda < (a_kmajor ? p.m : p.k) || p.ldb < (b_kmajor ? p.n : p.k) || p.ldc < p.n) return FP8GMM_ERR_BAD_SHAPE;
     const bool has_work = p.m > 0 && p.n > 0;
     if (has_work) {
       if (p.c == nullptr) return FP8GMM_ERR_NULL_POINTER;
       if (p.k > 0) {  // with k == 0 the operands are never read
         if (p.a == nullptr || p.b == nullptr) return FP8GMM_ERR_NULL_POINTER;
-        if ((p.k & 15) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
+        // a row-major operand is fetched in 16-byte pieces along k, a contraction-major one along its rows
+        if ((!(a_kmajor && b_kmajor) && (p.k & 15)) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
+        if ((a_kmajor && (p.m & 15)) || (b_kmajor && (p.n & 15))) return FP8GMM_ERR_ALIGNMENT;
         if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
           return FP8GMM_ERR_ALIGNMENT;
         // the kernel addresses each operand through a buffer descriptor with 32-bit byte offsets
-        if ((uint64_t)p.m * (uint64_t)p.lda > 0xffffffffull ||
+        if ((uint64_t)(a_kmajor ? p.k : p.m) * (uint64_t)p.lda > 0xffffffffull ||
             (uint64_t)(b_kmajor ? p.k : p.n) * (uint64_t)p.ldb > 0xffffffffull)
           return FP8GMM_ERR_BAD_SHAPE;
-        // a contraction-major b is fetched in 16-byte pieces along n
-        if (b_kmajor && (p.n & 15)) return FP8GMM_ERR_ALIGNMENT;
       }
     }
     const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;
@@ -751,8 +776,10 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
                         int out_kind, int epilogue, void* stream) {
   if (n < 0 || total_tiles < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_kind != FP8GMM_OUT_BF16 && out_kind != FP8GMM_E4M3 && out_kind != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
-  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
+  const bool a_kmajor = (epilogue & FP8GMM_GEMM_A_KMAJOR) != 0;
   const bool b_kmajor = (epilogue & FP8GMM_GEMM_B_KMAJOR) != 0;
+  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;
   epilogue &= FP8GMM_EPI_GELU;
   if ((a_fmt != FP8GMM_E4M3 && a_fmt != FP8GMM_E5M2) || (b_fmt != FP8GMM_E4M3 && b_fmt != FP8GMM_E5M2))
     return FP8GMM_ERR_BAD_FORMAT;
@@ -760,17 +787,22 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
   if (n == 0 || total_tiles == 0) return FP8GMM_OK;
   if (probs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (b_kmajor) {  // the data-gradient form: b is a forward weight, always e4m3
+  if (b_kmajor) {  // the gradient forms: b is a forward tensor (weight or activation), always e4m3
     if (b_fmt != FP8GMM_E4M3) return FP8GMM_ERR_BAD_FORMAT;
+    if (a_kmajor) {
+      if (a_fmt == FP8GMM_E4M3)
+        return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, true, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+      return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, true, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+    }
     if (a_fmt == FP8GMM_E4M3)
-      return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+      return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, false, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, false, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
   }
   if (a_fmt == FP8GMM_E4M3 && b_fmt == FP8GMM_E4M3)
-    return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+    return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
   if (a_fmt == FP8GMM_E5M2 && b_fmt == FP8GMM_E4M3)
-    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-  return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E5M2, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+  return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E5M2, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
 }
 
 }  // extern "C"

@@ -3,13 +3,16 @@
 Same surface and data flow as the reference's ``fp8_gmm/grouped_linear.py``
 (``_GroupedLinear`` :11-183, ``GroupedLinear`` :186-214):
 
-forward   one multi-tensor cast(+transpose) launch over the E activation slices and
-          the E weights (e4m3 under HYBRID), then one grouped GEMM
+forward   one multi-tensor cast launch over the E activation slices and the E weights
+          (e4m3 under HYBRID), then one grouped GEMM
           ``out[rows_i] = x_fp8[rows_i] . w_fp8[i]^T * (x_scale_inv_i * w_scale_inv_i)``.
-backward  one cast(+transpose) launch over the E slices of grad_out (e5m2), a grouped
-          dgrad GEMM against the transposed weights, and a grouped wgrad GEMM
-          ``dW[i] = dY_i^T[N, Mpad_i] . X_i^T[K, Mpad_i]^T`` whose contraction runs over
-          the expert's tokens padded to a multiple of 16 with zeros.
+backward  one cast launch over the E slices of grad_out (e5m2), a grouped dgrad GEMM
+          ``dX[rows_i] = dY_i . W_i`` and a grouped wgrad GEMM ``dW[i] = dY_i^T . X_i``.
+          In the reference's layout (``reference_layout=True``) the casts also write
+          transposed copies - the weights as ``[E, K, N]``, activations and gradients as
+          ``[features, Mpad_i]`` with the expert's rows padded to a multiple with zeros -
+          and both gradient GEMMs take those; by default they read the row-major fp8
+          tensors in place.
 
 Differences from the reference: experts with zero tokens are allowed (their weight
 gradient is zero), wgrad is a single launch instead of a per-expert loop, and the
@@ -108,8 +111,14 @@ class _GroupedLinear(torch.autograd.Function):
         have them, the cache of fp8 weights and whether this pass refreshes it."""
         wgrad_needed = is_grad_enabled and weight.requires_grad
         dgrad_needed = is_grad_enabled and input.requires_grad
+        # By default the gradient GEMMs read the row-major fp8 tensors in place; the reference's layout
+        # (transposed fp8 weights, padded transposed activations and gradients) is cast only on request, or when
+        # a feature count is not a multiple of 16 (the in-place GEMMs fetch 16-byte pieces along the features).
+        reference_layout = bool(fp8_meta.get("reference_layout", False)) or weight.size(1) % 16 != 0 \
+            or weight.size(2) % 16 != 0
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
-            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed,
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes,
+            need_padding=wgrad_needed and reference_layout,
             pad_multiple=fp8_meta.get("pad_multiple", PAD_MULTIPLE),
         )
         if cumsums[-1] != input.size(0):
@@ -126,7 +135,7 @@ class _GroupedLinear(torch.autograd.Function):
         input_t_fp8 = None
         x_scales = meta.get_meta_pointers(Fp8TensorType.kInputGroup1, MetaTensorType.kScale)
         x_amaxes = meta.get_meta_pointers(Fp8TensorType.kInputGroup1, MetaTensorType.kAmax)
-        if wgrad_needed:
+        if wgrad_needed and reference_layout:
             input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums,
                                                       fp8_dtype, dev)
             for lst, item in zip(with_t, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_t_views,
@@ -139,10 +148,8 @@ class _GroupedLinear(torch.autograd.Function):
 
         w_scales = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kScale)
         w_amaxes = meta.get_meta_pointers(Fp8TensorType.kWeightGroup1, MetaTensorType.kAmax)
-        # the data-gradient GEMM reads the row-major fp8 weights in place unless the reference's layout is asked for
-        transposed_weights = bool(fp8_meta.get("transposed_weights", False))
         weight_fp8, weight_t_fp8 = stage_weight_cast(
-            weight, fp8_dtype, dgrad_needed and transposed_weights, is_grad_enabled and transposed_weights,
+            weight, fp8_dtype, dgrad_needed and reference_layout, is_grad_enabled and reference_layout,
             weight_cache, update_fp8_weights, w_scales, w_amaxes, plain, with_t)
 
         if plain[0]:
@@ -160,9 +167,11 @@ class _GroupedLinear(torch.autograd.Function):
         )
 
         if is_grad_enabled:
-            ctx.save_for_backward(input_t_fp8, weight_t_fp8 if transposed_weights else
-                                  (weight_fp8 if dgrad_needed else None))
-            ctx.transposed_weights = transposed_weights
+            if reference_layout:
+                ctx.save_for_backward(input_t_fp8, weight_t_fp8)
+            else:
+                ctx.save_for_backward(input_fp8 if wgrad_needed else None, weight_fp8 if dgrad_needed else None)
+            ctx.reference_layout = reference_layout
             ctx.group_sizes = group_sizes
             meta.set_forward_scale_inv_cloned()
             ctx.meta = meta
@@ -179,7 +188,7 @@ class _GroupedLinear(torch.autograd.Function):
 
     @staticmethod
     def _backward(ctx, grad_out):
-        input_t_fp8, weight_for_dgrad = ctx.saved_tensors
+        input_for_wgrad, weight_for_dgrad = ctx.saved_tensors   # transposed copies in the reference's layout
         meta = ctx.meta
         cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
         grad_dtype = to_torch_dtype(get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=False))
@@ -191,7 +200,7 @@ class _GroupedLinear(torch.autograd.Function):
         g_scale_invs = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScaleInv)
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
         g_t_views = None
-        if ctx.weight_requires_grad:
+        if ctx.weight_requires_grad and ctx.reference_layout:
             _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
                                             dev)
             multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
@@ -204,17 +213,19 @@ class _GroupedLinear(torch.autograd.Function):
             grad_input = fp8_gmm(
                 grad_out_fp8, weight_for_dgrad, ctx.group_sizes, g_scale_invs,
                 meta.get_meta_pointers(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
-                backward=True, cutlass=ctx.cutlass, b_transposed=not ctx.transposed_weights,
+                backward=True, cutlass=ctx.cutlass, b_transposed=not ctx.reference_layout,
             )
 
         grad_weight = None
         if ctx.weight_requires_grad:
             grad_weight = torch.empty(ctx.weight_shape, dtype=torch.bfloat16, device=dev)
-            x_t_views = transposed_views(input_t_fp8, padded_cumsums if padded else cumsums)
-            grouped_gemm(
-                g_t_views, x_t_views, TensorBatch.stack_of(grad_weight), g_scale_invs,
-                meta.get_meta_pointers(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv),
-            )
+            x_scale_invs = meta.get_meta_pointers(Fp8TensorType.kForwardInputGroup1, MetaTensorType.kScaleInv)
+            if ctx.reference_layout:
+                x_t_views = transposed_views(input_for_wgrad, padded_cumsums if padded else cumsums)
+                grouped_gemm(g_t_views, x_t_views, TensorBatch.stack_of(grad_weight), g_scale_invs, x_scale_invs)
+            else:  # dW[i] = dY_i^T . X_i on the row-major slices, contraction over the expert's rows
+                grouped_gemm(row_slices(grad_out_fp8, cumsums), row_slices(input_for_wgrad, cumsums),
+                             TensorBatch.stack_of(grad_weight), g_scale_invs, x_scale_invs, transposed=True)
         return grad_input, grad_weight, None, None, None, None, None, None
 
 
@@ -223,18 +234,19 @@ class GroupedLinear(Fp8GroupedModuleBase):
 
     ``forward(input[tokens, in_features], group_sizes[E])`` where ``group_sizes`` is a CPU
     int64 tensor (or list) of rows per expert, in order; returns ``[tokens, out_features]`` bf16.
-    ``transposed_weights=True`` keeps the reference's buffers: a transposed fp8 copy ``[E, K, N]`` of the weights is
-    cast in the forward pass for the data-gradient GEMM; by default that GEMM reads the row-major copy in place
-    (same results, a quarter less cast traffic).
+    ``reference_layout=True`` keeps the reference's buffers: transposed fp8 weights ``[E, K, N]`` for the
+    data-gradient GEMM and zero-padded transposed fp8 activations / gradients for the weight-gradient GEMM.  By
+    default those GEMMs read the row-major fp8 tensors in place and none of the copies is cast: same results bit
+    for bit, less memory traffic, no padding.
     ``is_first_microbatch``: None casts the weights to fp8 on every pass; True casts them into buffers the
     module keeps; False reuses those buffers (gradient accumulation over micro-batches of one optimizer step).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False,
-                 pad_multiple=MODULE_PAD_MULTIPLE, transposed_weights=False):
+                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False):
         super().__init__()
         self.fp8_meta["pad_multiple"] = pad_multiple
-        self.fp8_meta["transposed_weights"] = transposed_weights
+        self.fp8_meta["reference_layout"] = reference_layout
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.in_features = in_features
         self.out_features = out_features
@@ -255,7 +267,7 @@ class GroupedLinear(Fp8GroupedModuleBase):
         if is_first_microbatch is None:
             return [None, None]
         dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
-        return list(self._weight_cache.buffers(self.weight_tensor, dtype, self.fp8_meta["transposed_weights"]))
+        return list(self._weight_cache.buffers(self.weight_tensor, dtype, self.fp8_meta["reference_layout"]))
 
     def forward(self, input, group_sizes, is_first_microbatch=None):
         with self.prepare_forward(input, is_first_microbatch, self.num_groups):

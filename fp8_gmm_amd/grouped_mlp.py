@@ -4,14 +4,18 @@ Same surface and data flow as the reference's ``fp8_gmm/grouped_mlp.py``
 (``_GroupedMlp`` :18-325, ``GroupedMlp`` :328-366).  ``GroupedMlp(in=H, out=F)`` owns
 ``fc1_weight [E, F, H]`` and ``fc2_weight [E, H, F]``.
 
-forward   one cast(+transpose) launch over the E activation slices and 2E weights;
+forward   one cast launch over the E activation slices and 2E weights;
           fc1 grouped GEMM with the GELU-aux epilogue (writes bf16 pre-GELU values and
           the e4m3 GELU output scaled by the InputGroup2 scale, recording its amax);
           fc2 grouped GEMM to bf16.
-backward  cast(+transpose) of grad_out to e5m2 and pad-transpose of the saved GELU
-          output; fc2 wgrad; fc2 dgrad; fused (dgelu * grad) cast(+transpose) under the
-          GradOutputGroup2 scale; fc1 dgrad (optionally all-reduced over a tensor-parallel
-          group, overlapped with fc1 wgrad); fc1 wgrad.
+backward  cast of grad_out to e5m2; fc2 wgrad; fc2 dgrad; fused (dgelu * grad) cast under
+          the GradOutputGroup2 scale; fc1 dgrad (optionally all-reduced over a
+          tensor-parallel group, overlapped with fc1 wgrad); fc1 wgrad.
+
+In the reference's layout (``reference_layout=True``) every cast also writes the transposed
+copy its gradient GEMM takes (weights ``[E, K, N]``; activations, the GELU output and the
+gradients zero-padded per expert), as grouped_mlp.py:60-150,196-262 does; by default the
+gradient GEMMs read the row-major fp8 tensors in place and no such copy exists.
 
 Experts with zero tokens are allowed; each wgrad is one grouped launch.
 """
@@ -60,8 +64,12 @@ class _GroupedMlp(torch.autograd.Function):
         wgrad_needed = is_grad_enabled and weight_requires_grad
         # fc2's transposed weights feed the fc2 dgrad, which both the input and the fc1 weight gradients need
         dgrad_needed = is_grad_enabled and (input_requires_grad or weight_requires_grad)
+        # in-place gradient GEMMs unless the reference's layout is asked for (see GroupedLinear)
+        reference_layout = bool(fp8_meta.get("reference_layout", False)) or fc1_weight.size(1) % 16 != 0 \
+            or fc1_weight.size(2) % 16 != 0
         num_groups, padded, cumsums, padded_cumsums = cumsum_group_sizes(
-            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes, need_padding=wgrad_needed,
+            group_sizes.tolist() if isinstance(group_sizes, torch.Tensor) else group_sizes,
+            need_padding=wgrad_needed and reference_layout,
             pad_multiple=fp8_meta.get("pad_multiple", PAD_MULTIPLE),
         )
         if cumsums[-1] != input.size(0):
@@ -78,7 +86,7 @@ class _GroupedMlp(torch.autograd.Function):
         input_t_fp8 = None
         x_scales = meta.get_meta_pointers(_T.kInputGroup1, _M.kScale)
         x_amaxes = meta.get_meta_pointers(_T.kInputGroup1, _M.kAmax)
-        if wgrad_needed:
+        if wgrad_needed and reference_layout:
             input_t_fp8, x_t_views = alloc_transposed(input.size(1), padded, cumsums, padded_cumsums, fp8_dtype, dev)
             for lst, item in zip(with_t, (row_slices(input, cumsums), row_slices(input_fp8, cumsums), x_t_views,
                                           x_scales, x_amaxes)):
@@ -88,8 +96,7 @@ class _GroupedMlp(torch.autograd.Function):
                                          x_amaxes)):
                 lst.append(item)
 
-        transposed_weights = bool(fp8_meta.get("transposed_weights", False))
-        need_t, cache_t = dgrad_needed and transposed_weights, is_grad_enabled and transposed_weights
+        need_t, cache_t = dgrad_needed and reference_layout, is_grad_enabled and reference_layout
         fc1_weight_fp8, fc1_weight_t_fp8 = stage_weight_cast(
             fc1_weight, fp8_dtype, need_t, cache_t, weight_caches[0], update_fp8_weights,
             meta.get_meta_pointers(_T.kWeightGroup1, _M.kScale), meta.get_meta_pointers(_T.kWeightGroup1, _M.kAmax),
@@ -130,13 +137,14 @@ class _GroupedMlp(torch.autograd.Function):
             gelu_out_fp8 = None
 
         if is_grad_enabled:
-            if transposed_weights:
-                w1_dgrad, w2_dgrad = fc1_weight_t_fp8, fc2_weight_t_fp8
-            else:  # the data-gradient GEMMs read the row-major copies in place
+            if reference_layout:
+                x_wgrad, w1_dgrad, w2_dgrad = input_t_fp8, fc1_weight_t_fp8, fc2_weight_t_fp8
+            else:  # the gradient GEMMs read the row-major copies in place
+                x_wgrad = input_fp8 if wgrad_needed else None
                 w1_dgrad = fc1_weight_fp8 if (dgrad_needed and input_requires_grad) else None
                 w2_dgrad = fc2_weight_fp8 if dgrad_needed else None
-            ctx.save_for_backward(input_t_fp8, w1_dgrad, w2_dgrad, pre_gelu_out, gelu_out_fp8)
-            ctx.transposed_weights = transposed_weights
+            ctx.save_for_backward(x_wgrad, w1_dgrad, w2_dgrad, pre_gelu_out, gelu_out_fp8)
+            ctx.reference_layout = reference_layout
             ctx.group_sizes = group_sizes
             meta.set_forward_scale_inv_cloned()
             ctx.meta = meta
@@ -157,8 +165,9 @@ class _GroupedMlp(torch.autograd.Function):
 
     @staticmethod
     def _backward(ctx, grad_out):
-        input_t_fp8, fc1_weight_dgrad, fc2_weight_dgrad, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
-        b_transposed = not ctx.transposed_weights
+        input_for_wgrad, fc1_weight_dgrad, fc2_weight_dgrad, pre_gelu_out, gelu_out_fp8 = ctx.saved_tensors
+        in_place = not ctx.reference_layout
+        b_transposed = in_place
         meta = ctx.meta
         cumsums, padded_cumsums, padded = ctx.cumsums, ctx.padded_cumsums, ctx.padded
         t_bounds = padded_cumsums if padded else cumsums
@@ -173,21 +182,25 @@ class _GroupedMlp(torch.autograd.Function):
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
 
         grad_fc2_weight = None
-        if wgrad:
+        if wgrad and not in_place:
             _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype, dev)
             _, gelu_t_views = alloc_transposed(gelu_out_fp8.size(1), padded, cumsums, padded_cumsums,
                                                gelu_out_fp8.dtype, dev)
             multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
                                  g1_scales, g1_amaxes)
             multi_transpose(row_slices(gelu_out_fp8, cumsums), gelu_t_views)
-            # fc2 wgrad: dW2[i][H, F] = dY_i^T[H, Mpad] . gelu_i^T[F, Mpad]^T
-            grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev)
-            grouped_gemm(
-                g_t_views, gelu_t_views, TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs,
-                meta.get_meta_pointers(_T.kForwardInputGroup2, _M.kScaleInv),
-            )
         else:
             multi_quantize(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g1_scales, g1_amaxes)
+        if wgrad:
+            # fc2 wgrad: dW2[i][H, F] = dY_i^T . gelu_i (reference layout: dY_i^T[H, Mpad] . gelu_i^T[F, Mpad]^T)
+            grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev)
+            gelu_scale_invs = meta.get_meta_pointers(_T.kForwardInputGroup2, _M.kScaleInv)
+            if in_place:
+                grouped_gemm(row_slices(grad_out_fp8, cumsums), row_slices(gelu_out_fp8, cumsums),
+                             TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs, gelu_scale_invs, transposed=True)
+            else:
+                grouped_gemm(g_t_views, gelu_t_views, TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs,
+                             gelu_scale_invs)
 
         # fc2 dgrad: d(gelu_out)[tokens, F]
         grad_gelu_out = fp8_gmm(
@@ -196,12 +209,13 @@ class _GroupedMlp(torch.autograd.Function):
             backward=True, cutlass=False, b_transposed=b_transposed,
         )
 
-        # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8; the padded transpose only feeds fc1 wgrad
-        # (the reference always transposes and notes the missing cast-only kernel, grouped_mlp.py:252-253)
+        # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8; the padded transpose only feeds fc1 wgrad in
+        # the reference's layout (the reference always transposes and notes the missing cast-only kernel,
+        # grouped_mlp.py:252-253)
         grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
         g2_scales = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale)
         g2_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax)
-        if wgrad:
+        if wgrad and not in_place:
             _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
                                                    dev)
             multi_cast_transpose_dgelu(
@@ -231,10 +245,13 @@ class _GroupedMlp(torch.autograd.Function):
         if wgrad:
             # fc1 wgrad: dW1[i][F, H] = d(pre)_i^T[F, Mpad] . X_i^T[H, Mpad]^T
             grad_fc1_weight = torch.empty(ctx.fc1_weight_shape, dtype=torch.bfloat16, device=dev)
-            grouped_gemm(
-                grad_pre_t_views, transposed_views(input_t_fp8, t_bounds), TensorBatch.stack_of(grad_fc1_weight),
-                g2_scale_invs, meta.get_meta_pointers(_T.kForwardInputGroup1, _M.kScaleInv),
-            )
+            x_scale_invs = meta.get_meta_pointers(_T.kForwardInputGroup1, _M.kScaleInv)
+            if in_place:
+                grouped_gemm(row_slices(grad_pre_fp8, cumsums), row_slices(input_for_wgrad, cumsums),
+                             TensorBatch.stack_of(grad_fc1_weight), g2_scale_invs, x_scale_invs, transposed=True)
+            else:
+                grouped_gemm(grad_pre_t_views, transposed_views(input_for_wgrad, t_bounds),
+                             TensorBatch.stack_of(grad_fc1_weight), g2_scale_invs, x_scale_invs)
         if handle is not None:
             handle.wait()
         return grad_input, grad_fc1_weight, grad_fc2_weight, None, None, None, None, None, None, None
@@ -244,15 +261,15 @@ class GroupedMlp(Fp8GroupedModuleBase):
     """E expert MLPs ``in_features -> out_features -> in_features`` with tanh-GELU, no biases.
 
     ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None, is_first_microbatch=None)``;
-    ``transposed_weights`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
+    ``reference_layout`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
     the module's fp8 weight buffers).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
-                 pad_multiple=MODULE_PAD_MULTIPLE, transposed_weights=False):
+                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False):
         super().__init__()
         self.fp8_meta["pad_multiple"] = pad_multiple
-        self.fp8_meta["transposed_weights"] = transposed_weights
+        self.fp8_meta["reference_layout"] = reference_layout
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.num_groups = num_groups
         self.fc1_weight = torch.nn.Parameter(
@@ -272,7 +289,7 @@ class GroupedMlp(Fp8GroupedModuleBase):
         if is_first_microbatch is None:
             return [None, None, None, None]
         dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
-        tw = self.fp8_meta["transposed_weights"]
+        tw = self.fp8_meta["reference_layout"]
         return list(self._weight_caches[0].buffers(self.fc1_weight, dtype, tw)) + \
             list(self._weight_caches[1].buffers(self.fc2_weight, dtype, tw))
 

@@ -138,6 +138,12 @@ typedef struct fp8gmm_gemm_problem {
  * (fp8_gmm/grouped_linear.py:69-74,163).  b must be e4m3, n a multiple of 16, k * ldb < 2^32.  Plan such tables
  * with fp8gmm_plan_grouped_gemm_layout(..., FP8GMM_GEMM_B_KMAJOR, ...). */
 #define FP8GMM_GEMM_B_KMAJOR 2
+/* a is stored contraction-major as well: a[k, m] with m contiguous and lda >= m, i.e.
+ * c[m, n] = epilogue( a[k, m]^T . b[k, n] ): the weight-gradient GEMM dW[N, K] = dY[M, N]^T . X[M, K] on the
+ * row-major gradient and activation, without the padded transposed copies the reference casts for it
+ * (fp8_gmm/grouped_linear.py:36-52,142-150).  Only together with FP8GMM_GEMM_B_KMAJOR; m and n multiples of
+ * 16, k arbitrary (rows past k contribute zeros), k * lda < 2^32. */
+#define FP8GMM_GEMM_A_KMAJOR 4
 
 /* ---- library info ------------------------------------------------------------------------- */
 int fp8gmm_version(void);
@@ -156,7 +162,8 @@ int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* tota
 /* Validates `probs[0..n)`, fills tile_begin / cost_begin, returns the tile count in *total_tiles.
  * Replaces the host half of CutlassFp8GroupedGemm (csrc/fp8_gmm.cu:82-135). */
 int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles);
-/* The same for a launch with layout flags (0 or FP8GMM_GEMM_B_KMAJOR): only the checks on b differ. */
+/* The same for a launch with layout flags (0, FP8GMM_GEMM_B_KMAJOR, or both KMAJOR flags): only the checks on
+ * the operands differ. */
 int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layout, int* total_tiles);
 
 /* ---- launches (descs_dev / probs_dev: DEVICE copies of planned tables) ------------------- */

@@ -506,3 +506,50 @@ def test_contraction_major_b_gives_the_same_bits(dev, a_dtype):
     with pytest.raises(RuntimeError):   # n must be a multiple of 16 in this layout
         backend.fp8_gmm(torch.zeros(4, 16, device=dev).to(a_dtype), torch.zeros(1, 16, 8, device=dev).to(E4M3),
                         [4], None, None, b_transposed=True)
+
+
+@pytest.mark.parametrize("a_dtype", [E4M3, E5M2])
+def test_contraction_major_a_and_b_give_the_weight_gradient(dev, a_dtype):
+    """grouped_gemm(..., transposed=True): c_i = a_i^T . b_i on row-major [rows_i, m] / [rows_i, n] slices, rows_i
+    ragged and not a multiple of anything.  Must equal, bit for bit, the row-major path on explicitly transposed and
+    zero-padded copies (the reference's data flow), and the fp32 matmul on exact data."""
+    backend = _backend()
+    g = torch.Generator(device=dev).manual_seed(123)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    for rows, m, n in [([137, 401, 0, 59, 403], 512, 256), ([1, 2, 700], 16, 48), ([1439, 909, 669], 1408, 2048),
+                       ([300], 272, 1040), ([4096], 256, 256)]:
+        e, total = len(rows), sum(rows)
+        dy = torch.randn(total, m, generator=g, device=dev).to(a_dtype)
+        x = torch.randn(total, n, generator=g, device=dev).to(E4M3)
+        bounds = [0]
+        for r in rows:
+            bounds.append(bounds[-1] + r)
+        a_list = [dy[bounds[i]: bounds[i + 1]] for i in range(e)]
+        b_list = [x[bounds[i]: bounds[i + 1]] for i in range(e)]
+        sa = torch.rand(e, generator=g, device=dev) + 0.5
+        sb = torch.rand(e, generator=g, device=dev) + 0.5
+        got = torch.full((e, m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        backend.grouped_gemm(a_list, b_list, list(got.unbind(0)), sa, sb, transposed=True)
+        # the reference's flow: transposed copies padded with zeros to a multiple of 16
+        a_t, b_t = [], []
+        for i, r in enumerate(rows):
+            rp = (r + 15) // 16 * 16
+            at = torch.zeros(m, rp, device=dev).to(a_dtype)
+            bt = torch.zeros(n, rp, device=dev).to(E4M3)
+            at[:, :r] = a_list[i].t()
+            bt[:, :r] = b_list[i].t()
+            a_t.append(at)
+            b_t.append(bt)
+        want = torch.empty(e, m, n, dtype=torch.bfloat16, device=dev)
+        backend.grouped_gemm(a_t, b_t, list(want.unbind(0)), sa, sb)
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"rows {rows} m {m} n {n}"
+        # exact data against fp32
+        dy2 = vals[torch.randint(0, 8, (total, m), generator=g, device=dev)].to(a_dtype)
+        x2 = vals[torch.randint(0, 8, (total, n), generator=g, device=dev)].to(E4M3)
+        ones = torch.ones(e, device=dev)
+        backend.grouped_gemm([dy2[bounds[i]: bounds[i + 1]] for i in range(e)],
+                             [x2[bounds[i]: bounds[i + 1]] for i in range(e)], list(got.unbind(0)), ones, ones,
+                             transposed=True)
+        for i in range(e):
+            ref32 = (dy2[bounds[i]: bounds[i + 1]].float().t() @ x2[bounds[i]: bounds[i + 1]].float()).to(torch.bfloat16)
+            assert torch.equal(got[i].view(torch.int16), ref32.view(torch.int16)), f"rows {rows} expert {i}"

@@ -222,10 +222,10 @@ def test_pad_multiple_does_not_change_results(dev, kind):
     results = []
     for pad in (16, 128):
         if kind == "linear":
-            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad)
+            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad, reference_layout=True)
             mod.weight_tensor.data.copy_(w1)
         else:
-            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad)
+            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, pad_multiple=pad, reference_layout=True)
             mod.fc1_weight.data.copy_(w1)
             mod.fc2_weight.data.copy_(w2)
         xd = x.clone().requires_grad_()
@@ -237,8 +237,8 @@ def test_pad_multiple_does_not_change_results(dev, kind):
         assert torch.equal(a.view(torch.int16), b.view(torch.int16))
 
 
-@pytest.mark.parametrize("transposed_weights", [False, True], ids=["in-place-dgrad", "reference-layout"])
-def test_grouped_linear_reuses_cached_fp8_weights(dev, transposed_weights):
+@pytest.mark.parametrize("reference_layout", [False, True], ids=["in-place", "reference-layout"])
+def test_grouped_linear_reuses_cached_fp8_weights(dev, reference_layout):
     """is_first_microbatch: True casts the weights into the module's buffers, False reuses them.  The weights
     are CHANGED between the two micro-batches, so only a pass that really reuses the cached bytes (and their
     scale_inv) can match the oracle, which is handed the first pass's fp8 weights; a later True picks up the
@@ -249,7 +249,7 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev, transposed_weights):
     g = gen(3001)
     w = randn_bf16((e, n, k), g, 0.02)
     w_changed = (w.float() * 1.5 + 0.01).to(torch.bfloat16)
-    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev, transposed_weights=transposed_weights)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev, reference_layout=reference_layout)
     fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
     fwd, bwd = orc.Meta(3 * e, hist), orc.Meta(2 * e, hist)
     weight_slots = [3 * i + 1 for i in range(e)]
@@ -279,7 +279,7 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev, transposed_weights):
             assert not gm["scaling_fwd"].amax_history[0][weight_slots].any()
         w_fp8, w_t_fp8 = module.get_fp8_weights_scratchpad(first)
         assert torch.equal(w_fp8.cpu().view(torch.uint8), cached["w_fp8"].view(torch.uint8)), f"step {step}"
-        if transposed_weights:
+        if reference_layout:
             assert torch.equal(w_t_fp8.cpu().view(torch.uint8), cached["w_t_fp8"].view(torch.uint8)), f"step {step}"
         else:
             assert w_t_fp8 is None   # the data-gradient GEMM reads w_fp8 in place
@@ -291,7 +291,7 @@ def test_grouped_linear_reuses_cached_fp8_weights(dev, transposed_weights):
 
 def test_cached_weights_need_a_first_microbatch(dev):
     pkg = _pkg()
-    module = pkg.GroupedLinear(64, 64, 2, torch.bfloat16, device=dev, transposed_weights=True)
+    module = pkg.GroupedLinear(64, 64, 2, torch.bfloat16, device=dev, reference_layout=True)
     x = torch.zeros(32, 64, dtype=torch.bfloat16, device=dev, requires_grad=True)
     with pytest.raises(RuntimeError, match="is_first_microbatch=False"):
         module(x, [16, 16], is_first_microbatch=False)
@@ -380,10 +380,10 @@ def test_grouped_mlp_frozen_weights_against_the_oracle(dev):
 
 
 @pytest.mark.parametrize("kind", ["linear", "mlp"])
-def test_in_place_dgrad_equals_the_reference_layout(dev, kind):
-    """By default no transposed fp8 weights are cast and the data-gradient GEMMs read the row-major copies in
-    place; with transposed_weights=True the reference's [E, K, N] copies are cast and used.  Same bits either way,
-    over three steps of delayed scaling."""
+def test_in_place_gradient_gemms_equal_the_reference_layout(dev, kind):
+    """By default no transposed fp8 copies are cast and the data- and weight-gradient GEMMs read the row-major
+    tensors in place; with reference_layout=True the reference's transposed weights [E, K, N] and padded transposed
+    activations / gradients are cast and used.  Same bits either way, over three steps of delayed scaling."""
     pkg = _pkg()
     sizes, h, f = [137, 0, 401, 59, 403], 256, 512
     e, m = len(sizes), sum(sizes)
@@ -391,9 +391,9 @@ def test_in_place_dgrad_equals_the_reference_layout(dev, kind):
     mods = []
     for tw in (False, True):
         if kind == "linear":
-            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, transposed_weights=tw)
+            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, reference_layout=tw)
         else:
-            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, transposed_weights=tw)
+            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, reference_layout=tw)
         mods.append(mod)
     mods[1].load_state_dict(mods[0].state_dict())
     out_cols = f if kind == "linear" else h
