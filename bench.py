@@ -346,6 +346,33 @@ def main():
             "ms_per_step": round(cached_ms, 4), "value": round(flops_per_step / (cached_ms * 1e-3) / 1e12, 2),
             "unit": "TFLOP/s"}}
 
+    # ... and the same step on the reference's buffers (transposed fp8 weights, padded transposed activations and
+    # gradients, written by the pad / cast / transpose kernels), which the default path no longer needs
+    if gs is not None and not args.headline_only:
+        ref_module = type(module)(hidden, ffn, experts, torch.bfloat16, device=dev, reference_layout=True)
+        ref_module.load_state_dict(module.state_dict())
+        main_module, module = module, ref_module
+        try:
+            for _ in range(3):
+                step()
+            torch.cuda.synchronize()
+            with kernel_timing() as rt:
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    step()
+                torch.cuda.synchronize()
+                ref_ms = (time.perf_counter() - t0) / args.steps * 1e3
+            ref_kernels = {name: {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
+                                  "GBps": round(d["work"] / (d["ms"] * 1e-3) / 1e9, 1)}
+                           for name, d in rt.summary().items() if name != "grouped_gemm"}
+        finally:
+            module = main_module
+        del ref_module
+        also = dict(also or {})
+        also["reference_layout"] = {"ms_per_step": round(ref_ms, 4),
+                                    "value": round(flops_per_step / (ref_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
+                                    "kernels": ref_kernels}
+
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
