@@ -780,6 +780,8 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
   const bool a_kmajor = (epilogue & FP8GMM_GEMM_A_KMAJOR) != 0;
   const bool b_kmajor = (epilogue & FP8GMM_GEMM_B_KMAJOR) != 0;
   if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;
+  // the contraction-major forms are the gradient GEMMs: b is a forward tensor (weight or activation), always e4m3
+  if (b_kmajor && b_fmt != FP8GMM_E4M3) return FP8GMM_ERR_BAD_FORMAT;
   epilogue &= FP8GMM_EPI_GELU;
   if ((a_fmt != FP8GMM_E4M3 && a_fmt != FP8GMM_E5M2) || (b_fmt != FP8GMM_E4M3 && b_fmt != FP8GMM_E5M2))
     return FP8GMM_ERR_BAD_FORMAT;
@@ -787,8 +789,7 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_t
   if (n == 0 || total_tiles == 0) return FP8GMM_OK;
   if (probs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (b_kmajor) {  // the gradient forms: b is a forward tensor (weight or activation), always e4m3
-    if (b_fmt != FP8GMM_E4M3) return FP8GMM_ERR_BAD_FORMAT;
+  if (b_kmajor) {
     if (a_kmajor) {
       if (a_fmt == FP8GMM_E4M3)
         return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, true, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);

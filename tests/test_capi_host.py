@@ -134,3 +134,39 @@ def test_launch_entry_points_validate_before_touching_the_gpu():
     assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 8, None) == -6  # unknown epilogue flag
     assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 0, None) == -1
     assert lib.fp8gmm_grouped_gemm(None, 0, 0, 0, 0, 2, 0, None) == 0
+
+
+def test_plan_grouped_gemm_layouts():
+    """Operands stored contraction-major: which pitch, alignment and size rules apply to which operand."""
+    lib = _lib.load()
+    total = ctypes.c_int(0)
+    B, A = _lib.GEMM_B_KMAJOR, _lib.GEMM_A_KMAJOR
+
+    def rc(t, layout):
+        return lib.fp8gmm_plan_grouped_gemm_layout(t.ctypes.data, len(t), layout, ctypes.byref(total))
+
+    # b[k, n]: ldb is the pitch of a k row (>= n), n must be a multiple of 16, a keeps the row-major rules
+    assert rc(_prob([100], [256], [512], ldb=256), B) == 0 and total.value == 1
+    assert rc(_prob([100], [256], [512], ldb=128), B) == -2      # pitch smaller than n
+    assert rc(_prob([100], [256], [512]), 0) == 0                # the same table row-major: ldb = k
+    assert rc(_prob([100], [264], [512], ldb=272), B) == -4      # n not a multiple of 16
+    assert rc(_prob([100], [256], [520], ldb=256), B) == -4      # a is still fetched in 16-byte pieces of k
+    assert rc(_prob([16], [65536], [65536], ldb=65536), B) == -2  # k * ldb >= 2^32
+    # a[k, m] and b[k, n]: k is a row count and may be anything; m and n multiples of 16
+    assert rc(_prob([512], [256], [137], lda=512, ldb=256), A | B) == 0
+    assert rc(_prob([512], [256], [137], lda=500, ldb=256), A | B) == -2
+    assert rc(_prob([520], [256], [137], lda=528, ldb=256), A | B) == -4
+    assert rc(_prob([512], [256], [0], lda=512, ldb=256, a=0, b=0), A | B) == 0   # an expert without rows
+    # a contraction-major a alone is not a layout the path uses; unknown bits are refused
+    assert rc(_prob([512], [256], [128], lda=512), A) == -6
+    assert rc(_prob([16], [16], [16]), 8) == -6
+    # the launch refuses the same combinations, and a contraction-major b that is not e4m3
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, A, None) == -6
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 1, 2, B, None) == -3
+    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, A | B | _lib.EPI_GELU, None) == -1   # valid flags, no table
+    t = _prob([137, 0, 401], [512, 512, 512], [300, 0, 77], lda=[137 + 7, 16, 416], ldb=512)
+    t["lda"] = [144, 16, 416]
+    assert rc(t, A | B) == -4     # m = 137 is not a multiple of 16
+    t = _prob([144, 0, 416], [512, 512, 512], [300, 0, 77], ldb=512)
+    t["lda"] = [144, 16, 416]
+    assert rc(t, A | B) == 0 and t["tile_begin"].tolist() == [0, 2, 2] and t["cost_begin"].tolist() == [0, 6, 6]
