@@ -660,25 +660,29 @@ std::atomic<bool> g_clock_probe_on{false};
 template <int A_FMT, int B_FMT, bool PROBE, bool A_TR, bool B_TR>
 int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
                    hipStream_t stream) {
-  static int num_cu = 0;
-  static bool attr_set = false;
+  // per device (a process may drive several): compute-unit count and "the kernel may use the whole LDS"
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> num_cu[kMaxDevices];
+  static std::atomic<bool> attr_set[kMaxDevices];
   const size_t lds_bytes = (size_t)RING * HS;
   auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE, A_TR, B_TR>;
-  if (!attr_set) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
+  if (!attr_set[dev].load(std::memory_order_acquire)) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds_bytes) != hipSuccess)
       return FP8GMM_ERR_LAUNCH;
-    attr_set = true;
+    attr_set[dev].store(true, std::memory_order_release);
   }
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
-  if (num_cu == 0) {
+  int cus = num_cu[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
-    num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    num_cu[dev].store(cus, std::memory_order_relaxed);
   }
   // one workgroup per CU, a multiple of 8 so that every XCD gets the same number of workgroups
-  int grid = (num_cu / kNumXcd) * kNumXcd;
+  int grid = (cus / kNumXcd) * kNumXcd;
   if (grid < kNumXcd) grid = kNumXcd;
   // tail balancing can only pay when the launch has few rounds; it needs the whole grid even for few tiles
   uint8_t* workspace = nullptr;
