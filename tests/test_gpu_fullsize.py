@@ -3,6 +3,7 @@
 The CPU oracle cannot finish these sizes in seconds, so the checks are properties that do not depend on size:
   * GEMMs on operands from {0, +-0.25 .. +-2}: every partial sum is exact in fp32, whatever the order, so the
     result must equal a plain fp32 matmul of the dequantised operands bit for bit (here torch's, on the GPU);
+    this for the forward, data-gradient and weight-gradient shapes, on transposed copies and in place;
   * a sample of rows of each result against the CPU oracle;
   * cast + transpose: the transposed copy is the transpose of the row-major copy plus zero padding, the
     row-major copy equals what the quantize kernel writes, amax equals max|x|, sampled rows equal the oracle's
@@ -192,3 +193,38 @@ def test_cast_pad_bandwidth_configuration_full_size(dev):
         for r in (0, m // 2, m - 1):
             want = ref.f32_to_fp8((ins[i][r: r + 1].float().cpu() * scales[i].item()).contiguous(), E4M3)
             assert_bytes_equal(outs[i][r: r + 1], want, f"tensor {i} row {r}")
+
+
+@pytest.mark.parametrize("k,n", [(FFN, HIDDEN), (HIDDEN, FFN)])
+def test_dgrad_in_place_full_size_exact(dev, k, n):
+    """Data-gradient shapes with the weight read in place (b[i] is [k, n]): bit-equal to the fp32 matmul."""
+    backend = _backend()
+    e = len(SIZES)
+    a = _exact_fp8((sum(SIZES), k), E5M2, dev, 3)
+    b = _exact_fp8((e, k, n), E4M3, dev, 4)
+    sa = torch.full((e,), 0.5, device=dev)
+    sb = torch.full((e,), 0.25, device=dev)
+    c = backend.fp8_gmm(a, b, torch.tensor(SIZES), sa, sb, backward=True, b_transposed=True)
+    bounds = _bounds(SIZES)
+    for i in range(e):
+        rows = slice(bounds[i], bounds[i + 1])
+        want = ((a[rows].float() @ b[i].float()) * 0.125).to(torch.bfloat16)
+        assert torch.equal(c[rows].view(torch.int16), want.view(torch.int16)), f"expert {i}"
+
+
+def test_wgrad_in_place_full_size_exact(dev):
+    """fc1 weight gradient on the row-major slices, dW[i] = dY_i^T . X_i, contraction over the expert's own
+    (unpadded, ragged) row count: bit-equal to the fp32 matmul."""
+    backend = _backend()
+    e, bounds = len(SIZES), _bounds(SIZES)
+    dy = _exact_fp8((sum(SIZES), FFN), E5M2, dev, 5)
+    x = _exact_fp8((sum(SIZES), HIDDEN), E4M3, dev, 6)
+    dw = torch.empty(e, FFN, HIDDEN, dtype=torch.bfloat16, device=dev)
+    ones = torch.ones(e, device=dev)
+    backend.grouped_gemm([dy[bounds[i]: bounds[i + 1]] for i in range(e)],
+                         [x[bounds[i]: bounds[i + 1]] for i in range(e)], list(dw.unbind(0)), ones, ones,
+                         transposed=True)
+    for i in range(e):
+        rows = slice(bounds[i], bounds[i + 1])
+        want = (dy[rows].float().t() @ x[rows].float()).to(torch.bfloat16)
+        assert torch.equal(dw[i].view(torch.int16), want.view(torch.int16)), f"expert {i}"
