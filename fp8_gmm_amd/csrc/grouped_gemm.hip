@@ -48,16 +48,18 @@
 namespace fp8gmm {
 namespace {
 
-constexpr int HK = 64;           // bytes of K per half-slot / per MFMA
-constexpr int HS = (BM + BN) * HK;  // 32768 bytes per half-slot
+constexpr int BK = kGemmTileK;    // bytes of K per main-loop step: one 128-byte line of every operand row
+constexpr int US = BM * BK;       // 32768 bytes per ring unit: the 256 rows of ONE operand for one step
 constexpr int RING = 5;
-constexpr int NTHREADS = 512;
-constexpr int WM = 128, WN = 64;  // wavefront sub-tile
+static_assert(BM == BN, "token and weight units share one size");
+constexpr int NWAVES = 4;         // one wavefront per SIMD: 256 accumulator + 256 other registers per lane
+constexpr int NTHREADS = 64 * NWAVES;
+constexpr int WM = 128, WN = 128;  // wavefront sub-tile
+constexpr int WAVES_N = BN / WN;  // wavefronts along n: 2 (x 2 along m)
 constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
-constexpr int NT = WN / 32;       // 2 MFMA tiles along n per wave
-constexpr int kPairLoads = 8;     // buffer_load ... lds instructions per wavefront per K = 128 pair
+constexpr int NT = WN / 32;       // 4 MFMA tiles along n per wave
+constexpr int kParts = US / 1024 / NWAVES;  // buffer_load ... lds instructions (1 KB each) per wavefront per unit: 8
 constexpr int kFastStores = MT * NT * 2;  // 16-byte stores per wavefront in the interior bf16 epilogue
-constexpr int kRelaxedWaits = 3;  // barriers after such an epilogue that need not wait for its stores
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -70,13 +72,30 @@ typedef unsigned u32pair __attribute__((ext_vector_type(2)));
 #define FP8GMM_DMA(lds_addr, voff, rsrc) \
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
 
+// One MFMA tile's accumulators as ordinary vector registers.  In the main kernel the 256 accumulators of a
+// lane live in the accumulation registers (the other 256 hold fragments and addresses); vector arithmetic
+// cannot read those, and left to itself the register allocator parks them in scratch memory on the way.
+// Reading them 16 at a time, where they are used, keeps the epilogue within the register file.
+template <bool FROM_ACC_REGS>
+__device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
+  if constexpr (FROM_ACC_REGS) {
+    f32x16 t;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
+    return t;
+  } else {
+    return a;
+  }
+}
+
 // Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
 // stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
+template <bool FROM_ACC_REGS>
 __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
                                               int out_kind, int epilogue) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int wave_m = wave >> 2, wave_n = wave & 3;
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, khalf = lane >> 5;
   const int M = pr.m, N = pr.n;
   bool fast = false;
@@ -99,13 +118,14 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
 #pragma unroll
           for (int gp = 0; gp < 2; ++gp) {
             const int ge = 8 * gp, go = 8 * gp + 4;  // accumulator index of g = 2 gp and g = 2 gp + 1
-            const uint32_t pe0 = pack_bf16x2(acc[i][j][ge + 0] * s, acc[i][j][ge + 1] * s);
-            const uint32_t pe1 = pack_bf16x2(acc[i][j][ge + 2] * s, acc[i][j][ge + 3] * s);
-            const uint32_t po0 = pack_bf16x2(acc[i][j][go + 0] * s, acc[i][j][go + 1] * s);
-            const uint32_t po1 = pack_bf16x2(acc[i][j][go + 2] * s, acc[i][j][go + 3] * s);
+            const uint32_t pe0 = pack_bf16x2(t[ge + 0] * s, t[ge + 1] * s);
+            const uint32_t pe1 = pack_bf16x2(t[ge + 2] * s, t[ge + 3] * s);
+            const uint32_t po0 = pack_bf16x2(t[go + 0] * s, t[go + 1] * s);
+            const uint32_t po1 = pack_bf16x2(t[go + 2] * s, t[go + 3] * s);
             const u32pair r0 = __builtin_amdgcn_permlane32_swap(pe0, po0, false, false);
             const u32pair r1 = __builtin_amdgcn_permlane32_swap(pe1, po1, false, false);
             const u32x4 o = {r0.x, r1.x, r0.y, r1.y};
@@ -125,6 +145,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -132,7 +153,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
             float v[4], r[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              v[q] = acc[i][j][g * 4 + q] * s;
+              v[q] = t[g * 4 + q] * s;
               r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
             }
             const int64_t off = (int64_t)m * ldc + n;
@@ -166,6 +187,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -173,7 +195,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
             float v[4], r[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-              v[q] = acc[i][j][g * 4 + q] * s;
+              v[q] = t[g * 4 + q] * s;
               r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
               if (n + q < N) amax = amax_step(amax, r[q]);
             }
@@ -214,18 +236,20 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
 }
 
 // Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
-// (r4 * 512 + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
+// (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
 __device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* slot) {
   float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
 #pragma unroll
   for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int j = 0; j < NT; ++j) {
+      const f32x16 t = tile_values<true>(acc[i][j]);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 v = {acc[i][j][4 * g + 0], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
         global_store(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4), v);
       }
+    }
 }
 __device__ __forceinline__ void partial_add(f32x16 (&acc)[MT][NT], const uint8_t* slot) {
   const float* base = reinterpret_cast<const float*>(slot) + threadIdx.x * 4;
@@ -289,33 +313,38 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wave_m = wave >> 2;  // 0..1
-  const int wave_n = wave & 3;   // 0..3
+  const int wave_m = wave / WAVES_N;  // 0..1
+  const int wave_n = wave % WAVES_N;  // 0..1
   const int l32 = lane & 31;
   const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
 
-  // DMA lane map: one wavefront instruction fills 16 rows x 64 B of a half-slot: lane -> row lane >> 2,
-  // slot chunk lane & 3.  With the swizzle (row >> 2) & 3 and row = 16 g + (lane >> 2) the GLOBAL chunk
-  // that has to land there is (lane & 3) ^ ((lane >> 4) & 3).
-  const int drow = lane >> 2;
-  const int dchunk = (lane & 3) ^ ((lane >> 4) & 3);
-  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 64 + 32 j + l32 (source 0)
-  const int fsw = (l32 >> 2) & 3;
-  const int fc0 = ((khalf * 2) ^ fsw) << 4;
-  const int fc1 = ((khalf * 2 + 1) ^ fsw) << 4;
-  const int fa_off = (wave_m * WM + l32) * HK;
-  const int fb_off = BM * HK + (wave_n * WN + l32) * HK;
-  // B_TR: row 32 khalf + b (+ 8 t per read), logical chunk wave_n * 4 + 2 j + g, byte 8 h; s = lane % 16 = 2 b + h
+  // DMA lane map, row-major operand: one wavefront instruction fills 8 rows x 128 B of a unit, i.e. whole
+  // cache lines: lane -> row lane >> 3 of the group, slot chunk lane & 7.  Chunk c of row r is kept at chunk
+  // c ^ ((r >> 1) & 7); for the rows of group wave + NWAVES j that is ((wave & 1) * 4 + (lane >> 4)) & 7, so the
+  // GLOBAL chunk that has to land in slot chunk lane & 7 is a per-lane constant.
+  const int drow = lane >> 3;
+  const int dchunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 128 + 32 j + l32
+  // (source 0); K half hh, lane half khalf -> chunks 4 hh + 2 khalf + {0, 1}; (row >> 1) & 7 = (l32 >> 1) & 7
+  const int fsw = (l32 >> 1) & 7;
+  int fc[2][2];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) fc[hh][q] = ((4 * hh + 2 * khalf + q) ^ fsw) << 4;
+  const int fa_off = (wave_m * WM + l32) * BK;
+  const int fb_off = (wave_n * WN + l32) * BK;
+  // contraction-major unit: 128 contraction rows x 256 B.  Fragment of K half hh: rows 64 hh + 32 khalf + b (+ 8 t
+  // per read), logical chunk wave_n * 8 + 2 j + g, byte 8 h; s = lane % 16 = 2 b + h
   const int tr_b = (lane & 15) >> 1, tr_h = lane & 1, tr_g = (lane >> 4) & 1;
-  const int fbt_row = BM * HK + (32 * khalf + tr_b) * 256 + 8 * tr_h;
-  const int fbt_off0 = fbt_row + (((wave_n * 4 + tr_g) ^ (2 * tr_b)) << 4);
-  const int fbt_off1 = fbt_row + (((wave_n * 4 + 2 + tr_g) ^ (2 * tr_b)) << 4);
-  // A_TR: logical chunk wave_m * 8 + 2 i + g of the token half of the half-slot
-  const int fat_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
+  const int tr_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
+  int fbt_off[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) fbt_off[j] = tr_row + (((wave_n * 8 + 2 * j + tr_g) ^ (2 * tr_b)) << 4);
   int fat_off[MT];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) fat_off[i] = fat_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
+  for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
 
   // ---- this workgroup's item sequence (uniform): strided tiles of its XCD's range, then its piece of
   // the range's stream-K region ----
@@ -328,13 +357,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   if (!cursor_valid(sch, wg_in_xcd, c_cp)) return;
   c_ld = c_cp;
 
-  // ---- load side: runs two pairs ahead of the compute side, possibly in the next tile ----
+  // ---- load side: runs two steps ahead of the compute side, possibly in the next tile ----
   bool ld_live = true;  // the load cursor still points at an item
   int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
   [[maybe_unused]] int ld_lda = 0, ld_ldb = 0, ld_trkmax = 0;  // contraction-major operands only
   i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
-  uint32_t a_base[2], b_base[2];
-  uint32_t ok_mask = 0;  // bit part: rows of that part exist
+  uint32_t a_base = 0, b_base = 0, a_step = 0, b_step = 0;  // part j of an operand starts at base + j * step
+  uint32_t ok_a = 0, ok_b = 0;                               // bit j: the rows / columns of part j exist
   auto load_setup = [&]() {
     while ((ld_live = cursor_valid(sch, wg_in_xcd, c_ld))) {
       const Item g = cursor_item(sch, xcd, wg_in_xcd, c_ld);
@@ -349,35 +378,41 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         rsrc_b[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pb);
         rsrc_b[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pb >> 32));
         rsrc_b[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sb > 0xffffffffull ? 0xffffffffull : sb));
-        ok_mask = 0;
+        // row-major operand: part j = rows (wave + NWAVES j) * 8 + drow of the tile.
+        // contraction-major operand: one instruction fills 4 contraction rows x 256 B: part j = rows
+        // (wave + NWAVES j) * 4 + lane / 16 of the unit, slot chunk lane % 16, which must receive global chunk
+        // p ^ 2 (row mod 8); row mod 8 is the same for every j.
+        const int krow = wave * 4 + (lane >> 4);
+        const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
+        ok_a = ok_b = 0;
+        if constexpr (!A_TR) {
+          const int ar = g.m0 + wave * 8 + drow;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int ar = g.m0 + (wave + 8 * j) * 16 + drow;
-          const int br = g.n0 + (wave + 8 * j) * 16 + drow;
-          // contraction-major operand: one instruction fills 4 contraction rows x 256 B: lane -> row
-          // (wave + 8 j) * 4 + lane / 16 of the half-slot, physical chunk lane % 16, which must receive
-          // global chunk p ^ 2 (row mod 8)
-          const int krow = (wave + 8 * j) * 4 + (lane >> 4);
-          const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
-          if constexpr (!A_TR) {
-            if (ar < pr.m) ok_mask |= 1u << j;
-            a_base[j] = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
-          } else {
-            if (g.m0 + tr_col < pr.m) ok_mask |= 1u << j;
-            a_base[j] = (uint32_t)krow * (uint32_t)pr.lda + (uint32_t)(g.m0 + tr_col);
-          }
-          if constexpr (!B_TR) {
-            if (br < pr.n) ok_mask |= 4u << j;
-            b_base[j] = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
-          } else {
-            if (g.n0 + tr_col < pr.n) ok_mask |= 4u << j;
-            b_base[j] = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)(g.n0 + tr_col);
-          }
+          for (int j = 0; j < kParts; ++j)
+            if (ar + NWAVES * 8 * j < pr.m) ok_a |= 1u << j;
+          a_base = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          a_step = NWAVES * 8 * (uint32_t)pr.lda;
+        } else {
+          if (g.m0 + tr_col < pr.m) ok_a = (1u << kParts) - 1;
+          a_base = (uint32_t)krow * (uint32_t)pr.lda + (uint32_t)(g.m0 + tr_col);
+          a_step = NWAVES * 4 * (uint32_t)pr.lda;
+          ld_lda = pr.lda;
         }
-        if constexpr (A_TR) ld_lda = pr.lda;
-        if constexpr (B_TR) ld_ldb = pr.ldb;
-        // row k0 + krow of part j of a contraction-major operand exists iff k0 + 32 j < ld_trkmax
-        if constexpr (A_TR || B_TR) ld_trkmax = pr.k - (wave * 4 + (lane >> 4));
+        if constexpr (!B_TR) {
+          const int br = g.n0 + wave * 8 + drow;
+#pragma unroll
+          for (int j = 0; j < kParts; ++j)
+            if (br + NWAVES * 8 * j < pr.n) ok_b |= 1u << j;
+          b_base = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
+          b_step = NWAVES * 8 * (uint32_t)pr.ldb;
+        } else {
+          if (g.n0 + tr_col < pr.n) ok_b = (1u << kParts) - 1;
+          b_base = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)(g.n0 + tr_col);
+          b_step = NWAVES * 4 * (uint32_t)pr.ldb;
+          ld_ldb = pr.ldb;
+        }
+        // row k0 + krow + 4 NWAVES j of a contraction-major operand exists iff k0 + 4 NWAVES j < ld_trkmax
+        if constexpr (A_TR || B_TR) ld_trkmax = pr.k - krow;
         ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
         ld_kt = g.k_begin;
         ld_nk = g.k_begin + g.nk;
@@ -386,35 +421,32 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       cursor_advance(sch, wg_in_xcd, c_ld);  // an item without K work needs no loads
     }
   };
-  // One quarter of a pair: part 0, 1 = token row groups wave, wave + 8; part 2, 3 = weight row groups.
-  // Low 64-byte half into slot_lo, high half into slot_hi.  Past the end of the stream the loads are
-  // issued all the same with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
-  auto dma_part = [&](int slot_lo, int slot_hi, int part) {
-    const int j = part & 1;
-    const bool is_b = (part >> 1) != 0;
-    const int k0 = ld_kt * 128;
-    const bool rok = ld_live && ((ok_mask >> part) & 1);
-    const uint32_t base = is_b ? b_base[j] : a_base[j];
-    uint32_t v_lo, v_hi;
-    if (is_b ? B_TR : A_TR) {
-      const uint32_t ld = (uint32_t)(is_b ? ld_ldb : ld_lda);
-      const uint32_t row0 = (uint32_t)k0 * ld;  // k * pitch < 2^32 is checked when the table is planned
-      v_lo = (rok && k0 + 32 * j < ld_trkmax) ? base + row0 : 0xffffffffu;
-      v_hi = (rok && k0 + 64 + 32 * j < ld_trkmax) ? base + row0 + 64u * ld : 0xffffffffu;
+  // One instruction of the K = 128 step the load cursor points at: part j (0..7) of the token operand into
+  // ring unit `unit`, or of the weight operand.  Past the end of the stream the loads are issued all the same
+  // with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
+  auto dma_a = [&](int unit, int j) {
+    const int k0 = ld_kt * BK;
+    const bool rok = ld_live && ((ok_a >> j) & 1);
+    uint32_t v;
+    if constexpr (A_TR) {  // k * pitch < 2^32 is checked when the table is planned
+      v = (rok && k0 + 4 * NWAVES * j < ld_trkmax) ? a_base + j * a_step + (uint32_t)k0 * (uint32_t)ld_lda : 0xffffffffu;
     } else {
-      v_lo = (rok && k0 < ld_kmax) ? base + k0 : 0xffffffffu;
-      v_hi = (rok && k0 + 64 < ld_kmax) ? base + k0 + 64 : 0xffffffffu;
+      v = (rok && k0 < ld_kmax) ? a_base + j * a_step + k0 : 0xffffffffu;
     }
-    const uint32_t off = (is_b ? BM * HK : 0) + (wave + 8 * j) * 1024;
-    const uint32_t l_lo = __builtin_amdgcn_readfirstlane(lds_base + slot_lo * HS + off);
-    const uint32_t l_hi = __builtin_amdgcn_readfirstlane(lds_base + slot_hi * HS + off);
-    if (!is_b) {
-      FP8GMM_DMA(l_lo, v_lo, rsrc_a);
-      FP8GMM_DMA(l_hi, v_hi, rsrc_a);
+    const uint32_t l = __builtin_amdgcn_readfirstlane(lds_base + unit * US + (wave + NWAVES * j) * 1024);
+    FP8GMM_DMA(l, v, rsrc_a);
+  };
+  auto dma_b = [&](int unit, int j) {
+    const int k0 = ld_kt * BK;
+    const bool rok = ld_live && ((ok_b >> j) & 1);
+    uint32_t v;
+    if constexpr (B_TR) {
+      v = (rok && k0 + 4 * NWAVES * j < ld_trkmax) ? b_base + j * b_step + (uint32_t)k0 * (uint32_t)ld_ldb : 0xffffffffu;
     } else {
-      FP8GMM_DMA(l_lo, v_lo, rsrc_b);
-      FP8GMM_DMA(l_hi, v_hi, rsrc_b);
+      v = (rok && k0 < ld_kmax) ? b_base + j * b_step + k0 : 0xffffffffu;
     }
+    const uint32_t l = __builtin_amdgcn_readfirstlane(lds_base + unit * US + (wave + NWAVES * j) * 1024);
+    FP8GMM_DMA(l, v, rsrc_b);
   };
   auto dma_advance = [&]() {
     if (!ld_live) return;
@@ -425,10 +457,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   };
   auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
 
-  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: even / odd half-steps
-  auto read_frag = [&](i32x8& f, const uint8_t* base) {
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc0);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc1);
+  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: low / high K half of a step
+  auto read_frag = [&](i32x8& f, const uint8_t* base, int hh) {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc[hh][0]);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc[hh][1]);
     f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
   };
 
@@ -441,46 +473,46 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
     f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
   };
-  // weight fragment j / token fragment i of the half-slot at `slot`
-  auto read_frag_b = [&](i32x8& f, const uint8_t* slot, int j) {
+  // weight fragment j / token fragment i, K half hh, of the unit at `unit`
+  auto read_frag_b = [&](i32x8& f, const uint8_t* unit, int j, int hh) {
     if constexpr (!B_TR) {
-      read_frag(f, slot + fb_off + j * 32 * HK);
+      read_frag(f, unit + fb_off + j * 32 * BK, hh);
     } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)slot + (j == 0 ? fbt_off0 : fbt_off1));
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * 256));
     }
   };
-  auto read_frag_a = [&](i32x8& f, const uint8_t* slot, int i) {
+  auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh) {
     if constexpr (!A_TR) {
-      read_frag(f, slot + fa_off + i * 32 * HK);
+      read_frag(f, unit + fa_off + i * 32 * BK, hh);
     } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)slot + fat_off[i]);
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * 256));
     }
   };
 
-  // ---- fill: pairs 0 and 1 of the stream into half-slots 0..3, first fragments into registers ----
+  // ---- fill: steps 0 and 1 of the stream into units 0..3, the first fragments into registers ----
   load_setup();
 #pragma unroll
-  for (int part = 0; part < 4; ++part) dma_part(0, 1, part);
+  for (int j = 0; j < kParts; ++j) dma_a(0, j);
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_b(1, j);
   dma_advance();
 #pragma unroll
-  for (int part = 0; part < 4; ++part) dma_part(2, 3, part);
+  for (int j = 0; j < kParts; ++j) dma_a(2, j);
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_b(3, j);
   dma_advance();
-  FP8GMM_WAIT_VM(kPairLoads);
+  FP8GMM_WAIT_VM(2 * kParts);
   __builtin_amdgcn_s_barrier();
-  {
-    read_frag_b(fb0[0], lds, 0);
-    read_frag_b(fb0[1], lds, 1);
-    read_frag_a(fa0[0], lds, 0);
-    read_frag_a(fa0[1], lds, 1);
-    read_frag_a(fa0[2], lds, 2);
-    read_frag_a(fa0[3], lds, 3);
-  }
-  int hs = 0;  // half-slot of the current even half-step
-  // vmcnt counts loads and stores in issue order.  A barrier needs the pair before the newest one, so it
-  // normally waits for "all but the newest 8".  Right after an interior epilogue the newest operations
-  // also include that epilogue's kFastStores stores, which nothing in LDS depends on: for the next
-  // kRelaxedWaits barriers the needed pair is older than those stores, so they may stay in flight.
-  int relaxed = 0;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + US, j, 0);
+#pragma unroll
+  for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds, i, 0);
+  int ua = 0;  // ring unit of the current step's token rows; its weight rows are in the next unit
+  // vmcnt counts loads and stores in issue order.  The barrier of a step needs the next step's units, which are
+  // older than the token loads issued during the low half-step: "all but the newest kParts".  Right after an
+  // interior epilogue the newest operations also include that epilogue's kFastStores stores, which nothing in
+  // LDS depends on: at the first barrier after it they may stay in flight.
+  bool relaxed = false;
 
 // source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
 #define FP8GMM_MF0(i, j) \
@@ -502,77 +534,102 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
     for (int kt = 0; kt < g.nk; ++kt) {
-      const int h1 = ring_inc(hs), h2 = ring_inc(h1);
-      const int free_lo = (hs + 4 >= RING) ? hs + 4 - RING : hs + 4;  // will hold half-step + 4
-      const int free_hi = hs;                                         // will hold half-step + 5
-      // The pair for half-steps + 4 / + 5 is fetched in four quarters spread over both half-steps (token
-      // rows in the even one, weight rows in the odd one, one quarter every fourth MFMA).  Issued in one
-      // burst, the 64 KB of a pair keep the texture-address unit busy for about a thousand cycles and every
-      // wavefront queues behind it with its MFMAs.
-      // ---- even half-step: its fragments are in fa0 / fb0.  The barrier proves that every wavefront has
-      // them too (lgkmcnt(0)), which frees half-slot hs, and that the pair holding half-step + 1 has landed
-      // (everything but the newest pair: 4 token-row + 4 weight-row loads).
-      if (relaxed > 0) {
-        FP8GMM_WAIT_VM_LGKM(kPairLoads + kFastStores);
-        --relaxed;
-      } else {
-        FP8GMM_WAIT_VM_LGKM(kPairLoads);
-      }
-      __builtin_amdgcn_s_barrier();
+      // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
+      // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
+      // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
+      // has read them.
+      const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
+      // ---- low K half: fragments in fa0 / fb0; fetch the high half's from the same units.  No barrier:
+      // nothing written since the last one is read here.
       {
-        const uint8_t* qb = lds + h1 * HS;
+        const uint8_t* qa = lds + ua * US;
+        const uint8_t* qb = lds + ub * US;
         FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 0);
+        dma_a(fa, 0);
         FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
-        read_frag_b(fb1[0], qb, 0);
-        read_frag_b(fb1[1], qb, 1);
-        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_MF0(1, 1); FP8GMM_SB();
-        read_frag_a(fa1[0], qb, 0);
-        read_frag_a(fa1[1], qb, 1);
+        read_frag_b(fb1[0], qb, 0, 1);
+        read_frag_b(fb1[1], qb, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 2); FP8GMM_SB();
+        dma_a(fa, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 3); FP8GMM_SB();
+        read_frag_b(fb1[2], qb, 2, 1);
+        read_frag_b(fb1[3], qb, 3, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
+        dma_a(fa, 2);
+        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        read_frag_a(fa1[0], qa, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 2); FP8GMM_SB();
+        dma_a(fa, 3);
+        FP8GMM_SB(); FP8GMM_MF0(1, 3); FP8GMM_SB();
+        read_frag_a(fa1[1], qa, 1, 1);
         FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 1);
+        dma_a(fa, 4);
         FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
-        read_frag_a(fa1[2], qb, 2);
-        read_frag_a(fa1[3], qb, 3);
-        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_MF0(3, 1); FP8GMM_SB();
+        read_frag_a(fa1[2], qa, 2, 1);
+        FP8GMM_SB(); FP8GMM_MF0(2, 2); FP8GMM_SB();
+        dma_a(fa, 5);
+        FP8GMM_SB(); FP8GMM_MF0(2, 3); FP8GMM_SB();
+        read_frag_a(fa1[3], qa, 3, 1);
+        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_SB();
+        dma_a(fa, 6);
+        FP8GMM_SB(); FP8GMM_MF0(3, 1); FP8GMM_SB();
+        dma_a(fa, 7);
+        FP8GMM_SB(); FP8GMM_MF0(3, 2); FP8GMM_MF0(3, 3); FP8GMM_SB();
       }
-      // ---- odd half-step: fragments in fa1 / fb1.  Half-step + 2 sits in the low half of the pair whose
-      // weight rows were issued one half-step ago; only the 4 token-row loads of the newest pair may still
-      // be in flight.
-      if (relaxed > 0) {
-        FP8GMM_WAIT_VM(kPairLoads / 2 + kFastStores);
-        --relaxed;
+      // ---- high K half: fragments in fa1 / fb1.  The barrier proves that every wavefront has read this
+      // step's units (lgkmcnt(0)) and that the next step's units have landed for all of them.
+      if (relaxed) {
+        FP8GMM_WAIT_VM_LGKM(kParts + kFastStores);
+        relaxed = false;
       } else {
-        FP8GMM_WAIT_VM(kPairLoads / 2);
+        FP8GMM_WAIT_VM_LGKM(kParts);
       }
       __builtin_amdgcn_s_barrier();
       {
-        const uint8_t* qb = lds + h2 * HS;
+        const uint8_t* qa = lds + na * US;
+        const uint8_t* qb = lds + nb * US;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 2);
+        dma_b(ua, 0);
         FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
-        read_frag_b(fb0[0], qb, 0);
-        read_frag_b(fb0[1], qb, 1);
-        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_MF1(1, 1); FP8GMM_SB();
-        read_frag_a(fa0[0], qb, 0);
-        read_frag_a(fa0[1], qb, 1);
+        read_frag_b(fb0[0], qb, 0, 0);
+        read_frag_b(fb0[1], qb, 1, 0);
+        FP8GMM_SB(); FP8GMM_MF1(0, 2); FP8GMM_SB();
+        dma_b(ua, 1);
+        FP8GMM_SB(); FP8GMM_MF1(0, 3); FP8GMM_SB();
+        read_frag_b(fb0[2], qb, 2, 0);
+        read_frag_b(fb0[3], qb, 3, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        dma_b(ua, 2);
+        FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
+        read_frag_a(fa0[0], qa, 0, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 2); FP8GMM_SB();
+        dma_b(ua, 3);
+        FP8GMM_SB(); FP8GMM_MF1(1, 3); FP8GMM_SB();
+        read_frag_a(fa0[1], qa, 1, 0);
         FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
-        dma_part(free_lo, free_hi, 3);
-        dma_advance();
+        dma_b(ua, 4);
         FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
-        read_frag_a(fa0[2], qb, 2);
-        read_frag_a(fa0[3], qb, 3);
-        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_MF1(3, 1); FP8GMM_SB();
+        read_frag_a(fa0[2], qa, 2, 0);
+        FP8GMM_SB(); FP8GMM_MF1(2, 2); FP8GMM_SB();
+        dma_b(ua, 5);
+        FP8GMM_SB(); FP8GMM_MF1(2, 3); FP8GMM_SB();
+        read_frag_a(fa0[3], qa, 3, 0);
+        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_SB();
+        dma_b(ua, 6);
+        FP8GMM_SB(); FP8GMM_MF1(3, 1); FP8GMM_SB();
+        dma_b(ua, 7);
+        dma_advance();
+        FP8GMM_SB(); FP8GMM_MF1(3, 2); FP8GMM_MF1(3, 3); FP8GMM_SB();
       }
-      hs = h2;
+      ua = na;
     }
     // ---- epilogue ----
     if (g.slot >= 0) {
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
       partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
-      relaxed = 0;
+      relaxed = false;
     } else {
-      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue) ? kRelaxedWaits : 0;
+      relaxed = tile_epilogue<true>(acc, pr, m0, n0, out_kind, epilogue);
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS
@@ -615,7 +672,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8g
   const fp8gmm_gemm_problem pr = probs[prob];
   int m0, n0;
   tile_origin(pr.m, pr.n, tile - pr.tile_begin, &m0, &n0);
-  tile_epilogue(acc, pr, m0, n0, out_kind, epilogue);
+  tile_epilogue<false>(acc, pr, m0, n0, out_kind, epilogue);
 }
 
 // Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)
@@ -664,7 +721,7 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles,
   constexpr int kMaxDevices = 64;
   static std::atomic<int> num_cu[kMaxDevices];
   static std::atomic<bool> attr_set[kMaxDevices];
-  const size_t lds_bytes = (size_t)RING * HS;
+  const size_t lds_bytes = (size_t)RING * US;
   auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE, A_TR, B_TR>;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
