@@ -312,12 +312,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   clock_probe_mark<PROBE>(0);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: what depends on it stays in scalar registers
   const int wave_m = wave / WAVES_N;  // 0..1
   const int wave_n = wave % WAVES_N;  // 0..1
   const int l32 = lane & 31;
   const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
 
   // DMA lane map, row-major operand: one wavefront instruction fills 8 rows x 128 B of a unit, i.e. whole
   // cache lines: lane -> row lane >> 3 of the group, slot chunk lane & 7.  Chunk c of row r is kept at chunk
@@ -360,10 +360,29 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   // ---- load side: runs two steps ahead of the compute side, possibly in the next tile ----
   bool ld_live = true;  // the load cursor still points at an item
   int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
-  [[maybe_unused]] int ld_lda = 0, ld_ldb = 0, ld_trkmax = 0;  // contraction-major operands only
+  [[maybe_unused]] int ld_lda = 0, ld_ldb = 0;  // contraction-major operands only
   i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
-  uint32_t a_base = 0, b_base = 0, a_step = 0, b_step = 0;  // part j of an operand starts at base + j * step
-  uint32_t ok_a = 0, ok_b = 0;                               // bit j: the rows / columns of part j exist
+  // Addresses of the K = 128 step the load cursor points at: part j of an operand is fetched from a_k + j * a_step
+  // (byte offsets into the operand's buffer, a_step uniform).  Rows past m / n are not masked: whatever they
+  // deliver only reaches accumulators of rows / columns that the epilogue never stores, and the descriptor keeps
+  // the access inside the operand.  The K tail is: a row-major lane whose 16-byte chunk lies past k gets an
+  // out-of-range offset (zero fill); contraction rows past k are out of the descriptor's range by themselves.
+  uint32_t a_base = 0, b_base = 0, a_step = 0, b_step = 0, a_k = 0, b_k = 0;
+  bool k_ok = false;  // row-major operands: this lane's chunk of the step exists
+  auto step_setup = [&]() {
+    const uint32_t k0 = (uint32_t)ld_kt * BK;
+    if constexpr (A_TR) {
+      a_k = a_base + k0 * (uint32_t)ld_lda;  // k * pitch < 2^32 is checked when the table is planned
+    } else {
+      a_k = a_base + k0;
+    }
+    if constexpr (B_TR) {
+      b_k = b_base + k0 * (uint32_t)ld_ldb;
+    } else {
+      b_k = b_base + k0;
+    }
+    k_ok = (int)k0 < ld_kmax;
+  };
   auto load_setup = [&]() {
     while ((ld_live = cursor_valid(sch, wg_in_xcd, c_ld))) {
       const Item g = cursor_item(sch, xcd, wg_in_xcd, c_ld);
@@ -384,68 +403,46 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         // p ^ 2 (row mod 8); row mod 8 is the same for every j.
         const int krow = wave * 4 + (lane >> 4);
         const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
-        ok_a = ok_b = 0;
         if constexpr (!A_TR) {
-          const int ar = g.m0 + wave * 8 + drow;
-#pragma unroll
-          for (int j = 0; j < kParts; ++j)
-            if (ar + NWAVES * 8 * j < pr.m) ok_a |= 1u << j;
-          a_base = (uint32_t)ar * (uint32_t)pr.lda + dchunk * 16;
+          a_base = (uint32_t)(g.m0 + wave * 8 + drow) * (uint32_t)pr.lda + dchunk * 16;
           a_step = NWAVES * 8 * (uint32_t)pr.lda;
         } else {
-          if (g.m0 + tr_col < pr.m) ok_a = (1u << kParts) - 1;
           a_base = (uint32_t)krow * (uint32_t)pr.lda + (uint32_t)(g.m0 + tr_col);
           a_step = NWAVES * 4 * (uint32_t)pr.lda;
           ld_lda = pr.lda;
         }
         if constexpr (!B_TR) {
-          const int br = g.n0 + wave * 8 + drow;
-#pragma unroll
-          for (int j = 0; j < kParts; ++j)
-            if (br + NWAVES * 8 * j < pr.n) ok_b |= 1u << j;
-          b_base = (uint32_t)br * (uint32_t)pr.ldb + dchunk * 16;
+          b_base = (uint32_t)(g.n0 + wave * 8 + drow) * (uint32_t)pr.ldb + dchunk * 16;
           b_step = NWAVES * 8 * (uint32_t)pr.ldb;
         } else {
-          if (g.n0 + tr_col < pr.n) ok_b = (1u << kParts) - 1;
           b_base = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)(g.n0 + tr_col);
           b_step = NWAVES * 4 * (uint32_t)pr.ldb;
           ld_ldb = pr.ldb;
         }
-        // row k0 + krow + 4 NWAVES j of a contraction-major operand exists iff k0 + 4 NWAVES j < ld_trkmax
-        if constexpr (A_TR || B_TR) ld_trkmax = pr.k - krow;
         ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
         ld_kt = g.k_begin;
         ld_nk = g.k_begin + g.nk;
+        step_setup();
         return;
       }
       cursor_advance(sch, wg_in_xcd, c_ld);  // an item without K work needs no loads
     }
+    // Past the end of the stream the loads are issued all the same, against empty descriptors (zero fill),
+    // which keeps the vmcnt arithmetic uniform.
+    rsrc_a[2] = 0;
+    rsrc_b[2] = 0;
   };
-  // One instruction of the K = 128 step the load cursor points at: part j (0..7) of the token operand into
-  // ring unit `unit`, or of the weight operand.  Past the end of the stream the loads are issued all the same
-  // with out-of-range offsets (zero fill), which keeps the vmcnt arithmetic uniform.
+  // One instruction of that step: part j (0..7) of the token operand into ring unit `unit`, or of the weights.
   auto dma_a = [&](int unit, int j) {
-    const int k0 = ld_kt * BK;
-    const bool rok = ld_live && ((ok_a >> j) & 1);
-    uint32_t v;
-    if constexpr (A_TR) {  // k * pitch < 2^32 is checked when the table is planned
-      v = (rok && k0 + 4 * NWAVES * j < ld_trkmax) ? a_base + j * a_step + (uint32_t)k0 * (uint32_t)ld_lda : 0xffffffffu;
-    } else {
-      v = (rok && k0 < ld_kmax) ? a_base + j * a_step + k0 : 0xffffffffu;
-    }
-    const uint32_t l = __builtin_amdgcn_readfirstlane(lds_base + unit * US + (wave + NWAVES * j) * 1024);
+    uint32_t v = a_k + j * a_step;
+    if constexpr (!A_TR) v = k_ok ? v : 0xffffffffu;
+    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
     FP8GMM_DMA(l, v, rsrc_a);
   };
   auto dma_b = [&](int unit, int j) {
-    const int k0 = ld_kt * BK;
-    const bool rok = ld_live && ((ok_b >> j) & 1);
-    uint32_t v;
-    if constexpr (B_TR) {
-      v = (rok && k0 + 4 * NWAVES * j < ld_trkmax) ? b_base + j * b_step + (uint32_t)k0 * (uint32_t)ld_ldb : 0xffffffffu;
-    } else {
-      v = (rok && k0 < ld_kmax) ? b_base + j * b_step + k0 : 0xffffffffu;
-    }
-    const uint32_t l = __builtin_amdgcn_readfirstlane(lds_base + unit * US + (wave + NWAVES * j) * 1024);
+    uint32_t v = b_k + j * b_step;
+    if constexpr (!B_TR) v = k_ok ? v : 0xffffffffu;
+    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
     FP8GMM_DMA(l, v, rsrc_b);
   };
   auto dma_advance = [&]() {
@@ -453,6 +450,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     if (++ld_kt == ld_nk) {
       cursor_advance(sch, wg_in_xcd, c_ld);
       load_setup();
+    } else {
+      step_setup();
     }
   };
   auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
@@ -815,8 +814,9 @@ int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layou
         if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
           return FP8GMM_ERR_ALIGNMENT;
         // the kernel addresses each operand through a buffer descriptor with 32-bit byte offsets
-        if ((uint64_t)(a_kmajor ? p.k : p.m) * (uint64_t)p.lda > 0xffffffffull ||
-            (uint64_t)(b_kmajor ? p.k : p.n) * (uint64_t)p.ldb > 0xffffffffull)
+        // (contraction rows up to 127 past k are addressed, and must fall outside the descriptor, not wrap)
+        if ((uint64_t)(a_kmajor ? p.k + 128 : p.m) * (uint64_t)p.lda > 0xffffffffull ||
+            (uint64_t)(b_kmajor ? p.k + 128 : p.n) * (uint64_t)p.ldb > 0xffffffffull)
           return FP8GMM_ERR_BAD_SHAPE;
       }
     }
