@@ -39,6 +39,7 @@
 #include <cstdlib>
 #include <map>
 #include <mutex>
+#include <type_traits>
 #include <utility>
 
 #include "device_utils.h"
@@ -532,7 +533,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    for (int kt = 0; kt < g.nk; ++kt) {
+    // One K = 128 step.  `same_item`: the load cursor stays inside its current item after this step (the caller
+    // knows), so advancing it is three additions; otherwise the general advance, which may switch items.
+    auto k_step = [&](auto same_item) {
       // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
       // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
       // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
@@ -617,11 +620,21 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         dma_b(ua, 6);
         FP8GMM_SB(); FP8GMM_MF1(3, 1); FP8GMM_SB();
         dma_b(ua, 7);
-        dma_advance();
+        if constexpr (decltype(same_item)::value) {
+          ++ld_kt;
+          step_setup();
+        } else {
+          dma_advance();
+        }
         FP8GMM_SB(); FP8GMM_MF1(3, 2); FP8GMM_MF1(3, 3); FP8GMM_SB();
       }
       ua = na;
-    }
+    };
+    // The load cursor runs two steps ahead of this loop: while at least three steps of the item remain, its
+    // next step lies in the same item.
+    int kt = 0;
+    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{});
+    for (; kt < g.nk; ++kt) k_step(std::false_type{});
     // ---- epilogue ----
     if (g.slot >= 0) {
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
