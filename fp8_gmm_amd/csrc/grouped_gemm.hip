@@ -91,9 +91,11 @@ __device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
 
 // Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
 // stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
+// `stage` (main kernel only): 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of
+// the staged path; the fix-up kernel passes null and stores straight from the MFMA layout.
 template <bool FROM_ACC_REGS>
 __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
-                                              int out_kind, int epilogue) {
+                                              int out_kind, int epilogue, uint8_t* stage) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
@@ -109,11 +111,47 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
     const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
     if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
         ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
-      // Interior tile, plain bf16 output: straight-line code with an exact store count.  A lane holds
-      // columns 8 g + 4 khalf .. + 3 of its row for g = 0..3; swapping the upper lanes of the even-g
+      // Interior tile, plain bf16 output: straight-line code with an exact store count.
+      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+      if (stage != nullptr) {
+        // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
+        // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
+        // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
+        // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
+        // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
+        uint8_t* mine = stage + wave * 8192;
+        const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
+        const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
+                               pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+              *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
+            }
+          }
+          // only this wavefront touches `mine`: its own LDS operations complete in order
+          u32x4 v[8];
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int r = 4 * it + rrow;
+            v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
+          }
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
+            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
+          }
+        }
+        __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
+      } else {
+      // A lane holds columns 8 g + 4 khalf .. + 3 of its row for g = 0..3; swapping the upper lanes of the even-g
       // registers with the lower lanes of the odd-g ones leaves 8 consecutive columns per lane:
       // lanes 0-31 take g even, lanes 32-63 g odd.  One 16-byte store each.
-      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
         const int m = m0 + wave_m * WM + i * 32 + l32;
@@ -134,6 +172,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
             global_store(C + (int64_t)m * ldc + n, o);
           }
         }
+      }
       }
       fast = true;
     } else if (out_kind == FP8GMM_OUT_BF16) {
@@ -641,7 +680,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
       relaxed = false;
     } else {
-      relaxed = tile_epilogue<true>(acc, pr, m0, n0, out_kind, epilogue);
+      // free until the next step's token loads: the unit that held the last step's weights
+      relaxed = tile_epilogue<true>(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS
@@ -684,7 +724,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8g
   const fp8gmm_gemm_problem pr = probs[prob];
   int m0, n0;
   tile_origin(pr.m, pr.n, tile - pr.tile_begin, &m0, &n0);
-  tile_epilogue<false>(acc, pr, m0, n0, out_kind, epilogue);
+  tile_epilogue<false>(acc, pr, m0, n0, out_kind, epilogue, nullptr);
 }
 
 // Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)
