@@ -291,22 +291,6 @@ __device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* sl
       }
     }
 }
-__device__ __forceinline__ void partial_add(f32x16 (&acc)[MT][NT], const uint8_t* slot) {
-  const float* base = reinterpret_cast<const float*>(slot) + threadIdx.x * 4;
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const float4 v = *reinterpret_cast<const float4*>(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4));
-        acc[i][j][4 * g + 0] += v.x;
-        acc[i][j][4 * g + 1] += v.y;
-        acc[i][j][4 * g + 2] += v.z;
-        acc[i][j][4 * g + 3] += v.w;
-      }
-}
-
 // Measurement hook (fp8gmm_gemm_clock_probe): 8 x 4 uint64 of device memory, or null.
 __device__ uint64_t* volatile d_clock_probe = nullptr;
 
@@ -695,12 +679,16 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 // Completes the tiles that the main kernel shared along K.  One workgroup per interior piece boundary of
 // every XCD's stream-K region; the FIRST boundary that falls strictly inside a tile owns that tile: it adds
 // the pieces in K order (workgroup j - 1 holds the piece from the tile's first pair step, workgroups j,
-// j + 1, ... the following ones) and runs the normal epilogue.
-__global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
-                                                                      int nprob, int total_tiles, int out_kind,
-                                                                      int epilogue,
-                                                                      const uint8_t* __restrict__ workspace,
-                                                                      int wgs_per_xcd) {
+// j + 1, ... the following ones) and applies the epilogue.
+// 1024 threads: thread T owns the 16-byte groups T + 1024 q (q = 0..15) of a slot, i.e. register group g = T / 256
+// of every MFMA tile (i, j) = q of main-kernel thread T % 256: 4 consecutive columns of one row each.  The sums and
+// the arithmetic are those of tile_epilogue's general paths, so a shared tile gets the same bits as a whole one.
+constexpr int kFixupThreads = 1024;
+static_assert(kFixupThreads == 4 * NTHREADS, "one register group of every MFMA tile per thread");
+
+__global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
+    const fp8gmm_gemm_problem* __restrict__ probs, int nprob, int total_tiles, int out_kind, int epilogue,
+    const uint8_t* __restrict__ workspace, int wgs_per_xcd) {
   const int xcd = blockIdx.x % kNumXcd;
   const int j = blockIdx.x / kNumXcd + 1;
   Sched sch;
@@ -709,22 +697,107 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_fixup_kernel(const fp8g
   const int tile = fixup_tile(sch, j, &n_following);
   if (tile < 0) return;
   const int prob = problem_of_tile(sch, tile);
-
-  f32x16 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int jj = 0; jj < NT; ++jj)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][jj][r] = 0.f;
-  partial_add(acc, workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + j - 1) + 1) * kPartialBytes);
-  for (int q = j; q < j + n_following; ++q)
-    partial_add(acc, workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + q)) * kPartialBytes);
-
   const fp8gmm_gemm_problem pr = probs[prob];
   int m0, n0;
   tile_origin(pr.m, pr.n, tile - pr.tile_begin, &m0, &n0);
-  tile_epilogue<false>(acc, pr, m0, n0, out_kind, epilogue, nullptr);
+
+  const int t = threadIdx.x % NTHREADS, g = threadIdx.x / NTHREADS;
+  const int lane = t & 63, wave = t >> 6;
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int l32 = lane & 31, khalf = lane >> 5;
+
+  f32x4 sum[MT * NT];
+  {
+    const f32x4* first = reinterpret_cast<const f32x4*>(
+        workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + j - 1) + 1) * kPartialBytes) + threadIdx.x;
+#pragma unroll
+    for (int q = 0; q < MT * NT; ++q) sum[q] = first[q * kFixupThreads];
+  }
+  for (int w = j; w < j + n_following; ++w) {
+    const f32x4* next = reinterpret_cast<const f32x4*>(
+        workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + w)) * kPartialBytes) + threadIdx.x;
+    f32x4 part[MT * NT];
+#pragma unroll
+    for (int q = 0; q < MT * NT; ++q) part[q] = next[q * kFixupThreads];
+#pragma unroll
+    for (int q = 0; q < MT * NT; ++q) sum[q] += part[q];
+  }
+
+  const int M = pr.m, N = pr.n;
+  const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
+  const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
+  const float s = sa_inv * sb_inv;
+  const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
+  const int64_t ldc = pr.ldc;
+  uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
+  const bool aux_ok = AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0;
+  const float cs = pr.c_scale ? *pr.c_scale : 1.f;
+  float amax = 0.f;
+#pragma unroll
+  for (int q = 0; q < MT * NT; ++q) {
+    const int i = q / NT, jj = q % NT;
+    const int m = m0 + wave_m * WM + i * 32 + l32;
+    const int n = n0 + wave_n * WN + jj * 32 + g * 8 + khalf * 4;
+    if (m >= M || n >= N) continue;
+    float v[4], r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] = sum[q][e] * s;
+      r[e] = gelu ? gelu_tanh_fast(v[e]) : v[e];
+    }
+    const int64_t off = (int64_t)m * ldc + n;
+    if (out_kind == FP8GMM_OUT_BF16) {
+      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) && aux_ok;
+      if (vec && n + 3 < N) {
+        const u32x2 o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+        global_store(C + off, o);
+        if (gelu && AUX != nullptr) {
+          const u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          global_store(AUX + off, a);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (n + e < N) {
+            global_store(C + off + e, (uint16_t)f32_to_bf16_bits(r[e]));
+            if (gelu && AUX != nullptr) global_store(AUX + off + e, (uint16_t)f32_to_bf16_bits(v[e]));
+          }
+        }
+      }
+    } else {
+      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
+      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 3) == 0) && aux_ok;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < N) amax = amax_step(amax, r[e]);
+      uint32_t w;
+      if (out_kind == FP8GMM_E4M3) {
+        w = cvt4_fp8<FP8GMM_E4M3>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
+      } else {
+        w = cvt4_fp8<FP8GMM_E5M2>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
+      }
+      if (vec && n + 3 < N) {
+        global_store(C + off, w);
+        if (gelu && AUX != nullptr) {
+          const u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+          global_store(AUX + off, a);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (n + e < N) {
+            global_store(C + off + e, (uint8_t)(w >> (8 * e)));
+            if (gelu && AUX != nullptr) global_store(AUX + off + e, (uint16_t)f32_to_bf16_bits(v[e]));
+          }
+        }
+      }
+    }
+  }
+  if (out_kind != FP8GMM_OUT_BF16 && pr.c_amax != nullptr) {
+    amax = wave_max(amax);
+    if (lane == 0 && amax > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= amax)) atomic_max_nonneg(pr.c_amax, amax);
+  }
 }
 
 // Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)
@@ -806,7 +879,7 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles,
   if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
   if (workspace != nullptr) {
     const int wgs_per_xcd = grid / kNumXcd;
-    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(kNumXcd * (wgs_per_xcd - 1)), dim3(NTHREADS), 0, stream,
+    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(kNumXcd * (wgs_per_xcd - 1)), dim3(kFixupThreads), 0, stream,
                        probs_dev, n, total_tiles, out_kind, epilogue, workspace, wgs_per_xcd);
     if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
   }
