@@ -63,7 +63,7 @@ def splits(kind, experts, tokens, seed):
 # summary is profiles/config2_mlp_step_hbm_traffic.md (counter units calibrated against a 256 MiB copy:
 # 2 KiB per FETCH_SIZE unit, 1 KiB per WRITE_SIZE unit).  Counters cannot be read from inside this process,
 # so the figure is carried here; the algorithmic bytes of one launch are 1.09 GB.
-GEMM_HBM_TRAFFIC_BYTES = {"config2": 2.53e9}
+GEMM_HBM_TRAFFIC_BYTES = {"config2": 2.73e9}
 
 
 def sample_shader_clock(work):
@@ -189,6 +189,45 @@ def bench_cast_pad(args):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None},
         "cpu_baseline": cpu,
     }))
+
+
+def dense_gemm_comparison(dev, m, n, k, reps=100):
+    """[m, k] x [n, k]^T -> bf16 [m, n], e4m3 operands: TFLOP/s of the grouped kernel (one group) and of the vendor GEMM."""
+    import fp8_gmm_amd.backend as backend
+
+    def quantized(t):
+        return (t * (448.0 / t.abs().max())).to(torch.float8_e4m3fn)
+
+    a = quantized(torch.randn(m, k, device=dev))
+    b = quantized(torch.randn(n, k, device=dev))
+    c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+    one = torch.ones(1, device=dev)
+    sizes = torch.tensor([m])
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    flops = 2.0 * m * n * k
+    out = {"shape": [m, n, k], "data": "N(0, 1) scaled to amax 448"}
+    mine, vendor = [], []
+    for _ in range(2):
+        mine.append(timed(lambda: backend.fp8_gmm(a, b.view(1, n, k), sizes, one, one, c)))
+        try:
+            vendor.append(timed(lambda: torch._scaled_mm(a, b.t(), scale_a=one[0], scale_b=one[0],
+                                                         out_dtype=torch.bfloat16, out=c)))
+        except Exception as exc:  # the private torch entry point may change; the comparison is optional
+            out["vendor_error"] = repr(exc)[:200]
+    out["this_kernel_tflops"] = round(flops / min(mine) / 1e12, 1)
+    if vendor:
+        out["torch_scaled_mm_tflops"] = round(flops / min(vendor) / 1e12, 1)
+    return out
 
 
 def main():
@@ -372,6 +411,13 @@ def main():
         also["reference_layout"] = {"ms_per_step": round(ref_ms, 4),
                                     "value": round(flops_per_step / (ref_ms * 1e-3) / 1e12, 2), "unit": "TFLOP/s",
                                     "kernels": ref_kernels}
+
+    # ... and, for scale, one dense e4m3 GEMM of the step's size (all tokens as one group, tokens x ffn x hidden)
+    # through this library's kernel and through the vendor library behind torch._scaled_mm, on the same Gaussian
+    # operands scaled to the fp8 range, timed alternately
+    if args.workload == "config2" and not args.headline_only:
+        also = dict(also or {})
+        also["dense_gemm_of_the_same_size"] = dense_gemm_comparison(dev, tokens, ffn, hidden)
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -30,7 +30,7 @@ constexpr int kNumXcd = 8;
 constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many pair steps
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
 constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
-constexpr int kPartialBytes = BM * BN * 4;  // one slot: the 128 accumulators of the 512 lanes
+constexpr int kPartialBytes = BM * BN * 4;  // one slot: the fp32 accumulators of one tile
 constexpr int kTileOverhead = 4;      // fixed cost of a tile (epilogue, switch) in K = 128 steps, measured
 constexpr int kSlotsPerWg = 2;        // a piece that starts inside a tile, one that ends inside a tile
 

@@ -12,29 +12,37 @@
 //     contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so that workgroups that
 //     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest within
 //     groups of 8 rows of tiles, so one round of an XCD's 32 workgroups is an 8 x 4 block of tiles.
-//   * a workgroup is 8 wavefronts (2 along m x 4 along n); a wavefront owns a 128 x 64
-//     sub-tile = 4 x 2 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4 (128 accumulator registers).
+//   * a workgroup is 4 wavefronts (2 along m x 2 along n), one per SIMD; a wavefront owns a
+//     128 x 128 sub-tile = 4 x 4 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4.  Its 256 accumulators
+//     live in the accumulation registers, the other 256 registers hold fragments and addresses.
 //     The weight operand is MFMA source 0 and the token operand source 1: every lane then
-//     holds 4 consecutive output columns of one row (8-byte bf16 stores, no shuffle).
+//     holds 4 consecutive output columns of one row.
 //
 // Data movement
 //   * operands go global -> LDS directly (`buffer_load_dwordx4 ... lds`), never through
 //     registers.  Buffer descriptors bound every operand, so rows past m / n and K tails read
 //     as zeros: m, n are arbitrary and k only has to be a multiple of 16.
-//   * LDS holds a ring of five 32 KB half-slots (all 160 KB); a half-slot is one K = 64 slice
-//     of the tile: 256 token rows + 256 weight rows of 64 bytes, the four 16-byte chunks of a
-//     row XOR-swizzled with (row >> 2) & 3, which makes the 16-byte fragment reads of a
-//     wavefront conflict-free.
-//   * every second step a wavefront issues the 8 loads of a K = 128 pair (the two 64-byte
-//     halves of each 128-byte line back to back, so the second half hits in L1) into the two
-//     half-slots that have just become free; the pair is first read three steps later.
-//   * the load stream, the fragment double buffer and the ring run CONTINUOUSLY across tile
-//     boundaries: while a tile's epilogue stores its result, the next tile's first two pairs
-//     are already in LDS and its first fragments in registers.
-//   * one s_barrier per K = 64 step.  After each barrier the MFMAs (whose fragments were
-//     fetched during the previous step) are issued first and the DMA issues / next-fragment
-//     LDS reads are interleaved between them (pinned with sched_barrier), so the MFMA pipe
-//     does not idle while the two wavefronts of a SIMD do their memory work.
+//   * a main-loop step consumes K = 128: one 128-byte line of each of the tile's 256 token rows
+//     and 256 weight rows.  LDS (all 160 KB) is a ring of five 32 KB units, a unit being the
+//     256 rows x 128 B of ONE operand for one step, its eight 16-byte chunks XOR-swizzled with
+//     (row >> 1) & 7 so that the 16-byte fragment reads of a wavefront are conflict-free.  Every
+//     load instruction fetches 8 whole lines (two half-line requests for one line, issued apart,
+//     meet in the L1 as a hit on a pending miss and stall it).
+//   * at any time the ring holds the units of the step being computed, of the next step, and
+//     the tokens of the step after; that step's weights replace the current tokens once the
+//     step's barrier has shown that every wavefront has read them.  The token loads of step + 2
+//     are issued during the low K half of a step, the weight loads during the high half, one
+//     after every second MFMA.
+//   * the load stream and the ring run CONTINUOUSLY across tile boundaries: while a tile's
+//     epilogue stores its result, the next tile's first two steps are already in LDS.
+//   * ONE s_barrier per step, between its two K = 64 halves.  The fragments of a half are read
+//     from LDS during the half before it, interleaved with the MFMAs (pinned with sched_barrier).
+//     With a single wavefront per SIMD nothing else fills an MFMA pipe, so whatever sits between
+//     two MFMAs has to issue within the 64 cycles the first one runs: addresses are two
+//     instructions per load, the load cursor advances without branches while it stays inside an
+//     item, and the scheduler arithmetic of an item switch runs once per tile.
+//   * epilogue: scale, convert, and - for interior bf16 tiles - a pass through the free ring unit
+//     that turns the MFMA layout into whole-line stores.
 #include <atomic>
 #include <cstdlib>
 #include <map>
@@ -60,7 +68,7 @@ constexpr int WAVES_N = BN / WN;  // wavefronts along n: 2 (x 2 along m)
 constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
 constexpr int NT = WN / 32;       // 4 MFMA tiles along n per wave
 constexpr int kParts = US / 1024 / NWAVES;  // buffer_load ... lds instructions (1 KB each) per wavefront per unit: 8
-constexpr int kFastStores = MT * NT * 2;  // 16-byte stores per wavefront in the interior bf16 epilogue
+constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the interior bf16 epilogue (8 per 32-row block)
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -68,7 +76,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
 #define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
 #define FP8GMM_WAIT_VM_LGKM(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(n) : "memory")
-typedef unsigned u32pair __attribute__((ext_vector_type(2)));
 // global -> LDS: lane i's 16 bytes land at M0 + 16 i; out-of-range offsets deliver zeros
 #define FP8GMM_DMA(lds_addr, voff, rsrc) \
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
@@ -77,23 +84,16 @@ typedef unsigned u32pair __attribute__((ext_vector_type(2)));
 // lane live in the accumulation registers (the other 256 hold fragments and addresses); vector arithmetic
 // cannot read those, and left to itself the register allocator parks them in scratch memory on the way.
 // Reading them 16 at a time, where they are used, keeps the epilogue within the register file.
-template <bool FROM_ACC_REGS>
 __device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
-  if constexpr (FROM_ACC_REGS) {
-    f32x16 t;
+  f32x16 t;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
-    return t;
-  } else {
-    return a;
-  }
+  for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
+  return t;
 }
 
 // Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
 // stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
-// `stage` (main kernel only): 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of
-// the staged path; the fix-up kernel passes null and stores straight from the MFMA layout.
-template <bool FROM_ACC_REGS>
+// `stage`: 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of the staged path.
 __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
                                               int out_kind, int epilogue, uint8_t* stage) {
   const int lane = threadIdx.x & 63;
@@ -113,67 +113,40 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
       // Interior tile, plain bf16 output: straight-line code with an exact store count.
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
-      if (stage != nullptr) {
-        // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
-        // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
-        // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
-        // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
-        // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
-        uint8_t* mine = stage + wave * 8192;
-        const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
-        const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
-                               pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
-              *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
-            }
-          }
-          // only this wavefront touches `mine`: its own LDS operations complete in order
-          u32x4 v[8];
-#pragma unroll
-          for (int it = 0; it < 8; ++it) {
-            const int r = 4 * it + rrow;
-            v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
-          }
-#pragma unroll
-          for (int it = 0; it < 8; ++it) {
-            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
-            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
-          }
-        }
-        __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
-      } else {
-      // A lane holds columns 8 g + 4 khalf .. + 3 of its row for g = 0..3; swapping the upper lanes of the even-g
-      // registers with the lower lanes of the odd-g ones leaves 8 consecutive columns per lane:
-      // lanes 0-31 take g even, lanes 32-63 g odd.  One 16-byte store each.
+      // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
+      // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
+      // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
+      // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
+      // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
+      uint8_t* mine = stage + wave * 8192;
+      const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
+      const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
+          const f32x16 t = tile_values(acc[i][j]);
 #pragma unroll
-          for (int gp = 0; gp < 2; ++gp) {
-            const int ge = 8 * gp, go = 8 * gp + 4;  // accumulator index of g = 2 gp and g = 2 gp + 1
-            const uint32_t pe0 = pack_bf16x2(t[ge + 0] * s, t[ge + 1] * s);
-            const uint32_t pe1 = pack_bf16x2(t[ge + 2] * s, t[ge + 3] * s);
-            const uint32_t po0 = pack_bf16x2(t[go + 0] * s, t[go + 1] * s);
-            const uint32_t po1 = pack_bf16x2(t[go + 2] * s, t[go + 3] * s);
-            const u32pair r0 = __builtin_amdgcn_permlane32_swap(pe0, po0, false, false);
-            const u32pair r1 = __builtin_amdgcn_permlane32_swap(pe1, po1, false, false);
-            const u32x4 o = {r0.x, r1.x, r0.y, r1.y};
-            const int n = n0 + wave_n * WN + j * 32 + (2 * gp + khalf) * 8;
-            global_store(C + (int64_t)m * ldc + n, o);
+          for (int g = 0; g < 4; ++g) {
+            const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
+                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
           }
         }
+        // only this wavefront touches `mine`: its own LDS operations complete in order
+        u32x4 v[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int r = 4 * it + rrow;
+          v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
+          global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
+        }
       }
-      }
+      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
     } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
@@ -185,7 +158,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
+          const f32x16 t = tile_values(acc[i][j]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -227,7 +200,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         const int m = m0 + wave_m * WM + i * 32 + l32;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values<FROM_ACC_REGS>(acc[i][j]);
+          const f32x16 t = tile_values(acc[i][j]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -283,7 +256,7 @@ __device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* sl
   for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const f32x16 t = tile_values<true>(acc[i][j]);
+      const f32x16 t = tile_values(acc[i][j]);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
@@ -319,7 +292,7 @@ __device__ __forceinline__ void clock_probe_mark(int which) {
 }
 
 // B_TR: operand b is stored contraction-major, b[k][n] with n contiguous and pitch ldb (the layout of a weight
-// stack [N_out.., ] seen from the data-gradient GEMM), instead of b[n][k].  Its half-slot in LDS then holds 64
+// stack [N_out.., ] seen from the data-gradient GEMM), instead of b[n][k].  Its ring unit then holds 128
 // contraction rows of 256 bytes; the 16-byte chunk c of row r sits at chunk c ^ 2 (r mod 8), and a fragment is
 // gathered with four transposing reads (ds_read_b64_tr_b8: in a group of 16 lanes, lane 8 h + i receives byte i
 // of the 8 bytes addressed by lanes 2 b + h, b = 0..7).  Everything else - schedule, MFMA order, epilogue -
@@ -665,7 +638,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       relaxed = false;
     } else {
       // free until the next step's token loads: the unit that held the last step's weights
-      relaxed = tile_epilogue<true>(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
+      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS

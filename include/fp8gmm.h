@@ -135,14 +135,14 @@ typedef struct fp8gmm_gemm_problem {
 /* b is stored contraction-major: b[k, n] with n contiguous and ldb >= n its row pitch, i.e.
  * c[m, n] = epilogue( a[m, k] . b[k, n] ).  This is a forward weight [N_fwd = k, K_fwd = n] as the data-gradient
  * GEMM needs it, read in place: the reference casts a transposed copy of every weight for that GEMM instead
- * (fp8_gmm/grouped_linear.py:69-74,163).  b must be e4m3, n a multiple of 16, k * ldb < 2^32.  Plan such tables
+ * (fp8_gmm/grouped_linear.py:69-74,163).  b must be e4m3, n a multiple of 16, (k + 128) * ldb < 2^32.  Plan such tables
  * with fp8gmm_plan_grouped_gemm_layout(..., FP8GMM_GEMM_B_KMAJOR, ...). */
 #define FP8GMM_GEMM_B_KMAJOR 2
 /* a is stored contraction-major as well: a[k, m] with m contiguous and lda >= m, i.e.
  * c[m, n] = epilogue( a[k, m]^T . b[k, n] ): the weight-gradient GEMM dW[N, K] = dY[M, N]^T . X[M, K] on the
  * row-major gradient and activation, without the padded transposed copies the reference casts for it
  * (fp8_gmm/grouped_linear.py:36-52,142-150).  Only together with FP8GMM_GEMM_B_KMAJOR; m and n multiples of
- * 16, k arbitrary (rows past k contribute zeros), k * lda < 2^32. */
+ * 16, k arbitrary (rows past k contribute zeros), (k + 128) * lda < 2^32. */
 #define FP8GMM_GEMM_A_KMAJOR 4
 
 /* ---- library info ------------------------------------------------------------------------- */
