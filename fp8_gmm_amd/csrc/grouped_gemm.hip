@@ -148,6 +148,90 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       }
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
+    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && interior && ((ldc & 15) == 0) &&
+               ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0) && ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0)) {
+      // Interior tile of the fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
+      // outputs go through the staging area like the plain form's, one 32-row block at a time - first the bf16
+      // block as 32 rows x 256 B, then, in a second pass over the same accumulators, the fp8 block as 32 rows x
+      // 128 B (chunk c of row r at chunk c ^ ((r >> 1) & 7)) - so that every store instruction writes whole
+      // lines: 12 per block instead of 32 that touch 32 rows each.
+      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
+      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
+      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
+      uint8_t* mine = stage + wave * 8192;
+      const int wr = l32 * 256 + khalf * 8;   // bf16 block: + ((4 j + g) ^ (l32 & 15)) * 16
+      const int wr8 = l32 * 128 + khalf * 4;  // fp8 block:  + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
+      const int rrow = lane >> 4, rchunk = lane & 15;
+      const int rrow8 = lane >> 3, rchunk8 = lane & 7;
+      float tile_amax = 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const u32x2 a = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
+                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = a;
+          }
+        }
+        {
+          u32x4 rb[8];
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int r = 4 * it + rrow;
+            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
+          }
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
+            global_store(AUX + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, rb[it]);
+          }
+        }
+        // the wavefront's LDS operations complete in order: the reads above are done before these writes land
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            float x[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float r = gelu_tanh_fast(t[g * 4 + q] * s);
+              // A chain of hardware max operations, pinned: written as compare + select, the compiler rebuilds
+              // the 256-element reduction as a tree and keeps far more values alive than there are registers.
+              // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
+              asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
+              // straight-line conversion: clamp, but hand a NaN to the converter as the positive canonical one,
+              // which it turns into 0x7F
+              const float y = r * cs;
+              x[q] = (y != y) ? __builtin_nanf("") : __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
+            }
+            const uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
+                x[2], x[3], __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
+            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) = w;
+          }
+        }
+        {
+          u32x4 rb[4];
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int r = 8 * it + rrow8;
+            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 128 + ((rchunk8 ^ ((r >> 1) & 7)) << 4));
+          }
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int m = m0 + wave_m * WM + i * 32 + 8 * it + rrow8;
+            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk8 * 16, rb[it]);
+          }
+        }
+      }
+      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
+      if (pr.c_amax != nullptr) {
+        const float am = wave_max(tile_amax);
+        if (lane == 0 && am > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= am)) atomic_max_nonneg(pr.c_amax, am);
+      }
     } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
