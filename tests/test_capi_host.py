@@ -152,6 +152,9 @@ def test_plan_grouped_gemm_layouts():
     assert rc(_prob([100], [264], [512], ldb=272), B) == -4      # n not a multiple of 16
     assert rc(_prob([100], [256], [520], ldb=256), B) == -4      # a is still fetched in 16-byte pieces of k
     assert rc(_prob([16], [65536], [65536], ldb=65536), B) == -2  # k * ldb >= 2^32
+    # rows up to 127 past k are addressed and must fall outside the 32-bit descriptor, not wrap: (k + 128) * ldb
+    assert rc(_prob([16], [65536], [65392], lda=65392, ldb=65536), B) == 0
+    assert rc(_prob([16], [65536], [65408], lda=65408, ldb=65536), B) == -2
     # a[k, m] and b[k, n]: k is a row count and may be anything; m and n multiples of 16
     assert rc(_prob([512], [256], [137], lda=512, ldb=256), A | B) == 0
     assert rc(_prob([512], [256], [137], lda=500, ldb=256), A | B) == -2
