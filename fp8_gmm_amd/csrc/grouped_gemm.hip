@@ -196,6 +196,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             float x[4];
+            uint32_t nan_bytes = 0;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const float r = gelu_tanh_fast(t[g * 4 + q] * s);
@@ -203,13 +204,15 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
               // the 256-element reduction as a tree and keeps far more values alive than there are registers.
               // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
               asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
-              // straight-line conversion: clamp, but hand a NaN to the converter as the positive canonical one,
-              // which it turns into 0x7F
+              // straight-line conversion (a branch here costs the register allocator its footing): clamp, convert,
+              // and patch the byte of a NaN to 0x7F afterwards (the median turns a NaN into -max)
               const float y = r * cs;
-              x[q] = (y != y) ? __builtin_nanf("") : __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
+              x[q] = __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
+              nan_bytes |= (y != y) ? (0xffu << (8 * q)) : 0u;
             }
-            const uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
+            uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
                 x[2], x[3], __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
+            w = (w & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
             *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) = w;
           }
         }

@@ -8,7 +8,7 @@ and exact equality wherever the arithmetic is exact (power-of-two data, identity
 import pytest
 import torch
 
-from helpers import assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
+from helpers import assert_bytes_equal, assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -553,3 +553,38 @@ def test_contraction_major_a_and_b_give_the_weight_gradient(dev, a_dtype):
         for i in range(e):
             ref32 = (dy2[bounds[i]: bounds[i + 1]].float().t() @ x2[bounds[i]: bounds[i + 1]].float()).to(torch.bfloat16)
             assert torch.equal(got[i].view(torch.int16), ref32.view(torch.int16)), f"rows {rows} expert {i}"
+
+
+@pytest.mark.gpu
+def test_gelu_epilogue_whole_line_stores_equal_the_per_group_path(dev):
+    """Interior tiles of the fused GELU form store through LDS; with a row pitch that is not a multiple of 16 every
+    tile takes the per-group path instead.  Same arithmetic, so the common columns must agree bit for bit -
+    saturated values and a NaN row included - and so must the amax (the extra weight rows are zero)."""
+    backend = _backend()
+    g = gen(4242)
+    m, k, n, extra = 700, 512, 1024, 8
+    a = _q(randn_bf16((m, k), g), E4M3)
+    a.view(torch.uint8)[3, 5] = 0x7F  # NaN: its whole output row
+    b = _q(randn_bf16((1, n, k), g), E4M3)
+    b_wide = torch.zeros(1, n + extra, k, dtype=torch.uint8).view(E4M3)
+    b_wide.view(torch.uint8)[:, :n] = b.view(torch.uint8)
+    gs = torch.tensor([m], dtype=torch.int64)
+    one = [torch.ones((), device=dev)]
+    scale = [torch.full((), 64.0, device=dev)]  # large enough for gelu(v) * scale to pass 448 here and there
+
+    def run(weights, cols):
+        c = torch.empty(m, cols, dtype=E4M3, device=dev)
+        pre = torch.empty(m, cols, dtype=torch.bfloat16, device=dev)
+        amax = [torch.zeros(1, device=dev)]
+        backend.fp8_gmm(a.to(dev), weights.to(dev), gs, one, one, c, E4M3, pre, scale, amax, False, False)
+        torch.cuda.synchronize()
+        return c.cpu(), pre.cpu(), amax[0].cpu()
+
+    c0, pre0, amax0 = run(b, n)
+    c1, pre1, amax1 = run(b_wide, n + extra)
+    assert (c0.view(torch.uint8) == 0x7E).any(), "the case is meant to contain saturated values"
+    assert (c0.view(torch.uint8)[3] == 0x7F).all(), "NaN row"
+    assert_bytes_equal(c0, c1[:, :n].contiguous(), "fp8 gelu output")
+    assert_bytes_equal(pre0.view(torch.int16), pre1[:, :n].contiguous().view(torch.int16), "pre-gelu output")
+    assert_scalar_bits_equal(amax0, amax1, "amax")
+    assert torch.isfinite(amax0).all() and amax0.item() > 0
