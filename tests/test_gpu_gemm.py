@@ -588,3 +588,25 @@ def test_gelu_epilogue_whole_line_stores_equal_the_per_group_path(dev):
     assert_bytes_equal(pre0.view(torch.int16), pre1[:, :n].contiguous().view(torch.int16), "pre-gelu output")
     assert_scalar_bits_equal(amax0, amax1, "amax")
     assert torch.isfinite(amax0).all() and amax0.item() > 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("a_dtype", [E4M3, E5M2], ids=["e4m3", "e5m2"])
+def test_bf16_epilogue_whole_line_stores_equal_the_per_group_path(dev, a_dtype):
+    """The same for the plain bf16 output: interior tiles go through LDS, a row pitch that is not a multiple of 8
+    sends every tile down the per-group path; the common columns must agree bit for bit (NaN row included)."""
+    backend = _backend()
+    g = gen(4243)
+    m, k, n, extra = 700, 384, 768, 4
+    a = _q(randn_bf16((m, k), g), a_dtype)
+    a.view(torch.uint8)[300, 7] = 0x7F  # NaN in both formats
+    b = _q(randn_bf16((1, n, k), g), E4M3)
+    b_wide = torch.zeros(1, n + extra, k, dtype=torch.uint8).view(E4M3)
+    b_wide.view(torch.uint8)[:, :n] = b.view(torch.uint8)
+    gs = torch.tensor([m], dtype=torch.int64)
+    sa, sb = [torch.full((), 0.37, device=dev)], [torch.full((), 1.9, device=dev)]
+    c0 = backend.fp8_gmm(a.to(dev), b.to(dev), gs, sa, sb)
+    c1 = backend.fp8_gmm(a.to(dev), b_wide.to(dev), gs, sa, sb)
+    torch.cuda.synchronize()
+    assert torch.isnan(c0[300].float()).all()
+    assert_bytes_equal(c0.cpu().view(torch.int16), c1[:, :n].contiguous().cpu().view(torch.int16), "bf16 output")
