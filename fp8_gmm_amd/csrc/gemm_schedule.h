@@ -24,10 +24,10 @@ constexpr int kNumXcd = 8;
 // ---- tail balancing (stream-K over the remainder of an XCD's tile range) ----
 // A range of n tiles on W workgroups takes ceil(n / W) rounds; when the last round is mostly empty the
 // remainder tiles (plus one full round when there are very few of them) are cut along K instead: the
-// region's K = 128 pair steps are dealt out in W equal contiguous pieces.  A piece that does not cover
+// region's K = 128 steps are dealt out in W equal contiguous pieces.  A piece that does not cover
 // a whole tile leaves its fp32 accumulators in a workspace slot; a second, small kernel adds the pieces
 // of such a tile in K order and runs the normal epilogue.  No workgroup ever waits for another one.
-constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many pair steps
+constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many K = 128 steps
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
 constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
 constexpr int kPartialBytes = BM * BN * 4;  // one slot: the fp32 accumulators of one tile
@@ -42,7 +42,7 @@ struct Sched {
   int dp_rounds;               // workgroup j takes tiles range_begin + j + wgs * i, i < dp_rounds
   int sk_begin;                // first tile of the stream-K region (== range_end: none)
   int sk_wgs;                  // workgroups that take a piece of the region
-  int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (pair steps)
+  int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (K = 128 steps)
   int64_t total_cost;          // cost of all tiles
 };
 
@@ -58,7 +58,7 @@ FP8GMM_HD int problem_of_tile(const Sched& s, int tile) {
   }
   return lo;
 }
-// A tile of problem p costs ceil(k / 128) pair steps (1 for k = 0: its epilogue still has to run).
+// A tile of problem p costs ceil(k / 128) main-loop steps (1 for k = 0: its epilogue still has to run).
 FP8GMM_HD int64_t tile_cost(const Sched& s, int p) {
   const int c = (s.probs[p].k + 127) / 128;
   return (int64_t)(c > 0 ? c : 1);
@@ -160,7 +160,7 @@ FP8GMM_HD void tile_origin(int m, int n, int local, int* m0, int* n0) {
 
 struct Item {
   int tile, prob, m0, n0;
-  int k_begin, nk;  // pair steps: first one, how many (0 for a problem without K)
+  int k_begin, nk;  // K = 128 steps: first one, how many (0 for a problem without K)
   int slot;         // workspace slot of a partial piece, -1: the piece is the whole tile
 };
 struct Cursor {
@@ -214,7 +214,7 @@ FP8GMM_HD void cursor_advance(const Sched& s, int j, Cursor& c) {
 
 // The tile that the workgroup of piece boundary j (1 <= j < sk_wgs) completes in the fix-up pass, or -1:
 // the FIRST boundary strictly inside a tile owns it.  `first_piece_wg` is the workgroup that holds the piece
-// from the tile's first pair step (slot kSlotsPerWg * wg + 1); the following pieces come from workgroups
+// from the tile's first K step (slot kSlotsPerWg * wg + 1); the following pieces come from workgroups
 // j, j + 1, ... (slot kSlotsPerWg * wg) while their boundary lies inside the tile.
 FP8GMM_HD int fixup_tile(const Sched& s, int j, int* n_following) {
   *n_following = 0;

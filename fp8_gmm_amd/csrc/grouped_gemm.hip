@@ -738,7 +738,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 
 // Completes the tiles that the main kernel shared along K.  One workgroup per interior piece boundary of
 // every XCD's stream-K region; the FIRST boundary that falls strictly inside a tile owns that tile: it adds
-// the pieces in K order (workgroup j - 1 holds the piece from the tile's first pair step, workgroups j,
+// the pieces in K order (workgroup j - 1 holds the piece from the tile's first K step, workgroups j,
 // j + 1, ... the following ones) and applies the epilogue.
 // 1024 threads: thread T owns the 16-byte groups T + 1024 q (q = 0..15) of a slot, i.e. register group g = T / 256
 // of every MFMA tile (i, j) = q of main-kernel thread T % 256: 4 consecutive columns of one row each.  The sums and
