@@ -346,18 +346,15 @@ def main():
                                      "source": "pp_dpm_sclk and hwmon power1_input (sysfs), 1 ms period, over 40 "
                                                "extra steps"}}
     # ... and the clock the GEMM launches really ran at: cycles / time counted inside a measurement build of the
-    # kernel by the first workgroup of every XCD (fp8gmm_gemm_clock_probe), over 5 more steps
+    # kernel by the first workgroup of every XCD (fp8gmm_grouped_gemm_timed), over 5 more steps
     if roofline is not None and not args.headline_only:
-        from fp8_gmm_amd import _lib
+        from fp8_gmm_amd import backend
 
         counters = torch.zeros(32, dtype=torch.int64, device=dev)
-        _lib.check(_lib.load().fp8gmm_gemm_clock_probe(counters.data_ptr()))
-        try:
+        with backend.gemm_clock_probe(counters):
             for _ in range(5):
                 step()
             torch.cuda.synchronize()
-        finally:
-            _lib.check(_lib.load().fp8gmm_gemm_clock_probe(None))
         c = counters.cpu().reshape(8, 4).to(torch.float64)
         if (c[:, 3] > 0).all():
             per_xcd = (c[:, 2] / c[:, 3] * 100.0).tolist()

@@ -69,11 +69,54 @@ GEMM_PROBLEM = np.dtype(
     align=False,
 )
 
+# struct fp8gmm_gemm_item (64 bytes): one record of a launch's work list
+GEMM_ITEM = np.dtype(
+    [
+        ("a", "<u8"),
+        ("b", "<u8"),
+        ("a_bytes", "<u4"),
+        ("b_bytes", "<u4"),
+        ("lda", "<i4"),
+        ("ldb", "<i4"),
+        ("k", "<i4"),
+        ("k_begin", "<i4"),
+        ("nk", "<i4"),
+        ("m0", "<i4"),
+        ("n0", "<i4"),
+        ("prob", "<i4"),
+        ("slot", "<i4"),
+        ("reserved", "<i4"),
+    ],
+    align=False,
+)
+
+# struct fp8gmm_gemm_fixup_desc (32 bytes): one tile that was shared along K
+GEMM_FIXUP = np.dtype(
+    [("prob", "<i4"), ("m0", "<i4"), ("n0", "<i4"), ("first_slot", "<i4"), ("n_pieces", "<i4"),
+     ("reserved", "<i4", (3,))],
+    align=False,
+)
+
+GEMM_SLOT_BYTES = 262144
+
+
+class GemmPlan(ctypes.Structure):
+    """struct fp8gmm_gemm_plan"""
+
+    _fields_ = [("grid", ctypes.c_int32), ("rounds", ctypes.c_int32), ("n_fixups", ctypes.c_int32),
+                ("n_slots", ctypes.c_int32), ("total_tiles", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
+
+
 EXPORTS = (
     "fp8gmm_version",
     "fp8gmm_status_string",
     "fp8gmm_sizeof_tensor_desc",
     "fp8gmm_sizeof_gemm_problem",
+    "fp8gmm_sizeof_gemm_item",
+    "fp8gmm_init",
+    "fp8gmm_gemm_grid",
+    "fp8gmm_plan_grouped_gemm_launch",
+    "fp8gmm_grouped_gemm_timed",
     "fp8gmm_gemm_tile_shape",
     "fp8gmm_plan_multi_tensor",
     "fp8gmm_plan_grouped_gemm",
@@ -86,7 +129,6 @@ EXPORTS = (
     "fp8gmm_multi_cast_dgelu",
     "fp8gmm_grouped_gemm",
     "fp8gmm_delayed_scaling_update",
-    "fp8gmm_gemm_clock_probe",
     "fp8gmm_route_workspace_bytes",
     "fp8gmm_route_sort",
     "fp8gmm_route_invert",
@@ -149,10 +191,19 @@ def load():
     L.fp8gmm_multi_pad_cast_transpose_dgelu.argtypes = [vp, ci, ci, ci, vp]
     L.fp8gmm_multi_cast_dgelu.restype = ci
     L.fp8gmm_multi_cast_dgelu.argtypes = [vp, ci, ci, ci, vp]
+    L.fp8gmm_sizeof_gemm_item.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_gemm_item.argtypes = []
+    L.fp8gmm_init.restype = ci
+    L.fp8gmm_init.argtypes = [ci]
+    L.fp8gmm_gemm_grid.restype = ci
+    L.fp8gmm_gemm_grid.argtypes = [ci]
+    pp = ctypes.POINTER(GemmPlan)
+    L.fp8gmm_plan_grouped_gemm_launch.restype = ci
+    L.fp8gmm_plan_grouped_gemm_launch.argtypes = [vp, ci, ci, ci, ci, vp, ci, vp, ci, pp]
     L.fp8gmm_grouped_gemm.restype = ci
-    L.fp8gmm_grouped_gemm.argtypes = [vp, ci, ci, ci, ci, ci, ci, vp]
-    L.fp8gmm_gemm_clock_probe.restype = ci
-    L.fp8gmm_gemm_clock_probe.argtypes = [vp]
+    L.fp8gmm_grouped_gemm.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp]
+    L.fp8gmm_grouped_gemm_timed.restype = ci
+    L.fp8gmm_grouped_gemm_timed.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp, vp]
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t
@@ -171,7 +222,8 @@ def load():
     L.fp8gmm_gemm_schedule.argtypes = [vp, ci, ci, ci, ci, ci, vp, ci]
     L.fp8gmm_gemm_fixup.restype = ci
     L.fp8gmm_gemm_fixup.argtypes = [vp, ci, ci, ci, ci, ip, vp, ci]
-    if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize:
+    if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize \
+            or L.fp8gmm_sizeof_gemm_item() != GEMM_ITEM.itemsize or ctypes.sizeof(GemmPlan) != 32:
         raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
     _lib = L
     return L
@@ -193,6 +245,52 @@ def plan_grouped_gemm(table, layout=0):
     total = ctypes.c_int(0)
     check(load().fp8gmm_plan_grouped_gemm_layout(table.ctypes.data, len(table), layout, ctypes.byref(total)))
     return total.value
+
+
+def plan_grouped_gemm_launch(table, layout, grid, stream_k):
+    """Validate a host problem table and write the work list of a launch with `grid` workgroups.
+    Returns (GemmPlan, items, fixups): numpy arrays of GEMM_ITEM [rounds * grid] and GEMM_FIXUP [n_fixups]."""
+    L = load()
+    plan = GemmPlan()
+    n = len(table)
+    # first guess: striding needs ceil(tiles / grid) records per workgroup, tail sharing a few more
+    guess = (int(np.ceil(max(1, _tiles_upper_bound(table)) / grid)) + 6) * grid
+    items = np.empty(guess, dtype=GEMM_ITEM)
+    fixups = np.empty(grid, dtype=GEMM_FIXUP)
+    rc = L.fp8gmm_plan_grouped_gemm_launch(table.ctypes.data, n, layout, grid, int(bool(stream_k)), items.ctypes.data,
+                                           len(items), fixups.ctypes.data, len(fixups), ctypes.byref(plan))
+    if rc == -8:  # FP8GMM_ERR_BUFFER_TOO_SMALL: the sizes are in the plan
+        items = np.empty(plan.rounds * plan.grid, dtype=GEMM_ITEM)
+        fixups = np.empty(max(1, plan.n_fixups), dtype=GEMM_FIXUP)
+        rc = L.fp8gmm_plan_grouped_gemm_launch(table.ctypes.data, n, layout, grid, int(bool(stream_k)),
+                                               items.ctypes.data, len(items), fixups.ctypes.data, len(fixups),
+                                               ctypes.byref(plan))
+    check(rc)
+    return plan, items[: plan.rounds * plan.grid], fixups[: plan.n_fixups]
+
+
+def _tiles_upper_bound(table):
+    m = table["m"].astype(np.int64)
+    n = table["n"].astype(np.int64)
+    return int((((m + 255) // 256) * ((n + 255) // 256)).clip(min=0).sum())
+
+
+_num_cu = {}
+
+
+def init(device_index):
+    """fp8gmm_init once per device: compute-unit count (cached)."""
+    cus = _num_cu.get(device_index)
+    if cus is None:
+        cus = load().fp8gmm_init(device_index)
+        if cus <= 0:
+            check(cus if cus < 0 else -7)
+        _num_cu[device_index] = cus
+    return cus
+
+
+def gemm_grid(num_cu):
+    return load().fp8gmm_gemm_grid(num_cu)
 
 
 def gemm_schedule(table, total_tiles, grid, stream_k, wg, max_items=4096):

@@ -1,7 +1,7 @@
 // Work decomposition of the grouped GEMM: which (tile, K range) items a workgroup processes, in which
 // order, and which workgroup completes a tile that several workgroups shared along K.  Pure integer
-// arithmetic on the problem table, compiled for the device (the kernels) and for the host (the
-// introspection entry point the CPU tests use), so both see exactly the same schedule.
+// arithmetic on the problem table.  It runs on the host: fp8gmm_plan_grouped_gemm_launch (plan.cpp) writes the
+// schedule out as the work list the kernels read, and the introspection entry points show it to the CPU tests.
 #pragma once
 
 #include <stdint.h>
@@ -16,10 +16,6 @@
 #endif
 
 namespace fp8gmm {
-
-constexpr int BM = kGemmTileM;  // 256
-constexpr int BN = kGemmTileN;  // 256
-constexpr int kNumXcd = 8;
 
 // ---- tail balancing (stream-K over the remainder of an XCD's tile range) ----
 // A range of n tiles on W workgroups takes ceil(n / W) rounds; when the last round is mostly empty the

@@ -1,745 +1,17 @@
-// Persistent FP8 grouped GEMM for gfx950 (MI355X).
+// C-ABI entry points of the grouped GEMM and the kernel that completes tiles shared along K.  The main kernel
+// lives in grouped_gemm_kernel.h and is instantiated per operand format / layout in gemm_variant.hip.
 //
-// Replaces the reference's CUTLASS grouped GEMM (csrc/fp8_gmm.cu:82-205) and its
-// per-expert cuBLASLt loops (fp8_gmm/backend.py:84-96, grouped_linear.py:173-182,
-// grouped_mlp.py:234-242,313-322) with ONE launch over a device-side problem table.
-//
-//   c[m, n] = epilogue( sum_k a[m, k] * b[n, k] ),   a, b fp8 (K contiguous), fp32 accumulation
-//
-// Work decomposition
-//   * the output of every problem is cut into 256 x 256 tiles; all tiles of all problems form
-//     one list walked by a persistent grid (one workgroup per CU).  The list is split into 8
-//     contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so that workgroups that
-//     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest within
-//     groups of 8 rows of tiles, so one round of an XCD's 32 workgroups is an 8 x 4 block of tiles.
-//   * a workgroup is 4 wavefronts (2 along m x 2 along n), one per SIMD; a wavefront owns a
-//     128 x 128 sub-tile = 4 x 4 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4.  Its 256 accumulators
-//     live in the accumulation registers, the other 256 registers hold fragments and addresses.
-//     The weight operand is MFMA source 0 and the token operand source 1: every lane then
-//     holds 4 consecutive output columns of one row.
-//
-// Data movement
-//   * operands go global -> LDS directly (`buffer_load_dwordx4 ... lds`), never through
-//     registers.  Buffer descriptors bound every operand, so rows past m / n and K tails read
-//     as zeros: m, n are arbitrary and k only has to be a multiple of 16.
-//   * a main-loop step consumes K = 128: one 128-byte line of each of the tile's 256 token rows
-//     and 256 weight rows.  LDS (all 160 KB) is a ring of five 32 KB units, a unit being the
-//     256 rows x 128 B of ONE operand for one step, its eight 16-byte chunks XOR-swizzled with
-//     (row >> 1) & 7 so that the 16-byte fragment reads of a wavefront are conflict-free.  Every
-//     load instruction fetches 8 whole lines (two half-line requests for one line, issued apart,
-//     meet in the L1 as a hit on a pending miss and stall it).
-//   * at any time the ring holds the units of the step being computed, of the next step, and
-//     the tokens of the step after; that step's weights replace the current tokens once the
-//     step's barrier has shown that every wavefront has read them.  The token loads of step + 2
-//     are issued during the low K half of a step, the weight loads during the high half, one
-//     after every second MFMA.
-//   * the load stream and the ring run CONTINUOUSLY across tile boundaries: while a tile's
-//     epilogue stores its result, the next tile's first two steps are already in LDS.
-//   * ONE s_barrier per step, between its two K = 64 halves.  The fragments of a half are read
-//     from LDS during the half before it, interleaved with the MFMAs (pinned with sched_barrier).
-//     With a single wavefront per SIMD nothing else fills an MFMA pipe, so whatever sits between
-//     two MFMAs has to issue within the 64 cycles the first one runs: addresses are two
-//     instructions per load, the load cursor advances without branches while it stays inside an
-//     item, and the scheduler arithmetic of an item switch runs once per tile.
-//   * epilogue: scale, convert, and - for interior bf16 tiles - a pass through the free ring unit
-//     that turns the MFMA layout into whole-line stores.
-#include <atomic>
-#include <cstdlib>
-#include <map>
-#include <mutex>
-#include <type_traits>
-#include <utility>
-
-#include "device_utils.h"
-#include "gemm_schedule.h"
-#include "tiling.h"
+// Replaces the reference's CUTLASS grouped GEMM (csrc/fp8_gmm.cu:82-205) and its per-expert cuBLASLt loops
+// (fp8_gmm/backend.py:84-96, grouped_linear.py:173-182, grouped_mlp.py:234-242,313-322) with ONE launch over
+// device-side tables written by the host planner (plan.cpp).
+#include "grouped_gemm_kernel.h"
 
 namespace fp8gmm {
 namespace {
 
-constexpr int BK = kGemmTileK;    // bytes of K per main-loop step: one 128-byte line of every operand row
-constexpr int US = BM * BK;       // 32768 bytes per ring unit: the 256 rows of ONE operand for one step
-constexpr int RING = 5;
-static_assert(BM == BN, "token and weight units share one size");
-constexpr int NWAVES = 4;         // one wavefront per SIMD: 256 accumulator + 256 other registers per lane
-constexpr int NTHREADS = 64 * NWAVES;
-constexpr int WM = 128, WN = 128;  // wavefront sub-tile
-constexpr int WAVES_N = BN / WN;  // wavefronts along n: 2 (x 2 along m)
-constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
-constexpr int NT = WN / 32;       // 4 MFMA tiles along n per wave
-constexpr int kParts = US / 1024 / NWAVES;  // buffer_load ... lds instructions (1 KB each) per wavefront per unit: 8
-constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the interior bf16 epilogue (8 per 32-row block)
-
-typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-
-#define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
-#define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
-#define FP8GMM_WAIT_VM_LGKM(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(n) : "memory")
-// global -> LDS: lane i's 16 bytes land at M0 + 16 i; out-of-range offsets deliver zeros
-#define FP8GMM_DMA(lds_addr, voff, rsrc) \
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
-
-// One MFMA tile's accumulators as ordinary vector registers.  In the main kernel the 256 accumulators of a
-// lane live in the accumulation registers (the other 256 hold fragments and addresses); vector arithmetic
-// cannot read those, and left to itself the register allocator parks them in scratch memory on the way.
-// Reading them 16 at a time, where they are used, keeps the epilogue within the register file.
-__device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
-  f32x16 t;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
-  return t;
-}
-
-// Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
-// stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
-// `stage`: 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of the staged path.
-__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
-                                              int out_kind, int epilogue, uint8_t* stage) {
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
-  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-  const int l32 = lane & 31, khalf = lane >> 5;
-  const int M = pr.m, N = pr.n;
-  bool fast = false;
-    const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
-    const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
-    const float s = sa_inv * sb_inv;
-    const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
-    const int64_t ldc = pr.ldc;
-    float amax = 0.f;
-    const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
-    if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
-        ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
-      // Interior tile, plain bf16 output: straight-line code with an exact store count.
-      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
-      // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
-      // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
-      // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
-      // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
-      // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
-      uint8_t* mine = stage + wave * 8192;
-      const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
-      const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
-                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
-            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
-          }
-        }
-        // only this wavefront touches `mine`: its own LDS operations complete in order
-        u32x4 v[8];
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const int r = 4 * it + rrow;
-          v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
-        }
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
-          global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
-        }
-      }
-      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
-      fast = true;
-    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && interior && ((ldc & 15) == 0) &&
-               ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0) && ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0)) {
-      // Interior tile of the fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
-      // outputs go through the staging area like the plain form's, one 32-row block at a time - first the bf16
-      // block as 32 rows x 256 B, then, in a second pass over the same accumulators, the fp8 block as 32 rows x
-      // 128 B (chunk c of row r at chunk c ^ ((r >> 1) & 7)) - so that every store instruction writes whole
-      // lines: 12 per block instead of 32 that touch 32 rows each.
-      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
-      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
-      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
-      uint8_t* mine = stage + wave * 8192;
-      const int wr = l32 * 256 + khalf * 8;   // bf16 block: + ((4 j + g) ^ (l32 & 15)) * 16
-      const int wr8 = l32 * 128 + khalf * 4;  // fp8 block:  + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
-      const int rrow = lane >> 4, rchunk = lane & 15;
-      const int rrow8 = lane >> 3, rchunk8 = lane & 7;
-      float tile_amax = 0.f;
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const u32x2 a = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
-                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
-            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = a;
-          }
-        }
-        {
-          u32x4 rb[8];
-#pragma unroll
-          for (int it = 0; it < 8; ++it) {
-            const int r = 4 * it + rrow;
-            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
-          }
-#pragma unroll
-          for (int it = 0; it < 8; ++it) {
-            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
-            global_store(AUX + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, rb[it]);
-          }
-        }
-        // the wavefront's LDS operations complete in order: the reads above are done before these writes land
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float x[4];
-            uint32_t nan_bytes = 0;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const float r = gelu_tanh_fast(t[g * 4 + q] * s);
-              // A chain of hardware max operations, pinned: written as compare + select, the compiler rebuilds
-              // the 256-element reduction as a tree and keeps far more values alive than there are registers.
-              // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
-              asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
-              // straight-line conversion (a branch here costs the register allocator its footing): clamp, convert,
-              // and patch the byte of a NaN to 0x7F afterwards (the median turns a NaN into -max)
-              const float y = r * cs;
-              x[q] = __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
-              nan_bytes |= (y != y) ? (0xffu << (8 * q)) : 0u;
-            }
-            uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
-                x[2], x[3], __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
-            w = (w & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
-            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) = w;
-          }
-        }
-        {
-          u32x4 rb[4];
-#pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int r = 8 * it + rrow8;
-            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 128 + ((rchunk8 ^ ((r >> 1) & 7)) << 4));
-          }
-#pragma unroll
-          for (int it = 0; it < 4; ++it) {
-            const int m = m0 + wave_m * WM + i * 32 + 8 * it + rrow8;
-            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk8 * 16, rb[it]);
-          }
-        }
-      }
-      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
-      if (pr.c_amax != nullptr) {
-        const float am = wave_max(tile_amax);
-        if (lane == 0 && am > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= am)) atomic_max_nonneg(pr.c_amax, am);
-      }
-    } else if (out_kind == FP8GMM_OUT_BF16) {
-      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
-      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
-      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) &&
-                       (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const int m = m0 + wave_m * WM + i * 32 + l32;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
-            if (m >= M || n >= N) continue;
-            float v[4], r[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              v[q] = t[g * 4 + q] * s;
-              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
-            }
-            const int64_t off = (int64_t)m * ldc + n;
-            if (vec && n + 3 < N) {
-              u32x2 o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
-              global_store(C + off, o);
-              if (gelu && AUX != nullptr) {
-                u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-                global_store(AUX + off, a);
-              }
-            } else {
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                if (n + q < N) {
-                  global_store(C + off + q, (uint16_t)f32_to_bf16_bits(r[q]));
-                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
-                }
-              }
-            }
-          }
-        }
-      }
-    } else {
-      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
-      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
-      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
-      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 3) == 0) &&
-                       (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const int m = m0 + wave_m * WM + i * 32 + l32;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
-            if (m >= M || n >= N) continue;
-            float v[4], r[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              v[q] = t[g * 4 + q] * s;
-              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
-              if (n + q < N) amax = amax_step(amax, r[q]);
-            }
-            uint32_t w;
-            if (out_kind == FP8GMM_E4M3) {
-              w = cvt4_fp8<FP8GMM_E4M3>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
-            } else {
-              w = cvt4_fp8<FP8GMM_E5M2>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
-            }
-            const int64_t off = (int64_t)m * ldc + n;
-            if (vec && n + 3 < N) {
-              global_store(C + off, w);
-              if (gelu && AUX != nullptr) {
-                u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
-                global_store(AUX + off, a);
-              }
-            } else {
-#pragma unroll
-              for (int q = 0; q < 4; ++q) {
-                if (n + q < N) {
-                  global_store(C + off + q, (uint8_t)(w >> (8 * q)));
-                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
-                }
-              }
-            }
-          }
-        }
-      }
-      if (pr.c_amax != nullptr) {
-        amax = wave_max(amax);
-        // amax only grows: once the slot holds a value at or above this wavefront's, the atomic is redundant
-        // (the slots of all experts share a cache line, and atomics on one line serialise)
-        if (lane == 0 && amax > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= amax))
-          atomic_max_nonneg(pr.c_amax, amax);
-      }
-    }
-    return fast;
-}
-
-// Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
-// (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
-__device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* slot) {
-  float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
-        global_store(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4), v);
-      }
-    }
-}
-// Measurement hook (fp8gmm_gemm_clock_probe): 8 x 4 uint64 of device memory, or null.
-__device__ uint64_t* volatile d_clock_probe = nullptr;
-
-// PROBE: measurement build of the same kernel.  The first workgroup of every XCD writes its shader-cycle counter
-// and the constant 100 MHz counter when it starts and adds the differences to two running totals when it ends,
-// so that the caller can derive the clock the launches really ran at (the counters of different compute units are
-// not comparable, hence the same workgroup takes both readings).  The production build (PROBE = false) contains none of it.
-template <bool PROBE>
-__device__ __forceinline__ void clock_probe_mark(int which) {
-  if constexpr (PROBE) {
-    if (blockIdx.x < kNumXcd && threadIdx.x == 0) {
-      volatile uint64_t* const p = d_clock_probe;
-      if (p != nullptr) {
-        volatile uint64_t* const q = p + 4 * blockIdx.x;
-        const uint64_t cycles = (uint64_t)clock64(), ticks = (uint64_t)wall_clock64();
-        if (which == 0) {
-          q[0] = cycles;
-          q[1] = ticks;
-        } else {  // totals over all launches since the counters were cleared
-          q[2] += cycles - q[0];
-          q[3] += ticks - q[1];
-        }
-      }
-    }
-  }
-}
-
-// B_TR: operand b is stored contraction-major, b[k][n] with n contiguous and pitch ldb (the layout of a weight
-// stack [N_out.., ] seen from the data-gradient GEMM), instead of b[n][k].  Its ring unit then holds 128
-// contraction rows of 256 bytes; the 16-byte chunk c of row r sits at chunk c ^ 2 (r mod 8), and a fragment is
-// gathered with four transposing reads (ds_read_b64_tr_b8: in a group of 16 lanes, lane 8 h + i receives byte i
-// of the 8 bytes addressed by lanes 2 b + h, b = 0..7).  Everything else - schedule, MFMA order, epilogue -
-// is shared, so both layouts produce the same bits.
-// A_TR: the same for operand a (a[k][m], pitch lda): with both, c = a^T . b contracts over the rows of two
-// row-major matrices, which is the weight-gradient GEMM on the un-transposed activations and gradients; rows
-// past k read as zeros, so the contraction length needs no padding.
-template <int A_FMT, int B_FMT, bool PROBE, bool A_TR, bool B_TR>
-__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
-                                                                int nprob, int total_tiles, int out_kind,
-                                                                int epilogue, uint8_t* __restrict__ workspace) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-  clock_probe_mark<PROBE>(0);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: what depends on it stays in scalar registers
-  const int wave_m = wave / WAVES_N;  // 0..1
-  const int wave_n = wave % WAVES_N;  // 0..1
-  const int l32 = lane & 31;
-  const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
-  const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
-
-  // DMA lane map, row-major operand: one wavefront instruction fills 8 rows x 128 B of a unit, i.e. whole
-  // cache lines: lane -> row lane >> 3 of the group, slot chunk lane & 7.  Chunk c of row r is kept at chunk
-  // c ^ ((r >> 1) & 7); for the rows of group wave + NWAVES j that is ((wave & 1) * 4 + (lane >> 4)) & 7, so the
-  // GLOBAL chunk that has to land in slot chunk lane & 7 is a per-lane constant.
-  const int drow = lane >> 3;
-  const int dchunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
-  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 128 + 32 j + l32
-  // (source 0); K half hh, lane half khalf -> chunks 4 hh + 2 khalf + {0, 1}; (row >> 1) & 7 = (l32 >> 1) & 7
-  const int fsw = (l32 >> 1) & 7;
-  int fc[2][2];
-#pragma unroll
-  for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-    for (int q = 0; q < 2; ++q) fc[hh][q] = ((4 * hh + 2 * khalf + q) ^ fsw) << 4;
-  const int fa_off = (wave_m * WM + l32) * BK;
-  const int fb_off = (wave_n * WN + l32) * BK;
-  // contraction-major unit: 128 contraction rows x 256 B.  Fragment of K half hh: rows 64 hh + 32 khalf + b (+ 8 t
-  // per read), logical chunk wave_n * 8 + 2 j + g, byte 8 h; s = lane % 16 = 2 b + h
-  const int tr_b = (lane & 15) >> 1, tr_h = lane & 1, tr_g = (lane >> 4) & 1;
-  const int tr_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
-  int fbt_off[NT];
-#pragma unroll
-  for (int j = 0; j < NT; ++j) fbt_off[j] = tr_row + (((wave_n * 8 + 2 * j + tr_g) ^ (2 * tr_b)) << 4);
-  int fat_off[MT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
-
-  // ---- this workgroup's item sequence (uniform): strided tiles of its XCD's range, then its piece of
-  // the range's stream-K region ----
-  const int xcd = blockIdx.x % kNumXcd;
-  const int wg_in_xcd = blockIdx.x / kNumXcd;
-  Sched sch;
-  sched_init(sch, probs, nprob, total_tiles, xcd, gridDim.x / kNumXcd, workspace != nullptr);  // gridDim.x % 8 == 0
-  Cursor c_cp, c_ld;
-  cursor_init(sch, wg_in_xcd, c_cp);
-  if (!cursor_valid(sch, wg_in_xcd, c_cp)) return;
-  c_ld = c_cp;
-
-  // ---- load side: runs two steps ahead of the compute side, possibly in the next tile ----
-  bool ld_live = true;  // the load cursor still points at an item
-  int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
-  [[maybe_unused]] int ld_lda = 0, ld_ldb = 0;  // contraction-major operands only
-  i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
-  // Addresses of the K = 128 step the load cursor points at: part j of an operand is fetched from a_k + j * a_step
-  // (byte offsets into the operand's buffer, a_step uniform).  Rows past m / n are not masked: whatever they
-  // deliver only reaches accumulators of rows / columns that the epilogue never stores, and the descriptor keeps
-  // the access inside the operand.  The K tail is: a row-major lane whose 16-byte chunk lies past k gets an
-  // out-of-range offset (zero fill); contraction rows past k are out of the descriptor's range by themselves.
-  uint32_t a_base = 0, b_base = 0, a_step = 0, b_step = 0, a_k = 0, b_k = 0;
-  bool k_ok = false;  // row-major operands: this lane's chunk of the step exists
-  auto step_setup = [&]() {
-    const uint32_t k0 = (uint32_t)ld_kt * BK;
-    if constexpr (A_TR) {
-      a_k = a_base + k0 * (uint32_t)ld_lda;  // k * pitch < 2^32 is checked when the table is planned
-    } else {
-      a_k = a_base + k0;
-    }
-    if constexpr (B_TR) {
-      b_k = b_base + k0 * (uint32_t)ld_ldb;
-    } else {
-      b_k = b_base + k0;
-    }
-    k_ok = (int)k0 < ld_kmax;
-  };
-  auto load_setup = [&]() {
-    while ((ld_live = cursor_valid(sch, wg_in_xcd, c_ld))) {
-      const Item g = cursor_item(sch, xcd, wg_in_xcd, c_ld);
-      if (g.nk > 0) {
-        const fp8gmm_gemm_problem pr = probs[g.prob];
-        const uint64_t pa = (uint64_t)pr.a, pb = (uint64_t)pr.b;
-        const uint64_t sa = (uint64_t)(A_TR ? pr.k : pr.m) * (uint64_t)pr.lda;
-        const uint64_t sb = (uint64_t)(B_TR ? pr.k : pr.n) * (uint64_t)pr.ldb;  // rows of b times its pitch
-        rsrc_a[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pa);
-        rsrc_a[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pa >> 32));
-        rsrc_a[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sa > 0xffffffffull ? 0xffffffffull : sa));
-        rsrc_b[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)pb);
-        rsrc_b[1] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(pb >> 32));
-        rsrc_b[2] = __builtin_amdgcn_readfirstlane((int)(uint32_t)(sb > 0xffffffffull ? 0xffffffffull : sb));
-        // row-major operand: part j = rows (wave + NWAVES j) * 8 + drow of the tile.
-        // contraction-major operand: one instruction fills 4 contraction rows x 256 B: part j = rows
-        // (wave + NWAVES j) * 4 + lane / 16 of the unit, slot chunk lane % 16, which must receive global chunk
-        // p ^ 2 (row mod 8); row mod 8 is the same for every j.
-        const int krow = wave * 4 + (lane >> 4);
-        const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
-        if constexpr (!A_TR) {
-          a_base = (uint32_t)(g.m0 + wave * 8 + drow) * (uint32_t)pr.lda + dchunk * 16;
-          a_step = NWAVES * 8 * (uint32_t)pr.lda;
-        } else {
-          a_base = (uint32_t)krow * (uint32_t)pr.lda + (uint32_t)(g.m0 + tr_col);
-          a_step = NWAVES * 4 * (uint32_t)pr.lda;
-          ld_lda = pr.lda;
-        }
-        if constexpr (!B_TR) {
-          b_base = (uint32_t)(g.n0 + wave * 8 + drow) * (uint32_t)pr.ldb + dchunk * 16;
-          b_step = NWAVES * 8 * (uint32_t)pr.ldb;
-        } else {
-          b_base = (uint32_t)krow * (uint32_t)pr.ldb + (uint32_t)(g.n0 + tr_col);
-          b_step = NWAVES * 4 * (uint32_t)pr.ldb;
-          ld_ldb = pr.ldb;
-        }
-        ld_kmax = pr.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
-        ld_kt = g.k_begin;
-        ld_nk = g.k_begin + g.nk;
-        step_setup();
-        return;
-      }
-      cursor_advance(sch, wg_in_xcd, c_ld);  // an item without K work needs no loads
-    }
-    // Past the end of the stream the loads are issued all the same, against empty descriptors (zero fill),
-    // which keeps the vmcnt arithmetic uniform.
-    rsrc_a[2] = 0;
-    rsrc_b[2] = 0;
-  };
-  // One instruction of that step: part j (0..7) of the token operand into ring unit `unit`, or of the weights.
-  auto dma_a = [&](int unit, int j) {
-    uint32_t v = a_k + j * a_step;
-    if constexpr (!A_TR) v = k_ok ? v : 0xffffffffu;
-    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
-    FP8GMM_DMA(l, v, rsrc_a);
-  };
-  auto dma_b = [&](int unit, int j) {
-    uint32_t v = b_k + j * b_step;
-    if constexpr (!B_TR) v = k_ok ? v : 0xffffffffu;
-    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
-    FP8GMM_DMA(l, v, rsrc_b);
-  };
-  auto dma_advance = [&]() {
-    if (!ld_live) return;
-    if (++ld_kt == ld_nk) {
-      cursor_advance(sch, wg_in_xcd, c_ld);
-      load_setup();
-    } else {
-      step_setup();
-    }
-  };
-  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
-
-  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: low / high K half of a step
-  auto read_frag = [&](i32x8& f, const uint8_t* base, int hh) {
-    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc[hh][0]);
-    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc[hh][1]);
-    f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
-  };
-
-  typedef int i32x2 __attribute__((ext_vector_type(2)));
-  typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
-  auto read_frag_tr = [&](i32x8& f, uint32_t a) {  // 4 x 8 contraction rows of the lane's column
-    const i32x2 t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a));
-    const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 2048));
-    const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 4096));
-    const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
-    f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
-  };
-  // weight fragment j / token fragment i, K half hh, of the unit at `unit`
-  auto read_frag_b = [&](i32x8& f, const uint8_t* unit, int j, int hh) {
-    if constexpr (!B_TR) {
-      read_frag(f, unit + fb_off + j * 32 * BK, hh);
-    } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * 256));
-    }
-  };
-  auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh) {
-    if constexpr (!A_TR) {
-      read_frag(f, unit + fa_off + i * 32 * BK, hh);
-    } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * 256));
-    }
-  };
-
-  // ---- fill: steps 0 and 1 of the stream into units 0..3, the first fragments into registers ----
-  load_setup();
-#pragma unroll
-  for (int j = 0; j < kParts; ++j) dma_a(0, j);
-#pragma unroll
-  for (int j = 0; j < kParts; ++j) dma_b(1, j);
-  dma_advance();
-#pragma unroll
-  for (int j = 0; j < kParts; ++j) dma_a(2, j);
-#pragma unroll
-  for (int j = 0; j < kParts; ++j) dma_b(3, j);
-  dma_advance();
-  FP8GMM_WAIT_VM(2 * kParts);
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + US, j, 0);
-#pragma unroll
-  for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds, i, 0);
-  int ua = 0;  // ring unit of the current step's token rows; its weight rows are in the next unit
-  // vmcnt counts loads and stores in issue order.  The barrier of a step needs the next step's units, which are
-  // older than the token loads issued during the low half-step: "all but the newest kParts".  Right after an
-  // interior epilogue the newest operations also include that epilogue's kFastStores stores, which nothing in
-  // LDS depends on: at the first barrier after it they may stay in flight.
-  bool relaxed = false;
-
-// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
-#define FP8GMM_MF0(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
-#define FP8GMM_MF1(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
-
-  for (; cursor_valid(sch, wg_in_xcd, c_cp); cursor_advance(sch, wg_in_xcd, c_cp)) {
-    const Item g = cursor_item(sch, xcd, wg_in_xcd, c_cp);
-    const fp8gmm_gemm_problem pr = probs[g.prob];
-    const int m0 = g.m0, n0 = g.n0;
-
-    f32x16 acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    // One K = 128 step.  `same_item`: the load cursor stays inside its current item after this step (the caller
-    // knows), so advancing it is three additions; otherwise the general advance, which may switch items.
-    auto k_step = [&](auto same_item) {
-      // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
-      // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
-      // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
-      // has read them.
-      const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
-      // ---- low K half: fragments in fa0 / fb0; fetch the high half's from the same units.  No barrier:
-      // nothing written since the last one is read here.
-      {
-        const uint8_t* qa = lds + ua * US;
-        const uint8_t* qb = lds + ub * US;
-        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
-        dma_a(fa, 0);
-        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
-        read_frag_b(fb1[0], qb, 0, 1);
-        read_frag_b(fb1[1], qb, 1, 1);
-        FP8GMM_SB(); FP8GMM_MF0(0, 2); FP8GMM_SB();
-        dma_a(fa, 1);
-        FP8GMM_SB(); FP8GMM_MF0(0, 3); FP8GMM_SB();
-        read_frag_b(fb1[2], qb, 2, 1);
-        read_frag_b(fb1[3], qb, 3, 1);
-        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
-        dma_a(fa, 2);
-        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
-        read_frag_a(fa1[0], qa, 0, 1);
-        FP8GMM_SB(); FP8GMM_MF0(1, 2); FP8GMM_SB();
-        dma_a(fa, 3);
-        FP8GMM_SB(); FP8GMM_MF0(1, 3); FP8GMM_SB();
-        read_frag_a(fa1[1], qa, 1, 1);
-        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
-        dma_a(fa, 4);
-        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
-        read_frag_a(fa1[2], qa, 2, 1);
-        FP8GMM_SB(); FP8GMM_MF0(2, 2); FP8GMM_SB();
-        dma_a(fa, 5);
-        FP8GMM_SB(); FP8GMM_MF0(2, 3); FP8GMM_SB();
-        read_frag_a(fa1[3], qa, 3, 1);
-        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_SB();
-        dma_a(fa, 6);
-        FP8GMM_SB(); FP8GMM_MF0(3, 1); FP8GMM_SB();
-        dma_a(fa, 7);
-        FP8GMM_SB(); FP8GMM_MF0(3, 2); FP8GMM_MF0(3, 3); FP8GMM_SB();
-      }
-      // ---- high K half: fragments in fa1 / fb1.  The barrier proves that every wavefront has read this
-      // step's units (lgkmcnt(0)) and that the next step's units have landed for all of them.
-      if (relaxed) {
-        FP8GMM_WAIT_VM_LGKM(kParts + kFastStores);
-        relaxed = false;
-      } else {
-        FP8GMM_WAIT_VM_LGKM(kParts);
-      }
-      __builtin_amdgcn_s_barrier();
-      {
-        const uint8_t* qa = lds + na * US;
-        const uint8_t* qb = lds + nb * US;
-        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
-        dma_b(ua, 0);
-        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
-        read_frag_b(fb0[0], qb, 0, 0);
-        read_frag_b(fb0[1], qb, 1, 0);
-        FP8GMM_SB(); FP8GMM_MF1(0, 2); FP8GMM_SB();
-        dma_b(ua, 1);
-        FP8GMM_SB(); FP8GMM_MF1(0, 3); FP8GMM_SB();
-        read_frag_b(fb0[2], qb, 2, 0);
-        read_frag_b(fb0[3], qb, 3, 0);
-        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
-        dma_b(ua, 2);
-        FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
-        read_frag_a(fa0[0], qa, 0, 0);
-        FP8GMM_SB(); FP8GMM_MF1(1, 2); FP8GMM_SB();
-        dma_b(ua, 3);
-        FP8GMM_SB(); FP8GMM_MF1(1, 3); FP8GMM_SB();
-        read_frag_a(fa0[1], qa, 1, 0);
-        FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
-        dma_b(ua, 4);
-        FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
-        read_frag_a(fa0[2], qa, 2, 0);
-        FP8GMM_SB(); FP8GMM_MF1(2, 2); FP8GMM_SB();
-        dma_b(ua, 5);
-        FP8GMM_SB(); FP8GMM_MF1(2, 3); FP8GMM_SB();
-        read_frag_a(fa0[3], qa, 3, 0);
-        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_SB();
-        dma_b(ua, 6);
-        FP8GMM_SB(); FP8GMM_MF1(3, 1); FP8GMM_SB();
-        dma_b(ua, 7);
-        if constexpr (decltype(same_item)::value) {
-          ++ld_kt;
-          step_setup();
-        } else {
-          dma_advance();
-        }
-        FP8GMM_SB(); FP8GMM_MF1(3, 2); FP8GMM_MF1(3, 3); FP8GMM_SB();
-      }
-      ua = na;
-    };
-    // The load cursor runs two steps ahead of this loop: while at least three steps of the item remain, its
-    // next step lies in the same item.
-    int kt = 0;
-    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{});
-    for (; kt < g.nk; ++kt) k_step(std::false_type{});
-    // ---- epilogue ----
-    if (g.slot >= 0) {
-      // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
-      partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
-      relaxed = false;
-    } else {
-      // free until the next step's token loads: the unit that held the last step's weights
-      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
-    }
-  }
-  // zero-fill loads issued past the end of the stream still target this workgroup's LDS
-  FP8GMM_WAIT_VM(0);
-  clock_probe_mark<PROBE>(1);
-}
-
-#undef FP8GMM_MF0
-#undef FP8GMM_MF1
-
-// Completes the tiles that the main kernel shared along K.  One workgroup per interior piece boundary of
-// every XCD's stream-K region; the FIRST boundary that falls strictly inside a tile owns that tile: it adds
-// the pieces in K order (workgroup j - 1 holds the piece from the tile's first K step, workgroups j,
-// j + 1, ... the following ones) and applies the epilogue.
+// Completes the tiles that the main kernel shared along K.  One workgroup per such tile (one record of the
+// fix-up list each): it adds the tile's pieces, which lie in consecutive workspace slots in K order, and
+// applies the epilogue.
 // 1024 threads: thread T owns the 16-byte groups T + 1024 q (q = 0..15) of a slot, i.e. register group g = T / 256
 // of every MFMA tile (i, j) = q of main-kernel thread T % 256: 4 consecutive columns of one row each.  The sums and
 // the arithmetic are those of tile_epilogue's general paths, so a shared tile gets the same bits as a whole one.
@@ -747,19 +19,11 @@ constexpr int kFixupThreads = 1024;
 static_assert(kFixupThreads == 4 * NTHREADS, "one register group of every MFMA tile per thread");
 
 __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
-    const fp8gmm_gemm_problem* __restrict__ probs, int nprob, int total_tiles, int out_kind, int epilogue,
-    const uint8_t* __restrict__ workspace, int wgs_per_xcd) {
-  const int xcd = blockIdx.x % kNumXcd;
-  const int j = blockIdx.x / kNumXcd + 1;
-  Sched sch;
-  sched_init(sch, probs, nprob, total_tiles, xcd, wgs_per_xcd, true);
-  int n_following = 0;
-  const int tile = fixup_tile(sch, j, &n_following);
-  if (tile < 0) return;
-  const int prob = problem_of_tile(sch, tile);
-  const fp8gmm_gemm_problem pr = probs[prob];
-  int m0, n0;
-  tile_origin(pr.m, pr.n, tile - pr.tile_begin, &m0, &n0);
+    const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_fixup_desc* __restrict__ fixups, int out_kind,
+    int epilogue, const uint8_t* __restrict__ workspace) {
+  const fp8gmm_gemm_fixup_desc fx = fixups[blockIdx.x];
+  const fp8gmm_gemm_problem pr = probs[fx.prob];
+  const int m0 = fx.m0, n0 = fx.n0;
 
   const int t = threadIdx.x % NTHREADS, g = threadIdx.x / NTHREADS;
   const int lane = t & 63, wave = t >> 6;
@@ -768,14 +32,12 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
 
   f32x4 sum[MT * NT];
   {
-    const f32x4* first = reinterpret_cast<const f32x4*>(
-        workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + j - 1) + 1) * kPartialBytes) + threadIdx.x;
+    const f32x4* first = reinterpret_cast<const f32x4*>(workspace + (size_t)fx.first_slot * kPartialBytes) + threadIdx.x;
 #pragma unroll
     for (int q = 0; q < MT * NT; ++q) sum[q] = first[q * kFixupThreads];
   }
-  for (int w = j; w < j + n_following; ++w) {
-    const f32x4* next = reinterpret_cast<const f32x4*>(
-        workspace + (size_t)(kSlotsPerWg * (xcd * wgs_per_xcd + w)) * kPartialBytes) + threadIdx.x;
+  for (int w = 1; w < fx.n_pieces; ++w) {
+    const f32x4* next = reinterpret_cast<const f32x4*>(workspace + (size_t)(fx.first_slot + w) * kPartialBytes) + threadIdx.x;
     f32x4 part[MT * NT];
 #pragma unroll
     for (int q = 0; q < MT * NT; ++q) part[q] = next[q * kFixupThreads];
@@ -860,100 +122,69 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
   }
 }
 
-// Workspace of the stream-K pieces: kSlotsPerWg slots per workgroup, allocated once per (device, stream)
-// and kept until the process ends.  Launches on one stream are ordered, so they can share it; a few
-// streams get a workspace each, further ones simply run without tail balancing.
-struct WorkspaceKey {
-  int device;
-  hipStream_t stream;
-  bool operator<(const WorkspaceKey& o) const {
-    return device != o.device ? device < o.device : reinterpret_cast<uintptr_t>(stream) < reinterpret_cast<uintptr_t>(o.stream);
-  }
-};
-constexpr size_t kMaxWorkspaces = 8;
 
-uint8_t* workspace_for(int device, hipStream_t stream, int grid) {
-  static std::mutex mu;
-  static std::map<WorkspaceKey, std::pair<uint8_t*, size_t>> cache;
-  const size_t bytes = (size_t)kSlotsPerWg * (size_t)grid * kPartialBytes;
-  std::lock_guard<std::mutex> lock(mu);
-  auto it = cache.find(WorkspaceKey{device, stream});
-  if (it != cache.end()) return it->second.second >= bytes ? it->second.first : nullptr;
-  if (cache.size() >= kMaxWorkspaces) return nullptr;
-  void* ptr = nullptr;
-  if (hipMalloc(&ptr, bytes) != hipSuccess) {
-    (void)hipGetLastError();  // e.g. under stream capture: run without tail balancing
-    return nullptr;
-  }
-  cache[WorkspaceKey{device, stream}] = {static_cast<uint8_t*>(ptr), bytes};
-  return static_cast<uint8_t*>(ptr);
-}
+// compute-unit count per device, looked up once (fp8gmm_init, or the first launch on the device)
+std::atomic<int> g_num_cu[kMaxDevices];
 
-bool stream_k_allowed() {
-  static const bool allowed = [] {
-    const char* e = getenv("FP8GMM_STREAMK");
-    return !(e != nullptr && e[0] == '0');
-  }();
-  return allowed;
-}
-
-std::atomic<bool> g_clock_probe_on{false};
-
-template <int A_FMT, int B_FMT, bool PROBE, bool A_TR, bool B_TR>
-int launch_variant(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
-                   hipStream_t stream) {
-  // per device (a process may drive several): compute-unit count and "the kernel may use the whole LDS"
-  constexpr int kMaxDevices = 64;
-  static std::atomic<int> num_cu[kMaxDevices];
-  static std::atomic<bool> attr_set[kMaxDevices];
-  const size_t lds_bytes = (size_t)RING * US;
-  auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, PROBE, A_TR, B_TR>;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
-  if (!attr_set[dev].load(std::memory_order_acquire)) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)lds_bytes) != hipSuccess)
-      return FP8GMM_ERR_LAUNCH;
-    attr_set[dev].store(true, std::memory_order_release);
-  }
-  int cus = num_cu[dev].load(std::memory_order_relaxed);
+int device_num_cu(int dev) {
+  if (dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
+  int cus = g_num_cu[dev].load(std::memory_order_relaxed);
   if (cus == 0) {
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
     cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    num_cu[dev].store(cus, std::memory_order_relaxed);
+    g_num_cu[dev].store(cus, std::memory_order_relaxed);
   }
-  // one workgroup per CU, a multiple of 8 so that every XCD gets the same number of workgroups
-  int grid = (cus / kNumXcd) * kNumXcd;
-  if (grid < kNumXcd) grid = kNumXcd;
-  // tail balancing can only pay when the launch has few rounds; it needs the whole grid even for few tiles
-  uint8_t* workspace = nullptr;
-  if (stream_k_allowed() && (int64_t)total_tiles <= (int64_t)kSkMaxRounds * grid && grid > kNumXcd)
-    workspace = workspace_for(dev, stream, grid);
-  if (workspace == nullptr) {
-    const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
-    if (grid > needed) grid = needed;
-  }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(NTHREADS), lds_bytes, stream, probs_dev, n, total_tiles, out_kind,
-                     epilogue, workspace);
-  if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
-  if (workspace != nullptr) {
-    const int wgs_per_xcd = grid / kNumXcd;
-    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(kNumXcd * (wgs_per_xcd - 1)), dim3(kFixupThreads), 0, stream,
-                       probs_dev, n, total_tiles, out_kind, epilogue, workspace, wgs_per_xcd);
+  return cus;
+}
+
+typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*, uint64_t*,
+                         hipStream_t);
+
+// the variant for a format / layout combination, or null when the combination does not exist
+launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor) {
+#define FP8GMM_PICK(AF, BF, AT, BT) \
+  if (a_fmt == AF && b_fmt == BF && a_kmajor == AT && b_kmajor == BT) return &launch_variant<AF, BF, AT, BT>;
+  FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_PICK)
+#undef FP8GMM_PICK
+  return nullptr;
+}
+
+int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                   const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
+                   int out_kind, int epilogue, void* workspace, size_t workspace_bytes, uint64_t* counters,
+                   void* stream) {
+  if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  if (n < 0 || plan->total_tiles < 0 || plan->rounds < 0 || plan->n_fixups < 0 || plan->n_slots < 0)
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if (out_kind != FP8GMM_OUT_BF16 && out_kind != FP8GMM_E4M3 && out_kind != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
+  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
+  const bool a_kmajor = (epilogue & FP8GMM_GEMM_A_KMAJOR) != 0;
+  const bool b_kmajor = (epilogue & FP8GMM_GEMM_B_KMAJOR) != 0;
+  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;
+  if ((a_fmt != FP8GMM_E4M3 && a_fmt != FP8GMM_E5M2) || (b_fmt != FP8GMM_E4M3 && b_fmt != FP8GMM_E5M2))
+    return FP8GMM_ERR_BAD_FORMAT;
+  // e5m2 x e5m2 does not exist (cuBLASLt rejects it too); the contraction-major forms are the gradient GEMMs,
+  // whose b is a forward tensor (weight or activation), always e4m3
+  const launch_fn launch = variant_for(a_fmt, b_fmt, a_kmajor, b_kmajor);
+  if (launch == nullptr) return FP8GMM_ERR_BAD_FORMAT;
+  if (n == 0 || plan->total_tiles == 0) return FP8GMM_OK;
+  if (plan->grid <= 0 || (plan->grid % kNumXcd) != 0 || plan->rounds < 1) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (probs_dev == nullptr || items_dev == nullptr || (plan->n_fixups > 0 && fixups_dev == nullptr))
+    return FP8GMM_ERR_NULL_POINTER;
+  if (plan->n_slots > 0 && (workspace == nullptr || workspace_bytes < (size_t)plan->n_slots * kPartialBytes ||
+                            (reinterpret_cast<uintptr_t>(workspace) & 255) != 0))
+    return FP8GMM_ERR_WORKSPACE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int rc = launch(probs_dev, items_dev, plan->grid, out_kind, epilogue & FP8GMM_EPI_GELU,
+                        static_cast<uint8_t*>(workspace), counters, s);
+  if (rc != FP8GMM_OK) return rc;
+  if (plan->n_fixups > 0) {
+    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups), dim3(kFixupThreads), 0, s, probs_dev,
+                       fixups_dev, out_kind, epilogue & FP8GMM_EPI_GELU, static_cast<const uint8_t*>(workspace));
     if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
   }
   return FP8GMM_OK;
-}
-
-template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
-int launch(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int out_kind, int epilogue,
-           hipStream_t stream) {
-  if constexpr (!A_TR && !B_TR) {  // the measurement build exists for the row-major layout only
-    if (g_clock_probe_on.load(std::memory_order_relaxed))
-      return launch_variant<A_FMT, B_FMT, true, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
-  }
-  return launch_variant<A_FMT, B_FMT, false, A_TR, B_TR>(probs_dev, n, total_tiles, out_kind, epilogue, stream);
 }
 
 }  // namespace
@@ -966,91 +197,38 @@ void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n) {
   if (tile_n) *tile_n = fp8gmm::BN;
 }
 
-int fp8gmm_gemm_clock_probe(uint64_t* dev_counters) {
-  // synchronous copy into the device-side pointer of the current device
-  if (hipMemcpyToSymbol(HIP_SYMBOL(fp8gmm::d_clock_probe), &dev_counters, sizeof(dev_counters)) != hipSuccess)
-    return FP8GMM_ERR_LAUNCH;
-  fp8gmm::g_clock_probe_on.store(dev_counters != nullptr, std::memory_order_relaxed);
-  return FP8GMM_OK;
-}
-
-int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles) {
-  return fp8gmm_plan_grouped_gemm_layout(probs, n, 0, total_tiles);
-}
-
-int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layout, int* total_tiles) {
-  if (n < 0 || (layout & ~(FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR))) return FP8GMM_ERR_BAD_ARGUMENT;
-  const bool a_kmajor = (layout & FP8GMM_GEMM_A_KMAJOR) != 0;
-  const bool b_kmajor = (layout & FP8GMM_GEMM_B_KMAJOR) != 0;
-  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;  // not a combination the path uses
-  if (total_tiles == nullptr || (n > 0 && probs == nullptr)) return FP8GMM_ERR_NULL_POINTER;
-  int64_t tiles = 0, cost = 0;
-  for (int i = 0; i < n; ++i) {
-    fp8gmm_gemm_problem& p = probs[i];
-    if (p.m < 0 || p.n < 0 || p.k < 0) return FP8GMM_ERR_BAD_SHAPE;
-    if (p.lda < (a_kmajor ? p.m : p.k) || p.ldb < (b_kmajor ? p.n : p.k) || p.ldc < p.n) return FP8GMM_ERR_BAD_SHAPE;
-    const bool has_work = p.m > 0 && p.n > 0;
-    if (has_work) {
-      if (p.c == nullptr) return FP8GMM_ERR_NULL_POINTER;
-      if (p.k > 0) {  // with k == 0 the operands are never read
-        if (p.a == nullptr || p.b == nullptr) return FP8GMM_ERR_NULL_POINTER;
-        // a row-major operand is fetched in 16-byte pieces along k, a contraction-major one along its rows
-        if ((!(a_kmajor && b_kmajor) && (p.k & 15)) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
-        if ((a_kmajor && (p.m & 15)) || (b_kmajor && (p.n & 15))) return FP8GMM_ERR_ALIGNMENT;
-        if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
-          return FP8GMM_ERR_ALIGNMENT;
-        // the kernel addresses each operand through a buffer descriptor with 32-bit byte offsets
-        // (contraction rows up to 127 past k are addressed, and must fall outside the descriptor, not wrap)
-        if ((uint64_t)(a_kmajor ? p.k + 128 : p.m) * (uint64_t)p.lda > 0xffffffffull ||
-            (uint64_t)(b_kmajor ? p.k + 128 : p.n) * (uint64_t)p.ldb > 0xffffffffull)
-          return FP8GMM_ERR_BAD_SHAPE;
-      }
-    }
-    const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;
-    const int64_t tn = (p.n + fp8gmm::BN - 1) / fp8gmm::BN;
-    p.tile_begin = (int32_t)tiles;
-    p.cost_begin = (int32_t)cost;  // a tile costs ceil(k / 128) steps of the main loop (1 for k = 0)
-    const int64_t steps = (p.k + 127) / 128;
-    tiles += tm * tn;
-    cost += tm * tn * (steps > 0 ? steps : 1);
-    if (tiles > INT32_MAX / 16 || cost > INT32_MAX / 2) return FP8GMM_ERR_BAD_SHAPE;
+int fp8gmm_init(int device) {
+  using namespace fp8gmm;
+  int current = 0;
+  if (hipGetDevice(&current) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
+  const int dev = device < 0 ? current : device;
+  if (dev != current && hipSetDevice(dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
+  int rc = device_num_cu(dev);
+#define FP8GMM_PREPARE(AF, BF, AT, BT) \
+  if (rc > 0) {                        \
+    const int e = prepare_variant<AF, BF, AT, BT>(dev); \
+    if (e != FP8GMM_OK) rc = e;        \
   }
-  *total_tiles = (int)tiles;
-  return FP8GMM_OK;
+  FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_PREPARE)
+#undef FP8GMM_PREPARE
+  if (dev != current) (void)hipSetDevice(current);
+  return rc;
 }
 
-int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int a_fmt, int b_fmt,
-                        int out_kind, int epilogue, void* stream) {
-  if (n < 0 || total_tiles < 0) return FP8GMM_ERR_BAD_ARGUMENT;
-  if (out_kind != FP8GMM_OUT_BF16 && out_kind != FP8GMM_E4M3 && out_kind != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
-  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
-  const bool a_kmajor = (epilogue & FP8GMM_GEMM_A_KMAJOR) != 0;
-  const bool b_kmajor = (epilogue & FP8GMM_GEMM_B_KMAJOR) != 0;
-  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;
-  // the contraction-major forms are the gradient GEMMs: b is a forward tensor (weight or activation), always e4m3
-  if (b_kmajor && b_fmt != FP8GMM_E4M3) return FP8GMM_ERR_BAD_FORMAT;
-  epilogue &= FP8GMM_EPI_GELU;
-  if ((a_fmt != FP8GMM_E4M3 && a_fmt != FP8GMM_E5M2) || (b_fmt != FP8GMM_E4M3 && b_fmt != FP8GMM_E5M2))
-    return FP8GMM_ERR_BAD_FORMAT;
-  if (a_fmt == FP8GMM_E5M2 && b_fmt == FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
-  if (n == 0 || total_tiles == 0) return FP8GMM_OK;
-  if (probs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (b_kmajor) {
-    if (a_kmajor) {
-      if (a_fmt == FP8GMM_E4M3)
-        return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, true, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-      return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, true, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-    }
-    if (a_fmt == FP8GMM_E4M3)
-      return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, false, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, false, true>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-  }
-  if (a_fmt == FP8GMM_E4M3 && b_fmt == FP8GMM_E4M3)
-    return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E4M3, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-  if (a_fmt == FP8GMM_E5M2 && b_fmt == FP8GMM_E4M3)
-    return fp8gmm::launch<FP8GMM_E5M2, FP8GMM_E4M3, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
-  return fp8gmm::launch<FP8GMM_E4M3, FP8GMM_E5M2, false, false>(probs_dev, n, total_tiles, out_kind, epilogue, s);
+int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                        const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
+                        int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+  return fp8gmm::launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
+                                workspace_bytes, nullptr, stream);
+}
+
+int fp8gmm_grouped_gemm_timed(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                              const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
+                              int b_fmt, int out_kind, int epilogue, void* workspace, size_t workspace_bytes,
+                              uint64_t* dev_counters, void* stream) {
+  if (dev_counters == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  return fp8gmm::launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
+                                workspace_bytes, dev_counters, stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,807 @@
+// Persistent FP8 grouped GEMM for gfx950 (MI355X): the kernel template and its launcher.  Included by
+// gemm_variant.hip, which is compiled once per operand format / layout combination, and by grouped_gemm.hip.
+//
+// Replaces the reference's CUTLASS grouped GEMM (csrc/fp8_gmm.cu:82-205) and its
+// per-expert cuBLASLt loops (fp8_gmm/backend.py:84-96, grouped_linear.py:173-182,
+// grouped_mlp.py:234-242,313-322) with ONE launch over a device-side problem table.
+//
+//   c[m, n] = epilogue( sum_k a[m, k] * b[n, k] ),   a, b fp8 (K contiguous), fp32 accumulation
+//
+// Work decomposition
+//   * the output of every problem is cut into 256 x 256 tiles; all tiles of all problems form
+//     one list walked by a persistent grid (one workgroup per CU).  The list is split into 8
+//     contiguous ranges, one per XCD (workgroup i runs on XCD i % 8), so that workgroups that
+//     share an L2 work on neighbouring tiles; inside a problem the m index runs fastest within
+//     groups of 8 rows of tiles, so one round of an XCD's 32 workgroups is an 8 x 4 block of tiles.
+//     All of that is decided on the host (gemm_schedule.h, fp8gmm_plan_grouped_gemm_launch): the kernel
+//     reads its work list, one 64-byte record per tile, and does no scheduling arithmetic of its own
+//     (binary searches over the problem table and integer divisions in the scalar unit cost a tile switch
+//     thousands of cycles, more with every expert).
+//   * a workgroup is 4 wavefronts (2 along m x 2 along n), one per SIMD; a wavefront owns a
+//     128 x 128 sub-tile = 4 x 4 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4.  Its 256 accumulators
+//     live in the accumulation registers, the other 256 registers hold fragments and addresses.
+//     The weight operand is MFMA source 0 and the token operand source 1: every lane then
+//     holds 4 consecutive output columns of one row.
+//
+// Data movement
+//   * operands go global -> LDS directly (`buffer_load_dwordx4 ... lds`), never through
+//     registers.  Buffer descriptors bound every operand, so rows past m / n and K tails read
+//     as zeros: m, n are arbitrary and k only has to be a multiple of 16.
+//   * a main-loop step consumes K = 128: one 128-byte line of each of the tile's 256 token rows
+//     and 256 weight rows.  LDS (all 160 KB) is a ring of five 32 KB units, a unit being the
+//     256 rows x 128 B of ONE operand for one step, its eight 16-byte chunks XOR-swizzled with
+//     (row >> 1) & 7 so that the 16-byte fragment reads of a wavefront are conflict-free.  Every
+//     load instruction fetches 8 whole lines (two half-line requests for one line, issued apart,
+//     meet in the L1 as a hit on a pending miss and stall it).
+//   * at any time the ring holds the units of the step being computed, of the next step, and
+//     the tokens of the step after; that step's weights replace the current tokens once the
+//     step's barrier has shown that every wavefront has read them.  The token loads of step + 2
+//     are issued during the low K half of a step, the weight loads during the high half, one
+//     after every second MFMA.
+//   * the load stream and the ring run CONTINUOUSLY across tile boundaries: while a tile's
+//     epilogue stores its result, the next tile's first two steps are already in LDS.
+//   * ONE s_barrier per step, between its two K = 64 halves.  The fragments of a half are read
+//     from LDS during the half before it, interleaved with the MFMAs (pinned with sched_barrier).
+//     With a single wavefront per SIMD nothing else fills an MFMA pipe, so whatever sits between
+//     two MFMAs has to issue within the 64 cycles the first one runs: addresses are two
+//     instructions per load, the load cursor advances without branches while it stays inside an
+//     item, and the scheduler arithmetic of an item switch runs once per tile.
+//   * epilogue: scale, convert, and - for interior bf16 tiles - a pass through the free ring unit
+//     that turns the MFMA layout into whole-line stores.
+#pragma once
+
+#include <atomic>
+#include <type_traits>
+
+#include "device_utils.h"
+#include "tiling.h"
+
+namespace fp8gmm {
+
+constexpr int kPartialBytes = FP8GMM_GEMM_SLOT_BYTES;  // one workspace slot: the fp32 accumulators of one tile
+static_assert(kPartialBytes == BM * BN * 4, "a slot holds one tile of fp32 accumulators");
+
+constexpr int BK = kGemmTileK;    // bytes of K per main-loop step: one 128-byte line of every operand row
+constexpr int US = BM * BK;       // 32768 bytes per ring unit: the 256 rows of ONE operand for one step
+constexpr int RING = 5;
+static_assert(BM == BN, "token and weight units share one size");
+constexpr int NWAVES = 4;         // one wavefront per SIMD: 256 accumulator + 256 other registers per lane
+constexpr int NTHREADS = 64 * NWAVES;
+constexpr int WM = 128, WN = 128;  // wavefront sub-tile
+constexpr int WAVES_N = BN / WN;  // wavefronts along n: 2 (x 2 along m)
+constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
+constexpr int NT = WN / 32;       // 4 MFMA tiles along n per wave
+constexpr int kParts = US / 1024 / NWAVES;  // buffer_load ... lds instructions (1 KB each) per wavefront per unit: 8
+constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the interior bf16 epilogue (8 per 32-row block)
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
+#define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
+#define FP8GMM_WAIT_VM_LGKM(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(n) : "memory")
+// global -> LDS: lane i's 16 bytes land at M0 + 16 i; out-of-range offsets deliver zeros
+#define FP8GMM_DMA(lds_addr, voff, rsrc) \
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
+
+// One MFMA tile's accumulators as ordinary vector registers.  In the main kernel the 256 accumulators of a
+// lane live in the accumulation registers (the other 256 hold fragments and addresses); vector arithmetic
+// cannot read those, and left to itself the register allocator parks them in scratch memory on the way.
+// Reading them 16 at a time, where they are used, keeps the epilogue within the register file.
+__device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
+  f32x16 t;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
+  return t;
+}
+
+// Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
+// stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
+// `stage`: 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of the staged path.
+__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
+                                              int out_kind, int epilogue, uint8_t* stage) {
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+  const int l32 = lane & 31, khalf = lane >> 5;
+  const int M = pr.m, N = pr.n;
+  bool fast = false;
+    const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
+    const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
+    const float s = sa_inv * sb_inv;
+    const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
+    const int64_t ldc = pr.ldc;
+    float amax = 0.f;
+    const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
+    if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
+        ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
+      // Interior tile, plain bf16 output: straight-line code with an exact store count.
+      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+      // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
+      // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
+      // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
+      // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
+      // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
+      uint8_t* mine = stage + wave * 8192;
+      const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
+      const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
+                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
+          }
+        }
+        // only this wavefront touches `mine`: its own LDS operations complete in order
+        u32x4 v[8];
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int r = 4 * it + rrow;
+          v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+          const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
+          global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
+        }
+      }
+      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
+      fast = true;
+    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && interior && ((ldc & 15) == 0) &&
+               ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0) && ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0)) {
+      // Interior tile of the fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
+      // outputs go through the staging area like the plain form's, one 32-row block at a time - first the bf16
+      // block as 32 rows x 256 B, then, in a second pass over the same accumulators, the fp8 block as 32 rows x
+      // 128 B (chunk c of row r at chunk c ^ ((r >> 1) & 7)) - so that every store instruction writes whole
+      // lines: 12 per block instead of 32 that touch 32 rows each.
+      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
+      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
+      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
+      uint8_t* mine = stage + wave * 8192;
+      const int wr = l32 * 256 + khalf * 8;   // bf16 block: + ((4 j + g) ^ (l32 & 15)) * 16
+      const int wr8 = l32 * 128 + khalf * 4;  // fp8 block:  + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
+      const int rrow = lane >> 4, rchunk = lane & 15;
+      const int rrow8 = lane >> 3, rchunk8 = lane & 7;
+      float tile_amax = 0.f;
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const u32x2 a = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
+                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = a;
+          }
+        }
+        {
+          u32x4 rb[8];
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int r = 4 * it + rrow;
+            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
+          }
+#pragma unroll
+          for (int it = 0; it < 8; ++it) {
+            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
+            global_store(AUX + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, rb[it]);
+          }
+        }
+        // the wavefront's LDS operations complete in order: the reads above are done before these writes land
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            float x[4];
+            uint32_t nan_bytes = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float r = gelu_tanh_fast(t[g * 4 + q] * s);
+              // A chain of hardware max operations, pinned: written as compare + select, the compiler rebuilds
+              // the 256-element reduction as a tree and keeps far more values alive than there are registers.
+              // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
+              asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
+              // straight-line conversion (a branch here costs the register allocator its footing): clamp, convert,
+              // and patch the byte of a NaN to 0x7F afterwards (the median turns a NaN into -max)
+              const float y = r * cs;
+              x[q] = __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
+              nan_bytes |= (y != y) ? (0xffu << (8 * q)) : 0u;
+            }
+            uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
+                x[2], x[3], __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
+            w = (w & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
+            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) = w;
+          }
+        }
+        {
+          u32x4 rb[4];
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int r = 8 * it + rrow8;
+            rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 128 + ((rchunk8 ^ ((r >> 1) & 7)) << 4));
+          }
+#pragma unroll
+          for (int it = 0; it < 4; ++it) {
+            const int m = m0 + wave_m * WM + i * 32 + 8 * it + rrow8;
+            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk8 * 16, rb[it]);
+          }
+        }
+      }
+      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
+      if (pr.c_amax != nullptr) {
+        const float am = wave_max(tile_amax);
+        if (lane == 0 && am > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= am)) atomic_max_nonneg(pr.c_amax, am);
+      }
+    } else if (out_kind == FP8GMM_OUT_BF16) {
+      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
+      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) &&
+                       (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int m = m0 + wave_m * WM + i * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
+            if (m >= M || n >= N) continue;
+            float v[4], r[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              v[q] = t[g * 4 + q] * s;
+              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
+            }
+            const int64_t off = (int64_t)m * ldc + n;
+            if (vec && n + 3 < N) {
+              u32x2 o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
+              global_store(C + off, o);
+              if (gelu && AUX != nullptr) {
+                u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                global_store(AUX + off, a);
+              }
+            } else {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if (n + q < N) {
+                  global_store(C + off + q, (uint16_t)f32_to_bf16_bits(r[q]));
+                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
+                }
+              }
+            }
+          }
+        }
+      }
+    } else {
+      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
+      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
+      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
+      const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 3) == 0) &&
+                       (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int m = m0 + wave_m * WM + i * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
+            if (m >= M || n >= N) continue;
+            float v[4], r[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              v[q] = t[g * 4 + q] * s;
+              r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
+              if (n + q < N) amax = amax_step(amax, r[q]);
+            }
+            uint32_t w;
+            if (out_kind == FP8GMM_E4M3) {
+              w = cvt4_fp8<FP8GMM_E4M3>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
+            } else {
+              w = cvt4_fp8<FP8GMM_E5M2>(r[0] * cs, r[1] * cs, r[2] * cs, r[3] * cs);
+            }
+            const int64_t off = (int64_t)m * ldc + n;
+            if (vec && n + 3 < N) {
+              global_store(C + off, w);
+              if (gelu && AUX != nullptr) {
+                u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+                global_store(AUX + off, a);
+              }
+            } else {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                if (n + q < N) {
+                  global_store(C + off + q, (uint8_t)(w >> (8 * q)));
+                  if (gelu && AUX != nullptr) global_store(AUX + off + q, (uint16_t)f32_to_bf16_bits(v[q]));
+                }
+              }
+            }
+          }
+        }
+      }
+      if (pr.c_amax != nullptr) {
+        amax = wave_max(amax);
+        // amax only grows: once the slot holds a value at or above this wavefront's, the atomic is redundant
+        // (the slots of all experts share a cache line, and atomics on one line serialise)
+        if (lane == 0 && amax > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= amax))
+          atomic_max_nonneg(pr.c_amax, amax);
+      }
+    }
+    return fast;
+}
+
+// Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
+// (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
+__device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* slot) {
+  float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
+        global_store(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4), v);
+      }
+    }
+}
+// Measurement on the side (fp8gmm_grouped_gemm_timed): when `counters` (8 x 4 uint64 of device memory) is not
+// null, the first workgroup of every XCD writes its shader-cycle counter and the constant 100 MHz counter when it
+// starts and adds the differences to two running totals when it ends, so that the caller can derive the clock
+// the launch really ran at (the counters of different compute units are not comparable, hence the same
+// workgroup takes both readings).  Two uniform branches per launch otherwise.
+__device__ __forceinline__ void clock_probe_mark(uint64_t* counters, int which) {
+  if (counters != nullptr && blockIdx.x < kNumXcd && threadIdx.x == 0) {
+    volatile uint64_t* const q = counters + 4 * blockIdx.x;
+    const uint64_t cycles = (uint64_t)clock64(), ticks = (uint64_t)wall_clock64();
+    if (which == 0) {
+      q[0] = cycles;
+      q[1] = ticks;
+    } else {  // totals over all launches since the counters were cleared
+      q[2] += cycles - q[0];
+      q[3] += ticks - q[1];
+    }
+  }
+}
+
+// The half of a work-list record (fp8gmm_gemm_item) that a side of the kernel needs, as scalar loads.
+struct ItemLoad {   // bytes 0..31: what the load stream needs besides ItemTile
+  uint64_t a, b;
+  uint32_t a_bytes, b_bytes;
+  int32_t lda, ldb;
+};
+struct ItemTile {   // bytes 32..63
+  int32_t k, k_begin, nk, m0, n0, prob, slot, reserved;
+};
+static_assert(sizeof(fp8gmm_gemm_item) == 64 && sizeof(ItemLoad) == 32 && sizeof(ItemTile) == 32, "record layout");
+static_assert(offsetof(fp8gmm_gemm_item, k) == 32 && offsetof(fp8gmm_gemm_item, lda) == 24, "record layout");
+
+// B_TR: operand b is stored contraction-major, b[k][n] with n contiguous and pitch ldb (the layout of a weight
+// stack [N_out.., ] seen from the data-gradient GEMM), instead of b[n][k].  Its ring unit then holds 128
+// contraction rows of 256 bytes; the 16-byte chunk c of row r sits at chunk c ^ 2 (r mod 8), and a fragment is
+// gathered with four transposing reads (ds_read_b64_tr_b8: in a group of 16 lanes, lane 8 h + i receives byte i
+// of the 8 bytes addressed by lanes 2 b + h, b = 0..7).  Everything else - schedule, MFMA order, epilogue -
+// is shared, so both layouts produce the same bits.
+// A_TR: the same for operand a (a[k][m], pitch lda): with both, c = a^T . b contracts over the rows of two
+// row-major matrices, which is the weight-gradient GEMM on the un-transposed activations and gradients; rows
+// past k read as zeros, so the contraction length needs no padding.
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
+__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
+                                                                const fp8gmm_gemm_item* __restrict__ items,
+                                                                int out_kind, int epilogue,
+                                                                uint8_t* __restrict__ workspace,
+                                                                uint64_t* __restrict__ counters) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+  clock_probe_mark(counters, 0);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: what depends on it stays in scalar registers
+  const int wave_m = wave / WAVES_N;  // 0..1
+  const int wave_n = wave % WAVES_N;  // 0..1
+  const int l32 = lane & 31;
+  const int khalf = lane >> 5;   // which 32-byte half of the 64-byte MFMA K slice this lane feeds
+  const uint32_t lds_base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+
+  // DMA lane map, row-major operand: one wavefront instruction fills 8 rows x 128 B of a unit, i.e. whole
+  // cache lines: lane -> row lane >> 3 of the group, slot chunk lane & 7.  Chunk c of row r is kept at chunk
+  // c ^ ((r >> 1) & 7); for the rows of group wave + NWAVES j that is ((wave & 1) * 4 + (lane >> 4)) & 7, so the
+  // GLOBAL chunk that has to land in slot chunk lane & 7 is a per-lane constant.
+  const int drow = lane >> 3;
+  const int dchunk = (lane & 7) ^ ((((wave & 1) << 2) + (lane >> 4)) & 7);
+  // fragment read map: token rows wave_m * 128 + 32 i + l32 (source 1), weight rows wave_n * 128 + 32 j + l32
+  // (source 0); K half hh, lane half khalf -> chunks 4 hh + 2 khalf + {0, 1}; (row >> 1) & 7 = (l32 >> 1) & 7
+  const int fsw = (l32 >> 1) & 7;
+  int fc[2][2];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) fc[hh][q] = ((4 * hh + 2 * khalf + q) ^ fsw) << 4;
+  const int fa_off = (wave_m * WM + l32) * BK;
+  const int fb_off = (wave_n * WN + l32) * BK;
+  // contraction-major unit: 128 contraction rows x 256 B.  Fragment of K half hh: rows 64 hh + 32 khalf + b (+ 8 t
+  // per read), logical chunk wave_n * 8 + 2 j + g, byte 8 h; s = lane % 16 = 2 b + h
+  const int tr_b = (lane & 15) >> 1, tr_h = lane & 1, tr_g = (lane >> 4) & 1;
+  const int tr_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
+  int fbt_off[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) fbt_off[j] = tr_row + (((wave_n * 8 + 2 * j + tr_g) ^ (2 * tr_b)) << 4);
+  int fat_off[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
+
+  // ---- this workgroup's work list (uniform): records blockIdx.x, blockIdx.x + grid, ... up to the end record.
+  // Both sides of the kernel walk it, the load side ahead of the compute side, and both read a record one item
+  // before they need it, so that a tile switch never waits for memory.
+  const uint8_t* const my_items = reinterpret_cast<const uint8_t*>(items + blockIdx.x);
+  const size_t item_stride = (size_t)gridDim.x * sizeof(fp8gmm_gemm_item);
+  auto item_load = [&](int r) { return *reinterpret_cast<const ItemLoad*>(my_items + r * item_stride); };
+  auto item_tile = [&](int r) { return *reinterpret_cast<const ItemTile*>(my_items + r * item_stride + 32); };
+  int r_ld = 0;                         // record the load side is in
+  ItemLoad ld_next_l = item_load(0);    // ... and the record it takes next, fetched ahead
+  ItemTile ld_next_t = item_tile(0);
+  if (ld_next_t.prob < 0) return;
+
+  // ---- load side: runs two steps ahead of the compute side, possibly in the next tile ----
+  bool ld_live = true;  // the load cursor still points at an item
+  int ld_kt = 0, ld_nk = 0, ld_kmax = 0;
+  [[maybe_unused]] int ld_lda = 0, ld_ldb = 0;  // contraction-major operands only
+  i32x4 rsrc_a = {0, 0, 0, 0x00020000}, rsrc_b = {0, 0, 0, 0x00020000};  // raw buffers; empty until set up
+  // Addresses of the K = 128 step the load cursor points at: part j of an operand is fetched from a_k + j * a_step
+  // (byte offsets into the operand's buffer, a_step uniform).  Rows past m / n are not masked: whatever they
+  // deliver only reaches accumulators of rows / columns that the epilogue never stores, and the descriptor keeps
+  // the access inside the operand.  The K tail is: a row-major lane whose 16-byte chunk lies past k gets an
+  // out-of-range offset (zero fill); contraction rows past k are out of the descriptor's range by themselves.
+  uint32_t a_base = 0, b_base = 0, a_step = 0, b_step = 0, a_k = 0, b_k = 0;
+  bool k_ok = false;  // row-major operands: this lane's chunk of the step exists
+  auto step_setup = [&]() {
+    const uint32_t k0 = (uint32_t)ld_kt * BK;
+    if constexpr (A_TR) {
+      a_k = a_base + k0 * (uint32_t)ld_lda;  // k * pitch < 2^32 is checked when the table is planned
+    } else {
+      a_k = a_base + k0;
+    }
+    if constexpr (B_TR) {
+      b_k = b_base + k0 * (uint32_t)ld_ldb;
+    } else {
+      b_k = b_base + k0;
+    }
+    k_ok = (int)k0 < ld_kmax;
+  };
+  // row-major operand: part j = rows (wave + NWAVES j) * 8 + drow of the tile.
+  // contraction-major operand: one instruction fills 4 contraction rows x 256 B: part j = rows
+  // (wave + NWAVES j) * 4 + lane / 16 of the unit, slot chunk lane % 16, which must receive global chunk
+  // p ^ 2 (row mod 8); row mod 8 is the same for every j.
+  // A record's operand addresses are those of the tile's first row / column, so these offsets depend on the
+  // pitch alone.
+  const int krow = wave * 4 + (lane >> 4);
+  const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
+  // Takes the record fetched ahead (r_ld), fetches the one after it, and sets up descriptors and offsets.
+  auto load_setup = [&]() {
+    for (;;) {
+      const ItemLoad gl = ld_next_l;
+      const ItemTile gt = ld_next_t;
+      ld_live = gt.prob >= 0;
+      if (!ld_live) break;
+      ld_next_l = item_load(r_ld + 1);  // every list ends with an end record, so r_ld + 1 exists
+      ld_next_t = item_tile(r_ld + 1);
+      if (gt.nk > 0) {
+        rsrc_a[0] = (int)(uint32_t)gl.a;
+        rsrc_a[1] = (int)(uint32_t)(gl.a >> 32);
+        rsrc_a[2] = (int)gl.a_bytes;
+        rsrc_b[0] = (int)(uint32_t)gl.b;
+        rsrc_b[1] = (int)(uint32_t)(gl.b >> 32);
+        rsrc_b[2] = (int)gl.b_bytes;
+        if constexpr (!A_TR) {
+          a_base = (uint32_t)(wave * 8 + drow) * (uint32_t)gl.lda + dchunk * 16;
+          a_step = NWAVES * 8 * (uint32_t)gl.lda;
+        } else {
+          a_base = (uint32_t)krow * (uint32_t)gl.lda + (uint32_t)tr_col;
+          a_step = NWAVES * 4 * (uint32_t)gl.lda;
+          ld_lda = gl.lda;
+        }
+        if constexpr (!B_TR) {
+          b_base = (uint32_t)(wave * 8 + drow) * (uint32_t)gl.ldb + dchunk * 16;
+          b_step = NWAVES * 8 * (uint32_t)gl.ldb;
+        } else {
+          b_base = (uint32_t)krow * (uint32_t)gl.ldb + (uint32_t)tr_col;
+          b_step = NWAVES * 4 * (uint32_t)gl.ldb;
+          ld_ldb = gl.ldb;
+        }
+        ld_kmax = gt.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
+        ld_kt = gt.k_begin;
+        ld_nk = gt.k_begin + gt.nk;
+        step_setup();
+        return;
+      }
+      ++r_ld;  // an item without K work needs no loads
+    }
+    // Past the end of the stream the loads are issued all the same, against empty descriptors (zero fill),
+    // which keeps the vmcnt arithmetic uniform.
+    rsrc_a[2] = 0;
+    rsrc_b[2] = 0;
+  };
+  // One instruction of that step: part j (0..7) of the token operand into ring unit `unit`, or of the weights.
+  auto dma_a = [&](int unit, int j) {
+    uint32_t v = a_k + j * a_step;
+    if constexpr (!A_TR) v = k_ok ? v : 0xffffffffu;
+    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
+    FP8GMM_DMA(l, v, rsrc_a);
+  };
+  auto dma_b = [&](int unit, int j) {
+    uint32_t v = b_k + j * b_step;
+    if constexpr (!B_TR) v = k_ok ? v : 0xffffffffu;
+    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
+    FP8GMM_DMA(l, v, rsrc_b);
+  };
+  auto dma_advance = [&]() {
+    if (!ld_live) return;
+    if (++ld_kt == ld_nk) {
+      ++r_ld;
+      load_setup();
+    } else {
+      step_setup();
+    }
+  };
+  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
+
+  i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];  // fragment double buffer: low / high K half of a step
+  auto read_frag = [&](i32x8& f, const uint8_t* base, int hh) {
+    const u32x4 lo = *reinterpret_cast<const u32x4*>(base + fc[hh][0]);
+    const u32x4 hi = *reinterpret_cast<const u32x4*>(base + fc[hh][1]);
+    f = i32x8{(int)lo.x, (int)lo.y, (int)lo.z, (int)lo.w, (int)hi.x, (int)hi.y, (int)hi.z, (int)hi.w};
+  };
+
+  typedef int i32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+  auto read_frag_tr = [&](i32x8& f, uint32_t a) {  // 4 x 8 contraction rows of the lane's column
+    const i32x2 t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a));
+    const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 2048));
+    const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 4096));
+    const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
+    f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
+  };
+  // weight fragment j / token fragment i, K half hh, of the unit at `unit`
+  auto read_frag_b = [&](i32x8& f, const uint8_t* unit, int j, int hh) {
+    if constexpr (!B_TR) {
+      read_frag(f, unit + fb_off + j * 32 * BK, hh);
+    } else {
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * 256));
+    }
+  };
+  auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh) {
+    if constexpr (!A_TR) {
+      read_frag(f, unit + fa_off + i * 32 * BK, hh);
+    } else {
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * 256));
+    }
+  };
+
+  // ---- fill: steps 0 and 1 of the stream into units 0..3, the first fragments into registers ----
+  load_setup();
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_a(0, j);
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_b(1, j);
+  dma_advance();
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_a(2, j);
+#pragma unroll
+  for (int j = 0; j < kParts; ++j) dma_b(3, j);
+  dma_advance();
+  FP8GMM_WAIT_VM(2 * kParts);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + US, j, 0);
+#pragma unroll
+  for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds, i, 0);
+  int ua = 0;  // ring unit of the current step's token rows; its weight rows are in the next unit
+  // vmcnt counts loads and stores in issue order.  The barrier of a step needs the next step's units, which are
+  // older than the token loads issued during the low half-step: "all but the newest kParts".  Right after an
+  // interior epilogue the newest operations also include that epilogue's kFastStores stores, which nothing in
+  // LDS depends on: at the first barrier after it they may stay in flight.
+  bool relaxed = false;
+
+// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
+#define FP8GMM_MF0(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+#define FP8GMM_MF1(i, j) \
+  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+
+  ItemTile cp_next = item_tile(0);  // the compute side's next record, fetched ahead like the load side's
+  for (int r_cp = 0;; ++r_cp) {
+    const ItemTile g = cp_next;
+    if (g.prob < 0) break;
+    cp_next = item_tile(r_cp + 1);
+    const fp8gmm_gemm_problem pr = probs[g.prob];  // only the epilogue needs it: the main loop hides the read
+    const int m0 = g.m0, n0 = g.n0;
+
+    f32x16 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    // One K = 128 step.  `same_item`: the load cursor stays inside its current item after this step (the caller
+    // knows), so advancing it is three additions; otherwise the general advance, which may switch items.
+    auto k_step = [&](auto same_item) {
+      // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
+      // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
+      // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
+      // has read them.
+      const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
+      // ---- low K half: fragments in fa0 / fb0; fetch the high half's from the same units.  No barrier:
+      // nothing written since the last one is read here.
+      {
+        const uint8_t* qa = lds + ua * US;
+        const uint8_t* qb = lds + ub * US;
+        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
+        dma_a(fa, 0);
+        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
+        read_frag_b(fb1[0], qb, 0, 1);
+        read_frag_b(fb1[1], qb, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 2); FP8GMM_SB();
+        dma_a(fa, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 3); FP8GMM_SB();
+        read_frag_b(fb1[2], qb, 2, 1);
+        read_frag_b(fb1[3], qb, 3, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
+        dma_a(fa, 2);
+        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        read_frag_a(fa1[0], qa, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 2); FP8GMM_SB();
+        dma_a(fa, 3);
+        FP8GMM_SB(); FP8GMM_MF0(1, 3); FP8GMM_SB();
+        read_frag_a(fa1[1], qa, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(2, 0); FP8GMM_SB();
+        dma_a(fa, 4);
+        FP8GMM_SB(); FP8GMM_MF0(2, 1); FP8GMM_SB();
+        read_frag_a(fa1[2], qa, 2, 1);
+        FP8GMM_SB(); FP8GMM_MF0(2, 2); FP8GMM_SB();
+        dma_a(fa, 5);
+        FP8GMM_SB(); FP8GMM_MF0(2, 3); FP8GMM_SB();
+        read_frag_a(fa1[3], qa, 3, 1);
+        FP8GMM_SB(); FP8GMM_MF0(3, 0); FP8GMM_SB();
+        dma_a(fa, 6);
+        FP8GMM_SB(); FP8GMM_MF0(3, 1); FP8GMM_SB();
+        dma_a(fa, 7);
+        FP8GMM_SB(); FP8GMM_MF0(3, 2); FP8GMM_MF0(3, 3); FP8GMM_SB();
+      }
+      // ---- high K half: fragments in fa1 / fb1.  The barrier proves that every wavefront has read this
+      // step's units (lgkmcnt(0)) and that the next step's units have landed for all of them.
+      if (relaxed) {
+        FP8GMM_WAIT_VM_LGKM(kParts + kFastStores);
+        relaxed = false;
+      } else {
+        FP8GMM_WAIT_VM_LGKM(kParts);
+      }
+      __builtin_amdgcn_s_barrier();
+      {
+        const uint8_t* qa = lds + na * US;
+        const uint8_t* qb = lds + nb * US;
+        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        dma_b(ua, 0);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        read_frag_b(fb0[0], qb, 0, 0);
+        read_frag_b(fb0[1], qb, 1, 0);
+        FP8GMM_SB(); FP8GMM_MF1(0, 2); FP8GMM_SB();
+        dma_b(ua, 1);
+        FP8GMM_SB(); FP8GMM_MF1(0, 3); FP8GMM_SB();
+        read_frag_b(fb0[2], qb, 2, 0);
+        read_frag_b(fb0[3], qb, 3, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        dma_b(ua, 2);
+        FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
+        read_frag_a(fa0[0], qa, 0, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 2); FP8GMM_SB();
+        dma_b(ua, 3);
+        FP8GMM_SB(); FP8GMM_MF1(1, 3); FP8GMM_SB();
+        read_frag_a(fa0[1], qa, 1, 0);
+        FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
+        dma_b(ua, 4);
+        FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
+        read_frag_a(fa0[2], qa, 2, 0);
+        FP8GMM_SB(); FP8GMM_MF1(2, 2); FP8GMM_SB();
+        dma_b(ua, 5);
+        FP8GMM_SB(); FP8GMM_MF1(2, 3); FP8GMM_SB();
+        read_frag_a(fa0[3], qa, 3, 0);
+        FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_SB();
+        dma_b(ua, 6);
+        FP8GMM_SB(); FP8GMM_MF1(3, 1); FP8GMM_SB();
+        dma_b(ua, 7);
+        if constexpr (decltype(same_item)::value) {
+          ++ld_kt;
+          step_setup();
+        } else {
+          dma_advance();
+        }
+        FP8GMM_SB(); FP8GMM_MF1(3, 2); FP8GMM_MF1(3, 3); FP8GMM_SB();
+      }
+      ua = na;
+    };
+    // The load cursor runs two steps ahead of this loop: while at least three steps of the item remain, its
+    // next step lies in the same item.
+    int kt = 0;
+    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{});
+    for (; kt < g.nk; ++kt) k_step(std::false_type{});
+    // ---- epilogue ----
+    if (g.slot >= 0) {
+      // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
+      partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
+      relaxed = false;
+    } else {
+      // free until the next step's token loads: the unit that held the last step's weights
+      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
+    }
+  }
+  // zero-fill loads issued past the end of the stream still target this workgroup's LDS
+  FP8GMM_WAIT_VM(0);
+  clock_probe_mark(counters, 1);
+}
+
+
+#undef FP8GMM_MF0
+#undef FP8GMM_MF1
+
+// Per device: "the GEMM kernels may use the whole LDS" has been set for this variant.  fp8gmm_init sets it for
+// every variant; a launch on a device that was never initialised sets its own.
+constexpr int kMaxDevices = 64;
+
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
+int prepare_variant(int dev) {
+  static std::atomic<bool> attr_set[kMaxDevices];
+  if (dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
+  if (!attr_set[dev].load(std::memory_order_acquire)) {
+    auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            RING * US) != hipSuccess)
+      return FP8GMM_ERR_LAUNCH;
+    attr_set[dev].store(true, std::memory_order_release);
+  }
+  return FP8GMM_OK;
+}
+
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
+int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item* items_dev, int grid, int out_kind,
+                   int epilogue, uint8_t* workspace, uint64_t* counters, hipStream_t stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
+  const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR>(dev);
+  if (rc != FP8GMM_OK) return rc;
+  hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR>), dim3(grid), dim3(NTHREADS), RING * US, stream,
+                     probs_dev, items_dev, out_kind, epilogue, workspace, counters);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+// One explicit instantiation per operand format / layout combination, each in its own translation unit
+// (gemm_variant.hip compiled with -DFP8GMM_VARIANT_*): the kernel takes most of a minute to compile.
+#define FP8GMM_FOR_EACH_GEMM_VARIANT(X)      \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, false)  \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, false)  \
+  X(FP8GMM_E4M3, FP8GMM_E5M2, false, false)  \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, true)   \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, true)   \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, true, true)    \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true)
+
+#define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT)                                                                     \
+  extern template int prepare_variant<AF, BF, AT, BT>(int);                                                        \
+  extern template int launch_variant<AF, BF, AT, BT>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, \
+                                                     int, uint8_t*, uint64_t*, hipStream_t);
+#ifndef FP8GMM_VARIANT_INDEX
+FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_DECLARE_VARIANT)
+#endif
+
+}  // namespace fp8gmm

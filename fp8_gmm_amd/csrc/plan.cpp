@@ -7,6 +7,8 @@
 // kernels pick the vector or the scalar path per tensor at run time.
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/fp8gmm.h"
 #include "gemm_schedule.h"
 #include "tiling.h"
@@ -25,12 +27,20 @@ const char* fp8gmm_status_string(int status) {
     case FP8GMM_ERR_LAUNCH: return "HIP kernel launch failed";
     case FP8GMM_ERR_BAD_ARGUMENT: return "inconsistent scalar argument";
     case FP8GMM_ERR_NO_DEVICE: return "no usable HIP device";
+    case FP8GMM_ERR_BUFFER_TOO_SMALL: return "output array of a planning call too small (required sizes returned)";
+    case FP8GMM_ERR_WORKSPACE: return "the launch needs more workspace than it was given";
     default: return "unknown fp8gmm status";
   }
 }
 
 size_t fp8gmm_sizeof_tensor_desc(void) { return sizeof(fp8gmm_tensor_desc); }
 size_t fp8gmm_sizeof_gemm_problem(void) { return sizeof(fp8gmm_gemm_problem); }
+size_t fp8gmm_sizeof_gemm_item(void) { return sizeof(fp8gmm_gemm_item); }
+
+int fp8gmm_gemm_grid(int num_cu) {
+  int grid = (num_cu / fp8gmm::kNumXcd) * fp8gmm::kNumXcd;
+  return grid < fp8gmm::kNumXcd ? fp8gmm::kNumXcd : grid;
+}
 
 int fp8gmm_plan_multi_tensor(fp8gmm_tensor_desc* descs, int n, int op, int* total_blocks) {
   if (n < 0) return FP8GMM_ERR_BAD_ARGUMENT;
@@ -120,6 +130,173 @@ int fp8gmm_gemm_fixup(const fp8gmm_gemm_problem* probs, int n, int total_tiles, 
   put(kSlotsPerWg * (xcd * wgs + j - 1) + 1);
   for (int q = j; q < j + n_following; ++q) put(kSlotsPerWg * (xcd * wgs + q));
   return count;
+}
+
+int fp8gmm_plan_grouped_gemm(fp8gmm_gemm_problem* probs, int n, int* total_tiles) {
+  return fp8gmm_plan_grouped_gemm_layout(probs, n, 0, total_tiles);
+}
+
+int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layout, int* total_tiles) {
+  if (n < 0 || (layout & ~(FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR))) return FP8GMM_ERR_BAD_ARGUMENT;
+  const bool a_kmajor = (layout & FP8GMM_GEMM_A_KMAJOR) != 0;
+  const bool b_kmajor = (layout & FP8GMM_GEMM_B_KMAJOR) != 0;
+  if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;  // not a combination the path uses
+  if (total_tiles == nullptr || (n > 0 && probs == nullptr)) return FP8GMM_ERR_NULL_POINTER;
+  int64_t tiles = 0, cost = 0;
+  for (int i = 0; i < n; ++i) {
+    fp8gmm_gemm_problem& p = probs[i];
+    if (p.m < 0 || p.n < 0 || p.k < 0) return FP8GMM_ERR_BAD_SHAPE;
+    if (p.lda < (a_kmajor ? p.m : p.k) || p.ldb < (b_kmajor ? p.n : p.k) || p.ldc < p.n) return FP8GMM_ERR_BAD_SHAPE;
+    const bool has_work = p.m > 0 && p.n > 0;
+    if (has_work) {
+      if (p.c == nullptr) return FP8GMM_ERR_NULL_POINTER;
+      if (p.k > 0) {  // with k == 0 the operands are never read
+        if (p.a == nullptr || p.b == nullptr) return FP8GMM_ERR_NULL_POINTER;
+        // a row-major operand is fetched in 16-byte pieces along k, a contraction-major one along its rows
+        if ((!(a_kmajor && b_kmajor) && (p.k & 15)) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
+        if ((a_kmajor && (p.m & 15)) || (b_kmajor && (p.n & 15))) return FP8GMM_ERR_ALIGNMENT;
+        if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
+          return FP8GMM_ERR_ALIGNMENT;
+        // the kernel addresses the rows of one tile (row-major operand) or the whole operand (contraction-major)
+        // through a buffer descriptor with 32-bit byte offsets; contraction rows up to 127 past k are addressed,
+        // and must fall outside the descriptor, not wrap
+        if ((uint64_t)(a_kmajor ? p.k + 128 : fp8gmm::BM) * (uint64_t)p.lda > 0xffffffffull ||
+            (uint64_t)(b_kmajor ? p.k + 128 : fp8gmm::BN) * (uint64_t)p.ldb > 0xffffffffull)
+          return FP8GMM_ERR_BAD_SHAPE;
+      }
+    }
+    const int64_t tm = (p.m + fp8gmm::BM - 1) / fp8gmm::BM;
+    const int64_t tn = (p.n + fp8gmm::BN - 1) / fp8gmm::BN;
+    p.tile_begin = (int32_t)tiles;
+    p.cost_begin = (int32_t)cost;  // a tile costs ceil(k / 128) steps of the main loop (1 for k = 0)
+    const int64_t steps = (p.k + 127) / 128;
+    tiles += tm * tn;
+    cost += tm * tn * (steps > 0 ? steps : 1);
+    if (tiles > INT32_MAX / 16 || cost > INT32_MAX / 2) return FP8GMM_ERR_BAD_SHAPE;
+  }
+  *total_tiles = (int)tiles;
+  return FP8GMM_OK;
+}
+
+// The work list of a launch: the schedule of gemm_schedule.h written out, one record per (workgroup, item), in
+// the order items[r * grid + workgroup]; the slots in use are renumbered from 0 in the order the workgroups
+// are walked, and the fix-up records name them by their new numbers.
+int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layout, int grid, int stream_k,
+                                    fp8gmm_gemm_item* items, int max_items, fp8gmm_gemm_fixup_desc* fixups,
+                                    int max_fixups, fp8gmm_gemm_plan* plan) {
+  using namespace fp8gmm;
+  if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  *plan = fp8gmm_gemm_plan{};
+  if (grid <= 0 || (grid % kNumXcd) != 0 || max_items < 0 || max_fixups < 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  int total_tiles = 0;
+  const int rc = fp8gmm_plan_grouped_gemm_layout(probs, n, layout, &total_tiles);
+  if (rc != FP8GMM_OK) return rc;
+  plan->total_tiles = total_tiles;
+  if (total_tiles == 0) return FP8GMM_OK;
+  // tail balancing can only pay when the launch has few rounds; it needs the whole grid even for few tiles
+  const bool sk = stream_k != 0 && (int64_t)total_tiles <= (int64_t)kSkMaxRounds * grid && grid > kNumXcd;
+  if (!sk) {
+    const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
+    if (grid > needed) grid = needed;
+  }
+  const int wgs = grid / kNumXcd;
+  const bool a_kmajor = (layout & FP8GMM_GEMM_A_KMAJOR) != 0, b_kmajor = (layout & FP8GMM_GEMM_B_KMAJOR) != 0;
+
+  // pass 1: sizes.  The tiles that were shared along K first: the pieces of such a tile get consecutive
+  // workspace slots, numbered from 0 over the launch, in K order.
+  std::vector<Sched> sched(kNumXcd);
+  for (int x = 0; x < kNumXcd; ++x) sched_init(sched[x], probs, n, total_tiles, x, wgs, sk);
+  std::vector<int32_t> slot_map((size_t)kSlotsPerWg * grid, -1);
+  std::vector<fp8gmm_gemm_fixup_desc> fix;
+  int n_slots = 0;
+  if (sk)
+    for (int x = 0; x < kNumXcd; ++x)
+      for (int j = 1; j < wgs; ++j) {
+        int nf = 0;
+        const int tile = fixup_tile(sched[x], j, &nf);
+        if (tile < 0) continue;
+        const int prob = problem_of_tile(sched[x], tile);
+        fp8gmm_gemm_fixup_desc o{};
+        o.prob = prob;
+        tile_origin(probs[prob].m, probs[prob].n, tile - probs[prob].tile_begin, &o.m0, &o.n0);
+        o.first_slot = n_slots;
+        o.n_pieces = nf + 1;
+        // uncompacted numbering: the piece from the tile's first K step sits in slot 2 (x wgs + j - 1) + 1,
+        // the following ones in slots 2 (x wgs + q), q = j, j + 1, ...
+        slot_map[kSlotsPerWg * (x * wgs + j - 1) + 1] = n_slots++;
+        for (int q = j; q < j + nf; ++q) slot_map[kSlotsPerWg * (x * wgs + q)] = n_slots++;
+        fix.push_back(o);
+      }
+  int rounds = 0;
+  for (int wg = 0; wg < grid; ++wg) {
+    const int x = wg % kNumXcd, j = wg / kNumXcd;
+    Cursor c;
+    cursor_init(sched[x], j, c);
+    int count = 0;
+    for (; cursor_valid(sched[x], j, c); cursor_advance(sched[x], j, c)) ++count;
+    if (count > rounds) rounds = count;
+  }
+  rounds += 1;  // every list ends with a record whose prob is -1
+  const int n_fixups = (int)fix.size();
+  plan->grid = grid;
+  plan->rounds = rounds;
+  plan->n_fixups = n_fixups;
+  plan->n_slots = n_slots;
+  if ((int64_t)rounds * grid > INT32_MAX / 64) return FP8GMM_ERR_BAD_SHAPE;
+  if ((int64_t)rounds * grid > max_items || n_fixups > max_fixups) return FP8GMM_ERR_BUFFER_TOO_SMALL;
+  if (items == nullptr || (n_fixups > 0 && fixups == nullptr)) return FP8GMM_ERR_NULL_POINTER;
+
+  // pass 2: records
+  for (int f = 0; f < n_fixups; ++f) fixups[f] = fix[f];
+  fp8gmm_gemm_item end_record{};
+  end_record.prob = -1;
+  end_record.slot = -1;
+  for (int i = 0; i < rounds * grid; ++i) items[i] = end_record;
+  for (int wg = 0; wg < grid; ++wg) {
+    const int x = wg % kNumXcd, j = wg / kNumXcd;
+    Cursor c;
+    cursor_init(sched[x], j, c);
+    int r = 0;
+    for (; cursor_valid(sched[x], j, c); cursor_advance(sched[x], j, c), ++r) {
+      const Item it = cursor_item(sched[x], x, j, c);
+      const fp8gmm_gemm_problem& p = probs[it.prob];
+      fp8gmm_gemm_item& o = items[(size_t)r * grid + wg];
+      o = fp8gmm_gemm_item{};
+      const int64_t rows = p.m - it.m0 < BM ? p.m - it.m0 : BM;
+      const int64_t cols = p.n - it.n0 < BN ? p.n - it.n0 : BN;
+      if (p.k > 0) {
+        // extents: up to the last byte of the tile's last row (row-major) / of the operand's last contraction row
+        if (!a_kmajor) {
+          o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0 * (uint64_t)p.lda;
+          o.a_bytes = (uint32_t)((rows - 1) * p.lda + p.k);
+        } else {
+          o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0;
+          o.a_bytes = (uint32_t)((int64_t)(p.k - 1) * p.lda + (p.m - it.m0));
+        }
+        if (!b_kmajor) {
+          o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0 * (uint64_t)p.ldb;
+          o.b_bytes = (uint32_t)((cols - 1) * p.ldb + p.k);
+        } else {
+          o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0;
+          o.b_bytes = (uint32_t)((int64_t)(p.k - 1) * p.ldb + (p.n - it.n0));
+        }
+      }
+      o.lda = p.lda;
+      o.ldb = p.ldb;
+      o.k = p.k;
+      o.k_begin = it.k_begin;
+      o.nk = it.nk;
+      o.m0 = it.m0;
+      o.n0 = it.n0;
+      o.prob = it.prob;
+      o.slot = -1;
+      if (it.slot >= 0) {
+        o.slot = slot_map[it.slot];
+        if (o.slot < 0) return FP8GMM_ERR_BAD_ARGUMENT;  // a partial item that no fix-up record completes
+      }
+    }
+  }
+  return FP8GMM_OK;
 }
 
 }  // extern "C"

@@ -18,5 +18,8 @@ constexpr int kPtTileCols = 128;                 // tile extent along the featur
 constexpr int kGemmTileM = 256;                  // rows of c per workgroup tile
 constexpr int kGemmTileN = 256;                  // columns of c per workgroup tile
 constexpr int kGemmTileK = 128;                  // bytes of K consumed per main-loop step
+constexpr int BM = kGemmTileM;
+constexpr int BN = kGemmTileN;
+constexpr int kNumXcd = 8;                       // workgroup i of a launch runs on XCD i % 8
 
 }  // namespace fp8gmm

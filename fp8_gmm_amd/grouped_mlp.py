@@ -125,6 +125,9 @@ class _GroupedMlp(torch.autograd.Function):
             c_amaxes=meta.get_meta_pointers(_T.kInputGroup2, _M.kAmax),
             backward=False, cutlass=False,
         )
+        capture = fp8_meta.get("capture")
+        if capture is not None:  # see GroupedMlp.capture_intermediates
+            capture.update(pre_gelu_out=pre_gelu_out, gelu_out_fp8=gelu_out_fp8)
         if not is_grad_enabled:
             pre_gelu_out = None
         out = fp8_gmm(
@@ -226,6 +229,9 @@ class _GroupedMlp(torch.autograd.Function):
             multi_cast_dgelu(row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums),
                              row_slices(grad_pre_fp8, cumsums), g2_scales, g2_amaxes)
         g2_scale_invs = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScaleInv)
+        capture = ctx.fp8_meta.get("capture")
+        if capture is not None:
+            capture.update(grad_gelu_out=grad_gelu_out, grad_pre_fp8=grad_pre_fp8)
 
         grad_input = None
         handle = None
@@ -282,6 +288,15 @@ class GroupedMlp(Fp8GroupedModuleBase):
         torch.nn.init.uniform_(self.fc1_weight.data, -b1, b1)
         torch.nn.init.uniform_(self.fc2_weight.data, -b2, b2)
         self._weight_caches.extend([Fp8WeightCache(), Fp8WeightCache()])
+
+    def capture_intermediates(self, store):
+        """Keep references to the tensors a pass produces between its kernels in the dict ``store`` (None: stop):
+        ``pre_gelu_out`` bf16 and ``gelu_out_fp8`` of the forward pass, ``grad_gelu_out`` bf16 and ``grad_pre_fp8``
+        of the backward pass.  For checks that follow the data flow stage by stage; costs nothing when unset."""
+        if store is None:
+            self.fp8_meta.pop("capture", None)
+        else:
+            self.fp8_meta["capture"] = store
 
     def get_fp8_weights_scratchpad(self, is_first_microbatch):
         """``[fc1_weight_fp8, fc1_weight_t_fp8, fc2_weight_fp8, fc2_weight_t_fp8]`` kept across micro-batches, or

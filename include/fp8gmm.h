@@ -4,10 +4,10 @@
  * This is the boundary that replaces the reference's pybind11 module
  * `fp8_gmm_backend` (csrc/ops.cu:9-16).  Every function is `extern "C"`,
  * takes plain pointers and integers, returns an int status (0 = success,
- * negative = fp8gmm_status) and never throws, frees or synchronises.  The only
- * allocation is fp8gmm_grouped_gemm's tail-balancing workspace (128 MB, once per
- * device and stream, for up to 8 streams; kept until the process ends; skipped,
- * without error, when the allocation is refused or FP8GMM_STREAMK=0 is set).
+ * negative = fp8gmm_status) and never throws, allocates, frees or synchronises:
+ * scratch memory (the grouped GEMM's tail-balancing workspace, the router's
+ * counters) is passed in by the caller.  fp8gmm_init is the one call that talks to
+ * the runtime about anything but a launch.
  * All device work is enqueued on the HIP stream passed in (`hipStream_t`,
  * passed as `void*`; NULL = the default stream).
  *
@@ -16,11 +16,12 @@
  * argument structs, csrc/multi_pointwise.cu:13, csrc/multi_pad_fusion.cu:14).
  * The protocol is:
  *   1. the caller fills an array of descriptors in host memory;
- *   2. `fp8gmm_plan_*` validates it and fills the scheduling fields
- *      (`block_begin` / `tile_begin`) and returns the launch size;
- *   3. the caller copies the array to device memory on the same stream;
+ *   2. `fp8gmm_plan_*` validates it, fills the scheduling fields
+ *      (`block_begin` / `tile_begin`) and returns the launch size; for the GEMM
+ *      it also writes the launch's work list (one record per workgroup and tile);
+ *   3. the caller copies the arrays to device memory on the same stream;
  *   4. `fp8gmm_multi_*` / `fp8gmm_grouped_gemm` launches one kernel over the
- *      device copy.
+ *      device copies.
  * The library never owns memory; outputs are written in place.
  */
 #ifndef FP8GMM_H_
@@ -33,7 +34,7 @@
 extern "C" {
 #endif
 
-#define FP8GMM_VERSION 1
+#define FP8GMM_VERSION 2
 
 /* fp8 formats (OCP): e4m3fn = torch.float8_e4m3fn, e5m2 = torch.float8_e5m2 */
 #define FP8GMM_E4M3 0
@@ -49,7 +50,9 @@ typedef enum fp8gmm_status {
   FP8GMM_ERR_ALIGNMENT = -4,      /* GEMM operand not 16-byte aligned / K or pitch not a multiple of 16 */
   FP8GMM_ERR_LAUNCH = -5,         /* the HIP runtime rejected the launch */
   FP8GMM_ERR_BAD_ARGUMENT = -6,   /* inconsistent scalar arguments (count < 0, total mismatch, ...) */
-  FP8GMM_ERR_NO_DEVICE = -7       /* no usable gfx950 device */
+  FP8GMM_ERR_NO_DEVICE = -7,      /* no usable gfx950 device */
+  FP8GMM_ERR_BUFFER_TOO_SMALL = -8, /* an output array of a planning call cannot hold the result (sizes are returned) */
+  FP8GMM_ERR_WORKSPACE = -9       /* the launch needs more workspace than it was given */
 } fp8gmm_status;
 
 /*
@@ -102,8 +105,8 @@ typedef struct fp8gmm_tensor_desc {
  * Both operands are K-contiguous ("TN"), the only layout the reference uses
  * (fp8_gmm/backend.py:25,57; csrc/fp8_gmm.h:7-11).  Pitches are in elements.
  * a, b must be 16-byte aligned and k, lda, ldb multiples of 16 (the same
- * divisibility cuBLASLt demands of the reference, grouped_linear.py:68); one operand of one problem
- * may span at most 4 GiB (m * lda, n * ldb < 2^32).
+ * divisibility cuBLASLt demands of the reference, grouped_linear.py:68); 256 rows of an operand
+ * may span at most 4 GiB (256 * lda, 256 * ldb < 2^32).
  * k == 0 is allowed and writes epilogue(0); m == 0 or n == 0 produce no work.
  *
  * Epilogue:  v = acc * (*a_scale_inv * *b_scale_inv)        (NULL scale = 1)
@@ -145,11 +148,67 @@ typedef struct fp8gmm_gemm_problem {
  * 16, k arbitrary (rows past k contribute zeros), (k + 128) * lda < 2^32. */
 #define FP8GMM_GEMM_A_KMAJOR 4
 
+/*
+ * Work list of a grouped-GEMM launch, written by fp8gmm_plan_grouped_gemm_launch on the host and read by the
+ * kernel: the launch has `grid` persistent workgroups (a multiple of 8; workgroup i runs on XCD i % 8), and
+ * workgroup w processes the records items[r * grid + w], r = 0, 1, ..., up to the first record with
+ * prob == -1.  A record is one 256 x 256 tile of one problem's c, or - for the tail tiles that the
+ * workgroups of an XCD share along K - a contiguous range of K = 128 steps of one, whose fp32 partial sums go
+ * to a workspace slot.  The record carries what the kernel's load stream needs (operand addresses of the
+ * tile, extents for the bounds check, pitches), so that switching tiles costs it one 64-byte read.
+ * No counterpart in the reference: CUTLASS's tile scheduler computes the equivalent on the device
+ * (csrc/fp8_gmm.cu:73-80,146-159).
+ */
+typedef struct fp8gmm_gemm_item {
+  uint64_t a;          /* first byte of the tile's rows of operand a (row-major: a + m0 * lda; contraction-major: a + m0) */
+  uint64_t b;          /* the same for operand b and n0 */
+  uint32_t a_bytes;    /* bytes addressable from `a`: reads past them deliver zeros */
+  uint32_t b_bytes;
+  int32_t lda, ldb;
+  int32_t k;           /* contraction length of the problem */
+  int32_t k_begin;     /* first K = 128 step of this record */
+  int32_t nk;          /* number of K = 128 steps (0: a problem without K, only the epilogue runs) */
+  int32_t m0, n0;      /* origin of the tile in c */
+  int32_t prob;        /* index into the problem table; -1 ends a workgroup's list */
+  int32_t slot;        /* -1: whole tile, the epilogue runs; else the workspace slot that receives the partial sums */
+  int32_t reserved;
+} fp8gmm_gemm_item;    /* 64 bytes */
+
+/* One tile that was shared along K: the fix-up launch adds the partial sums of the workspace slots first_slot,
+ * first_slot + 1, ..., first_slot + n_pieces - 1 (the tile's pieces in K order) and runs the epilogue. */
+typedef struct fp8gmm_gemm_fixup_desc {
+  int32_t prob, m0, n0;
+  int32_t first_slot, n_pieces;
+  int32_t reserved[3];
+} fp8gmm_gemm_fixup_desc;   /* 32 bytes */
+
+/* Sizes of a planned launch. */
+typedef struct fp8gmm_gemm_plan {
+  int32_t grid;        /* workgroups of the main launch */
+  int32_t rounds;      /* records per workgroup, end record included: items has rounds * grid entries */
+  int32_t n_fixups;    /* tiles shared along K = workgroups of the fix-up launch (0: no such launch) */
+  int32_t n_slots;     /* workspace slots the launch writes: it needs n_slots * FP8GMM_GEMM_SLOT_BYTES bytes */
+  int32_t total_tiles;
+  int32_t reserved[3];
+} fp8gmm_gemm_plan;    /* 32 bytes */
+
+#define FP8GMM_GEMM_SLOT_BYTES 262144  /* fp32 accumulators of one 256 x 256 tile */
+
 /* ---- library info ------------------------------------------------------------------------- */
 int fp8gmm_version(void);
 const char* fp8gmm_status_string(int status);
 size_t fp8gmm_sizeof_tensor_desc(void);   /* lets a binding check its struct layout */
 size_t fp8gmm_sizeof_gemm_problem(void);
+size_t fp8gmm_sizeof_gemm_item(void);
+/*
+ * Once per device, before the first launch on it (with that device current or named here; -1 = the current one):
+ * looks up the device's compute-unit count and lets the GEMM kernels use the whole LDS.  Returns the number of
+ * compute units (> 0) or a negative status.  Launches on a device that was never initialised do this themselves
+ * on their first call; calling it explicitly keeps that work out of a timed or captured region.
+ */
+int fp8gmm_init(int device);
+/* grid of a grouped-GEMM launch on a device with `num_cu` compute units: one workgroup per unit, a multiple of 8 */
+int fp8gmm_gemm_grid(int num_cu);
 /* workgroup tile of the GEMM kernel (rows of c, columns of c), for callers that size grids */
 void fp8gmm_gemm_tile_shape(int* tile_m, int* tile_n);
 
@@ -186,25 +245,46 @@ int fp8gmm_multi_pad_cast_transpose_dgelu(fp8gmm_tensor_desc* descs_dev, int n, 
 int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream);
 
 /*
- * One persistent launch over all tiles of all problems.
- * replaces Fp8GroupedGemm, csrc/fp8_gmm.cu:163 (pybind name fp8_gmm, csrc/ops.cu:10) and the
- * per-expert cuBLASLt loop of fp8_gmm/backend.py:84-96 and grouped_linear.py:173-182.
- *   a_fmt, b_fmt : FP8GMM_E4M3 / FP8GMM_E5M2 (e5m2 x e5m2 is rejected, as cuBLASLt does)
- *   out_kind     : FP8GMM_OUT_BF16, or FP8GMM_E4M3 / FP8GMM_E5M2 for an fp8 `c`
- *   epilogue     : 0 or FP8GMM_EPI_GELU
+ * Validates `probs[0..n)` like fp8gmm_plan_grouped_gemm_layout, fills tile_begin / cost_begin, and writes the work
+ * list of a launch with `grid` workgroups (fp8gmm_gemm_grid) into items[0 .. rounds * grid) and
+ * fixups[0 .. n_fixups).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
+ * the last round would otherwise be mostly idle; the launch then needs plan->n_slots workspace slots (never more
+ * than 2 * grid).  stream_k == 0: every record is a whole tile, no workspace, no fix-up launch.
+ * The sizes are returned in *plan even when max_items / max_fixups are too small (FP8GMM_ERR_BUFFER_TOO_SMALL,
+ * nothing written to the arrays): call again with larger arrays.  Host only, no GPU needed.
  */
-int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, int total_tiles, int a_fmt, int b_fmt,
-                        int out_kind, int epilogue, void* stream);
+int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layout, int grid, int stream_k,
+                                    fp8gmm_gemm_item* items, int max_items, fp8gmm_gemm_fixup_desc* fixups,
+                                    int max_fixups, fp8gmm_gemm_plan* plan);
 
 /*
- * Measurement hook, no counterpart in the reference.  While `dev_counters` (device memory, 8 x 4 uint64, one
- * group of four per XCD) is set, fp8gmm_grouped_gemm launches a measurement build of its kernel in which the
- * first workgroup of every XCD writes {shader-cycle counter, 100 MHz counter} when it starts ([0], [1]) and adds
- * the elapsed cycles and ticks to [2], [3] when it ends (clear them first): [2] / [3] * 100 MHz is the clock the
- * launches really ran at, which the clock the driver reports overstates while the chip is power-limited.  NULL (the default) restores the normal kernel.
- * Applies to the current device; the call synchronises.  bench.py reports the figure.
+ * One persistent launch over all tiles of all problems (plus a small second launch when tiles were shared along K).
+ * replaces Fp8GroupedGemm, csrc/fp8_gmm.cu:163 (pybind name fp8_gmm, csrc/ops.cu:10) and the
+ * per-expert cuBLASLt loop of fp8_gmm/backend.py:84-96 and grouped_linear.py:173-182.
+ *   probs_dev, items_dev, fixups_dev : DEVICE copies of the planned arrays (fixups_dev may be NULL when n_fixups == 0)
+ *   plan         : the host struct fp8gmm_plan_grouped_gemm_launch filled
+ *   a_fmt, b_fmt : FP8GMM_E4M3 / FP8GMM_E5M2 (e5m2 x e5m2 is rejected, as cuBLASLt does)
+ *   out_kind     : FP8GMM_OUT_BF16, or FP8GMM_E4M3 / FP8GMM_E5M2 for an fp8 `c`
+ *   epilogue     : FP8GMM_EPI_GELU and the layout flags the table was planned with
+ *   workspace    : device memory, workspace_bytes >= plan->n_slots * FP8GMM_GEMM_SLOT_BYTES, 256-byte aligned,
+ *                  contents irrelevant; may be NULL when n_slots == 0.  Launches that overlap in time (different
+ *                  streams) need different workspaces.  Too small: FP8GMM_ERR_WORKSPACE, nothing is launched.
  */
-int fp8gmm_gemm_clock_probe(uint64_t* dev_counters);
+int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                        const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
+                        int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The same launch with a measurement on the side, no counterpart in the reference: `dev_counters` (device memory,
+ * 8 x 4 uint64, one group of four per XCD, cleared by the caller) receives from the first workgroup of every XCD
+ * {shader-cycle counter, 100 MHz counter} when it starts ([0], [1]) and the elapsed cycles and ticks added to
+ * [2], [3] when it ends: [2] / [3] * 100 MHz is the clock the launch really ran at, which the clock the driver
+ * reports overstates while the chip is power-limited.  Same kernel, same results; bench.py reports the figure.
+ */
+int fp8gmm_grouped_gemm_timed(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                              const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
+                              int b_fmt, int out_kind, int epilogue, void* workspace, size_t workspace_bytes,
+                              uint64_t* dev_counters, void* stream);
 
 /*
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:
@@ -268,7 +348,8 @@ int fp8gmm_moe_scatter_wgrad(const void* x, const void* grad_out, const int32_t*
  * processes, in order, for the HOST table `probs` (after fp8gmm_plan_grouped_gemm).  stream_k != 0:
  * as in a launch that shares the tail tiles of each XCD's range along K.  Writes up to max_items records
  * of 7 int32 - tile, problem, m0, n0, k_begin, nk, slot (k_begin / nk in steps of 128 bytes of K; slot = -1
- * when the item is a whole tile, else the workspace slot that receives its partial sums) - and returns the
+ * when the item is a whole tile, else its position 2 * workgroup or 2 * workgroup + 1 in the launch's uncompacted
+ * slot numbering; fp8gmm_plan_grouped_gemm_launch renumbers the slots in use from 0) - and returns the
  * number of items.  No counterpart in the reference (its CUTLASS scheduler is not observable); it lets the
  * schedule be checked without a GPU.
  */

@@ -120,9 +120,15 @@ def grouped_linear_step(x, w, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn
 
 
 def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2,
-                     cached=None):
+                     cached=None, given=None):
     """One forward + backward of GroupedMlp. x [M, H], w1 [E, F, H], w2 [E, H, F], dy [M, H].
-    ``cached``: the result of an earlier step whose fp8 weights are reused."""
+    ``cached``: the result of an earlier step whose fp8 weights are reused.
+
+    ``given``: intermediates of another implementation's run of the same step (any of ``pre``, ``gelu_fp8``,
+    ``grad_gelu``, ``dpre_fp8``).  A given tensor replaces this function's own from the point where it is
+    produced, so that everything downstream is computed from identical bytes and can be compared GEMM by GEMM;
+    this function's own values are returned beside them under ``own_*`` (the amax it records stays its own)."""
+    given = given or {}
     e = len(sizes)
     b = _bounds(sizes)
     x1 = [3 * i for i in range(e)]
@@ -143,6 +149,9 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
     gelu_fp8 = torch.zeros(m, ffn, dtype=fwd_dtype)
     ref.fp8_gmm(x_fp8, w1_fp8, sizes, [fwd.scale_inv[s] for s in x1], [fwd.scale_inv[s] for s in w1s], gelu_fp8,
                 fwd_dtype, pre, [fwd.scale[s: s + 1] for s in x2], [fwd.amax(s) for s in x2])
+    own = dict(own_pre=pre, own_gelu_fp8=gelu_fp8)
+    pre = given.get("pre", pre)
+    gelu_fp8 = given.get("gelu_fp8", gelu_fp8)
     out = _gmm_bf16(gelu_fp8, w2_fp8, sizes, [fwd.scale_inv[s] for s in x2], [fwd.scale_inv[s] for s in w2s])
     fwd_inv = fwd.scale_inv.clone()
 
@@ -156,6 +165,8 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
         gelu_ts.append(t)
     grad_w2 = _wgrad(dy_ts, gelu_ts, g1_inv, [fwd_inv[s] for s in x2])
     grad_gelu = _gmm_bf16(dy_fp8, w2_t, sizes, g1_inv, [fwd_inv[s] for s in w2s])
+    own["own_grad_gelu"] = grad_gelu
+    grad_gelu = given.get("grad_gelu", grad_gelu)
 
     dpre_fp8 = torch.empty(m, ffn, dtype=bwd_dtype)
     dpre_ts = []
@@ -167,8 +178,16 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
                                        [o], [t], [bwd.scale[g2[i]: g2[i] + 1]], [bwd.amax(g2[i])])
         dpre_fp8[b[i]: b[i + 1]] = o
         dpre_ts.append(t)
+    own["own_dpre_fp8"] = dpre_fp8
+    if "dpre_fp8" in given:
+        dpre_fp8 = given["dpre_fp8"]
+        dpre_ts = []
+        for i, s in enumerate(sizes):
+            t = torch.empty(ffn, (s + 15) // 16 * 16, dtype=bwd_dtype)
+            ref.multi_transpose([dpre_fp8[b[i]: b[i + 1]].contiguous()], [t])
+            dpre_ts.append(t)
     g2_inv = [bwd.scale_inv[s] for s in g2]
     grad_input = _gmm_bf16(dpre_fp8, w1_t, sizes, g2_inv, [fwd_inv[s] for s in w1s])
     grad_w1 = _wgrad(dpre_ts, x_ts, g2_inv, [fwd_inv[s] for s in x1])
-    return dict(out=out, grad_input=grad_input, grad_w1=grad_w1, grad_w2=grad_w2, pre=pre, gelu_fp8=gelu_fp8,
+    return dict(own, out=out, grad_input=grad_input, grad_w1=grad_w1, grad_w2=grad_w2, pre=pre, gelu_fp8=gelu_fp8,
                 grad_gelu=grad_gelu, dpre_fp8=dpre_fp8, w1_fp8=w1_fp8, w1_t_fp8=w1_t, w2_fp8=w2_fp8, w2_t_fp8=w2_t)

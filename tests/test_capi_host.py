@@ -36,7 +36,11 @@ def test_struct_layouts_match_the_binding():
     assert lib.fp8gmm_sizeof_gemm_problem() == _lib.GEMM_PROBLEM.itemsize == 96
     assert _lib.TENSOR_DESC.fields["rows"][1] == 48 and _lib.TENSOR_DESC.fields["block_begin"][1] == 60
     assert _lib.GEMM_PROBLEM.fields["m"][1] == 64 and _lib.GEMM_PROBLEM.fields["tile_begin"][1] == 88
-    assert lib.fp8gmm_version() == 1
+    assert lib.fp8gmm_sizeof_gemm_item() == _lib.GEMM_ITEM.itemsize == 64 and _lib.GEMM_FIXUP.itemsize == 32
+    assert _lib.GEMM_ITEM.fields["lda"][1] == 24 and _lib.GEMM_ITEM.fields["k"][1] == 32
+    assert _lib.GEMM_ITEM.fields["prob"][1] == 52
+    assert ctypes.sizeof(_lib.GemmPlan) == 32
+    assert lib.fp8gmm_version() == 2
     assert _lib.gemm_tile_shape() == (256, 256)
     assert lib.fp8gmm_status_string(0) == b"ok"
     assert b"NULL" in lib.fp8gmm_status_string(-1)
@@ -118,7 +122,8 @@ def test_plan_grouped_gemm_error_codes():
     assert rc(_prob([16], [16], [32], c=0)) == -1
     assert rc(_prob([16], [16], [32], b=0)) == -1
     assert rc(_prob([-1], [16], [32])) == -2
-    assert rc(_prob([70000], [16], [65536])) == -2      # operand larger than 4 GiB
+    assert rc(_prob([70000], [16], [65536])) == 0       # a large operand is fine: descriptors span one tile's rows
+    assert rc(_prob([16], [16], [1 << 24], lda=1 << 24, ldb=1 << 24)) == -2   # ... 256 rows must stay below 4 GiB
     assert rc(_prob([16], [16], [0], a=0, b=0)) == 0     # k == 0 never reads the operands
     assert rc(_prob([0], [16], [32], a=0, b=0, c=0)) == 0 and total.value == 0
 
@@ -129,11 +134,28 @@ def test_launch_entry_points_validate_before_touching_the_gpu():
     assert lib.fp8gmm_multi_quantize(None, 1, 1, 7, None) == -3         # unknown format
     assert lib.fp8gmm_multi_quantize(None, 1, 1, 0, None) == -1         # table missing
     assert lib.fp8gmm_multi_pad_cast_transpose(None, -1, 0, 0, None) == -6
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 1, 1, 2, 0, None) == -3  # e5m2 x e5m2
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 9, 0, None) == -3  # unknown output kind
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 8, None) == -6  # unknown epilogue flag
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, 0, None) == -1
-    assert lib.fp8gmm_grouped_gemm(None, 0, 0, 0, 0, 2, 0, None) == 0
+    plan = _lib.GemmPlan(grid=8, rounds=2, total_tiles=1)
+
+    def gemm(n, a_fmt, b_fmt, out_kind, epilogue, plan=plan, workspace=None, workspace_bytes=0, items=None):
+        return lib.fp8gmm_grouped_gemm(None, n, items, None, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
+                                       workspace_bytes, None)
+
+    assert gemm(1, 1, 1, 2, 0) == -3  # e5m2 x e5m2
+    assert gemm(1, 0, 0, 9, 0) == -3  # unknown output kind
+    assert gemm(1, 0, 0, 2, 8) == -6  # unknown epilogue flag
+    assert gemm(1, 0, 0, 2, 0) == -1  # tables missing
+    assert gemm(0, 0, 0, 2, 0) == 0   # nothing to do
+    assert gemm(1, 0, 0, 2, 0, plan=_lib.GemmPlan()) == 0   # a plan without tiles
+    assert lib.fp8gmm_grouped_gemm(None, 1, None, None, None, 0, 0, 2, 0, None, 0, None) == -1   # no plan
+    # a launch that shares tiles along K needs its workspace, large enough and 256-byte aligned
+    sk = _lib.GemmPlan(grid=8, rounds=2, total_tiles=1, n_fixups=1, n_slots=2)
+    assert gemm(1, 0, 0, 2, 0, plan=sk, items=0x1000) == -1                       # tables first
+    fake = 0x10000  # never dereferenced: validation ends before any launch
+    assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, None, 0, None) == -9
+    assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake, 2 * 262144 - 1, None) == -9
+    assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake + 8, 2 * 262144, None) == -9
+    assert lib.fp8gmm_grouped_gemm_timed(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake, 2 * 262144, None, None) == -1
+    assert b"workspace" in lib.fp8gmm_status_string(-9)
 
 
 def test_plan_grouped_gemm_layouts():
@@ -164,12 +186,39 @@ def test_plan_grouped_gemm_layouts():
     assert rc(_prob([512], [256], [128], lda=512), A) == -6
     assert rc(_prob([16], [16], [16]), 8) == -6
     # the launch refuses the same combinations, and a contraction-major b that is not e4m3
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, A, None) == -6
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 1, 2, B, None) == -3
-    assert lib.fp8gmm_grouped_gemm(None, 1, 1, 0, 0, 2, A | B | _lib.EPI_GELU, None) == -1   # valid flags, no table
+    plan = _lib.GemmPlan(grid=8, rounds=2, total_tiles=1)
+    assert lib.fp8gmm_grouped_gemm(None, 1, None, None, plan, 0, 0, 2, A, None, 0, None) == -6
+    assert lib.fp8gmm_grouped_gemm(None, 1, None, None, plan, 0, 1, 2, B, None, 0, None) == -3
+    assert lib.fp8gmm_grouped_gemm(None, 1, None, None, plan, 0, 0, 2, A | B | _lib.EPI_GELU, None, 0,
+                                   None) == -1   # valid flags, no table
     t = _prob([137, 0, 401], [512, 512, 512], [300, 0, 77], lda=[137 + 7, 16, 416], ldb=512)
     t["lda"] = [144, 16, 416]
     assert rc(t, A | B) == -4     # m = 137 is not a multiple of 16
     t = _prob([144, 0, 416], [512, 512, 512], [300, 0, 77], ldb=512)
     t["lda"] = [144, 16, 416]
     assert rc(t, A | B) == 0 and t["tile_begin"].tolist() == [0, 2, 2] and t["cost_begin"].tolist() == [0, 6, 6]
+
+
+def test_gemm_grid_is_one_workgroup_per_compute_unit_in_multiples_of_eight():
+    assert [_lib.gemm_grid(c) for c in (256, 304, 250, 8, 3, 0)] == [256, 304, 248, 8, 8, 8]
+
+
+def test_launch_plan_reports_sizes_before_it_writes():
+    """Arrays too small: status -8, the required sizes in the plan, nothing written; then the same call with room."""
+    lib = _lib.load()
+    t = _prob([1000, 300], [512, 512], [256, 256])
+    plan = _lib.GemmPlan()
+    items = np.full(4, 0x55, dtype=np.uint8).view(np.uint8)
+    rc = lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, items.ctypes.data, 0, None, 0,
+                                             ctypes.byref(plan))
+    assert rc == -8 and (items == 0x55).all()
+    # 4 x 2 + 2 x 2 = 12 tiles on 16 workgroups: one record each plus the end record
+    assert (plan.total_tiles, plan.grid, plan.rounds, plan.n_fixups, plan.n_slots) == (12, 16, 2, 0, 0)
+    p2, it, fx = _lib.plan_grouped_gemm_launch(t, 0, 16, False)
+    assert (p2.grid, p2.rounds) == (16, 2) and len(it) == 32 and len(fx) == 0
+    assert sorted(it["prob"][:16].tolist()) == [-1] * 4 + [0] * 8 + [1] * 4 and (it["prob"][16:] == -1).all()
+    # a launch never has more workgroups than tiles (rounded up to a multiple of 8) when nothing is shared along K
+    p3, it3, _ = _lib.plan_grouped_gemm_launch(_prob([100], [100], [128]), 0, 256, False)
+    assert (p3.grid, p3.rounds, p3.total_tiles) == (8, 2, 1) and (it3["prob"] >= 0).sum() == 1
+    assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 12, 0, None, 0, None, 0, ctypes.byref(plan)) == -6
+    assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, None, 0, None, 0, None) == -1

@@ -103,7 +103,78 @@ def check_schedule(shapes, grid, stream_k):
                 pos += nk
             assert pos == nk_of[tile_prob[tile]]
     assert done == set(cut_tiles)
+    check_launch_plan(shapes, table, total, grid, stream_k)
     return n_partial_items
+
+
+def check_launch_plan(shapes, table, total, grid, stream_k):
+    """The work list the kernels read (fp8gmm_plan_grouped_gemm_launch) is the schedule above written out:
+    record r of workgroup w sits at items[r * grid + w], lists end with prob == -1, the slots of a shared
+    tile are consecutive in K order, and every record carries the addresses and extents of its tile's operands."""
+    plan, items, fixups = _lib.plan_grouped_gemm_launch(table.copy(), 0, grid, stream_k)
+    assert plan.total_tiles == total
+    if total == 0:
+        return
+    sk = stream_k and total <= 24 * grid and grid > 8
+    g = plan.grid
+    assert g == (grid if sk else min(grid, (total + 7) // 8 * 8)) and len(items) == plan.rounds * g
+    items = items.reshape(plan.rounds, g)
+    slot_name = {}      # uncompacted slot -> slot of the plan
+    pieces_of = {}      # (prob, m0, n0) -> [(k_begin, plan slot)]
+    longest = 0
+    for wg in range(g):
+        want = _lib.gemm_schedule(table, total, g, sk, wg).tolist()
+        longest = max(longest, len(want))
+        col = items[:, wg]
+        assert (col["prob"][len(want):] == -1).all() and len(want) < plan.rounds
+        for rec, (tile, prob, m0, n0, k_begin, nk, slot) in zip(col, want):
+            assert (rec["prob"], rec["m0"], rec["n0"], rec["k_begin"], rec["nk"]) == (prob, m0, n0, k_begin, nk)
+            m, n, k = shapes[prob]
+            lda = ldb = max(k, 16)
+            assert (rec["k"], rec["lda"], rec["ldb"]) == (k, lda, ldb)
+            if k > 0:
+                assert rec["a"] == 0x10000 + m0 * lda and rec["b"] == 0x20000 + n0 * ldb
+                assert rec["a_bytes"] == (min(m - m0, TILE) - 1) * lda + k
+                assert rec["b_bytes"] == (min(n - n0, TILE) - 1) * ldb + k
+            if slot < 0:
+                assert rec["slot"] == -1
+            else:
+                assert 0 <= rec["slot"] < plan.n_slots and slot not in slot_name
+                slot_name[slot] = int(rec["slot"])
+                pieces_of.setdefault((prob, m0, n0), []).append((k_begin, int(rec["slot"])))
+    assert plan.rounds == longest + 1
+    assert sorted(slot_name.values()) == list(range(plan.n_slots))   # renumbered from 0 without gaps
+    assert plan.n_fixups == len(fixups) == len(pieces_of)
+    seen = set()
+    for f in fixups:
+        key = (int(f["prob"]), int(f["m0"]), int(f["n0"]))
+        assert key in pieces_of and key not in seen
+        seen.add(key)
+        slots_in_k_order = [s for _, s in sorted(pieces_of[key])]
+        assert slots_in_k_order == list(range(f["first_slot"], f["first_slot"] + f["n_pieces"]))
+
+
+def test_launch_plan_of_contraction_major_operands():
+    """Addresses and extents of the records when operands are stored contraction-major (gradient GEMMs)."""
+    t = np.zeros(2, dtype=_lib.GEMM_PROBLEM)
+    t["a"], t["b"], t["c"] = 0x10000, 0x20000, 0x30000
+    t["m"], t["n"], t["k"] = [512, 272], [768, 768], [300, 77]
+    t["lda"], t["ldb"], t["ldc"] = [512, 288], [768, 800], 768
+    for layout in (_lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR | _lib.GEMM_A_KMAJOR):
+        tt = t.copy()
+        if not layout & _lib.GEMM_A_KMAJOR:
+            tt["k"] = tt["lda"] = [304, 80]   # a is [m, k] here, fetched in 16-byte pieces of k
+        plan, items, _ = _lib.plan_grouped_gemm_launch(tt, layout, 16, False)
+        recs = items[items["prob"] >= 0]
+        assert len(recs) == plan.total_tiles == 2 * 3 + 2 * 3
+        for r in recs:
+            p = int(r["prob"])
+            m, n, k, lda, ldb = (int(tt[f][p]) for f in ("m", "n", "k", "lda", "ldb"))
+            assert r["b"] == 0x20000 + r["n0"] and r["b_bytes"] == (k - 1) * ldb + (n - r["n0"])
+            if layout & _lib.GEMM_A_KMAJOR:
+                assert r["a"] == 0x10000 + r["m0"] and r["a_bytes"] == (k - 1) * lda + (m - r["m0"])
+            else:
+                assert r["a"] == 0x10000 + r["m0"] * lda and r["a_bytes"] == (min(m - r["m0"], 256) - 1) * lda + k
 
 
 MLP = [1439, 3146, 3993, 1820, 909, 3499, 669, 909]

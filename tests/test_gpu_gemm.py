@@ -78,10 +78,10 @@ def test_tiles_shared_along_k_are_exact(dev, a_dtype, sizes, n, k):
         table[i]["m"], table[i]["n"], table[i]["k"] = m, n, k
         table[i]["lda"] = table[i]["ldb"] = k
         table[i]["ldc"] = n
-    total = _lib.plan_grouped_gemm(table)
-    grid = torch.cuda.get_device_properties(dev).multi_processor_count // 8 * 8
-    cut = sum(int((_lib.gemm_schedule(table, total, grid, True, wg)[:, 6] >= 0).sum()) for wg in range(grid))
-    assert cut > 0, "this shape was meant to exercise the shared-tile path"
+    grid = _lib.gemm_grid(torch.cuda.get_device_properties(dev).multi_processor_count)
+    plan, items, fixups = _lib.plan_grouped_gemm_launch(table, 0, grid, True)
+    assert plan.n_fixups > 0 and (items["slot"] >= 0).sum() == plan.n_slots >= 2, \
+        "this shape was meant to exercise the shared-tile path"
 
     g = gen(7 + n + k)
     vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
@@ -305,10 +305,9 @@ def test_argument_errors_raise(dev):
 
 
 def test_shared_tiles_on_concurrent_streams(dev):
-    """Launches that cut tiles along K keep their partial sums in a workspace owned by (device, stream): GEMMs
-    running at the same time on different streams must not see each other's partial sums, and streams beyond
-    the number of workspaces the library keeps simply run without tail balancing.  Exact data, so any
-    cross-talk shows up as a bit difference."""
+    """Launches that cut tiles along K keep their partial sums in a workspace the caller passes in; the backend
+    keeps one per (device, stream): GEMMs running at the same time on different streams must not see each
+    other's partial sums.  Exact data, so any cross-talk shows up as a bit difference."""
     backend = _backend()
     m, n, k = 300, 512, 8192
     vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
@@ -386,11 +385,9 @@ def test_batched_uploads_runs_the_queued_launches_in_order(dev):
     assert c2.any()
 
 
-def test_clock_probe_build_gives_the_same_results_and_a_plausible_clock(dev):
-    """The measurement build of the GEMM kernel (fp8gmm_gemm_clock_probe) must compute exactly what the normal
-    build computes, and its counters must describe a shader clock inside the chip's range."""
-    from fp8_gmm_amd import _lib
-
+def test_timed_launch_gives_the_same_results_and_a_plausible_clock(dev):
+    """The launch with the clock measurement on the side (fp8gmm_grouped_gemm_timed) must compute exactly what the
+    plain launch computes, and its counters must describe a shader clock inside the chip's range."""
     backend = _backend()
     g = torch.Generator(device=dev).manual_seed(77)
     sizes = [700, 0, 1300, 48]
@@ -401,21 +398,17 @@ def test_clock_probe_build_gives_the_same_results_and_a_plausible_clock(dev):
     sb = torch.full((len(sizes),), 0.25, device=dev)
     want = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
     counters = torch.zeros(32, dtype=torch.int64, device=dev)
-    L = _lib.load()
-    _lib.check(L.fp8gmm_gemm_clock_probe(counters.data_ptr()))
-    try:
+    with backend.gemm_clock_probe(counters):
         got = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
         got2 = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)
         torch.cuda.synchronize()
-    finally:
-        _lib.check(L.fp8gmm_gemm_clock_probe(None))
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     assert torch.equal(got2.view(torch.int16), want.view(torch.int16))
     c = counters.cpu().reshape(8, 4).double()
     assert (c[:, 3] > 0).all(), "every XCD's first workgroup must have reported"
     mhz = c[:, 2] / c[:, 3] * 100.0
     assert ((mhz > 300) & (mhz < 2600)).all(), mhz.tolist()
-    after = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)     # back on the normal build
+    after = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb)     # back on the plain launch
     assert torch.equal(after.view(torch.int16), want.view(torch.int16))
 
 

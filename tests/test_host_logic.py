@@ -122,19 +122,26 @@ def test_delayed_scaling_update_rule():
 
 
 def test_update_rule_equals_the_oracle_restatement():
+    """The oracle's Meta.update is pinned by hand-worked numbers (tests/test_oracle_pins.py::test_meta_update_*);
+    the product's rule is then held against the oracle over several updates, for every option."""
     g = torch.Generator().manual_seed(3)
     hist = torch.rand(5, 12, generator=g) * torch.tensor([0.0, 1.0, 10.0] * 4)
-    a = fp8.Fp8MetaTensors(12, 5, torch.device("cpu"))
-    a.amax_history.copy_(hist)
-    b = orc.Meta(12, 5)
-    b.amax_history = hist.clone()
-    for _ in range(3):
-        fp8.amax_and_scale_update(a, 448.0, fp8.DelayedScaling(amax_history_len=5))
-        b.update(448.0)
-        assert torch.equal(a.scale, b.scale) and torch.equal(a.scale_inv, b.scale_inv)
-        assert torch.equal(a.amax_history, b.amax_history)
-        a.amax_history[0] += 1.5
-        b.amax_history[0] += 1.5
+    hist[2, 5] = float("inf")
+    hist[1, 7] = float("nan")
+    for algo, margin, keep in (("max", 0, None), ("most_recent", 0, None), ("max", 2, None), ("max", 0, (3, 1))):
+        want = orc.Meta(12, 5)
+        want.amax_history = hist.clone()
+        got = fp8.Fp8MetaTensors(12, 5, torch.device("cpu"))
+        got.amax_history.copy_(hist)
+        recipe = fp8.DelayedScaling(amax_history_len=5, amax_compute_algo=algo, margin=margin)
+        kept = [s for s in range(12) if keep and s % keep[0] == keep[1]]
+        for _ in range(7):
+            want.update(448.0, margin=margin, algo=algo, keep_scale_inv=kept)
+            fp8.amax_and_scale_update(got, 448.0, recipe, keep_scale_inv=keep)
+            assert torch.equal(got.scale, want.scale) and torch.equal(got.scale_inv, want.scale_inv), (algo, margin)
+            assert torch.equal(got.amax_history.nan_to_num(nan=-1.0), want.amax_history.nan_to_num(nan=-1.0))
+            want.amax_history[0] += 1.5
+            got.amax_history[0] += 1.5
 
 
 def test_recipe_and_autocast():

@@ -279,3 +279,63 @@ def test_scale_mul_is_left_to_right():
     ref.multi_scale_mul([y], [s1], [s2])
     expect = ((x.float() * s1) * s2).to(torch.bfloat16)
     assert torch.equal(y.view(torch.int16), expect.view(torch.int16))
+
+
+# ---- delayed-scaling bookkeeping of oracle.modules.Meta, pinned by hand-worked numbers ------------------
+# (every expected value below is worked out by hand from the rule: amax = max over the history rows, or
+# row 0 for "most_recent"; scale = fp8_max / amax / 2^margin where amax is finite and > 0, else the old
+# scale; scale_inv = 1 / scale except for the kept slots; the history moves up one row, the last row
+# receives the old row 0, and row 0 is cleared)
+def test_meta_update_hand_worked_max():
+    from oracle.modules import Meta
+
+    m = Meta(4, 3)
+    m.amax_history = torch.tensor([[2.0, 0.0, float("inf"), 7.0], [4.0, 0.0, 1.0, 1.0], [1.0, 0.0, 1.0, 28.0]])
+    m.scale = torch.tensor([9.0, 9.0, 9.0, 9.0])
+    m.scale_inv = torch.tensor([5.0, 5.0, 5.0, 5.0])
+    m.update(448.0, margin=1)
+    # slot 0: max 4 -> 448 / 4 / 2 = 56; slot 1: amax 0 -> old scale; slot 2: inf -> old scale; slot 3: 448 / 28 / 2 = 8
+    assert m.scale.tolist() == [56.0, 9.0, 9.0, 8.0]
+    # reciprocals as the correctly rounded fp32 values of the exact quotients
+    assert torch.equal(m.scale_inv, torch.tensor([1.0 / 56.0, 1.0 / 9.0, 1.0 / 9.0, 0.125], dtype=torch.float32))
+    assert m.amax_history.tolist() == [[0.0, 0.0, 0.0, 0.0], [1.0, 0.0, 1.0, 28.0], [2.0, 0.0, float("inf"), 7.0]]
+
+
+def test_meta_update_hand_worked_most_recent_and_nan():
+    from oracle.modules import Meta
+
+    m = Meta(3, 2)
+    m.amax_history = torch.tensor([[2.0, float("nan"), 0.5], [100.0, 3.0, 1000.0]])
+    m.scale = torch.tensor([1.0, 7.0, 1.0])
+    m.update(448.0, algo="most_recent")
+    assert m.scale.tolist() == [224.0, 7.0, 896.0]          # row 0 only; the NaN slot keeps its scale
+    assert torch.equal(m.scale_inv, torch.tensor([1.0 / 224.0, 1.0 / 7.0, 1.0 / 896.0], dtype=torch.float32))
+    assert m.amax_history[0].tolist() == [0.0, 0.0, 0.0]
+    assert m.amax_history[1, 0].item() == 2.0 and m.amax_history[1, 2].item() == 0.5
+    assert math.isnan(m.amax_history[1, 1].item())
+
+
+def test_meta_update_hand_worked_history_of_one():
+    from oracle.modules import Meta
+
+    m = Meta(2, 1)
+    m.amax_history = torch.tensor([[8.0, 0.0]])
+    m.update(57344.0)
+    assert m.scale.tolist() == [7168.0, 1.0]
+    assert torch.equal(m.scale_inv, torch.tensor([1.0 / 7168.0, 1.0], dtype=torch.float32))
+    assert m.amax_history.tolist() == [[0.0, 0.0]]          # no roll: the single row is cleared
+    m.amax_history[0, 0] = 16.0
+    m.update(57344.0, margin=2)
+    assert m.scale.tolist() == [896.0, 1.0]                 # 57344 / 16 / 4
+
+
+def test_meta_update_hand_worked_keep_scale_inv():
+    from oracle.modules import Meta
+
+    m = Meta(6, 2)
+    m.amax_history = torch.tensor([[1.0, 2.0, 4.0, 8.0, 16.0, 32.0], [0.0] * 6])
+    m.scale_inv = torch.tensor([3.0, 3.0, 3.0, 3.0, 3.0, 3.0])
+    m.update(448.0, keep_scale_inv=[1, 4])                  # the weight slots of two GEMMs
+    assert m.scale.tolist() == [448.0, 224.0, 112.0, 56.0, 28.0, 14.0]   # every scale moves ...
+    assert torch.equal(m.scale_inv, torch.tensor([1.0 / 448.0, 3.0, 1.0 / 112.0, 1.0 / 56.0, 3.0, 1.0 / 14.0],
+                                                 dtype=torch.float32))                    # ... kept slots do not
