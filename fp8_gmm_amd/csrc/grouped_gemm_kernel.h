@@ -72,7 +72,7 @@ constexpr int WAVES_N = BN / WN;  // wavefronts along n: 2 (x 2 along m)
 constexpr int MT = WM / 32;       // 4 MFMA tiles along m per wave
 constexpr int NT = WN / 32;       // 4 MFMA tiles along n per wave
 constexpr int kParts = US / 1024 / NWAVES;  // buffer_load ... lds instructions (1 KB each) per wavefront per unit: 8
-constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the interior bf16 epilogue (8 per 32-row block)
+constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the staged bf16 epilogue (8 per 32-row block)
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -95,36 +95,71 @@ __device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
   return t;
 }
 
+// Per-problem scalars (scaling factors, the current amax) are read through the scalar unit: they are uniform,
+// and a vector load would have to be waited for with vmcnt(0), i.e. together with every operand load the
+// load stream has in flight for the next tile - thousands of cycles per tile when those come from HBM.
+typedef __attribute__((address_space(4))) const float scalar_float;
+__device__ __forceinline__ float load_scale(const float* p) {   // constant while the kernel runs; null means 1
+  return p != nullptr ? *reinterpret_cast<scalar_float*>(reinterpret_cast<uintptr_t>(p)) : 1.f;
+}
+// The running maximum another workgroup may be raising at this moment: any value read is a lower bound of it.
+__device__ __forceinline__ float peek_amax(const float* p) {
+  float v;
+  asm volatile("s_load_dword %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(p) : "memory");
+  return v;
+}
+// amax only grows: once the slot holds a value at or above this wavefront's, the atomic is redundant
+// (the slots of all experts share a cache line, and atomics on one line serialise)
+__device__ __forceinline__ void merge_amax(float* slot, float wave_amax, int lane) {
+  if (slot != nullptr && wave_amax > 0.f && !(peek_amax(slot) >= wave_amax) && lane == 0)
+    atomic_max_nonneg(slot, wave_amax);
+}
+
 // Epilogue of one 256 x 256 tile whose accumulators are complete: scales, optional GELU, conversion,
-// stores, amax.  Returns true when the interior bf16 path ran (exactly kFastStores stores per wavefront).
+// stores, amax.  Returns true when the staged bf16 path ran (exactly kFastStores stores per wavefront).
 // `stage`: 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of the staged path.
+// `oob_zero`: accumulators of rows past m and columns past n are exactly zero (both operands row-major: what
+// lies outside the tile's rows is outside the load descriptors).
+//
+// The staged paths store through a buffer descriptor that spans the tile's valid rows: rows past m fall outside
+// it and are dropped by the hardware, lanes whose columns lie past n carry an offset beyond any descriptor.
+// Edge tiles therefore run the same straight-line code as interior ones, with the same number of store
+// instructions (a ragged expert's last row of tiles used to take a per-element path several times as slow,
+// and the workgroups that drew those tiles set the duration of the launch).
+constexpr uint32_t kMaskedOffset = 0x80000000u;  // + any row offset of a tile (< 2^30) stays out of range
+
+// `s` = a_scale_inv * b_scale_inv and `cs` = c_scale of the problem, read by the caller ahead of time.
 __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
-                                              int out_kind, int epilogue, uint8_t* stage) {
+                                              int out_kind, int epilogue, uint8_t* stage, bool oob_zero, float s,
+                                              float cs) {
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, khalf = lane >> 5;
   const int M = pr.m, N = pr.n;
   bool fast = false;
-    const float sa_inv = pr.a_scale_inv ? *pr.a_scale_inv : 1.f;
-    const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
-    const float s = sa_inv * sb_inv;
     const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
     const int64_t ldc = pr.ldc;
     float amax = 0.f;
     const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
-    if (out_kind == FP8GMM_OUT_BF16 && !gelu && interior && ((ldc & 7) == 0) &&
-        ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0)) {
-      // Interior tile, plain bf16 output: straight-line code with an exact store count.
-      uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
+    const int rv = M - m0 < BM ? M - m0 : BM;   // valid rows and columns of this tile
+    const int cv = N - n0 < BN ? N - n0 : BN;
+    // 16-byte pieces of the tile's rows can be addressed with 32-bit offsets below 2^30
+    const bool desc_ok = ((ldc & 7) == 0) && ldc < (1 << 21) && ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0);
+    if (out_kind == FP8GMM_OUT_BF16 && !gelu && desc_ok && (interior || (cv & 7) == 0)) {
+      // Plain bf16 output: straight-line code with an exact store count.
       // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
       // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
       // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
       // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
       // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
+      uint16_t* const C = static_cast<uint16_t*>(pr.c) + (int64_t)m0 * ldc + n0;
+      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       uint8_t* mine = stage + wave * 8192;
       const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
       const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
+      const int col = wave_n * WN + rchunk * 8;
+      const uint32_t lane_off = col < cv ? (uint32_t)((rrow * (int)ldc + col) * 2) : kMaskedOffset;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
 #pragma unroll
@@ -146,27 +181,32 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         }
 #pragma unroll
         for (int it = 0; it < 8; ++it) {
-          const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
-          global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, v[it]);
+          const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 4 * it) * (int)ldc * 2);  // uniform
+          buf_store16(v[it], rc, lane_off + row_off);
         }
       }
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
-    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && interior && ((ldc & 15) == 0) &&
-               ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0) && ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0)) {
-      // Interior tile of the fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
+    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
+               ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0) && (interior || (oob_zero && (cv & 15) == 0))) {
+      // The fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
       // outputs go through the staging area like the plain form's, one 32-row block at a time - first the bf16
       // block as 32 rows x 256 B, then, in a second pass over the same accumulators, the fp8 block as 32 rows x
       // 128 B (chunk c of row r at chunk c ^ ((r >> 1) & 7)) - so that every store instruction writes whole
-      // lines: 12 per block instead of 32 that touch 32 rows each.
-      uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
-      uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
-      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
+      // lines: 12 per block instead of 32 that touch 32 rows each.  On an edge tile the accumulators outside
+      // the problem are zero (oob_zero), and gelu(0) = 0 leaves the amax alone.
+      uint8_t* const C = static_cast<uint8_t*>(pr.c) + (int64_t)m0 * ldc + n0;
+      uint16_t* const AUX = static_cast<uint16_t*>(pr.aux) + (int64_t)m0 * ldc + n0;
+      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
+      const __amdgpu_buffer_rsrc_t ra = make_rsrc(AUX, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       uint8_t* mine = stage + wave * 8192;
       const int wr = l32 * 256 + khalf * 8;   // bf16 block: + ((4 j + g) ^ (l32 & 15)) * 16
       const int wr8 = l32 * 128 + khalf * 4;  // fp8 block:  + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
       const int rrow = lane >> 4, rchunk = lane & 15;
       const int rrow8 = lane >> 3, rchunk8 = lane & 7;
+      const int col = wave_n * WN + rchunk * 8, col8 = wave_n * WN + rchunk8 * 16;
+      const uint32_t lane_off = col < cv ? (uint32_t)((rrow * (int)ldc + col) * 2) : kMaskedOffset;
+      const uint32_t lane_off8 = col8 < cv ? (uint32_t)(rrow8 * (int)ldc + col8) : kMaskedOffset;
       float tile_amax = 0.f;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
@@ -189,8 +229,8 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
           }
 #pragma unroll
           for (int it = 0; it < 8; ++it) {
-            const int m = m0 + wave_m * WM + i * 32 + 4 * it + rrow;
-            global_store(AUX + (int64_t)m * ldc + n0 + wave_n * WN + rchunk * 8, rb[it]);
+            const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 4 * it) * (int)ldc * 2);
+            buf_store16(rb[it], ra, lane_off + row_off);
           }
         }
         // the wavefront's LDS operations complete in order: the reads above are done before these writes land
@@ -229,16 +269,13 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
           }
 #pragma unroll
           for (int it = 0; it < 4; ++it) {
-            const int m = m0 + wave_m * WM + i * 32 + 8 * it + rrow8;
-            global_store(C + (int64_t)m * ldc + n0 + wave_n * WN + rchunk8 * 16, rb[it]);
+            const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 8 * it) * (int)ldc);
+            buf_store16(rb[it], rc, lane_off8 + row_off);
           }
         }
       }
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
-      if (pr.c_amax != nullptr) {
-        const float am = wave_max(tile_amax);
-        if (lane == 0 && am > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= am)) atomic_max_nonneg(pr.c_amax, am);
-      }
+      merge_amax(pr.c_amax, wave_max(tile_amax), lane);
     } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
@@ -283,7 +320,6 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
     } else {
       uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
-      const float cs = pr.c_scale ? *pr.c_scale : 1.f;
       const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 3) == 0) &&
                        (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
 #pragma unroll
@@ -328,13 +364,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
           }
         }
       }
-      if (pr.c_amax != nullptr) {
-        amax = wave_max(amax);
-        // amax only grows: once the slot holds a value at or above this wavefront's, the atomic is redundant
-        // (the slots of all experts share a cache line, and atomics on one line serialise)
-        if (lane == 0 && amax > 0.f && !(__builtin_nontemporal_load(pr.c_amax) >= amax))
-          atomic_max_nonneg(pr.c_amax, amax);
-      }
+      merge_amax(pr.c_amax, wave_max(amax), lane);
     }
     return fast;
 }
@@ -623,7 +653,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     const ItemTile g = cp_next;
     if (g.prob < 0) break;
     cp_next = item_tile(r_cp + 1);
-    const fp8gmm_gemm_problem pr = probs[g.prob];  // only the epilogue needs it: the main loop hides the read
+    // only the epilogue needs the problem's record and its scaling factors: the main loop hides the reads
+    const fp8gmm_gemm_problem pr = probs[g.prob];
+    const float scale_ab = load_scale(pr.a_scale_inv) * load_scale(pr.b_scale_inv);
+    const float scale_c = load_scale(pr.c_scale);
     const int m0 = g.m0, n0 = g.n0;
 
     f32x16 acc[MT][NT];
@@ -743,7 +776,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       relaxed = false;
     } else {
       // free until the next step's token loads: the unit that held the last step's weights
-      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US);
+      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US, !A_TR && !B_TR, scale_ab,
+                              scale_c);
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS

@@ -603,3 +603,58 @@ def test_bf16_epilogue_whole_line_stores_equal_the_per_group_path(dev, a_dtype):
     torch.cuda.synchronize()
     assert torch.isnan(c0[300].float()).all()
     assert_bytes_equal(c0.cpu().view(torch.int16), c1[:, :n].contiguous().cpu().view(torch.int16), "bf16 output")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("form", ["bf16", "gelu"])
+def test_edge_tiles_store_nothing_outside_the_problem(dev, form):
+    """Edge tiles take the same whole-line store path as interior ones, bounded by a buffer descriptor (rows) and
+    by per-lane masks (columns).  Ragged problems written into column slices of wider, sentinel-filled buffers:
+    the valid region must equal the exact result, every byte outside it must keep the sentinel, and the rows of
+    the neighbouring problem in the same buffer must be untouched by this one's last row of tiles."""
+    backend = _backend()
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    g = torch.Generator(device=dev).manual_seed(99)
+    shapes = [(1, 8), (129, 264), (255, 136), (257, 248), (300, 520), (512, 16), (31, 1000)] if form == "bf16" else \
+        [(1, 16), (129, 272), (255, 144), (257, 240), (300, 528), (31, 1008)]
+    k, pad = 256, 24
+    a_list, b_list, c_views, pre_views, wides, pre_wides = [], [], [], [], [], []
+    for m, n in shapes:
+        a_list.append(vals[torch.randint(0, 8, (m, k), generator=g, device=dev)].to(E4M3))
+        b_list.append(vals[torch.randint(0, 8, (n, k), generator=g, device=dev)].to(E4M3))
+        if form == "bf16":
+            wide = torch.full((m + 3, n + pad), -7.0, dtype=torch.bfloat16, device=dev)
+        else:
+            wide = torch.full((m + 3, n + 2 * pad), 0x55, dtype=torch.uint8, device=dev).view(E4M3)
+            pre_wide = torch.full((m + 3, n + 2 * pad), -7.0, dtype=torch.bfloat16, device=dev)
+            pre_wides.append(pre_wide)
+            pre_views.append(pre_wide[:m, :n])
+        wides.append(wide)
+        c_views.append(wide[:m, :n])
+    e = len(shapes)
+    ones = torch.ones(e, device=dev)
+    if form == "bf16":
+        backend.grouped_gemm(a_list, b_list, c_views, ones, ones)
+    else:
+        amax = torch.zeros(e, device=dev)
+        backend.grouped_gemm(a_list, b_list, c_views, ones, ones, pre_gelu_outs=pre_views,
+                             c_scales=torch.full((e,), 0.5, device=dev), c_amaxes=amax)
+    torch.cuda.synchronize()
+    for i, (m, n) in enumerate(shapes):
+        acc = a_list[i].float() @ b_list[i].float().t()
+        if form == "bf16":
+            assert torch.equal(wides[i][:m, :n], acc.to(torch.bfloat16)), f"problem {i}"
+            outside = wides[i].clone()
+            outside[:m, :n] = -7.0
+            assert (outside == -7.0).all(), f"problem {i}: wrote outside its [m, n] region"
+        else:
+            assert torch.equal(pre_wides[i][:m, :n], acc.to(torch.bfloat16)), f"problem {i} pre-gelu"
+            gelu = torch.nn.functional.gelu(acc, approximate="tanh")
+            got = wides[i][:m, :n].float()
+            want = (gelu * 0.5).clamp(-448, 448)
+            assert ((got - want).abs() <= 0.07 * want.abs() + 2e-3).all(), f"problem {i} gelu output"
+            assert abs(amax[i].item() - gelu.abs().max().item()) <= 1e-3 * gelu.abs().max().item() + 1e-6
+            out8, outp = wides[i].view(torch.uint8).clone(), pre_wides[i].clone()
+            out8[:m, :n] = 0x55
+            outp[:m, :n] = -7.0
+            assert (out8 == 0x55).all() and (outp == -7.0).all(), f"problem {i}: wrote outside its [m, n] region"
