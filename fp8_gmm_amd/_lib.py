@@ -98,6 +98,7 @@ GEMM_FIXUP = np.dtype(
 )
 
 GEMM_SLOT_BYTES = 262144
+GEMM_STATIC_SLOTS = 256
 
 
 class GemmPlan(ctypes.Structure):
@@ -117,6 +118,7 @@ EXPORTS = (
     "fp8gmm_gemm_grid",
     "fp8gmm_plan_grouped_gemm_launch",
     "fp8gmm_grouped_gemm_timed",
+    "fp8gmm_grouped_gemm_static",
     "fp8gmm_gemm_tile_shape",
     "fp8gmm_plan_multi_tensor",
     "fp8gmm_plan_grouped_gemm",
@@ -202,6 +204,8 @@ def load():
     L.fp8gmm_plan_grouped_gemm_launch.argtypes = [vp, ci, ci, ci, ci, vp, ci, vp, ci, pp]
     L.fp8gmm_grouped_gemm.restype = ci
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp]
+    L.fp8gmm_grouped_gemm_static.restype = ci
+    L.fp8gmm_grouped_gemm_static.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp]
     L.fp8gmm_grouped_gemm_timed.restype = ci
     L.fp8gmm_grouped_gemm_timed.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp, vp]
     L.fp8gmm_delayed_scaling_update.restype = ci

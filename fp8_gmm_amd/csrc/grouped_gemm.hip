@@ -6,6 +6,13 @@
 // device-side tables written by the host planner (plan.cpp).
 #include "grouped_gemm_kernel.h"
 
+// Scratch of fp8gmm_grouped_gemm_static: the tail-balancing workspace for callers that cannot allocate one.
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.
+// In host code the name stands for the symbol, not for device memory: the per-device address is looked up once
+// (scratch_for) and only that address is ever handed to a kernel.
+constexpr int kStaticSlots = FP8GMM_GEMM_STATIC_SLOTS;
+static __device__ __align__(256) uint8_t scratch[(size_t)kStaticSlots * FP8GMM_GEMM_SLOT_BYTES];
+
 namespace fp8gmm {
 namespace {
 
@@ -138,6 +145,25 @@ int device_num_cu(int dev) {
   return cus;
 }
 
+// device address of `scratch` on device `dev`, which must be the current device; looked up once per device
+std::atomic<uint8_t*> g_scratch[kMaxDevices];
+
+int scratch_for(int dev, uint8_t** out) {
+  if (dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
+  uint8_t* p = g_scratch[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* addr = nullptr;
+    if (hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)) != hipSuccess || addr == nullptr) {
+      (void)hipGetLastError();
+      return FP8GMM_ERR_NO_DEVICE;
+    }
+    p = static_cast<uint8_t*>(addr);
+    g_scratch[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return FP8GMM_OK;
+}
+
 typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*, uint64_t*,
                          hipStream_t);
 
@@ -211,6 +237,11 @@ int fp8gmm_init(int device) {
   }
   FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_PREPARE)
 #undef FP8GMM_PREPARE
+  if (rc > 0) {
+    uint8_t* unused = nullptr;
+    const int e = scratch_for(dev, &unused);
+    if (e != FP8GMM_OK) rc = e;
+  }
   if (dev != current) (void)hipSetDevice(current);
   return rc;
 }
@@ -229,6 +260,23 @@ int fp8gmm_grouped_gemm_timed(const fp8gmm_gemm_problem* probs_dev, int n, const
   if (dev_counters == nullptr) return FP8GMM_ERR_NULL_POINTER;
   return fp8gmm::launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
                                 workspace_bytes, dev_counters, stream);
+}
+
+int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                               const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
+                               int b_fmt, int out_kind, int epilogue, void* stream) {
+  using namespace fp8gmm;
+  if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  if (plan->n_slots > kStaticSlots) return FP8GMM_ERR_WORKSPACE;  // plan the launch with stream_k = 0, or pass a workspace
+  uint8_t* ws = nullptr;
+  if (plan->n_slots > 0) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
+    const int rc = scratch_for(dev, &ws);
+    if (rc != FP8GMM_OK) return rc;
+  }
+  return launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, ws,
+                        (size_t)kStaticSlots * FP8GMM_GEMM_SLOT_BYTES, nullptr, stream);
 }
 
 }  // extern "C"

@@ -193,6 +193,7 @@ typedef struct fp8gmm_gemm_plan {
 } fp8gmm_gemm_plan;    /* 32 bytes */
 
 #define FP8GMM_GEMM_SLOT_BYTES 262144  /* fp32 accumulators of one 256 x 256 tile */
+#define FP8GMM_GEMM_STATIC_SLOTS 256   /* slots of the library's own scratch (fp8gmm_grouped_gemm_static): 64 MiB */
 
 /* ---- library info ------------------------------------------------------------------------- */
 int fp8gmm_version(void);
@@ -273,6 +274,21 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
 int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
                         const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
                         int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * fp8gmm_grouped_gemm for callers that cannot allocate a workspace (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc).  No counterpart in the reference.  The partial sums of tiles shared along K
+ * go to a scratch array that is part of the library's device image: 64 MiB (FP8GMM_GEMM_STATIC_SLOTS slots) on
+ * every GPU the library runs on, held until the process ends.  The call allocates and frees nothing.  A plan
+ * with more slots is refused with FP8GMM_ERR_WORKSPACE and nothing is launched (plan it with stream_k = 0, which
+ * needs no slots, or call fp8gmm_grouped_gemm with a workspace).  All calls on one GPU share the array: calls
+ * that overlap in time (different streams, or threads) race on it; calls on one stream are ordered and safe.
+ * Nothing needs clearing between calls: a launch writes every slot before it reads it.  The device address of
+ * the array is looked up by fp8gmm_init (or by the first call on a device that was never initialised).
+ */
+int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                               const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
+                               int b_fmt, int out_kind, int epilogue, void* stream);
 
 /*
  * The same launch with a measurement on the side, no counterpart in the reference: `dev_counters` (device memory,
