@@ -127,3 +127,112 @@ def assert_close_multistage(c_gpu, ref_t, fro_tol=5e-3, what=""):
     rms = r.pow(2).mean().sqrt()
     bad = err.abs() > 0.02 * r.abs() + 0.25 * rms
     assert not bad.any(), f"{what}: {int(bad.sum())} elements outside 0.02|ref| + 0.25 rms"
+
+
+def fp8_code_distance(a, b):
+    """|difference| in fp8 code steps between two same-dtype fp8 tensors (sign-magnitude codes)."""
+    ia = a.view(torch.uint8).to(torch.int32)
+    ib = b.view(torch.uint8).to(torch.int32)
+    sa = torch.where(ia >= 128, -(ia - 128), ia)
+    sb = torch.where(ib >= 128, -(ib - 128), ib)
+    return (sa - sb).abs()
+
+
+def _mini_meta(gpu_meta, slots):
+    """The scaling state of `slots` of a module's GPU meta as an oracle Meta with history length 1 (amax row
+    cleared: the oracle records its own)."""
+    from oracle import modules as orc
+
+    m = orc.Meta(len(slots), 1)
+    m.scale = gpu_meta.scale.detach().cpu()[slots].clone()
+    m.scale_inv = gpu_meta.scale_inv.detach().cpu()[slots].clone()
+    return m
+
+
+def check_linear_expert_against_oracle(module, i, sizes, x, dy, out, grad_input, tol=1e-2, what=""):
+    """One expert of a GroupedLinear step against the CPU oracle, with the scales the GPU pass used: output,
+    input gradient and weight gradient within `tol`, the amax of every directly cast tensor bit-exact.
+    To be called after the step, before the next forward pass updates the scales."""
+    from oracle import modules as orc
+
+    e = len(sizes)
+    r0 = sum(sizes[:i])
+    r1 = r0 + sizes[i]
+    gm = module.fp8_meta
+    fwd = _mini_meta(gm["scaling_fwd"], [3 * i, 3 * i + 1, 3 * i + 2])
+    bwd = _mini_meta(gm["scaling_bwd"], [2 * i, 2 * i + 1])
+    w = module.weight_tensor.detach()[i: i + 1].cpu()
+    o = orc.grouped_linear_step(x[r0:r1].cpu().contiguous(), w, [sizes[i]], dy[r0:r1].cpu().contiguous(), fwd, bwd)
+    tag = f"{what} expert {i} ({sizes[i]} rows)"
+    assert_gemm_close(out[r0:r1], o["out"].float(), tol, f"{tag} out")
+    assert_gemm_close(grad_input[r0:r1], o["grad_input"].float(), tol, f"{tag} grad_input")
+    assert_gemm_close(module.weight_tensor.grad[i], o["grad_weight"][0].float(), tol, f"{tag} grad_weight")
+    g_fwd = gm["scaling_fwd"].amax_history[0].detach().cpu()
+    g_bwd = gm["scaling_bwd"].amax_history[0].detach().cpu()
+    assert_scalar_bits_equal(g_fwd[[3 * i, 3 * i + 1]], fwd.amax_history[0][[0, 1]], f"{tag} forward amax")
+    assert_scalar_bits_equal(g_bwd[[2 * i]], bwd.amax_history[0][[0]], f"{tag} grad_out amax")
+    assert e == module.num_groups
+
+
+def check_mlp_expert_against_oracle(module, captured, i, sizes, x, dy, out, grad_input, tol=1e-2, what=""):
+    """One expert of a GroupedMlp step against the CPU oracle, stage by stage.
+
+    The fp8 re-quantisations inside the layer (GELU output, d(pre-GELU)) make an end-to-end comparison loose: a
+    value on a rounding boundary may land one fp8 code apart and move what it feeds.  So the oracle is handed
+    the GPU's own intermediates (`captured`, from GroupedMlp.capture_intermediates) at each such point, and every
+    stage is held to its own bar:
+      pre-GELU, d(GELU output)                     within `tol` of the oracle's own values (GEMM + bf16)
+      fp8 GELU output                              at most one code step from the oracle's epilogue of the pre-GELU copy
+      d(pre-GELU) fp8 bytes and its amax           bit-exact, given the GPU's bf16 inputs of that cast
+      output, input and weight gradients           within `tol` of the oracle's GEMMs on the GPU's fp8 bytes
+      amax of x, both weights, grad_out            bit-exact"""
+    from oracle import modules as orc
+
+    e = len(sizes)
+    r0 = sum(sizes[:i])
+    r1 = r0 + sizes[i]
+    gm = module.fp8_meta
+    fwd = _mini_meta(gm["scaling_fwd"], [3 * i, 3 * i + 1, 3 * i + 2, 3 * (e + i), 3 * (e + i) + 1, 3 * (e + i) + 2])
+    bwd = _mini_meta(gm["scaling_bwd"], [2 * i, 2 * i + 1, 2 * (e + i), 2 * (e + i) + 1])
+    w1 = module.fc1_weight.detach()[i: i + 1].cpu()
+    w2 = module.fc2_weight.detach()[i: i + 1].cpu()
+    given = {"pre": captured["pre_gelu_out"][r0:r1].cpu().contiguous(),
+             "gelu_fp8": captured["gelu_out_fp8"][r0:r1].cpu().contiguous(),
+             "grad_gelu": captured["grad_gelu_out"][r0:r1].cpu().contiguous(),
+             "dpre_fp8": captured["grad_pre_fp8"][r0:r1].cpu().contiguous()}
+    o = orc.grouped_mlp_step(x[r0:r1].cpu().contiguous(), w1, w2, [sizes[i]], dy[r0:r1].cpu().contiguous(), fwd, bwd,
+                             given=given)
+    tag = f"{what} expert {i} ({sizes[i]} rows)"
+    assert_gemm_close(given["pre"], o["own_pre"].float(), tol, f"{tag} pre-GELU")
+    # The fp8 GELU output is formed from the fp32 accumulator, of which the bf16 pre-GELU copy is a rounding: the
+    # oracle's epilogue applied to that copy lands at most one code step away.  (Against the oracle's OWN
+    # accumulator a value near zero can differ by several codes: a contraction of thousands of terms that cancels
+    # to 1e-3 of its scale carries the summation-order noise at full weight.)
+    acc = given["pre"].float().contiguous()
+    from_pre = torch.empty_like(given["gelu_fp8"])
+    scratch_amax = torch.zeros(1)
+    ref.lib().orc_epilogue_gelu_fp8(acc.data_ptr(), acc.numel(), 1.0, 1.0, fwd.scale[3:4].data_ptr(),
+                                    ref.fmt_of(from_pre.dtype), None, from_pre.data_ptr(), scratch_amax.data_ptr())
+    dist = fp8_code_distance(given["gelu_fp8"], from_pre)
+    if dist.max() > 1:
+        at = tuple((dist == dist.max()).nonzero()[0].tolist())
+        raise AssertionError(
+            f"{tag}: fp8 GELU output {int(dist.max())} code steps from the oracle at {at} ({int((dist > 1).sum())} such): "
+            f"gpu byte 0x{int(given['gelu_fp8'].view(torch.uint8)[at]):02x}, oracle byte "
+            f"0x{int(from_pre.view(torch.uint8)[at]):02x}, pre {given['pre'][at].item()!r}, c_scale {fwd.scale[3].item()!r}")
+    assert (dist != 0).float().mean() <= 0.08, f"{tag}: {(dist != 0).float().mean():.3f} of the GELU bytes differ"
+    own = fp8_code_distance(given["gelu_fp8"], o["own_gelu_fp8"])
+    assert (own > 1).float().mean() <= 1e-4, f"{tag}: GELU bytes far from the oracle's own"
+    assert_gemm_close(out[r0:r1], o["out"].float(), tol, f"{tag} out")
+    assert_gemm_close(given["grad_gelu"], o["own_grad_gelu"].float(), tol, f"{tag} d(GELU output)")
+    assert_bytes_equal(given["dpre_fp8"], o["own_dpre_fp8"], f"{tag} d(pre-GELU) fp8 bytes")
+    assert_gemm_close(grad_input[r0:r1], o["grad_input"].float(), tol, f"{tag} grad_input")
+    assert_gemm_close(module.fc1_weight.grad[i], o["grad_w1"][0].float(), tol, f"{tag} grad_fc1")
+    assert_gemm_close(module.fc2_weight.grad[i], o["grad_w2"][0].float(), tol, f"{tag} grad_fc2")
+    g_fwd = gm["scaling_fwd"].amax_history[0].detach().cpu()
+    g_bwd = gm["scaling_bwd"].amax_history[0].detach().cpu()
+    assert_scalar_bits_equal(g_fwd[[3 * i, 3 * i + 1, 3 * (e + i) + 1]], fwd.amax_history[0][[0, 1, 4]],
+                             f"{tag} amax of x, fc1 weight, fc2 weight")
+    assert_scalar_bits_equal(g_bwd[[2 * i, 2 * (e + i)]], bwd.amax_history[0][[0, 2]],
+                             f"{tag} amax of grad_out and d(pre-GELU)")
+    assert torch.allclose(g_fwd[3 * (e + i)], fwd.amax_history[0][3], rtol=1e-3, atol=0), f"{tag} GELU amax"

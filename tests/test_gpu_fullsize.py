@@ -1,4 +1,8 @@
-"""Parity at the full size of the headline workload (E = 8, 4096 -> 14336, 16384 tokens, ragged split).
+"""Parity at the full size of the benchmark workloads: the headline one (config 2: E = 8, 4096 -> 14336, 16384
+tokens, ragged split) and the two the reference itself cannot run - config 3 (GroupedLinear, E = 64, 2048 -> 1408,
+24576 tokens split by Zipf popularity: experts with no rows and with fewer than 16, amax history 16; the reference
+asserts `0 not in group_sizes`, fp8_gmm/grouped_linear.py:205) and config 4 (GroupedMlp, E = 128, 2048 -> 768,
+65536 tokens: 384 tensors in one cast launch where the reference stops at 64, csrc/multi_pad_fusion.cu:512).
 
 The CPU oracle cannot finish these sizes in seconds, so the checks are properties that do not depend on size:
   * GEMMs on operands from {0, +-0.25 .. +-2}: every partial sum is exact in fp32, whatever the order, so the
@@ -8,12 +12,18 @@ The CPU oracle cannot finish these sizes in seconds, so the checks are propertie
   * cast + transpose: the transposed copy is the transpose of the row-major copy plus zero padding, the
     row-major copy equals what the quantize kernel writes, amax equals max|x|, sampled rows equal the oracle's
     bytes, and casting the dequantised bytes again returns the same bytes;
-  * the whole GroupedMlp step against an fp32 autograd model of the same layer (cosine similarity).
+  * the whole module steps: sampled experts against the CPU oracle stage by stage (helpers.check_*_against_oracle),
+    and the scaling state (scale, scale_inv, amax history) bit for bit against the oracle's update rule fed with
+    max|x| of the tensors that were cast.
 """
 import pytest
 import torch
 
-from helpers import assert_bytes_equal, gen
+import numpy as np
+
+from helpers import (assert_bytes_equal, assert_scalar_bits_equal, check_linear_expert_against_oracle,
+                     check_mlp_expert_against_oracle, gen)
+from oracle import modules as orc
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -123,40 +133,191 @@ def test_cast_transpose_full_size_properties(dev, dtype):
 
 
 def test_grouped_mlp_full_size_step(dev):
-    """Two training steps of the config-2 layer; the second (real scales) against an fp32 autograd model."""
+    """Two training steps of the config-2 layer; the second (real scales) against the CPU oracle on two experts
+    (the smallest and a ragged mid-sized one), stage by stage."""
     import fp8_gmm_amd as pkg
 
     e = len(SIZES)
     g = torch.Generator(device=dev).manual_seed(9)
     module = pkg.GroupedMlp(HIDDEN, FFN, e, torch.bfloat16, device=dev)
+    module.fc1_weight.data.normal_(0, 0.02, generator=g)
+    module.fc2_weight.data.normal_(0, 0.02, generator=g)
     x = torch.randn(sum(SIZES), HIDDEN, generator=g, device=dev).to(torch.bfloat16)
     dy = (torch.randn(sum(SIZES), HIDDEN, generator=g, device=dev) * 1e-2).to(torch.bfloat16)
     gs = torch.tensor(SIZES)
+    captured = {}
+    module.capture_intermediates(captured)
     for _ in range(2):
         xd = x.clone().requires_grad_()
         module.zero_grad()
         with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=2)):
             out = module(xd, gs)
         out.backward(dy)
-    bounds = _bounds(SIZES)
-
-    def cos(a, b):
-        a, b = a.detach().float().flatten(), b.detach().float().flatten()
-        return (torch.dot(a, b) / (a.norm() * b.norm())).item()
-
-    # expert by expert, to bound the fp32 model's memory
-    for i in range(e):
-        rows = slice(bounds[i], bounds[i + 1])
-        xr = x[rows].float().requires_grad_()
-        w1 = module.fc1_weight.data[i].float().requires_grad_()
-        w2 = module.fc2_weight.data[i].float().requires_grad_()
-        ref_out = torch.nn.functional.gelu(xr @ w1.t(), approximate="tanh") @ w2.t()
-        ref_out.backward(dy[rows].float())
-        assert cos(out[rows], ref_out) > 0.995, f"expert {i} output"
-        assert cos(xd.grad[rows], xr.grad) > 0.99, f"expert {i} grad_input"
-        assert cos(module.fc1_weight.grad[i], w1.grad) > 0.99, f"expert {i} fc1 grad"
-        assert cos(module.fc2_weight.grad[i], w2.grad) > 0.99, f"expert {i} fc2 grad"
+    torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all() and torch.isfinite(module.fc1_weight.grad.float()).all()
+    for i in (6, 4):   # 669 and 909 rows: what the CPU oracle finishes in seconds at these feature counts
+        check_mlp_expert_against_oracle(module, captured, i, SIZES, x, dy, out, xd.grad, 1e-2, "config 2")
+
+
+def _bench_splits(kind, experts, tokens, seed):
+    """The split bench.py draws for its workloads (same generator, same seed)."""
+    rng = np.random.default_rng(seed)
+    if kind == "zipf":
+        p = 1.0 / np.arange(1, experts + 1) ** 1.1
+        p /= p.sum()
+    else:
+        p = np.full(experts, 1.0 / experts)
+    return [int(v) for v in rng.multinomial(tokens, p)]
+
+
+def _slice_amax(t, bounds):
+    """max|t[rows of expert i]| per expert, exactly (0 for an expert without rows)."""
+    a = t.float().abs().amax(dim=1)
+    out = torch.zeros(len(bounds) - 1)
+    for i in range(len(bounds) - 1):
+        if bounds[i + 1] > bounds[i]:
+            out[i] = a[bounds[i]: bounds[i + 1]].max().item()
+    return out
+
+
+def test_config3_grouped_linear_seventeen_steps(dev):
+    """Config 3 at its real size, 18 training steps with an amax history of 16: after every step scale, scale_inv
+    and the whole amax history must equal, bit for bit, the oracle's delayed-scaling rule applied to max|x| of each
+    tensor that was cast (the history wraps once); experts without rows leave their amax at zero, keep their
+    scale and get a zero weight gradient; on the last step four experts - the largest, a mid-sized one, the
+    smallest ones with rows - are checked against the CPU oracle."""
+    import fp8_gmm_amd as pkg
+
+    e, k, n, tokens, hist, steps = 64, 2048, 1408, 24576, 16, 18
+    sizes = _bench_splits("zipf", e, tokens, 1003)
+    assert sum(sizes) == tokens and len(sizes) == e
+    # the split bench.py uses has no empty expert and none under 16 rows by itself; this workload is defined
+    # by having both, so the two least popular experts hand their rows to the first
+    order = np.argsort(sizes)
+    sizes[0] += sizes[order[0]] + sizes[order[1]] - 7
+    sizes[order[0]], sizes[order[1]] = 0, 7
+    assert sum(sizes) == tokens and 0 in sizes and any(0 < s < 16 for s in sizes)
+    bounds = _bounds(sizes)
+    g = torch.Generator(device=dev).manual_seed(1003)
+    module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev)
+    module.weight_tensor.data.normal_(0, 0.02, generator=g)
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=hist)
+    fwd, bwd = orc.Meta(3 * e, hist), orc.Meta(2 * e, hist)
+    w_amax = module.weight_tensor.detach().float().abs().amax(dim=(1, 2)).cpu()
+    gs = torch.tensor(sizes)
+    xs = [3 * i for i in range(e)]
+    ws = [3 * i + 1 for i in range(e)]
+    for step in range(steps):
+        x = (torch.randn(tokens, k, generator=g, device=dev) * (1.0 + 0.25 * step)).to(torch.bfloat16)
+        dy = (torch.randn(tokens, n, generator=g, device=dev) * 1e-2 / (1.0 + step)).to(torch.bfloat16)
+        if step > 0:
+            fwd.update(448.0)
+            bwd.update(57344.0)
+        fwd.amax_history[0][xs] = _slice_amax(x, bounds)
+        fwd.amax_history[0][ws] = w_amax
+        bwd.amax_history[0][[2 * i for i in range(e)]] = _slice_amax(dy, bounds)
+        xd = x.clone().requires_grad_()
+        module.weight_tensor.grad = None
+        with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
+            out = module(xd, gs)
+        out.backward(dy)
+        gm = module.fp8_meta
+        for name, got, want in (("fwd", gm["scaling_fwd"], fwd), ("bwd", gm["scaling_bwd"], bwd)):
+            assert_scalar_bits_equal(got.scale, want.scale, f"step {step} {name} scale")
+            assert_scalar_bits_equal(got.scale_inv, want.scale_inv, f"step {step} {name} scale_inv")
+            assert_scalar_bits_equal(got.amax_history, want.amax_history, f"step {step} {name} amax history")
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    grad_w = module.weight_tensor.grad
+    for i, s in enumerate(sizes):
+        if s == 0:
+            assert not grad_w[i].any(), f"expert {i} has no rows: its weight gradient must be zero"
+            assert gm["scaling_fwd"].scale[3 * i].item() == 1.0    # never saw an amax: still the initial scale
+    live = [i for i in np.argsort(sizes) if sizes[i] > 0]
+    for i in (int(np.argmax(sizes)), int(live[len(live) // 2]), int(live[0]), int(live[1])):
+        check_linear_expert_against_oracle(module, i, sizes, x, dy, out, xd.grad, 1e-2, "config 3")
+
+
+@pytest.mark.parametrize("a_dtype,form", [(E4M3, "fwd"), (E5M2, "dgrad"), (E5M2, "wgrad")])
+def test_config3_gemms_exact(dev, a_dtype, form):
+    """The three GEMMs of config 3 (64 problems; N = 1408 is 5.5 tiles wide, rows from 0 to thousands per expert)
+    on operands whose every partial sum is exact: bit-equal to the fp32 matmul."""
+    backend = _backend()
+    e, k, n = 64, 2048, 1408
+    sizes = _bench_splits("zipf", e, 24576, 1003)
+    sizes[3] += sizes[-1]
+    sizes[-1] = 0
+    bounds = _bounds(sizes)
+    x = _exact_fp8((sum(sizes), k), E4M3, dev, 41)
+    w = _exact_fp8((e, n, k), E4M3, dev, 42)
+    dy = _exact_fp8((sum(sizes), n), E5M2, dev, 43)
+    sa = torch.full((e,), 0.5, device=dev)
+    sb = torch.full((e,), 0.25, device=dev)
+    if form == "fwd":
+        c = backend.fp8_gmm(x, w, torch.tensor(sizes), sa, sb)
+        for i in range(e):
+            rows = slice(bounds[i], bounds[i + 1])
+            want = ((x[rows].float() @ w[i].float().t()) * 0.125).to(torch.bfloat16)
+            assert torch.equal(c[rows].view(torch.int16), want.view(torch.int16)), f"expert {i} ({sizes[i]} rows)"
+    elif form == "dgrad":
+        c = backend.fp8_gmm(dy, w, torch.tensor(sizes), sa, sb, backward=True, b_transposed=True)
+        for i in range(e):
+            rows = slice(bounds[i], bounds[i + 1])
+            want = ((dy[rows].float() @ w[i].float()) * 0.125).to(torch.bfloat16)
+            assert torch.equal(c[rows].view(torch.int16), want.view(torch.int16)), f"expert {i} ({sizes[i]} rows)"
+    else:
+        dw = torch.full((e, n, k), float("nan"), dtype=torch.bfloat16, device=dev)
+        backend.grouped_gemm(backend.TensorBatch.rows_of(dy, bounds), backend.TensorBatch.rows_of(x, bounds),
+                             backend.TensorBatch.stack_of(dw), sa, sb, transposed=True)
+        for i in range(e):
+            rows = slice(bounds[i], bounds[i + 1])
+            want = ((dy[rows].float().t() @ x[rows].float()) * 0.125).to(torch.bfloat16)
+            assert torch.equal(dw[i].view(torch.int16), want.view(torch.int16)), f"expert {i} ({sizes[i]} rows)"
+
+
+def test_config4_grouped_mlp_many_experts(dev):
+    """Config 4 at its real size: 128 experts, 384 tensors in the forward cast launch, 128-problem tables in all
+    six GEMMs.  Two steps; after the second, scales of the directly cast tensors bit-exact against the oracle's
+    rule, and four experts (smallest, largest, first, last) against the CPU oracle stage by stage."""
+    import fp8_gmm_amd as pkg
+
+    e, h, f, tokens = 128, 2048, 768, 65536
+    sizes = _bench_splits("uniform", e, tokens, 1004)
+    bounds = _bounds(sizes)
+    g = torch.Generator(device=dev).manual_seed(1004)
+    module = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+    module.fc1_weight.data.normal_(0, 0.02, generator=g)
+    module.fc2_weight.data.normal_(0, 0.02, generator=g)
+    x = torch.randn(tokens, h, generator=g, device=dev).to(torch.bfloat16)
+    dy = (torch.randn(tokens, h, generator=g, device=dev) * 1e-2).to(torch.bfloat16)
+    gs = torch.tensor(sizes)
+    captured = {}
+    module.capture_intermediates(captured)
+    for _ in range(2):
+        xd = x.clone().requires_grad_()
+        module.zero_grad()
+        with pkg.fp8_autocast(fp8_recipe=pkg.DelayedScaling(amax_history_len=4)):
+            out = module(xd, gs)
+        out.backward(dy)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    # second step ran with scale = 448 / amax of the first: the rule, from max|x| of what was cast
+    gm = module.fp8_meta
+    want = orc.Meta(6 * e, 4)
+    want.amax_history[0][[3 * i for i in range(e)]] = _slice_amax(x, bounds)
+    want.amax_history[0][[3 * i + 1 for i in range(e)]] = module.fc1_weight.detach().float().abs().amax(dim=(1, 2)).cpu()
+    want.amax_history[0][[3 * (e + i) + 1 for i in range(e)]] = \
+        module.fc2_weight.detach().float().abs().amax(dim=(1, 2)).cpu()
+    want.update(448.0)
+    direct = [3 * i for i in range(e)] + [3 * i + 1 for i in range(e)] + [3 * (e + i) + 1 for i in range(e)]
+    assert_scalar_bits_equal(gm["scaling_fwd"].scale[direct], want.scale[direct], "forward scales of cast tensors")
+    want_b = orc.Meta(4 * e, 4)
+    want_b.amax_history[0][[2 * i for i in range(e)]] = _slice_amax(dy, bounds)
+    want_b.update(57344.0)
+    g1 = [2 * i for i in range(e)]
+    assert_scalar_bits_equal(gm["scaling_bwd"].scale[g1], want_b.scale[g1], "grad_out scales")
+    for i in (int(np.argmin(sizes)), int(np.argmax(sizes)), 0, e - 1):
+        check_mlp_expert_against_oracle(module, captured, i, sizes, x, dy, out, xd.grad, 1e-2, "config 4")
 
 
 def test_cast_pad_bandwidth_configuration_full_size(dev):

@@ -8,7 +8,8 @@ and exact equality wherever the arithmetic is exact (power-of-two data, identity
 import pytest
 import torch
 
-from helpers import assert_bytes_equal, assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
+from helpers import (assert_bytes_equal, assert_gemm_close, assert_scalar_bits_equal, fp8_code_distance, gen,
+                     randn_bf16)
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -32,13 +33,7 @@ def _scalars(vals, dev=None):
     return [t.to(dev) for t in ts] if dev is not None else ts
 
 
-def _fp8_code_distance(a, b):
-    """|difference| in fp8 code steps between two same-dtype fp8 tensors (sign-magnitude codes)."""
-    ia = a.view(torch.uint8).to(torch.int32)
-    ib = b.view(torch.uint8).to(torch.int32)
-    sa = torch.where(ia >= 128, -(ia - 128), ia)
-    sb = torch.where(ib >= 128, -(ib - 128), ib)
-    return (sa - sb).abs()
+_fp8_code_distance = fp8_code_distance
 
 
 @pytest.mark.parametrize("a_dtype", [E4M3, E5M2])

@@ -7,7 +7,8 @@ compare outputs, gradients and the recorded scaling state.
 import pytest
 import torch
 
-from helpers import assert_close_multistage, assert_gemm_close, assert_scalar_bits_equal, gen, randn_bf16
+from helpers import (assert_close_multistage, assert_gemm_close, assert_scalar_bits_equal,
+                     check_mlp_expert_against_oracle, gen, randn_bf16)
 from oracle import modules as orc
 
 pytestmark = pytest.mark.gpu
@@ -148,10 +149,18 @@ def test_grouped_mlp_fwd_bwd(dev, case):
         xd = x.to(dev).requires_grad_()
         module.fc1_weight.grad = None
         module.fc2_weight.grad = None
+        captured = {}
+        module.capture_intermediates(captured)
         with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
             out = module(xd, torch.tensor(sizes, dtype=torch.int64))
         out.backward(dy.to(dev))
         torch.cuda.synchronize()
+        module.capture_intermediates(None)
+        # stage by stage, with the oracle fed the GPU's own fp8 intermediates: every GEMM within 1e-2, the
+        # directly cast bytes and amaxes bit-exact (the end-to-end comparison further down is the loose one)
+        for i, rows in enumerate(sizes):
+            if rows:
+                check_mlp_expert_against_oracle(module, captured, i, sizes, x, dy, out, xd.grad, 1e-2, f"step {step}")
         gm = module.fp8_meta
         assert_scalar_bits_equal(gm["scaling_fwd"].scale, fwd.scale, f"step {step} fwd scale")
         assert_scalar_bits_equal(gm["scaling_bwd"].scale, bwd.scale, f"step {step} bwd scale")
