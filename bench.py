@@ -7,12 +7,15 @@ HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and
 delayed-scaling update.  Prints ONE JSON line.
 
   value     whole-step throughput in TFLOP/s: algorithmic GEMM flops of the step (unpadded rows,
-            2 * sum_i M_i * N * K per grouped GEMM) / wall time of the step
+            2 * sum_i M_i * N * K per grouped GEMM) / wall time of the step, timed over `--steps` steps
+            with nothing else running (no per-kernel events)
   roofline  the dominant kernel (grouped GEMM): algorithmic flops per launch / mean launch
-            duration from HIP events recorded around every launch inside the timed region,
-            against the dense FP8 MFMA peak of 5.0 PFLOP/s
+            duration from HIP events recorded around every launch during a second pass of
+            `--steps` identical steps, against the dense FP8 MFMA peak of 5.0 PFLOP/s
   kernels   the same event timing for every kernel of the step (GB/s against 8 TB/s for the
             cast / transpose / pad kernels)
+  parity    after the timed passes: sampled rows of every GEMM result of one more step against an fp32
+            matmul (torch, on the GPU) of the dequantised fp8 operands, max |err| / max |ref| per result
   also      the step time of a later micro-batch that reuses the first one's fp8 weights (not the headline:
             the reference casts the weights on every pass)
   cpu_baseline  the per-expert quantize-dequantize-fp32-matmul loop (oracle/cpu_baseline.py) on
@@ -59,11 +62,97 @@ def splits(kind, experts, tokens, seed):
     return [int(v) for v in rng.multinomial(tokens, p)]
 
 
-# HBM bytes per grouped-GEMM launch (reads + writes), from the rocprofv3 FETCH_SIZE / WRITE_SIZE runs whose
-# summary is profiles/config2_mlp_step_hbm_traffic.md (counter units calibrated against a 256 MiB copy:
-# 2 KiB per FETCH_SIZE unit, 1 KiB per WRITE_SIZE unit).  Counters cannot be read from inside this process,
-# so the figure is carried here; the algorithmic bytes of one launch are 1.09 GB.
-GEMM_HBM_TRAFFIC_BYTES = {"config2": 2.85e9}
+def gemm_hbm_traffic(workload):
+    """HBM bytes per grouped-GEMM launch (reads + writes) as the rocprofv3 FETCH_SIZE / WRITE_SIZE runs measured
+    them: hardware counters cannot be read from inside this process, so the figure is taken from the committed
+    summary of those runs (a line `gemm_hbm_bytes_per_launch: <number>` in profiles/<workload>_mlp_step_hbm_traffic.md)
+    and is None when no such summary is at hand."""
+    import glob
+    import re
+
+    for path in glob.glob(os.path.join(ROOT, "profiles", f"{workload}_*hbm_traffic.md")):
+        m = re.search(r"gemm_hbm_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read())
+        if m:
+            return float(m.group(1))
+    return None
+
+
+def seeded_normal(shape, seed, std, dev, dtype=torch.bfloat16):
+    """N(0, std) drawn on the CPU from numpy's seeded generator, then copied: the same bits on every machine."""
+    rng = np.random.default_rng(seed)
+    out = torch.empty(shape, dtype=dtype, device=dev)
+    flat = out.view(-1)
+    chunk = 1 << 26
+    for start in range(0, flat.numel(), chunk):
+        n = min(chunk, flat.numel() - start)
+        vals = torch.from_numpy(rng.standard_normal(n, dtype=np.float32))
+        flat[start: start + n] = (vals * std).to(dtype).to(dev)
+    return out
+
+
+def _fp8_cast(t, scale, dtype):
+    fmax = 448.0 if dtype == torch.float8_e4m3fn else 57344.0
+    return (t.float() * scale).clamp(-fmax, fmax).to(dtype)
+
+
+def parity_check(module, kind, x, dy, sizes, run_step):
+    """One more step, then sampled rows of each GEMM result against torch's fp32 matmul of the dequantised fp8
+    operands (the fp8 operands re-derived here with torch casts from the bf16 tensors and the scales the step
+    used).  Returns {"max_rel_err": worst max|err| / max|ref| over the results, "per_result": {...}, "ok": bool}."""
+    e = len(sizes)
+    captured = {}
+    if kind == "mlp":
+        module.capture_intermediates(captured)
+    out, xgrad = run_step()
+    torch.cuda.synchronize()
+    if kind == "mlp":
+        module.capture_intermediates(None)
+    fwd, bwd = module.fp8_meta["scaling_fwd"], module.fp8_meta["scaling_bwd"]
+    s, si, sb, sbi = fwd.scale, fwd.scale_inv, bwd.scale, bwd.scale_inv
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    bounds = np.concatenate([[0], np.cumsum(sizes)])
+    live = [i for i in range(e) if sizes[i] > 0]
+    picks = sorted({live[0], live[-1], max(live, key=lambda i: sizes[i])})
+    errs = {}
+
+    def note(name, got, ref):
+        r = ((got.float() - ref).abs().max() / ref.abs().max().clamp_min(1e-30)).item()
+        errs[name] = max(errs.get(name, 0.0), r)
+
+    for i in picks:
+        r0, r1 = int(bounds[i]), int(bounds[i + 1])
+        rows = torch.arange(r0, r1, max(1, (r1 - r0) // 48), device=x.device)[:64]
+        if kind == "mlp":
+            x1, w1s, x2, w2s, g1, g2 = 3 * i, 3 * i + 1, 3 * (e + i), 3 * (e + i) + 1, 2 * i, 2 * (e + i)
+            w1 = _fp8_cast(module.fc1_weight.detach()[i], s[w1s], E4).float()
+            w2 = _fp8_cast(module.fc2_weight.detach()[i], s[w2s], E4).float()
+            x8 = _fp8_cast(x.detach()[r0:r1], s[x1], E4).float()
+            dy8 = _fp8_cast(dy[r0:r1], sb[g1], E5).float()
+            gelu8 = captured["gelu_out_fp8"][r0:r1].float()
+            dpre8 = captured["grad_pre_fp8"][r0:r1].float()
+            loc = rows - r0
+            note("fc1 pre-activation", captured["pre_gelu_out"][rows], (x8[loc] @ w1.t()) * (si[x1] * si[w1s]))
+            note("fc2 output", out[rows], (gelu8[loc] @ w2.t()) * (si[x2] * si[w2s]))
+            note("fc2 dgrad", captured["grad_gelu_out"][rows], (dy8[loc] @ w2) * (sbi[g1] * si[w2s]))
+            note("fc1 dgrad", xgrad[rows], (dpre8[loc] @ w1) * (sbi[g2] * si[w1s]))
+            hs = torch.arange(0, w2.shape[0], max(1, w2.shape[0] // 48), device=x.device)[:64]
+            note("fc2 wgrad", module.fc2_weight.grad[i][hs], (dy8[:, hs].t() @ gelu8) * (sbi[g1] * si[x2]))
+            fs = torch.arange(0, w1.shape[0], max(1, w1.shape[0] // 48), device=x.device)[:64]
+            note("fc1 wgrad", module.fc1_weight.grad[i][fs], (dpre8[:, fs].t() @ x8) * (sbi[g2] * si[x1]))
+        else:
+            xs, ws, g1 = 3 * i, 3 * i + 1, 2 * i
+            w = _fp8_cast(module.weight_tensor.detach()[i], s[ws], E4).float()
+            x8 = _fp8_cast(x.detach()[r0:r1], s[xs], E4).float()
+            dy8 = _fp8_cast(dy[r0:r1], sb[g1], E5).float()
+            loc = rows - r0
+            note("output", out[rows], (x8[loc] @ w.t()) * (si[xs] * si[ws]))
+            note("dgrad", xgrad[rows], (dy8[loc] @ w) * (sbi[g1] * si[ws]))
+            ns = torch.arange(0, w.shape[0], max(1, w.shape[0] // 48), device=x.device)[:64]
+            note("wgrad", module.weight_tensor.grad[i][ns], (dy8[:, ns].t() @ x8) * (sbi[g1] * si[xs]))
+    worst = max(errs.values())
+    return {"max_rel_err": float(f"{worst:.3e}"), "tolerance": 1e-2, "ok": bool(worst <= 1e-2),
+            "per_result": {k: float(f"{v:.3e}") for k, v in errs.items()},
+            "checked": f"64 sampled rows of experts {picks} against torch fp32 matmul of the dequantised fp8 operands"}
 
 
 def sample_shader_clock(work):
@@ -132,13 +221,12 @@ def bench_cast_pad(args):
     rng = np.random.default_rng(1005)
     rows = [int(v) for v in rng.integers(1, 8192, size=8)]
     cols, pad = 4096, 128
-    torch.manual_seed(1005)
     ins, outs, touts, scales = [], [], [], []
-    for m in rows:
-        x = torch.randn(m, cols, device=dev)
-        hit = torch.rand(m, cols, device=dev) < 1e-3
-        sign = torch.where(torch.rand(m, cols, device=dev) < 0.5, -200.0, 200.0)
-        x = torch.where(hit, sign, x).to(torch.bfloat16)
+    for m in rows:   # drawn on the CPU from the workload's seed and copied: the same bits on every machine
+        vals = rng.standard_normal((m, cols), dtype=np.float32)
+        hit = rng.random((m, cols), dtype=np.float32) < 1e-3
+        vals[hit] = np.where(rng.random(int(hit.sum())) < 0.5, -200.0, 200.0)
+        x = torch.from_numpy(vals).to(torch.bfloat16).to(dev)
         ins.append(x)
         outs.append(torch.empty(m, cols, dtype=torch.float8_e4m3fn, device=dev))
         touts.append(torch.empty(cols, (m + pad - 1) // pad * pad, dtype=torch.float8_e4m3fn, device=dev))
@@ -237,7 +325,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-kernel-events", action="store_true", help="skip per-kernel HIP events (pure wall time)")
+    ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
+    ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the extra passes after the timed region (clock / power sampling, cached-weights "
                          "step): what a profiler should see")
@@ -255,9 +344,10 @@ def main():
 
     kind, experts, hidden, ffn, tokens, splitter = WORKLOADS[args.workload]
     idx = int(args.workload[-1]) if args.workload[-1].isdigit() else 9
-    sizes = splits(splitter, experts, tokens, 1000 + idx) if splitter != "router" else None
+    seed = 1000 + idx
+    sizes = splits(splitter, experts, tokens, seed) if splitter != "router" else None
     dev = torch.device("cuda:0")
-    torch.manual_seed(1000 + idx)
+    torch.manual_seed(seed)
     top_k = 2
     if kind == "routed_mlp":
         from fp8_gmm_amd.moe import Fp8MlpModule
@@ -266,16 +356,17 @@ def main():
         out_features, gemms = hidden, 6
     elif kind == "mlp":
         module = pkg.GroupedMlp(hidden, ffn, experts, torch.bfloat16, device=dev)
-        module.fc1_weight.data.normal_(0, 0.02)
-        module.fc2_weight.data.normal_(0, 0.02)
+        module.fc1_weight.data.copy_(seeded_normal(module.fc1_weight.shape, seed + 100, 0.02, dev))
+        module.fc2_weight.data.copy_(seeded_normal(module.fc2_weight.shape, seed + 200, 0.02, dev))
         out_features, gemms = hidden, 6
     else:
         module = pkg.GroupedLinear(hidden, ffn, experts, torch.bfloat16, device=dev)
-        module.weight_tensor.data.normal_(0, 0.02)
+        module.weight_tensor.data.copy_(seeded_normal(module.weight_tensor.shape, seed + 100, 0.02, dev))
         out_features, gemms = ffn, 3
     in_rows = tokens // top_k if kind == "routed_mlp" else tokens
-    x = torch.randn(in_rows, hidden, device=dev, dtype=torch.bfloat16).requires_grad_()
-    dy = (torch.randn(in_rows, out_features, device=dev) * 1e-2).to(torch.bfloat16)
+    # inputs are drawn on the CPU from the workload's seed and copied, so every run sees the same bits
+    x = seeded_normal((in_rows, hidden), seed + 300, 1.0, dev).requires_grad_()
+    dy = seeded_normal((in_rows, out_features), seed + 400, 1e-2, dev)
     gs = torch.tensor(sizes, dtype=torch.int64) if sizes is not None else None
     fp8_recipe = pkg.DelayedScaling(amax_history_len=16)
     flops_per_gemm = 2.0 * tokens * hidden * ffn
@@ -287,6 +378,11 @@ def main():
         with pkg.fp8_autocast(enabled=True, fp8_recipe=fp8_recipe):
             out = module(x) if gs is None else module(x, gs, is_first_microbatch=first)
         out.backward(dy)
+        return out, x.grad
+
+    from fp8_gmm_amd import backend
+
+    backend.warm_up(dev)   # library initialisation and the GEMM's workspace: not inside the timed region
 
     for _ in range(args.warmup):
         step()
@@ -297,20 +393,18 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    # the same steps again, with HIP events around every kernel launch: per-kernel durations
     timing = None
-    if args.no_kernel_events:
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            step()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    else:
+    if not args.no_kernel_events:
         with kernel_timing() as timing:
-            t0 = time.perf_counter()
             for _ in range(args.steps):
                 step()
             torch.cuda.synchronize()
-            elapsed = time.perf_counter() - t0
     ms_per_step = elapsed / args.steps * 1e3
     value = flops_per_step / (ms_per_step * 1e-3) / 1e12
 
@@ -325,7 +419,9 @@ def main():
                                  "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4)}
                 roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
                             "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),
-                            "traffic": GEMM_HBM_TRAFFIC_BYTES.get(args.workload)}
+                            "traffic": gemm_hbm_traffic(args.workload),
+                            "timed_over": f"a second pass of {args.steps} identical steps with HIP events around "
+                                          "every launch"}
             else:
                 gbs = d["work"] / (d["ms"] * 1e-3) / 1e9
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
@@ -348,8 +444,6 @@ def main():
     # ... and the clock the GEMM launches really ran at: cycles / time counted inside a measurement build of the
     # kernel by the first workgroup of every XCD (fp8gmm_grouped_gemm_timed), over 5 more steps
     if roofline is not None and not args.headline_only:
-        from fp8_gmm_amd import backend
-
         counters = torch.zeros(32, dtype=torch.int64, device=dev)
         with backend.gemm_clock_probe(counters):
             for _ in range(5):
@@ -416,6 +510,11 @@ def main():
         also = dict(also or {})
         also["dense_gemm_of_the_same_size"] = dense_gemm_comparison(dev, tokens, ffn, hidden)
 
+    # correctness gate, after everything that is timed
+    parity = None
+    if gs is not None and not args.no_parity:
+        parity = parity_check(module, kind, x, dy, sizes, step)
+
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import cpu_baseline
@@ -430,7 +529,8 @@ def main():
 
     names = {"mlp": "GroupedMlp", "linear": "GroupedLinear", "routed_mlp": "Fp8MlpModule (router, gather, GroupedMlp, scatter)"}
     line = {
-        "metric": "FP8 grouped-GEMM TFLOP/s fwd+bwd, % of MI355X FP8 MFMA peak, E=8 MoE MLP",
+        "metric": f"FP8 grouped-GEMM TFLOP/s fwd+bwd, % of MI355X FP8 MFMA peak, E={experts} MoE "
+                  f"{'MLP' if kind != 'linear' else 'Linear'}" + (" (routed layer)" if kind == "routed_mlp" else ""),
         "value": round(value, 2),
         "unit": "TFLOP/s",
         "pct_of_fp8_mfma_peak": round(100.0 * value / FP8_PEAK_TFLOPS, 2),
@@ -450,6 +550,7 @@ def main():
                    "gemm_flops_per_step": flops_per_step},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "parity": parity,
         "kernels": kernels,
         "clock": clock,
         "also": also,
