@@ -16,19 +16,23 @@ static __device__ __align__(256) uint8_t scratch[(size_t)kStaticSlots * FP8GMM_G
 namespace fp8gmm {
 namespace {
 
-// Completes the tiles that the main kernel shared along K.  One workgroup per such tile (one record of the
-// fix-up list each): it adds the tile's pieces, which lie in consecutive workspace slots in K order, and
-// applies the epilogue.
-// 1024 threads: thread T owns the 16-byte groups T + 1024 q (q = 0..15) of a slot, i.e. register group g = T / 256
-// of every MFMA tile (i, j) = q of main-kernel thread T % 256: 4 consecutive columns of one row each.  The sums and
-// the arithmetic are those of tile_epilogue's general paths, so a shared tile gets the same bits as a whole one.
+// Completes the tiles that the main kernel shared along K.  MT workgroups per such tile (one record of the
+// fix-up list): together they add the tile's pieces, which lie in consecutive workspace slots in K order, and
+// apply the epilogue.  A launch has few shared tiles (64 at most on 256 compute units), each with a megabyte of
+// partial sums to read: four workgroups per tile put the whole chip to it.
+// 1024 threads: thread T owns the 16-byte groups T + 1024 q of a slot, i.e. register group g = T / 256 of the
+// MFMA tiles (i, j) = q of main-kernel thread T % 256: 4 consecutive columns of one row each; workgroup `part`
+// of a tile takes i = part (q = part * NT .. part * NT + NT - 1).  The sums and the arithmetic are those of
+// tile_epilogue's general paths, so a shared tile gets the same bits as a whole one.
 constexpr int kFixupThreads = 1024;
+constexpr int kFixupSplit = MT;  // workgroups per shared tile
 static_assert(kFixupThreads == 4 * NTHREADS, "one register group of every MFMA tile per thread");
 
 __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
     const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_fixup_desc* __restrict__ fixups, int out_kind,
     int epilogue, const uint8_t* __restrict__ workspace) {
-  const fp8gmm_gemm_fixup_desc fx = fixups[blockIdx.x];
+  const fp8gmm_gemm_fixup_desc fx = fixups[blockIdx.x / kFixupSplit];
+  const int part = blockIdx.x % kFixupSplit;
   const fp8gmm_gemm_problem pr = probs[fx.prob];
   const int m0 = fx.m0, n0 = fx.n0;
 
@@ -37,19 +41,21 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, khalf = lane >> 5;
 
-  f32x4 sum[MT * NT];
+  f32x4 sum[NT];
   {
-    const f32x4* first = reinterpret_cast<const f32x4*>(workspace + (size_t)fx.first_slot * kPartialBytes) + threadIdx.x;
+    const f32x4* first = reinterpret_cast<const f32x4*>(workspace + (size_t)fx.first_slot * kPartialBytes) +
+                         (size_t)part * NT * kFixupThreads + threadIdx.x;
 #pragma unroll
-    for (int q = 0; q < MT * NT; ++q) sum[q] = first[q * kFixupThreads];
+    for (int q = 0; q < NT; ++q) sum[q] = first[q * kFixupThreads];
   }
   for (int w = 1; w < fx.n_pieces; ++w) {
-    const f32x4* next = reinterpret_cast<const f32x4*>(workspace + (size_t)(fx.first_slot + w) * kPartialBytes) + threadIdx.x;
-    f32x4 part[MT * NT];
+    const f32x4* next = reinterpret_cast<const f32x4*>(workspace + (size_t)(fx.first_slot + w) * kPartialBytes) +
+                        (size_t)part * NT * kFixupThreads + threadIdx.x;
+    f32x4 piece[NT];
 #pragma unroll
-    for (int q = 0; q < MT * NT; ++q) part[q] = next[q * kFixupThreads];
+    for (int q = 0; q < NT; ++q) piece[q] = next[q * kFixupThreads];
 #pragma unroll
-    for (int q = 0; q < MT * NT; ++q) sum[q] += part[q];
+    for (int q = 0; q < NT; ++q) sum[q] += piece[q];
   }
 
   const int M = pr.m, N = pr.n;
@@ -63,8 +69,8 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
   const float cs = pr.c_scale ? *pr.c_scale : 1.f;
   float amax = 0.f;
 #pragma unroll
-  for (int q = 0; q < MT * NT; ++q) {
-    const int i = q / NT, jj = q % NT;
+  for (int q = 0; q < NT; ++q) {
+    const int i = part, jj = q;
     const int m = m0 + wave_m * WM + i * 32 + l32;
     const int n = n0 + wave_n * WN + jj * 32 + g * 8 + khalf * 4;
     if (m >= M || n >= N) continue;
@@ -206,7 +212,7 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
                         static_cast<uint8_t*>(workspace), counters, s);
   if (rc != FP8GMM_OK) return rc;
   if (plan->n_fixups > 0) {
-    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups), dim3(kFixupThreads), 0, s, probs_dev,
+    hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups * kFixupSplit), dim3(kFixupThreads), 0, s, probs_dev,
                        fixups_dev, out_kind, epilogue & FP8GMM_EPI_GELU, static_cast<const uint8_t*>(workspace));
     if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
   }

@@ -189,12 +189,13 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       fast = true;
     } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
                ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0) && (interior || (oob_zero && (cv & 15) == 0))) {
-      // The fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both
-      // outputs go through the staging area like the plain form's, one 32-row block at a time - first the bf16
-      // block as 32 rows x 256 B, then, in a second pass over the same accumulators, the fp8 block as 32 rows x
-      // 128 B (chunk c of row r at chunk c ^ ((r >> 1) & 7)) - so that every store instruction writes whole
-      // lines: 12 per block instead of 32 that touch 32 rows each.  On an edge tile the accumulators outside
-      // the problem are zero (oob_zero), and gelu(0) = 0 leaves the amax alone.
+      // The fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both outputs go
+      // through the staging area like the plain form's, one 32-row block at a time, in ONE pass over the
+      // accumulators: the bf16 values are staged as they are formed (32 rows x 256 B), the fp8 bytes of the
+      // block wait in 16 registers until the bf16 block has been read back, then take its place (32 rows x 128 B,
+      // chunk c of row r at chunk c ^ ((r >> 1) & 7)).  Every store instruction writes whole lines: 12 per
+      // block instead of 32 that touch 32 rows each.  On an edge tile the accumulators outside the problem are
+      // zero (oob_zero), and gelu(0) = 0 leaves the amax alone.
       uint8_t* const C = static_cast<uint8_t*>(pr.c) + (int64_t)m0 * ldc + n0;
       uint16_t* const AUX = static_cast<uint16_t*>(pr.aux) + (int64_t)m0 * ldc + n0;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
@@ -210,14 +211,48 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       float tile_amax = 0.f;
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
+        uint32_t f8[NT][4];
+        bool any_nan = false;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           const f32x16 t = tile_values(acc[i][j]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const u32x2 a = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
-                             pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
+            float v[4], x[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = t[g * 4 + q] * s;
+            const u32x2 a = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
             *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = a;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const float r = gelu_tanh_fast(v[q]);
+              // A chain of hardware max operations, pinned: written as compare + select, the compiler rebuilds
+              // the 256-element reduction as a tree and keeps far more values alive than there are registers.
+              // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
+              asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
+              const float y = r * cs;
+              any_nan |= (y != y);   // rare: dealt with once per block, below (the median turns a NaN into -max)
+              x[q] = __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
+            }
+            f8[j][g] = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3],
+                                                       __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
+          }
+        }
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(any_nan) != 0, 0)) {
+          // some lane of this block saw a NaN: form the block's bytes again, with 0x7F in place of every NaN
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const f32x16 t = tile_values(acc[i][j]);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              uint32_t nan_bytes = 0;
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const float y = gelu_tanh_fast(t[g * 4 + q] * s) * cs;
+                nan_bytes |= (y != y) ? (0xffu << (8 * q)) : 0u;
+              }
+              f8[j][g] = (f8[j][g] & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
+            }
           }
         }
         {
@@ -235,31 +270,11 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         }
         // the wavefront's LDS operations complete in order: the reads above are done before these writes land
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
+        for (int j = 0; j < NT; ++j)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float x[4];
-            uint32_t nan_bytes = 0;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const float r = gelu_tanh_fast(t[g * 4 + q] * s);
-              // A chain of hardware max operations, pinned: written as compare + select, the compiler rebuilds
-              // the 256-element reduction as a tree and keeps far more values alive than there are registers.
-              // r is computed, hence never a signalling NaN, and a quiet NaN loses against the running maximum.
-              asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(r));
-              // straight-line conversion (a branch here costs the register allocator its footing): clamp, convert,
-              // and patch the byte of a NaN to 0x7F afterwards (the median turns a NaN into -max)
-              const float y = r * cs;
-              x[q] = __builtin_amdgcn_fmed3f(y, -448.0f, 448.0f);
-              nan_bytes |= (y != y) ? (0xffu << (8 * q)) : 0u;
-            }
-            uint32_t w = __builtin_amdgcn_cvt_pk_fp8_f32(
-                x[2], x[3], __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
-            w = (w & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
-            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) = w;
-          }
-        }
+          for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) =
+                f8[j][g];
         {
           u32x4 rb[4];
 #pragma unroll
