@@ -155,42 +155,59 @@ __device__ __forceinline__ void block_amax_merge(float local, uint32_t* target, 
   if (amax != nullptr && p > 0.f) atomic_max_nonneg(amax, p);
 }
 
-// tanh from a fixed sequence of IEEE single-precision operations (mul, add, fma,
-// one correctly rounded division), so that a CPU following the same sequence gets
-// the same bits.  |error| < 2e-7.
-//   a = min(|u|, 9); z = a * 2/ln2; n = rne(z); f = z - n; e = 2^f * 2^n = exp(2a)
-//   tanh = (e - 1) / (e + 1), sign of u restored.
-__device__ __forceinline__ float det_tanh(float u) {
-  float a = fabsf(u);
-  a = (a > 9.0f) ? 9.0f : a;
-  float z = a * 2.8853900817779268f;
+// exp(-2a) and 1 / (1 + exp(-2a)) for a >= 0, from a fixed sequence of IEEE single-precision operations (add, mul,
+// fma, integer add / shift: no division, no hardware approximation), so that a CPU following the same sequence
+// gets the same bits.  Input z = a * 2 / ln 2 >= 0 (NaN is taken as large):
+//   z = min(z, 125); n = rne(z) by adding 1.5 * 2^23, f = z - n in [-0.5, 0.5];
+//   q = 2^-f * 2^-n: degree-5 minimax polynomial for 2^-f with constant term exactly 1 (1.5e-7 relative; exact at f = 0), the exponent subtracted in the integer
+//   domain (the low bits of magic - z hold -n);
+//   r = 1 / (1 + q): quadratic first guess on q in [0, 1] (1 % off), two Newton steps r += r (1 - d r).
+// tanh(a) = (1 - q) r;  0.5 (1 + tanh(a)) = r;  0.5 (1 - tanh(a)) = q r.
+// The dGELU cast is bound by vector arithmetic, not by memory: this sequence is 21 operations where a polynomial
+// with one more term, an exactly rounded division and separate rounding steps took 31.
+__device__ __forceinline__ void det_exp_rcp(float z, float* q_out, float* r_out) {
+  z = __builtin_fminf(z, 125.0f);
   const float magic = 12582912.0f;
-  float zr = z + magic;
-  int n = (int)(__float_as_uint(zr) - __float_as_uint(magic));
-  float nf = zr - magic;
-  float f = z - nf;
-  float p = 1.5403530393381609e-4f;
-  p = __builtin_fmaf(p, f, 1.3333558146428443e-3f);
-  p = __builtin_fmaf(p, f, 9.6181291076284772e-3f);
-  p = __builtin_fmaf(p, f, 5.5504108664821580e-2f);
-  p = __builtin_fmaf(p, f, 2.4022650695910071e-1f);
-  p = __builtin_fmaf(p, f, 6.9314718055994531e-1f);
+  const float zr = magic - z;
+  const float nf = zr - magic;
+  const float f = z + nf;
+  float p = -1.3400432653725147e-3f;
+  p = __builtin_fmaf(p, f, 9.666378609836102e-3f);
+  p = __builtin_fmaf(p, f, -5.550333112478256e-2f);
+  p = __builtin_fmaf(p, f, 2.402234822511673e-1f);
+  p = __builtin_fmaf(p, f, -6.931471824645996e-1f);
   p = __builtin_fmaf(p, f, 1.0f);
-  float e = __uint_as_float(__float_as_uint(p) + ((uint32_t)n << 23));
-  float t = (e - 1.0f) / (e + 1.0f);
-  return __builtin_copysignf(t, u);
+  const float q = __uint_as_float(__float_as_uint(p) + (__float_as_uint(zr) << 23));
+  const float d = 1.0f + q;
+  float r = __builtin_fmaf(__builtin_fmaf(0.3232323229312897f, q, -0.808080792427063f), q, 0.9898989796638489f);
+  r = __builtin_fmaf(r, __builtin_fmaf(-d, r, 1.0f), r);
+  r = __builtin_fmaf(r, __builtin_fmaf(-d, r, 1.0f), r);
+  *q_out = q;
+  *r_out = r;
 }
 
-// d/dc of tanh-GELU with the constants of the reference (csrc/multi_pad_fusion.cu:39-44).
+// |error| < 2e-7.
+__device__ __forceinline__ float det_tanh(float u) {
+  float q, r;
+  det_exp_rcp(fabsf(u) * 2.8853900817779268f, &q, &r);
+  const float t = __builtin_copysignf(__builtin_fmaf(-q, r, r), u);
+  return (u != u) ? u : t;   // the clamp above takes a NaN for a large value
+}
+
+// d/dc of tanh-GELU with the constants of the reference (csrc/multi_pad_fusion.cu:39-44):
+//   0.5 c (1 - t^2)(0.79788456 + 0.1070322243 c^2) + 0.5 (1 + t),  t = tanh(u),  u = 0.79788456 c (1 + 0.044715 c^2)
+// With s = 0.5 (1 + t) = 1 / (1 + exp(-2u)):  1 - t^2 = 4 s (1 - s), and s (1 - s) = q r^2 for either sign of u, so
+//   dgelu = s + c (1.59576912 + 0.2140644486 c^2) q r^2,   s = r for c >= 0, q r otherwise.
 __device__ __forceinline__ float dgelu(float c) {
-  float c2 = c * c;
-  float u = (0.79788456f * c) * __builtin_fmaf(0.044715f, c2, 1.0f);
-  float t = det_tanh(u);
-  float dt = __builtin_fmaf(-t, t, 1.0f);
-  float g = __builtin_fmaf(0.1070322243f, c2, 0.79788456f);
-  float left = (0.5f * c) * (dt * g);
-  float right = __builtin_fmaf(0.5f, t, 0.5f);
-  return left + right;
+  const float c2 = c * c;
+  const float w = __builtin_fmaf(0.044715f, c2, 1.0f);
+  float q, r;
+  det_exp_rcp(fabsf((2.3022082f * c) * w), &q, &r);   // 2.3022082 = 0.79788456 * 2 / ln 2
+  const float t1 = q * r;
+  const float s1 = t1 * r;
+  const float sig = (c >= 0.0f) ? r : t1;
+  const float g2 = __builtin_fmaf(0.2140644486f, c2, 1.59576912f);
+  return __builtin_fmaf(c * g2, s1, sig);
 }
 
 __device__ __forceinline__ float gelu_tanh(float v) {

@@ -208,54 +208,64 @@ void orc_pad_cast_transpose(const uint16_t* x, int64_t m, int64_t n, int64_t mpa
 }
 
 /*
- * tanh evaluated with a fixed sequence of IEEE-754 single-precision operations
- * (multiply, add, fma, one division) so that a CPU and a GPU that both follow
- * the sequence produce identical bits.  The reference calls tanhf under
- * --use_fast_math (csrc/multi_pad_fusion.cu:41, setup.py:21), i.e. a hardware
- * approximation with ~2^-11 relative error whose bits cannot be restated; this
- * sequence is within 2e-7 absolute of the true tanh.
- *
- *   a = min(|u|, 9);  z = a * (2/ln 2);  n = round(z);  f = z - n  in [-1/2, 1/2]
- *   2^f by a degree-6 polynomial (Horner, fma);  e = 2^f * 2^n = exp(2a)
- *   tanh(a) = (e - 1) / (e + 1);  sign restored afterwards.
+ * exp(-2a) and 1 / (1 + exp(-2a)) for a >= 0 from a fixed sequence of IEEE single-precision operations (add, mul,
+ * fma, integer add / shift; no division), the sequence the HIP kernels follow (csrc/device_utils.h, det_exp_rcp),
+ * so that both sides produce the same bits.  Input z = a * 2 / ln 2 >= 0:
+ *   z = min(z, 125); n = rne(z) by adding 1.5 * 2^23 (adding it rounds to an integer), f = z - n in [-0.5, 0.5];
+ *   q = 2^-f * 2^-n with a degree-5 minimax polynomial for 2^-f (constant term exactly 1: tanh(0) = 0), the exponent subtracted in the integer domain;
+ *   r = 1 / (1 + q): quadratic first guess, two Newton steps.
+ * tanh(a) = (1 - q) r.  The reference evaluates tanhf under --use_fast_math (csrc/multi_pad_fusion.cu:39-44,
+ * setup.py:21), which no CPU can restate bit for bit: this order of operations is this build's rule, pinned
+ * against the double-precision closed forms (tests/test_oracle_pins.py).
  */
-float orc_tanh(float u) {
-  float a = fabsf(u);
-  a = (a > 9.0f) ? 9.0f : a; /* NaN stays NaN */
-  float z = a * 2.8853900817779268f;
-  const float magic = 12582912.0f; /* 1.5 * 2^23: adding it rounds to an integer (RNE) */
-  float zr = z + magic;
-  int32_t n = (int32_t)(f2u(zr) - f2u(magic));
+static void orc_exp_rcp(float z, float* q_out, float* r_out) {
+  z = fminf(z, 125.0f); /* NaN counts as large */
+  const float magic = 12582912.0f;
+  float zr = magic - z;
   float nf = zr - magic;
-  float f = z - nf;
-  float p = 1.5403530393381609e-4f;
-  p = fmaf(p, f, 1.3333558146428443e-3f);
-  p = fmaf(p, f, 9.6181291076284772e-3f);
-  p = fmaf(p, f, 5.5504108664821580e-2f);
-  p = fmaf(p, f, 2.4022650695910071e-1f);
-  p = fmaf(p, f, 6.9314718055994531e-1f);
+  float f = z + nf;
+  float p = -1.3400432653725147e-3f;
+  p = fmaf(p, f, 9.666378609836102e-3f);
+  p = fmaf(p, f, -5.550333112478256e-2f);
+  p = fmaf(p, f, 2.402234822511673e-1f);
+  p = fmaf(p, f, -6.931471824645996e-1f);
   p = fmaf(p, f, 1.0f);
-  float e = u2f(f2u(p) + ((uint32_t)n << 23));
-  float t = (e - 1.0f) / (e + 1.0f);
-  return copysignf(t, u);
+  float q = u2f(f2u(p) + (f2u(zr) << 23));
+  float d = 1.0f + q;
+  float r = fmaf(fmaf(0.3232323229312897f, q, -0.808080792427063f), q, 0.9898989796638489f);
+  r = fmaf(r, fmaf(-d, r, 1.0f), r);
+  r = fmaf(r, fmaf(-d, r, 1.0f), r);
+  *q_out = q;
+  *r_out = r;
+}
+
+float orc_tanh(float u) {
+  float q, r;
+  orc_exp_rcp(fabsf(u) * 2.8853900817779268f, &q, &r);
+  float t = copysignf(fmaf(-q, r, r), u);
+  return (u != u) ? u : t; /* the clamp above takes a NaN for a large value */
 }
 
 /*
  * Derivative of tanh-GELU, reference csrc/multi_pad_fusion.cu:39-44 (same
  * constants; python twin fp8_gmm/test.py:32-34):
- *   t = tanh(0.79788456 c (1 + 0.044715 c^2))
+ *   t = tanh(u), u = 0.79788456 c (1 + 0.044715 c^2)
  *   dgelu = 0.5 c (1 - t^2)(0.79788456 + 0.1070322243 c^2) + 0.5 (1 + t)
- * The operation order below is this build's rule (see orc_tanh).
+ * evaluated through s = 0.5 (1 + t) = 1 / (1 + exp(-2u)):  1 - t^2 = 4 s (1 - s) and s (1 - s) = q r^2, so
+ *   dgelu = s + c (1.59576912 + 0.2140644486 c^2) q r^2,   s = r for c >= 0 and q r otherwise.
+ * The operation order below is this build's rule (see orc_exp_rcp).  Where c^2 overflows (|c| > 1.8e19) the
+ * reference's form gives NaN (0 * inf) and this one an infinity; neither is a value an activation takes.
  */
 float orc_dgelu(float c) {
   float c2 = c * c;
-  float u = (0.79788456f * c) * fmaf(0.044715f, c2, 1.0f);
-  float t = orc_tanh(u);
-  float dt = fmaf(-t, t, 1.0f);
-  float g = fmaf(0.1070322243f, c2, 0.79788456f);
-  float left = (0.5f * c) * (dt * g);
-  float right = fmaf(0.5f, t, 0.5f);
-  return left + right;
+  float w = fmaf(0.044715f, c2, 1.0f);
+  float q, r;
+  orc_exp_rcp(fabsf((2.3022082f * c) * w), &q, &r); /* 2.3022082 = 0.79788456 * 2 / ln 2 */
+  float t1 = q * r;
+  float s1 = t1 * r;
+  float sig = (c >= 0.0f) ? r : t1;
+  float g2 = fmaf(0.2140644486f, c2, 1.59576912f);
+  return fmaf(c * g2, s1, sig);
 }
 
 /* tanh-GELU forward, the epilogue of the fc1 GEMM (the GELU-aux epilogue the
