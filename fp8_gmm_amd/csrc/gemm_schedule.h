@@ -26,6 +26,8 @@ namespace fp8gmm {
 constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many K = 128 steps
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
 constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
+constexpr int kSkMinSavedSteps = 24;  // sharing must shorten the launch by this many K = 128 steps (about 30 us):
+                                      // the second launch that completes the shared tiles costs 10 - 30 us itself
 constexpr int kPartialBytes = BM * BN * 4;  // one slot: the fp32 accumulators of one tile
 constexpr int kTileOverhead = 4;      // fixed cost of a tile (epilogue, switch) in K = 128 steps, measured
 constexpr int kSlotsPerWg = 2;        // a piece that starts inside a tile, one that ends inside a tile
@@ -115,8 +117,16 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   s.sk_cost = 0;
   const int full = n_x / W, rem = n_x % W;
   if (!sk_enable || rem == 0 || full > kSkMaxRounds) return;
-  // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves 4 %
+  // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves 4 % ...
   if ((int64_t)(W - rem) * 25 < (int64_t)W * (full + 1)) return;
+  // ... and more time than the pass that completes the shared tiles takes: the last round shrinks from one
+  // tile's duration to rem / W of it.  (Tiles of 16 steps, as in a layer with 2048 input features, are not worth
+  // sharing: at 128 experts x 768 outputs the second launch took 75 us to save 10.)
+  {
+    const int64_t tail_cost = cost_before(s, s.range_end) - cost_before(s, s.range_end - rem);
+    const int64_t tile_steps = tail_cost / rem + kTileOverhead;
+    if (tile_steps * (W - rem) < (int64_t)kSkMinSavedSteps * W) return;
+  }
   int n_sk = rem;
   int rounds = full;
   if (rem * 4 < W && full >= 1) {  // very few tiles: cut a full round with them, pieces of about a tile
