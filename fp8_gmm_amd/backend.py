@@ -582,7 +582,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         _fail("fp8_gmm_amd: a contraction-major b must be float8_e4m3fn")
     layout = (_lib.GEMM_B_KMAJOR if b_kmajor else 0) | (_lib.GEMM_A_KMAJOR if a_kmajor else 0)
     grid = _lib.gemm_grid(_lib.init(device.index if device.index is not None else torch.cuda.current_device()))
-    plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout, grid, _STREAM_K)
+    plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | (_lib.EPI_GELU if gelu else 0), grid, _STREAM_K)
     if plan.total_tiles == 0:
         return
     n = len(table)

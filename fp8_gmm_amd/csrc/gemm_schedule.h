@@ -19,15 +19,19 @@ namespace fp8gmm {
 
 // ---- tail balancing (stream-K over the remainder of an XCD's tile range) ----
 // A range of n tiles on W workgroups takes ceil(n / W) rounds; when the last round is mostly empty the
-// remainder tiles (plus one full round when there are very few of them) are cut along K instead: the
-// region's K = 128 steps are dealt out in W equal contiguous pieces.  A piece that does not cover
+// remainder tiles are cut along K instead: the region's K = 128 steps are dealt out in equal contiguous
+// pieces, up to W of them.  A piece that does not cover
 // a whole tile leaves its fp32 accumulators in a workspace slot; a second, small kernel adds the pieces
 // of such a tile in K order and runs the normal epilogue.  No workgroup ever waits for another one.
 constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many K = 128 steps
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
 constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
-constexpr int kSkMinSavedSteps = 24;  // sharing must shorten the launch by this many K = 128 steps (about 30 us):
-                                      // the second launch that completes the shared tiles costs 10 - 30 us itself
+// The second launch, which completes the shared tiles, costs about kSkFixupLaunch K = 128 steps of time (5 us:
+// the gap between two launches) plus kSkFixupPerTile / 100 steps per shared tile of the XCD (four workgroups per
+// tile on 256 compute units, a megabyte of partial sums each), three times that when it has the GELU epilogue to
+// apply; sharing has to save half as much again.
+constexpr int kSkFixupLaunch = 4;
+constexpr int kSkFixupPerTile = 75;
 constexpr int kPartialBytes = BM * BN * 4;  // one slot: the fp32 accumulators of one tile
 constexpr int kTileOverhead = 4;      // fixed cost of a tile (epilogue, switch) in K = 128 steps, measured
 constexpr int kSlotsPerWg = 2;        // a piece that starts inside a tile, one that ends inside a tile
@@ -42,6 +46,7 @@ struct Sched {
   int sk_wgs;                  // workgroups that take a piece of the region
   int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (K = 128 steps)
   int64_t total_cost;          // cost of all tiles
+  int fixup_weight;            // 1, or 3 when completing a shared tile includes the GELU epilogue
 };
 
 FP8GMM_HD int problem_end_tile(const Sched& s, int p) {
@@ -96,7 +101,8 @@ FP8GMM_HD int first_tile_at_work(const Sched& s, int64_t c, int ov) {
 // tile costs its K steps plus a fixed part (epilogue, tile switch) worth about kTileOverhead steps: balancing
 // K steps alone left the XCDs that hold the short-K problems 17 % more work than the others.
 FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob, int total_tiles,
-                                           int xcd, int wgs_per_xcd, bool sk_enable) {
+                                           int xcd, int wgs_per_xcd, bool sk_enable, int fixup_weight = 1) {
+  s.fixup_weight = fixup_weight;
   s.probs = probs;
   s.nprob = nprob;
   s.total_tiles = total_tiles;
@@ -119,20 +125,8 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   if (!sk_enable || rem == 0 || full > kSkMaxRounds) return;
   // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves 4 % ...
   if ((int64_t)(W - rem) * 25 < (int64_t)W * (full + 1)) return;
-  // ... and more time than the pass that completes the shared tiles takes: the last round shrinks from one
-  // tile's duration to rem / W of it.  (Tiles of 16 steps, as in a layer with 2048 input features, are not worth
-  // sharing: at 128 experts x 768 outputs the second launch took 75 us to save 10.)
-  {
-    const int64_t tail_cost = cost_before(s, s.range_end) - cost_before(s, s.range_end - rem);
-    const int64_t tile_steps = tail_cost / rem + kTileOverhead;
-    if (tile_steps * (W - rem) < (int64_t)kSkMinSavedSteps * W) return;
-  }
-  int n_sk = rem;
-  int rounds = full;
-  if (rem * 4 < W && full >= 1) {  // very few tiles: cut a full round with them, pieces of about a tile
-    n_sk += W;
-    rounds -= 1;
-  }
+  const int n_sk = rem;
+  const int rounds = full;
   const int sk_begin = s.range_begin + rounds * W;
   const int64_t c0 = cost_before(s, sk_begin);
   const int64_t cost = cost_before(s, s.range_end) - c0;
@@ -140,6 +134,14 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   if (w > cost / kSkMinPairs) w = cost / kSkMinPairs;
   if (w > (int64_t)n_sk * kSkMaxPieces) w = (int64_t)n_sk * kSkMaxPieces;
   if (w <= n_sk) return;  // nothing to gain: at most one piece per tile
+  // ... and more time than the launch that completes the shared tiles takes: the last round shrinks from one
+  // tile's duration to that of one piece.  (128 experts x 768 outputs x 2048 inputs with the GELU epilogue: 24
+  // shared tiles of 16 steps per XCD, the second launch took 75 us to save 10.)
+  {
+    const int64_t saved_x100 = (cost / n_sk - cost / w) * 100;
+    const int64_t fixup_x100 = kSkFixupLaunch * 100 + (int64_t)n_sk * kSkFixupPerTile * s.fixup_weight;
+    if (saved_x100 * 2 < fixup_x100 * 3) return;
+  }
   s.dp_rounds = rounds;
   s.sk_begin = sk_begin;
   s.sk_wgs = (int)w;

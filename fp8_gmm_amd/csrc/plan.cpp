@@ -188,6 +188,8 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
   *plan = fp8gmm_gemm_plan{};
   if (grid <= 0 || (grid % kNumXcd) != 0 || max_items < 0 || max_fixups < 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  const bool gelu = (layout & FP8GMM_EPI_GELU) != 0;  // only weighs the decision to share tiles along K
+  layout &= ~FP8GMM_EPI_GELU;
   int total_tiles = 0;
   const int rc = fp8gmm_plan_grouped_gemm_layout(probs, n, layout, &total_tiles);
   if (rc != FP8GMM_OK) return rc;
@@ -205,7 +207,7 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   // pass 1: sizes.  The tiles that were shared along K first: the pieces of such a tile get consecutive
   // workspace slots, numbered from 0 over the launch, in K order.
   std::vector<Sched> sched(kNumXcd);
-  for (int x = 0; x < kNumXcd; ++x) sched_init(sched[x], probs, n, total_tiles, x, wgs, sk);
+  for (int x = 0; x < kNumXcd; ++x) sched_init(sched[x], probs, n, total_tiles, x, wgs, sk, gelu ? 3 : 1);
   std::vector<int32_t> slot_map((size_t)kSlotsPerWg * grid, -1);
   std::vector<fp8gmm_gemm_fixup_desc> fix;
   int n_slots = 0;

@@ -248,7 +248,8 @@ int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_bloc
 /*
  * Validates `probs[0..n)` like fp8gmm_plan_grouped_gemm_layout, fills tile_begin / cost_begin, and writes the work
  * list of a launch with `grid` workgroups (fp8gmm_gemm_grid) into items[0 .. rounds * grid) and
- * fixups[0 .. n_fixups).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
+ * fixups[0 .. n_fixups).  `layout` takes the launch's flags: the KMAJOR flags as for the plain plan, and
+ * FP8GMM_EPI_GELU, which only weighs the decision below (completing a shared tile costs more with that epilogue).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
  * the last round would otherwise be mostly idle; the launch then needs plan->n_slots workspace slots (never more
  * than 2 * grid).  stream_k == 0: every record is a whole tile, no workspace, no fix-up launch.
  * The sizes are returned in *plan even when max_items / max_fixups are too small (FP8GMM_ERR_BUFFER_TOO_SMALL,
