@@ -41,7 +41,7 @@ struct Sched {
   int nprob, total_tiles;
   int wgs;                     // workgroups per XCD
   int range_begin, range_end;  // tiles of this XCD
-  int dp_rounds;               // workgroup j takes tiles range_begin + j + wgs * i, i < dp_rounds
+  int dp_rounds;               // workgroup j takes tile dp_tile(j, i) of rounds i < dp_rounds
   int sk_begin;                // first tile of the stream-K region (== range_end: none)
   int sk_wgs;                  // workgroups that take a piece of the region
   int64_t sk_c0, sk_cost;      // cost before the region, cost of the region (K = 128 steps)
@@ -176,18 +176,28 @@ struct Cursor {
   int sk_tile;  // next tile of this workgroup's stream-K piece, -1: none left
 };
 
+// The tile that workgroup j of the XCD takes in round i of the strided part.  The position inside the round
+// rotates from round to round: how fast a workgroup's steps run depends on where its tile sits in the round's
+// 8 x 4 block (which operand slabs it shares with its neighbours, which memory channels those fall into - up to
+// 6 % between columns of a weight-gradient problem), and a workgroup that kept one position for the whole launch
+// would finish that much earlier or later than the others.
+constexpr int kRoundRotation = 5;  // coprime to every workgroup count in use (multiples of 8 per XCD: 32, 38, ...)
+FP8GMM_HD int dp_tile(const Sched& s, int j, int i) {
+  return s.range_begin + s.wgs * i + (j + kRoundRotation * i) % s.wgs;
+}
+
 FP8GMM_HD void cursor_init(const Sched& s, int j, Cursor& c) {
   c.dp_i = 0;
   c.sk_tile = -1;
   if (j < s.sk_wgs && sk_bound(s, j) < sk_bound(s, j + 1)) c.sk_tile = tile_holding_cost(s, s.sk_c0 + sk_bound(s, j));
 }
 FP8GMM_HD bool cursor_valid(const Sched& s, int j, const Cursor& c) {
-  return (c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin) || c.sk_tile >= 0;
+  return (c.dp_i < s.dp_rounds && dp_tile(s, j, c.dp_i) < s.sk_begin) || c.sk_tile >= 0;
 }
 FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c) {
-  const bool dp = c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin;
+  const bool dp = c.dp_i < s.dp_rounds && dp_tile(s, j, c.dp_i) < s.sk_begin;
   Item it;
-  it.tile = dp ? s.range_begin + j + s.wgs * c.dp_i : c.sk_tile;
+  it.tile = dp ? dp_tile(s, j, c.dp_i) : c.sk_tile;
   it.prob = problem_of_tile(s, it.tile);
   tile_origin(s.probs[it.prob].m, s.probs[it.prob].n, it.tile - s.probs[it.prob].tile_begin, &it.m0, &it.n0);
   const int real_nk = (s.probs[it.prob].k + 127) / 128;  // a K tail is zero-filled
@@ -208,7 +218,7 @@ FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c) {
   return it;
 }
 FP8GMM_HD void cursor_advance(const Sched& s, int j, Cursor& c) {
-  if (c.dp_i < s.dp_rounds && s.range_begin + j + s.wgs * c.dp_i < s.sk_begin) {
+  if (c.dp_i < s.dp_rounds && dp_tile(s, j, c.dp_i) < s.sk_begin) {
     ++c.dp_i;
     return;
   }
