@@ -150,41 +150,50 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       // Plain bf16 output: straight-line code with an exact store count.
       // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
       // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
-      // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages one 32-row
-      // block of its sub-tile at a time (32 x 256 B in its own 8 KB; the 16-byte chunk c of row r sits at chunk
-      // c ^ (r mod 16)) and reads it back row-major: 4 rows x 256 contiguous bytes per store instruction.
+      // pieces per instruction, which the memory pipeline takes one by one.  Each wavefront stages its sub-tile
+      // in units of 32 rows x 64 columns (32 x 128 B; the 16-byte chunk c of row r sits at chunk
+      // c ^ ((r >> 1) & 7)) and reads a unit back row-major: 8 rows x 128 contiguous bytes per store instruction.
+      // Two 4 KB staging buffers alternate, so that the read-back of one unit is under way while the next unit is
+      // converted: the round trip through LDS, a third of the epilogue when exposed, hides behind the arithmetic.
       uint16_t* const C = static_cast<uint16_t*>(pr.c) + (int64_t)m0 * ldc + n0;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       uint8_t* mine = stage + wave * 8192;
-      const int wr = l32 * 256 + khalf * 8;              // + ((4 j + g) ^ (l32 & 15)) * 16
-      const int rrow = lane >> 4, rchunk = lane & 15;     // read-back: row 4 it + rrow, chunk rchunk
-      const int col = wave_n * WN + rchunk * 8;
-      const uint32_t lane_off = col < cv ? (uint32_t)((rrow * (int)ldc + col) * 2) : kMaskedOffset;
+      const int wr = l32 * 128 + khalf * 8;              // + ((4 jl + g) ^ ((l32 >> 1) & 7)) * 16, jl = j & 1
+      const int rrow = lane >> 3, rchunk = lane & 7;      // read-back: row 8 it + rrow, chunk rchunk
+      u32x4 v[4];
+      auto store_unit = [&](int i, int jj) {
+        const int col = wave_n * WN + jj * 64 + rchunk * 8;
+        const uint32_t lane_off = col < cv ? (uint32_t)((rrow * (int)ldc + col) * 2) : kMaskedOffset;
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
+        for (int it = 0; it < 4; ++it) {
+          const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 8 * it) * (int)ldc * 2);  // uniform
+          buf_store16(v[it], rc, lane_off + row_off);
+        }
+      };
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
+      for (int u = 0; u < MT * 2; ++u) {
+        const int i = u >> 1, jj = u & 1;
+        uint8_t* buf = mine + (u & 1) * 4096;
+#pragma unroll
+        for (int jl = 0; jl < 2; ++jl) {
+          const f32x16 t = tile_values(acc[i][2 * jj + jl]);
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
                              pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
-            *reinterpret_cast<u32x2*>(mine + wr + (((4 * j + g) ^ (l32 & 15)) << 4)) = o;
+            *reinterpret_cast<u32x2*>(buf + wr + (((4 * jl + g) ^ ((l32 >> 1) & 7)) << 4)) = o;
           }
         }
-        // only this wavefront touches `mine`: its own LDS operations complete in order
-        u32x4 v[8];
+        // the previous unit's read-back was issued before this unit's conversion: store it now
+        if (u > 0) store_unit((u - 1) >> 1, (u - 1) & 1);
+        // only this wavefront touches `mine`, and its LDS operations complete in order
 #pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const int r = 4 * it + rrow;
-          v[it] = *reinterpret_cast<const u32x4*>(mine + r * 256 + ((rchunk ^ (r & 15)) << 4));
-        }
-#pragma unroll
-        for (int it = 0; it < 8; ++it) {
-          const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 4 * it) * (int)ldc * 2);  // uniform
-          buf_store16(v[it], rc, lane_off + row_off);
+        for (int it = 0; it < 4; ++it) {
+          const int r = 8 * it + rrow;
+          v[it] = *reinterpret_cast<const u32x4*>(buf + r * 128 + ((rchunk ^ ((r >> 1) & 7)) << 4));
         }
       }
+      store_unit(MT - 1, 1);
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
     } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
