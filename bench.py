@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -279,6 +279,103 @@ def bench_cast_pad(args):
     }))
 
 
+def bench_hbm_ceiling(args):
+    """hbm_ceiling: what this machine's memory system sustains for the read : write mixes of the library's
+    bandwidth-bound kernels, measured with plain streaming kernels (fp8_gmm_amd/csrc/hbm_probe.hip) that do no
+    arithmetic, next to the library's own kernels moving the same bytes.  Every launch moves at least 512 MiB, twice
+    the 256 MB memory-side cache.  Each mix is swept over the grid size (256 ... 16384 workgroups of 256 threads),
+    plain / streaming-hinted accesses and two walks (a trip's accesses a whole grid apart, or 16 KiB contiguous per
+    workgroup); `probes` holds the best launch of each mix and the whole sweep."""
+    import ctypes
+
+    import fp8_gmm_amd as pkg  # noqa: F401
+    from fp8_gmm_amd import backend
+
+    path = os.path.join(ROOT, "fp8_gmm_amd", "libfp8gmm_probe.so")
+    if not os.path.exists(path):
+        sys.exit("bench.py: fp8_gmm_amd/libfp8gmm_probe.so is not built (make -C fp8_gmm_amd/csrc)")
+    probe = ctypes.CDLL(path).fp8gmm_probe_stream
+    probe.restype = ctypes.c_int
+    probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
+                      ctypes.c_int, ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    mib = 1 << 20
+    src = torch.empty(1024 * mib, dtype=torch.uint8, device=dev)
+    src.view(torch.int32).random_(0, 2**31 - 1)
+    dst = torch.empty(512 * mib, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        ev[0].record()
+        for i in range(args.steps):
+            fn()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        return min(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)) * 1e-3   # best launch, seconds
+
+    # (name, input streams, writes, MiB per stream)
+    mixes = [("read only", 1, 0, 1024), ("4 : 1", 4, 1, 256), ("2 : 1", 2, 1, 256), ("1 : 1", 1, 1, 512),
+             ("write only", 0, 1, 512)]
+    rows = []
+    for name, reads, write, per in mixes:
+        best, sweep = None, []
+        for nt in (0, 1, 2, 3):
+            for blocks in (256, 512, 1024, 2048, 4096, 8192, 16384):
+                def fn():
+                    rc = probe(reads, write, nt, src.data_ptr(), dst.data_ptr(), per * mib, blocks, stream)
+                    assert rc == 0, f"probe launch failed: {rc}"
+                secs = timed(fn)
+                gbs = (reads + write) * per * mib / secs / 1e9
+                sweep.append([blocks, nt, round(gbs)])
+                if best is None or gbs > best["GB/s"]:
+                    best = {"mix": name, "MiB_read": reads * per, "MiB_written": write * per, "GB/s": round(gbs, 1),
+                            "us": round(secs * 1e6, 1), "blocks": blocks, "nontemporal": bool(nt & 1),
+                            "blocked": bool(nt & 2)}
+        best["sweep"] = sweep   # [workgroups, flags (1 = streaming hint, 2 = blocked walk), GB/s]
+        rows.append(best)
+        print(f"# probe {name}: {best}", file=sys.stderr, flush=True)
+
+    # the library's kernels on the same bytes: 8 tensors of 32 Mi elements
+    n, numel = 8, 32 * mib
+    x0, g0 = (seeded_normal((numel // 4096, 4096), seed, 1.0, dev) for seed in (7000, 7100))
+    xs, gs = [x0] + [x0.clone() for _ in range(n - 1)], [g0] + [g0.clone() for _ in range(n - 1)]
+    os_ = [torch.empty(numel // 4096, 4096, dtype=torch.float8_e4m3fn, device=dev) for _ in range(n)]
+    ts = [torch.empty(4096, numel // 4096, dtype=torch.float8_e4m3fn, device=dev) for _ in range(n)]
+    scales = [torch.full((1,), 64.0, device=dev) for _ in range(n)]
+    amaxes = torch.zeros(n, device=dev)
+    kernels = []
+    for name, mix, nbytes, fn in (
+            ("multi_quantize (bf16 -> e4m3 + amax)", "2 : 1", 3 * n * numel,
+             lambda: backend.multi_quantize(xs, os_, scales, amaxes)),
+            ("multi_cast_dgelu (bf16 grad, bf16 pre-GELU -> e5m2 + amax)", "4 : 1", 5 * n * numel,
+             lambda: backend.multi_cast_dgelu(xs, gs, [o.view(torch.float8_e5m2) for o in os_], scales, amaxes)),
+            ("multi_cast_transpose (bf16 -> e4m3 + transposed copy + amax)", "1 : 1", 4 * n * numel,
+             lambda: backend.multi_cast_transpose(xs, os_, ts, scales, amaxes))):
+        secs = timed(fn)   # launch + the amax merge that follows it
+        kernels.append({"kernel": name, "mix": mix, "MiB": nbytes // mib, "GB/s": round(nbytes / secs / 1e9, 1),
+                        "us": round(secs * 1e6, 1)})
+        print(f"# library {kernels[-1]}", file=sys.stderr, flush=True)
+    by_mix = {r["mix"]: r["GB/s"] for r in rows}
+    for k in kernels:
+        k["of_probe"] = round(k["GB/s"] / by_mix[k["mix"]], 3)
+    print(json.dumps({
+        "metric": "sustained HBM GB/s of plain streaming kernels by read : write mix (best launch of each sweep)",
+        "value": by_mix["2 : 1"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic", "config": {"workload": "hbm_ceiling: 512-1280 MiB per launch, grids 256-16384 x 256 "
+                                                    "threads, plain and streaming-hinted accesses, strided and "
+                                                    "blocked walks"},
+        "probes": rows, "library_kernels": kernels,
+        "roofline": {"kernel": "stream_kernel<2 reads, 1 write>", "bound": "hbm", "achieved": by_mix["2 : 1"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by_mix["2 : 1"] / HBM_PEAK_GBS, 4),
+                     "traffic": None},
+        "cpu_baseline": None,
+    }))
+
+
 def dense_gemm_comparison(dev, m, n, k, reps=100):
     """[m, k] x [n, k]^T -> bf16 [m, n], e4m3 operands: TFLOP/s of the grouped kernel (one group) and of the vendor GEMM."""
     import fp8_gmm_amd.backend as backend
@@ -323,7 +420,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
@@ -338,6 +435,8 @@ def main():
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
     if args.workload == "config5":
         return bench_cast_pad(args)
+    if args.workload == "hbm_ceiling":
+        return bench_hbm_ceiling(args)
 
     import fp8_gmm_amd as pkg
     from fp8_gmm_amd.backend import kernel_timing
