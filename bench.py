@@ -516,11 +516,17 @@ def main():
                 ach = flops_per_gemm / (d["ms"] * 1e-3) / 1e12
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
                                  "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4)}
+                traffic = gemm_hbm_traffic(args.workload)
                 roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
                             "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),
-                            "traffic": gemm_hbm_traffic(args.workload),
+                            "traffic": traffic,
                             "timed_over": f"a second pass of {args.steps} identical steps with HIP events around "
                                           "every launch"}
+                if traffic is not None:
+                    # the same launches seen from the memory side: short contractions (configs 3 and 4) move
+                    # almost as many bytes per flop as the memory system can deliver
+                    gbs = traffic / (d["ms"] * 1e-3) / 1e9
+                    roofline["memory_side"] = {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
             else:
                 gbs = d["work"] / (d["ms"] * 1e-3) / 1e9
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
