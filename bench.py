@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling|small_tile]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -376,6 +376,60 @@ def bench_hbm_ceiling(args):
     }))
 
 
+def bench_small_tile(args):
+    """small_tile: grouped GEMMs that do not fill the machine with full 256 x 256 tiles - few tiles, or problems
+    of up to 128 rows - through both tile sizes (FP8GMM_GEMM_TILE_128 against the default), with the choice the
+    backend makes by itself; HIP events around every launch, mean of `--steps` launches."""
+    import fp8_gmm_amd as pkg  # noqa: F401
+    from fp8_gmm_amd import backend
+    from fp8_gmm_amd.backend import kernel_timing
+
+    dev = torch.device("cuda:0")
+    backend.warm_up(dev)
+    rows = []
+    # experts, rows per expert, n, k
+    shapes = [(8, 64, 2048, 4096), (8, 256, 2048, 4096), (8, 512, 2048, 4096), (8, 1024, 2048, 4096),
+              (8, 2048, 2048, 4096), (16, 128, 4096, 4096), (16, 256, 4096, 4096), (64, 64, 1408, 2048),
+              (64, 128, 1408, 2048), (128, 64, 768, 2048), (128, 128, 2048, 768), (4, 250, 512, 256),
+              (8, 100, 4096, 14336), (8, 300, 14336, 4096)]
+    for e, me, n, k in shapes:
+        m = e * me
+        a = _fp8_cast(seeded_normal((m, k), 9000 + e + me, 1.0, dev), 1.0, torch.float8_e4m3fn)
+        b = _fp8_cast(seeded_normal((e, n, k), 9100 + n, 1.0, dev), 1.0, torch.float8_e4m3fn)
+        ones = torch.ones(e, device=dev)
+        sizes = [me] * e
+        us, outs = {}, {}
+        for tile in ("256", "128", "auto"):
+            backend._TILE = tile
+            c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+            for _ in range(args.warmup):
+                backend.fp8_gmm(a, b, sizes, ones, ones, c)
+            torch.cuda.synchronize()
+            with kernel_timing() as t:
+                for _ in range(args.steps):
+                    backend.fp8_gmm(a, b, sizes, ones, ones, c)
+                torch.cuda.synchronize()
+            us[tile] = t.summary()["grouped_gemm"]["ms"] * 1e3
+            outs[tile] = c
+        backend._TILE = "auto"
+        large = e * ((me + 255) // 256) * ((n + 255) // 256)
+        small = e * ((me + 127) // 128) * ((n + 127) // 128)
+        rows.append({"experts": e, "rows": me, "n": n, "k": k, "tiles_256": large, "tiles_128": small,
+                     "us_256": round(us["256"], 1), "us_128": round(us["128"], 1), "us_auto": round(us["auto"], 1),
+                     "speedup_128": round(us["256"] / us["128"], 2),
+                     "same_bits": bool(torch.equal(outs["256"].view(torch.int16), outs["128"].view(torch.int16)))})
+        print(f"# {rows[-1]}", file=sys.stderr, flush=True)
+    best = sum(min(r["us_256"], r["us_128"]) for r in rows)
+    auto = sum(r["us_auto"] for r in rows)
+    print(json.dumps({
+        "metric": "grouped GEMM launch time, 128 x 128 against 256 x 256 tiles, launches that do not fill the machine",
+        "value": round(best / auto, 4), "unit": "sum of the better tile's times / sum of the chosen tile's times",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp8", "data": "synthetic",
+        "config": {"workload": "small_tile: fp8_gmm forward, bf16 output, equal rows per expert"},
+        "launches": rows, "roofline": None, "cpu_baseline": None}))
+
+
 def dense_gemm_comparison(dev, m, n, k, reps=100):
     """[m, k] x [n, k]^T -> bf16 [m, n], e4m3 operands: TFLOP/s of the grouped kernel (one group) and of the vendor GEMM."""
     import fp8_gmm_amd.backend as backend
@@ -420,7 +474,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling"])
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling", "small_tile"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
@@ -437,6 +491,8 @@ def main():
         return bench_cast_pad(args)
     if args.workload == "hbm_ceiling":
         return bench_hbm_ceiling(args)
+    if args.workload == "small_tile":
+        return bench_small_tile(args)
 
     import fp8_gmm_amd as pkg
     from fp8_gmm_amd.backend import kernel_timing

@@ -19,6 +19,7 @@ OUT_BF16 = 2
 EPI_GELU = 1
 GEMM_B_KMAJOR = 2
 GEMM_A_KMAJOR = 4
+GEMM_TILE_128 = 0x100   # planning flag: 128 x 128 tiles, two workgroups per compute unit
 
 OP_QUANTIZE = 0
 OP_SCALE_MUL = 1
@@ -105,7 +106,8 @@ class GemmPlan(ctypes.Structure):
     """struct fp8gmm_gemm_plan"""
 
     _fields_ = [("grid", ctypes.c_int32), ("rounds", ctypes.c_int32), ("n_fixups", ctypes.c_int32),
-                ("n_slots", ctypes.c_int32), ("total_tiles", ctypes.c_int32), ("reserved", ctypes.c_int32 * 3)]
+                ("n_slots", ctypes.c_int32), ("total_tiles", ctypes.c_int32), ("tile", ctypes.c_int32),
+                ("reserved", ctypes.c_int32 * 2)]
 
 
 EXPORTS = (
@@ -258,7 +260,8 @@ def plan_grouped_gemm_launch(table, layout, grid, stream_k):
     plan = GemmPlan()
     n = len(table)
     # first guess: striding needs ceil(tiles / grid) records per workgroup, tail sharing a few more
-    guess = (int(np.ceil(max(1, _tiles_upper_bound(table)) / grid)) + 6) * grid
+    tiles = max(1, _tiles_upper_bound(table)) * (4 if layout & GEMM_TILE_128 else 1)
+    guess = (int(np.ceil(tiles / grid)) + 6) * grid
     items = np.empty(guess, dtype=GEMM_ITEM)
     fixups = np.empty(grid, dtype=GEMM_FIXUP)
     rc = L.fp8gmm_plan_grouped_gemm_launch(table.ctypes.data, n, layout, grid, int(bool(stream_k)), items.ctypes.data,

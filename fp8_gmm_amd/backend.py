@@ -582,7 +582,11 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         _fail("fp8_gmm_amd: a contraction-major b must be float8_e4m3fn")
     layout = (_lib.GEMM_B_KMAJOR if b_kmajor else 0) | (_lib.GEMM_A_KMAJOR if a_kmajor else 0)
     grid = _lib.gemm_grid(_lib.init(device.index if device.index is not None else torch.cuda.current_device()))
-    plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | (_lib.EPI_GELU if gelu else 0), grid, _STREAM_K)
+    if not gelu and _small_tiles(table):
+        plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
+    else:
+        plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | (_lib.EPI_GELU if gelu else 0), grid,
+                                                            _STREAM_K)
     if plan.total_tiles == 0:
         return
     n = len(table)
@@ -612,6 +616,25 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         _lib.check(rc)
 
     _submit(blob, device, launch, keep)
+
+
+# Tile size of a grouped GEMM.  The 256 x 256 tile is the fast one per flop.  The 128 x 128 tile (two workgroups per
+# compute unit, twice the operand traffic from L2) wins where the large tile leaves the machine idle: launches with
+# fewer large tiles than about half the compute units, and launches whose problems are so short or narrow that the
+# large tiles are mostly padding (measured 1.1 - 1.7 x there, 0.8 - 0.9 x on launches that fill the machine with
+# full tiles; same bits either way).  FP8GMM_TILE=256 / 128 forces one of them.
+_TILE = os.environ.get("FP8GMM_TILE", "auto")
+
+
+def _small_tiles(table):
+    if _TILE != "auto":
+        return _TILE == "128"
+    m, n = table["m"].astype(np.int64), table["n"].astype(np.int64)
+    large = int((((m + 255) // 256) * ((n + 255) // 256)).sum())
+    if large == 0:
+        return False
+    small = int((((m + 127) // 128) * ((n + 127) // 128)).sum())
+    return large <= 160 or 2 * small <= 5 * large
 
 
 # Tail balancing of the grouped GEMM (the workgroups of an XCD share their range's last tiles along K) needs

@@ -1,8 +1,8 @@
 // One instantiation of the grouped-GEMM kernel and its launcher: compiled once per entry of
-// FP8GMM_FOR_EACH_GEMM_VARIANT with -DFP8GMM_VARIANT_INDEX=0..6 (see the Makefile), so that the variants build in
-// parallel.
+// FP8GMM_FOR_EACH_GEMM_VARIANT with -DFP8GMM_VARIANT_INDEX=0..13 (see the Makefile), so that the variants build in
+// parallel.  0..6: the 256 x 256 tile, 7..13: the same operand formats and layouts with the 128 x 128 tile.
 #ifndef FP8GMM_VARIANT_INDEX
-#error "compile with -DFP8GMM_VARIANT_INDEX=<0..6>"
+#error "compile with -DFP8GMM_VARIANT_INDEX=<0..13>"
 #endif
 #include "grouped_gemm_kernel.h"
 
@@ -10,18 +10,25 @@ namespace fp8gmm {
 
 #define FP8GMM_CAT_(a, b) a##b
 #define FP8GMM_CAT(a, b) FP8GMM_CAT_(a, b)
-#define FP8GMM_INSTANTIATE(AF, BF, AT, BT)                                                                     \
-  template int prepare_variant<AF, BF, AT, BT>(int);                                                           \
-  template int launch_variant<AF, BF, AT, BT>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, \
-                                              uint8_t*, uint64_t*, hipStream_t);
+#define FP8GMM_INSTANTIATE(AF, BF, AT, BT, TL)                                                                     \
+  template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                           \
+  template int launch_variant<AF, BF, AT, BT, TL>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, \
+                                                  uint8_t*, uint64_t*, hipStream_t);
 
-#define FP8GMM_V0 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, false)
-#define FP8GMM_V1 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, false)
-#define FP8GMM_V2 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E5M2, false, false)
-#define FP8GMM_V3 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, true)
-#define FP8GMM_V4 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, true)
-#define FP8GMM_V5 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, true, true)
-#define FP8GMM_V6 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, true, true)
+#define FP8GMM_V0 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, false, 256)
+#define FP8GMM_V1 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, false, 256)
+#define FP8GMM_V2 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E5M2, false, false, 256)
+#define FP8GMM_V3 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, true, 256)
+#define FP8GMM_V4 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, true, 256)
+#define FP8GMM_V5 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, true, true, 256)
+#define FP8GMM_V6 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 256)
+#define FP8GMM_V7 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, false, 128)
+#define FP8GMM_V8 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, false, 128)
+#define FP8GMM_V9 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E5M2, false, false, 128)
+#define FP8GMM_V10 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, true, 128)
+#define FP8GMM_V11 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, true, 128)
+#define FP8GMM_V12 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, true, true, 128)
+#define FP8GMM_V13 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 128)
 
 FP8GMM_CAT(FP8GMM_V, FP8GMM_VARIANT_INDEX)
 

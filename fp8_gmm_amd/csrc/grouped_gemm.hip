@@ -174,9 +174,10 @@ typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, in
                          hipStream_t);
 
 // the variant for a format / layout combination, or null when the combination does not exist
-launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor) {
-#define FP8GMM_PICK(AF, BF, AT, BT) \
-  if (a_fmt == AF && b_fmt == BF && a_kmajor == AT && b_kmajor == BT) return &launch_variant<AF, BF, AT, BT>;
+launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor, int tile) {
+#define FP8GMM_PICK(AF, BF, AT, BT, TL)                                              \
+  if (a_fmt == AF && b_fmt == BF && a_kmajor == AT && b_kmajor == BT && tile == TL) \
+    return &launch_variant<AF, BF, AT, BT, TL>;
   FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_PICK)
 #undef FP8GMM_PICK
   return nullptr;
@@ -198,7 +199,12 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
     return FP8GMM_ERR_BAD_FORMAT;
   // e5m2 x e5m2 does not exist (cuBLASLt rejects it too); the contraction-major forms are the gradient GEMMs,
   // whose b is a forward tensor (weight or activation), always e4m3
-  const launch_fn launch = variant_for(a_fmt, b_fmt, a_kmajor, b_kmajor);
+  const int tile = plan->tile == 0 ? kGemmTileM : plan->tile;
+  if (tile != kGemmTileM && tile != FP8GMM_GEMM_SMALL_TILE) return FP8GMM_ERR_BAD_ARGUMENT;
+  // the small tile is never shared along K and has no fused GELU epilogue
+  if (tile != kGemmTileM && (plan->n_slots != 0 || plan->n_fixups != 0 || (epilogue & FP8GMM_EPI_GELU)))
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  const launch_fn launch = variant_for(a_fmt, b_fmt, a_kmajor, b_kmajor, tile);
   if (launch == nullptr) return FP8GMM_ERR_BAD_FORMAT;
   if (n == 0 || plan->total_tiles == 0) return FP8GMM_OK;
   if (plan->grid <= 0 || (plan->grid % kNumXcd) != 0 || plan->rounds < 1) return FP8GMM_ERR_BAD_ARGUMENT;
@@ -236,10 +242,10 @@ int fp8gmm_init(int device) {
   const int dev = device < 0 ? current : device;
   if (dev != current && hipSetDevice(dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
   int rc = device_num_cu(dev);
-#define FP8GMM_PREPARE(AF, BF, AT, BT) \
-  if (rc > 0) {                        \
-    const int e = prepare_variant<AF, BF, AT, BT>(dev); \
-    if (e != FP8GMM_OK) rc = e;        \
+#define FP8GMM_PREPARE(AF, BF, AT, BT, TL)                  \
+  if (rc > 0) {                                             \
+    const int e = prepare_variant<AF, BF, AT, BT, TL>(dev); \
+    if (e != FP8GMM_OK) rc = e;                             \
   }
   FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_PREPARE)
 #undef FP8GMM_PREPARE

@@ -129,9 +129,13 @@ __device__ __forceinline__ void merge_amax(float* slot, float wave_amax, int lan
 constexpr uint32_t kMaskedOffset = 0x80000000u;  // + any row offset of a tile (< 2^30) stays out of range
 
 // `s` = a_scale_inv * b_scale_inv and `cs` = c_scale of the problem, read by the caller ahead of time.
-__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gmm_gemm_problem& pr, int m0, int n0,
-                                              int out_kind, int epilogue, uint8_t* stage, bool oob_zero, float s,
-                                              float cs) {
+// TILE: 256 (the namespace's constants) or 128 (the small tile: 64 x 64 per wavefront, 16 KB of staging).
+template <int TILE>
+__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64], const fp8gmm_gemm_problem& pr,
+                                              int m0, int n0, int out_kind, int epilogue, uint8_t* stage,
+                                              bool oob_zero, float s, float cs) {
+  constexpr int BM = TILE, BN = TILE, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
+  constexpr int kStageBytes = TILE * 32;   // per wavefront: a quarter of one ring unit
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
@@ -157,7 +161,10 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
       // converted: the round trip through LDS, a third of the epilogue when exposed, hides behind the arithmetic.
       uint16_t* const C = static_cast<uint16_t*>(pr.c) + (int64_t)m0 * ldc + n0;
       const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
-      uint8_t* mine = stage + wave * 8192;
+      // (the small tile's staging area holds one unit per wavefront: a wavefront's LDS operations complete in
+      // order, so the read-back of a unit is done before the next unit's writes land in the same place)
+      uint8_t* mine = stage + wave * kStageBytes;
+      constexpr int kUnitsPerRow = NT / 2;               // units of 64 columns per 32-row block of the sub-tile
       const int wr = l32 * 128 + khalf * 8;              // + ((4 jl + g) ^ ((l32 >> 1) & 7)) * 16, jl = j & 1
       const int rrow = lane >> 3, rchunk = lane & 7;      // read-back: row 8 it + rrow, chunk rchunk
       u32x4 v[4];
@@ -171,9 +178,9 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
         }
       };
 #pragma unroll
-      for (int u = 0; u < MT * 2; ++u) {
-        const int i = u >> 1, jj = u & 1;
-        uint8_t* buf = mine + (u & 1) * 4096;
+      for (int u = 0; u < MT * kUnitsPerRow; ++u) {
+        const int i = u / kUnitsPerRow, jj = u % kUnitsPerRow;
+        uint8_t* buf = mine + (kStageBytes >= 8192 ? (u & 1) * 4096 : 0);
 #pragma unroll
         for (int jl = 0; jl < 2; ++jl) {
           const f32x16 t = tile_values(acc[i][2 * jj + jl]);
@@ -185,7 +192,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
           }
         }
         // the previous unit's read-back was issued before this unit's conversion: store it now
-        if (u > 0) store_unit((u - 1) >> 1, (u - 1) & 1);
+        if (u > 0) store_unit((u - 1) / kUnitsPerRow, (u - 1) % kUnitsPerRow);
         // only this wavefront touches `mine`, and its LDS operations complete in order
 #pragma unroll
         for (int it = 0; it < 4; ++it) {
@@ -193,10 +200,10 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
           v[it] = *reinterpret_cast<const u32x4*>(buf + r * 128 + ((rchunk ^ ((r >> 1) & 7)) << 4));
         }
       }
-      store_unit(MT - 1, 1);
+      store_unit(MT - 1, kUnitsPerRow - 1);
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
-    } else if (out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
+    } else if (TILE == 256 && out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
                ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0) && (interior || (oob_zero && (cv & 15) == 0))) {
       // The fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both outputs go
       // through the staging area like the plain form's, one 32-row block at a time, in ONE pass over the
@@ -395,7 +402,9 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[MT][NT], const fp8gm
 
 // Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
 // (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
-__device__ __forceinline__ void partial_store(f32x16 (&acc)[MT][NT], uint8_t* slot) {
+template <int TILE>
+__device__ __forceinline__ void partial_store(f32x16 (&acc)[TILE / 64][TILE / 64], uint8_t* slot) {
+  constexpr int MT = TILE / 64, NT = TILE / 64;
   float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
 #pragma unroll
   for (int i = 0; i < MT; ++i)
@@ -449,13 +458,26 @@ static_assert(offsetof(fp8gmm_gemm_item, k) == 32 && offsetof(fp8gmm_gemm_item, 
 // A_TR: the same for operand a (a[k][m], pitch lda): with both, c = a^T . b contracts over the rows of two
 // row-major matrices, which is the weight-gradient GEMM on the un-transposed activations and gradients; rows
 // past k read as zeros, so the contraction length needs no padding.
-template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
-__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gemm_problem* __restrict__ probs,
-                                                                const fp8gmm_gemm_item* __restrict__ items,
-                                                                int out_kind, int epilogue,
-                                                                uint8_t* __restrict__ workspace,
-                                                                uint64_t* __restrict__ counters) {
+// TILE = 128: the small tile.  Same structure with every extent halved: 128 x 128 per workgroup, 64 x 64 = 2 x 2 MFMA
+// tiles per wavefront, 16 KB ring units, 80 KB of LDS and at most 256 registers per lane, so that TWO workgroups
+// share a compute unit.  It pays where the large tile leaves the machine idle: launches with fewer large tiles
+// than compute units (four times as many small ones), and problems of up to 128 rows, half of whose large tiles
+// would be padding - 1.1 to 1.7 times faster there.  It moves twice the operand bytes from L2 per flop: at the
+// MFMA's pace that is 64 B per clock and compute unit, the L2's peak, so on launches that fill the machine with
+// full tiles it is 10 - 20 % slower however short the contraction.  Which tile a launch takes is decided when it
+// is planned (FP8GMM_GEMM_TILE_128); the results are the same bits either way.  No sharing along K and no fused
+// GELU epilogue in this form.
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
+__global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_kernel(
+    const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items, int out_kind,
+    int epilogue, uint8_t* __restrict__ workspace, uint64_t* __restrict__ counters) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // the tile's extents shadow the namespace's (which are those of the 256 x 256 tile)
+  [[maybe_unused]] constexpr int BM = TILE;
+  constexpr int BN = TILE, US = TILE * BK, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
+  constexpr int kParts = US / 1024 / NWAVES;        // 8 or 4 load instructions per wavefront and unit
+  constexpr int kFastStores = MT * (NT / 2) * 4;    // stores per wavefront in the staged bf16 epilogue
+  static_assert(TILE == 256 || TILE == 128, "tile sizes with a step sequence below");
 
   clock_probe_mark(counters, 0);
   const int tid = threadIdx.x;
@@ -485,14 +507,18 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   const int fb_off = (wave_n * WN + l32) * BK;
   // contraction-major unit: 128 contraction rows x 256 B.  Fragment of K half hh: rows 64 hh + 32 khalf + b (+ 8 t
   // per read), logical chunk wave_n * 8 + 2 j + g, byte 8 h; s = lane % 16 = 2 b + h
+  // (small tile: 128 contraction rows x 128 B, 8 chunks per row; rows r and r + 2 share their banks, and chunk c
+  // of row r sits at chunk c ^ (r & 6))
   const int tr_b = (lane & 15) >> 1, tr_h = lane & 1, tr_g = (lane >> 4) & 1;
-  const int tr_row = (32 * khalf + tr_b) * 256 + 8 * tr_h;
+  constexpr int kTrPitch = BN;                         // bytes per contraction row of a unit
+  const int tr_swz = TILE == 256 ? 2 * tr_b : (tr_b & 6);
+  const int tr_row = (32 * khalf + tr_b) * kTrPitch + 8 * tr_h;
   int fbt_off[NT];
 #pragma unroll
-  for (int j = 0; j < NT; ++j) fbt_off[j] = tr_row + (((wave_n * 8 + 2 * j + tr_g) ^ (2 * tr_b)) << 4);
+  for (int j = 0; j < NT; ++j) fbt_off[j] = tr_row + (((wave_n * (WN / 16) + 2 * j + tr_g) ^ tr_swz) << 4);
   int fat_off[MT];
 #pragma unroll
-  for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * 8 + 2 * i + tr_g) ^ (2 * tr_b)) << 4);
+  for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * (WM / 16) + 2 * i + tr_g) ^ tr_swz) << 4);
 
   // ---- this workgroup's work list (uniform): records blockIdx.x, blockIdx.x + grid, ... up to the end record.
   // Both sides of the kernel walk it, the load side ahead of the compute side, and both read a record one item
@@ -538,8 +564,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   // p ^ 2 (row mod 8); row mod 8 is the same for every j.
   // A record's operand addresses are those of the tile's first row / column, so these offsets depend on the
   // pitch alone.
-  const int krow = wave * 4 + (lane >> 4);
-  const int tr_col = ((lane & 15) ^ (2 * (krow & 7))) << 4;
+  // (small tile: one instruction fills 8 contraction rows x 128 B; part j = rows (wave + NWAVES j) * 8 + lane / 8)
+  constexpr int kTrRows = 1024 / kTrPitch;             // contraction rows per load instruction: 4 or 8
+  const int krow = wave * kTrRows + lane / (kTrPitch / 16);
+  const int tr_col = TILE == 256 ? ((lane & 15) ^ (2 * (krow & 7))) << 4 : ((lane & 7) ^ (krow & 6)) << 4;
   // Takes the record fetched ahead (r_ld), fetches the one after it, and sets up descriptors and offsets.
   auto load_setup = [&]() {
     for (;;) {
@@ -561,7 +589,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
           a_step = NWAVES * 8 * (uint32_t)gl.lda;
         } else {
           a_base = (uint32_t)krow * (uint32_t)gl.lda + (uint32_t)tr_col;
-          a_step = NWAVES * 4 * (uint32_t)gl.lda;
+          a_step = NWAVES * kTrRows * (uint32_t)gl.lda;
           ld_lda = gl.lda;
         }
         if constexpr (!B_TR) {
@@ -569,7 +597,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
           b_step = NWAVES * 8 * (uint32_t)gl.ldb;
         } else {
           b_base = (uint32_t)krow * (uint32_t)gl.ldb + (uint32_t)tr_col;
-          b_step = NWAVES * 4 * (uint32_t)gl.ldb;
+          b_step = NWAVES * kTrRows * (uint32_t)gl.ldb;
           ld_ldb = gl.ldb;
         }
         ld_kmax = gt.k - dchunk * 16;  // this lane's chunk exists iff k0 < ld_kmax
@@ -620,9 +648,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
   typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
   auto read_frag_tr = [&](i32x8& f, uint32_t a) {  // 4 x 8 contraction rows of the lane's column
     const i32x2 t0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a));
-    const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 2048));
-    const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 4096));
-    const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 6144));
+    const i32x2 t1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 8 * kTrPitch));
+    const i32x2 t2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 16 * kTrPitch));
+    const i32x2 t3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32(reinterpret_cast<lds_i32x2*>(a + 24 * kTrPitch));
     f = i32x8{t0.x, t0.y, t1.x, t1.y, t2.x, t2.y, t3.x, t3.y};
   };
   // weight fragment j / token fragment i, K half hh, of the unit at `unit`
@@ -630,14 +658,14 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     if constexpr (!B_TR) {
       read_frag(f, unit + fb_off + j * 32 * BK, hh);
     } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * 256));
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * kTrPitch));
     }
   };
   auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh) {
     if constexpr (!A_TR) {
       read_frag(f, unit + fa_off + i * 32 * BK, hh);
     } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * 256));
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * kTrPitch));
     }
   };
 
@@ -701,7 +729,22 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
       const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
       // ---- low K half: fragments in fa0 / fb0; fetch the high half's from the same units.  No barrier:
       // nothing written since the last one is read here.
-      {
+      if constexpr (TILE == 128) {
+        const uint8_t* qa = lds + ua * US;
+        const uint8_t* qb = lds + ub * US;
+        FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
+        dma_a(fa, 0);
+        read_frag_b(fb1[0], qb, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
+        dma_a(fa, 1);
+        read_frag_b(fb1[1], qb, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
+        dma_a(fa, 2);
+        read_frag_a(fa1[0], qa, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        dma_a(fa, 3);
+        read_frag_a(fa1[1], qa, 1, 1);
+      } else {
         const uint8_t* qa = lds + ua * US;
         const uint8_t* qb = lds + ub * US;
         FP8GMM_SB(); FP8GMM_MF0(0, 0); FP8GMM_SB();
@@ -745,7 +788,28 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
         FP8GMM_WAIT_VM_LGKM(kParts);
       }
       __builtin_amdgcn_s_barrier();
-      {
+      if constexpr (TILE == 128) {
+        const uint8_t* qa = lds + na * US;
+        const uint8_t* qb = lds + nb * US;
+        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        dma_b(ua, 0);
+        read_frag_b(fb0[0], qb, 0, 0);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        dma_b(ua, 1);
+        read_frag_b(fb0[1], qb, 1, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        dma_b(ua, 2);
+        read_frag_a(fa0[0], qa, 0, 0);
+        FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
+        dma_b(ua, 3);
+        read_frag_a(fa0[1], qa, 1, 0);
+        if constexpr (decltype(same_item)::value) {
+          ++ld_kt;
+          step_setup();
+        } else {
+          dma_advance();
+        }
+      } else {
         const uint8_t* qa = lds + na * US;
         const uint8_t* qb = lds + nb * US;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
@@ -796,11 +860,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
     // ---- epilogue ----
     if (g.slot >= 0) {
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
-      partial_store(acc, workspace + (size_t)g.slot * kPartialBytes);
+      partial_store<TILE>(acc, workspace + (size_t)g.slot * kPartialBytes);
       relaxed = false;
     } else {
       // free until the next step's token loads: the unit that held the last step's weights
-      relaxed = tile_epilogue(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US, !A_TR && !B_TR, scale_ab,
+      relaxed = tile_epilogue<TILE>(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US, !A_TR && !B_TR, scale_ab,
                               scale_c);
     }
   }
@@ -817,47 +881,54 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const fp8gmm_gem
 // every variant; a launch on a device that was never initialised sets its own.
 constexpr int kMaxDevices = 64;
 
-template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 int prepare_variant(int dev) {
   static std::atomic<bool> attr_set[kMaxDevices];
   if (dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
   if (!attr_set[dev].load(std::memory_order_acquire)) {
-    auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR>;
+    auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RING * US) != hipSuccess)
+                            RING * TILE * BK) != hipSuccess)
       return FP8GMM_ERR_LAUNCH;
     attr_set[dev].store(true, std::memory_order_release);
   }
   return FP8GMM_OK;
 }
 
-template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
+template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item* items_dev, int grid, int out_kind,
                    int epilogue, uint8_t* workspace, uint64_t* counters, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
-  const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR>(dev);
+  const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR, TILE>(dev);
   if (rc != FP8GMM_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR>), dim3(grid), dim3(NTHREADS), RING * US, stream,
-                     probs_dev, items_dev, out_kind, epilogue, workspace, counters);
+  hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>), dim3(grid), dim3(NTHREADS),
+                     RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace, counters);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
 // One explicit instantiation per operand format / layout combination, each in its own translation unit
 // (gemm_variant.hip compiled with -DFP8GMM_VARIANT_*): the kernel takes most of a minute to compile.
-#define FP8GMM_FOR_EACH_GEMM_VARIANT(X)      \
-  X(FP8GMM_E4M3, FP8GMM_E4M3, false, false)  \
-  X(FP8GMM_E5M2, FP8GMM_E4M3, false, false)  \
-  X(FP8GMM_E4M3, FP8GMM_E5M2, false, false)  \
-  X(FP8GMM_E4M3, FP8GMM_E4M3, false, true)   \
-  X(FP8GMM_E5M2, FP8GMM_E4M3, false, true)   \
-  X(FP8GMM_E4M3, FP8GMM_E4M3, true, true)    \
-  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true)
+#define FP8GMM_FOR_EACH_GEMM_VARIANT(X)           \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, false, 256)  \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, false, 256)  \
+  X(FP8GMM_E4M3, FP8GMM_E5M2, false, false, 256)  \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, true, 256)   \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, true, 256)   \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, true, true, 256)    \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 256)    \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, false, 128)  \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, false, 128)  \
+  X(FP8GMM_E4M3, FP8GMM_E5M2, false, false, 128)  \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, true, 128)   \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, true, 128)   \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, true, true, 128)    \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 128)
 
-#define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT)                                                                     \
-  extern template int prepare_variant<AF, BF, AT, BT>(int);                                                        \
-  extern template int launch_variant<AF, BF, AT, BT>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, \
-                                                     int, uint8_t*, uint64_t*, hipStream_t);
+#define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT, TL)                                                                     \
+  extern template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                        \
+  extern template int launch_variant<AF, BF, AT, BT, TL>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, \
+                                                         int, uint8_t*, uint64_t*, hipStream_t);
 #ifndef FP8GMM_VARIANT_INDEX
 FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_DECLARE_VARIANT)
 #endif

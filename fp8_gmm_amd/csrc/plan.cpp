@@ -7,6 +7,7 @@
 // kernels pick the vector or the scalar path per tensor at run time.
 #include <stdint.h>
 
+#include <algorithm>
 #include <vector>
 
 #include "../../include/fp8gmm.h"
@@ -181,6 +182,107 @@ int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layou
 // The work list of a launch: the schedule of gemm_schedule.h written out, one record per (workgroup, item), in
 // the order items[r * grid + workgroup]; the slots in use are renumbered from 0 in the order the workgroups
 // are walked, and the fix-up records name them by their new numbers.
+// The same launch cut into 128 x 128 tiles (FP8GMM_GEMM_TILE_128): whole tiles only, the tile list in 8 contiguous
+// ranges of equal work, the workgroups of an XCD striding through their range.
+static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int grid, fp8gmm_gemm_item* items,
+                            int max_items, fp8gmm_gemm_plan* plan) {
+  using namespace fp8gmm;
+  constexpr int T = FP8GMM_GEMM_SMALL_TILE;
+  constexpr int kOverhead = 3;   // epilogue and switch of a small tile, in K = 128 steps of a workgroup that shares its CU
+  int unused = 0;
+  const int rc = fp8gmm_plan_grouped_gemm_layout(probs, n, layout, &unused);
+  if (rc != FP8GMM_OK) return rc;
+  const bool a_kmajor = (layout & FP8GMM_GEMM_A_KMAJOR) != 0, b_kmajor = (layout & FP8GMM_GEMM_B_KMAJOR) != 0;
+  // tiles and work per problem
+  std::vector<int64_t> tile_begin((size_t)n + 1, 0), work_begin((size_t)n + 1, 0);
+  for (int p = 0; p < n; ++p) {
+    const int64_t tiles = (int64_t)((probs[p].m + T - 1) / T) * ((probs[p].n + T - 1) / T);
+    const int64_t steps = (probs[p].k + 127) / 128;
+    tile_begin[p + 1] = tile_begin[p] + tiles;
+    work_begin[p + 1] = work_begin[p] + tiles * ((steps > 0 ? steps : 1) + kOverhead);
+    if (tile_begin[p + 1] > INT32_MAX / 16) return FP8GMM_ERR_BAD_SHAPE;
+  }
+  const int total_tiles = (int)tile_begin[n];
+  plan->total_tiles = total_tiles;
+  plan->tile = T;
+  if (total_tiles == 0) return FP8GMM_OK;
+  {
+    const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
+    if (grid > needed) grid = needed;
+  }
+  const int wgs = grid / kNumXcd;
+  // XCD x takes the tiles [cut[x], cut[x + 1]): the first tile at or past x / 8 of the work
+  int cut[kNumXcd + 1];
+  cut[0] = 0;
+  cut[kNumXcd] = total_tiles;
+  {
+    int p = 0;
+    for (int x = 1; x < kNumXcd; ++x) {
+      const int64_t target = (work_begin[n] * x + kNumXcd - 1) / kNumXcd;
+      while (p < n && work_begin[p + 1] <= target) ++p;
+      if (p >= n) {
+        cut[x] = total_tiles;
+        continue;
+      }
+      const int64_t per_tile = (work_begin[p + 1] - work_begin[p]) / (tile_begin[p + 1] - tile_begin[p]);
+      cut[x] = (int)(tile_begin[p] + (target - work_begin[p] + per_tile - 1) / per_tile);
+    }
+  }
+  int rounds = 0;
+  for (int x = 0; x < kNumXcd; ++x) rounds = std::max(rounds, (cut[x + 1] - cut[x] + wgs - 1) / wgs);
+  rounds += 1;  // every list ends with a record whose prob is -1
+  plan->grid = grid;
+  plan->rounds = rounds;
+  if ((int64_t)rounds * grid > INT32_MAX / 64) return FP8GMM_ERR_BAD_SHAPE;
+  if ((int64_t)rounds * grid > max_items) return FP8GMM_ERR_BUFFER_TOO_SMALL;
+  if (items == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  fp8gmm_gemm_item end_record{};
+  end_record.prob = -1;
+  end_record.slot = -1;
+  for (int i = 0; i < rounds * grid; ++i) items[i] = end_record;
+  for (int x = 0; x < kNumXcd; ++x) {
+    int p = 0;
+    for (int t = cut[x]; t < cut[x + 1]; ++t) {
+      while (tile_begin[p + 1] <= t) ++p;
+      const fp8gmm_gemm_problem& pr = probs[p];
+      const int local = t - cut[x];
+      const int r = local / wgs, j = (local + kRoundRotation * r) % wgs;   // position in the round rotates
+      fp8gmm_gemm_item& o = items[(size_t)r * grid + (size_t)j * kNumXcd + x];
+      o = fp8gmm_gemm_item{};
+      int m0 = 0, n0 = 0;
+      tile_origin(pr.m, pr.n, (int)(t - tile_begin[p]), T, &m0, &n0);
+      const int64_t rows = pr.m - m0 < T ? pr.m - m0 : T;
+      const int64_t cols = pr.n - n0 < T ? pr.n - n0 : T;
+      if (pr.k > 0) {
+        if (!a_kmajor) {
+          o.a = (uint64_t)reinterpret_cast<uintptr_t>(pr.a) + (uint64_t)m0 * (uint64_t)pr.lda;
+          o.a_bytes = (uint32_t)((rows - 1) * pr.lda + pr.k);
+        } else {
+          o.a = (uint64_t)reinterpret_cast<uintptr_t>(pr.a) + (uint64_t)m0;
+          o.a_bytes = (uint32_t)((int64_t)(pr.k - 1) * pr.lda + (pr.m - m0));
+        }
+        if (!b_kmajor) {
+          o.b = (uint64_t)reinterpret_cast<uintptr_t>(pr.b) + (uint64_t)n0 * (uint64_t)pr.ldb;
+          o.b_bytes = (uint32_t)((cols - 1) * pr.ldb + pr.k);
+        } else {
+          o.b = (uint64_t)reinterpret_cast<uintptr_t>(pr.b) + (uint64_t)n0;
+          o.b_bytes = (uint32_t)((int64_t)(pr.k - 1) * pr.ldb + (pr.n - n0));
+        }
+      }
+      o.lda = pr.lda;
+      o.ldb = pr.ldb;
+      o.k = pr.k;
+      o.k_begin = 0;
+      o.nk = (pr.k + 127) / 128;
+      o.m0 = m0;
+      o.n0 = n0;
+      o.prob = p;
+      o.slot = -1;
+    }
+  }
+  return FP8GMM_OK;
+}
+
 int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layout, int grid, int stream_k,
                                     fp8gmm_gemm_item* items, int max_items, fp8gmm_gemm_fixup_desc* fixups,
                                     int max_fixups, fp8gmm_gemm_plan* plan) {
@@ -188,6 +290,11 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
   *plan = fp8gmm_gemm_plan{};
   if (grid <= 0 || (grid % kNumXcd) != 0 || max_items < 0 || max_fixups < 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (layout & FP8GMM_GEMM_TILE_128) {
+    if (layout & FP8GMM_EPI_GELU) return FP8GMM_ERR_BAD_ARGUMENT;
+    return plan_small_tiles(probs, n, layout & ~FP8GMM_GEMM_TILE_128, grid, items, max_items, plan);
+  }
+  plan->tile = kGemmTileM;
   const bool gelu = (layout & FP8GMM_EPI_GELU) != 0;  // only weighs the decision to share tiles along K
   layout &= ~FP8GMM_EPI_GELU;
   int total_tiles = 0;

@@ -147,6 +147,15 @@ typedef struct fp8gmm_gemm_problem {
  * (fp8_gmm/grouped_linear.py:36-52,142-150).  Only together with FP8GMM_GEMM_B_KMAJOR; m and n multiples of
  * 16, k arbitrary (rows past k contribute zeros), (k + 128) * lda < 2^32. */
 #define FP8GMM_GEMM_A_KMAJOR 4
+/* Planning flag (fp8gmm_plan_grouped_gemm_launch's `layout` only): cut the outputs into 128 x 128 tiles instead of
+ * 256 x 256 and run two workgroups per compute unit (pass a grid of 2 * fp8gmm_gemm_grid()).  For launches whose
+ * contraction is short (K up to about 2048) or whose problems have few rows: a workgroup's epilogue, tile switch and
+ * waits for operands then overlap the other workgroup's arithmetic, and ragged problems pad to 128 rows.  Costs
+ * twice the operand traffic from L2 per flop.  Never shares tiles along K (stream_k is ignored); not available with
+ * FP8GMM_EPI_GELU.  No counterpart in the reference (CUTLASS picks its tile shape at compile time,
+ * csrc/fp8_gmm.cu:82-110). */
+#define FP8GMM_GEMM_TILE_128 0x100
+#define FP8GMM_GEMM_SMALL_TILE 128
 
 /*
  * Work list of a grouped-GEMM launch, written by fp8gmm_plan_grouped_gemm_launch on the host and read by the
@@ -189,7 +198,8 @@ typedef struct fp8gmm_gemm_plan {
   int32_t n_fixups;    /* tiles shared along K = workgroups of the fix-up launch (0: no such launch) */
   int32_t n_slots;     /* workspace slots the launch writes: it needs n_slots * FP8GMM_GEMM_SLOT_BYTES bytes */
   int32_t total_tiles;
-  int32_t reserved[3];
+  int32_t tile;        /* rows = columns of a tile: 256, or 128 when planned with FP8GMM_GEMM_TILE_128 (0 reads as 256) */
+  int32_t reserved[2];
 } fp8gmm_gemm_plan;    /* 32 bytes */
 
 #define FP8GMM_GEMM_SLOT_BYTES 262144  /* fp32 accumulators of one 256 x 256 tile */

@@ -253,3 +253,74 @@ def test_consecutive_tiles_form_compact_blocks():
             rows = {tiles[t][0] for t in range(start, start + 32)}
             cols = {tiles[t][1] for t in range(start, start + 32)}
             assert len(rows) + len(cols) <= 12, (shape, start, len(rows), len(cols))
+
+
+def test_small_tile_plan():
+    """FP8GMM_GEMM_TILE_128: the same launch cut into 128 x 128 tiles, whole tiles only.  Every 128 x 128 block of
+    every output exactly once, records with the addresses and extents of a 128-row / 128-column slab, XCD ranges
+    contiguous and in order, no workspace, no fix-up launch; not available together with the GELU epilogue."""
+    rng = np.random.default_rng(7)
+    cases = [[(137, 512, 256), (401, 512, 256), (0, 512, 256), (59, 512, 256)],
+             [(64, 1408, 2048)] * 64,
+             [(1, 16, 16)],
+             [(300, 520, 1040), (129, 128, 0), (128, 129, 4096)]]
+    for _ in range(20):
+        cases.append([(int(rng.choice([0, 1, 100, 128, 129, 300, 700])), int(rng.choice([16, 128, 144, 1000])),
+                       int(rng.choice([0, 16, 128, 1040, 4096]))) for _ in range(int(rng.integers(1, 10)))])
+    for shapes in cases:
+        for layout in (0, _lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR | _lib.GEMM_A_KMAJOR):
+            t = np.zeros(len(shapes), dtype=_lib.GEMM_PROBLEM)
+            for i, (m, n, k) in enumerate(shapes):
+                if layout & _lib.GEMM_A_KMAJOR:
+                    m = (m + 15) // 16 * 16
+                if layout & _lib.GEMM_B_KMAJOR:
+                    n = (n + 15) // 16 * 16
+                t[i]["a"], t[i]["b"], t[i]["c"] = 0x10000, 0x20000, 0x30000
+                t[i]["m"], t[i]["n"], t[i]["k"] = m, n, k
+                t[i]["lda"] = max(m if layout & _lib.GEMM_A_KMAJOR else k, 16)
+                t[i]["ldb"] = max(n if layout & _lib.GEMM_B_KMAJOR else k, 16)
+                t[i]["ldc"] = max(n, 1)
+            grid = 512
+            plan, items, fixups = _lib.plan_grouped_gemm_launch(t.copy(), layout | _lib.GEMM_TILE_128, grid, True)
+            want = {(p, i * 128, j * 128) for p in range(len(t))
+                    for i in range((int(t["m"][p]) + 127) // 128) for j in range((int(t["n"][p]) + 127) // 128)}
+            assert plan.tile == 128 and plan.total_tiles == len(want) and plan.n_slots == 0 and plan.n_fixups == 0
+            assert len(fixups) == 0
+            if not want:
+                continue
+            assert plan.grid == min(grid, (len(want) + 7) // 8 * 8) and len(items) == plan.rounds * plan.grid
+            items = items.reshape(plan.rounds, plan.grid)
+            seen, order = set(), {}
+            for wg in range(plan.grid):
+                col = items[:, wg]
+                count = int((col["prob"] >= 0).sum())
+                assert (col["prob"][:count] >= 0).all() and (col["prob"][count:] == -1).all() and count < plan.rounds
+                for r in col[:count]:
+                    p, m0, n0 = int(r["prob"]), int(r["m0"]), int(r["n0"])
+                    m, n, k, lda, ldb = (int(t[f][p]) for f in ("m", "n", "k", "lda", "ldb"))
+                    assert (p, m0, n0) in want and (p, m0, n0) not in seen
+                    seen.add((p, m0, n0))
+                    order.setdefault(wg % 8, []).append(p)
+                    assert (r["k_begin"], r["nk"], r["slot"], r["k"]) == (0, (k + 127) // 128, -1, k)
+                    if k > 0:
+                        if layout & _lib.GEMM_A_KMAJOR:
+                            assert r["a"] == 0x10000 + m0 and r["a_bytes"] == (k - 1) * lda + (m - m0)
+                        else:
+                            assert r["a"] == 0x10000 + m0 * lda and r["a_bytes"] == (min(m - m0, 128) - 1) * lda + k
+                        if layout & _lib.GEMM_B_KMAJOR:
+                            assert r["b"] == 0x20000 + n0 and r["b_bytes"] == (k - 1) * ldb + (n - n0)
+                        else:
+                            assert r["b"] == 0x20000 + n0 * ldb and r["b_bytes"] == (min(n - n0, 128) - 1) * ldb + k
+            assert seen == want
+            # the XCD ranges follow the problem order
+            last = -1
+            for x in range(8):
+                if x in order:
+                    assert min(order[x]) >= last
+                    last = max(order[x])
+    # no fused GELU epilogue with the small tile
+    t, _ = make_table([(256, 256, 128)])
+    import ctypes
+    plan = _lib.GemmPlan()
+    assert _lib.load().fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 1, _lib.GEMM_TILE_128 | _lib.EPI_GELU, 16, 0,
+                                                       None, 0, None, 0, ctypes.byref(plan)) < 0

@@ -56,17 +56,19 @@ def test_power_of_two_operands_are_exact(dev, a_dtype, m, n, k):
 
 @pytest.mark.parametrize("a_dtype", [E4M3, E5M2])
 @pytest.mark.parametrize("sizes,n,k", [([256], 256, 4096), ([700], 520, 4112), ([300, 0, 513, 90], 512, 7168)])
-def test_tiles_shared_along_k_are_exact(dev, a_dtype, sizes, n, k):
+def test_tiles_shared_along_k_are_exact(dev, a_dtype, sizes, n, k, monkeypatch):
     """Few tiles and a long K: the launch cuts tiles along K, leaves fp32 partial sums in its workspace and
     completes them in the fix-up pass.  With operands from {0, +-0.25 .. +-2} every partial sum is exact, so
     the result must still equal the exactly rounded oracle result bit for bit: a piece that is dropped,
-    added twice or taken from the wrong slot cannot pass.  The schedule introspection call proves that
-    this launch really does cut tiles."""
+    added twice or taken from the wrong slot cannot pass.  The plan proves that this launch really does cut
+    tiles (the 256 x 256 tile is forced: left to itself the backend gives a launch this small the 128 x 128 tile,
+    which is never shared)."""
     import numpy as np
 
     from fp8_gmm_amd import _lib
 
     backend = _backend()
+    monkeypatch.setattr(backend, "_TILE", "256")
     table = np.zeros(len(sizes), dtype=_lib.GEMM_PROBLEM)
     for i, m in enumerate(sizes):
         table[i]["a"], table[i]["b"], table[i]["c"] = 0x1000, 0x1000, 0x1000
@@ -299,11 +301,12 @@ def test_argument_errors_raise(dev):
                                [torch.zeros(1)])
 
 
-def test_shared_tiles_on_concurrent_streams(dev):
+def test_shared_tiles_on_concurrent_streams(dev, monkeypatch):
     """Launches that cut tiles along K keep their partial sums in a workspace the caller passes in; the backend
     keeps one per (device, stream): GEMMs running at the same time on different streams must not see each
     other's partial sums.  Exact data, so any cross-talk shows up as a bit difference."""
     backend = _backend()
+    monkeypatch.setattr(backend, "_TILE", "256")   # the tile that is shared along K
     m, n, k = 300, 512, 8192
     vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
     streams = [torch.cuda.Stream(device=dev) for _ in range(10)]
@@ -579,11 +582,14 @@ def test_gelu_epilogue_whole_line_stores_equal_the_per_group_path(dev):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("tile", ["256", "128"])
 @pytest.mark.parametrize("a_dtype", [E4M3, E5M2], ids=["e4m3", "e5m2"])
-def test_bf16_epilogue_whole_line_stores_equal_the_per_group_path(dev, a_dtype):
+def test_bf16_epilogue_whole_line_stores_equal_the_per_group_path(dev, a_dtype, tile, monkeypatch):
     """The same for the plain bf16 output: interior tiles go through LDS, a row pitch that is not a multiple of 8
-    sends every tile down the per-group path; the common columns must agree bit for bit (NaN row included)."""
+    sends every tile down the per-group path; the common columns must agree bit for bit (NaN row included).
+    Both tile sizes have the two paths."""
     backend = _backend()
+    monkeypatch.setattr(backend, "_TILE", tile)
     g = gen(4243)
     m, k, n, extra = 700, 384, 768, 4
     a = _q(randn_bf16((m, k), g), a_dtype)
@@ -601,13 +607,15 @@ def test_bf16_epilogue_whole_line_stores_equal_the_per_group_path(dev, a_dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("form", ["bf16", "gelu"])
-def test_edge_tiles_store_nothing_outside_the_problem(dev, form):
+@pytest.mark.parametrize("form", ["bf16", "bf16-small-tile", "gelu"])
+def test_edge_tiles_store_nothing_outside_the_problem(dev, form, monkeypatch):
     """Edge tiles take the same whole-line store path as interior ones, bounded by a buffer descriptor (rows) and
     by per-lane masks (columns).  Ragged problems written into column slices of wider, sentinel-filled buffers:
     the valid region must equal the exact result, every byte outside it must keep the sentinel, and the rows of
     the neighbouring problem in the same buffer must be untouched by this one's last row of tiles."""
     backend = _backend()
+    monkeypatch.setattr(backend, "_TILE", "128" if form == "bf16-small-tile" else "256")
+    form = form.split("-")[0]
     vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
     g = torch.Generator(device=dev).manual_seed(99)
     shapes = [(1, 8), (129, 264), (255, 136), (257, 248), (300, 520), (512, 16), (31, 1000)] if form == "bf16" else \
@@ -653,3 +661,74 @@ def test_edge_tiles_store_nothing_outside_the_problem(dev, form):
             out8[:m, :n] = 0x55
             outp[:m, :n] = -7.0
             assert (out8 == 0x55).all() and (outp == -7.0).all(), f"problem {i}: wrote outside its [m, n] region"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("a_dtype", [E4M3, E5M2], ids=["e4m3", "e5m2"])
+def test_small_tile_gives_the_same_bits_as_the_large_tile(dev, a_dtype, monkeypatch):
+    """The 128 x 128 tile (two workgroups per compute unit) is chosen per launch when the launch is planned; it walks K
+    in the same order with the same MFMA, so every output must equal the 256 x 256 tile's bit for bit: row-major
+    operands, a contraction-major b (data gradient), both contraction-major (weight gradient, ragged K), ragged and
+    empty problems, unaligned outputs, an fp8 output with its amax."""
+    backend = _backend()
+    g = torch.Generator(device=dev).manual_seed(321)
+
+    def both(fn):
+        out = {}
+        for tile in ("256", "128"):
+            monkeypatch.setattr(backend, "_TILE", tile)
+            out[tile] = fn()
+        monkeypatch.setattr(backend, "_TILE", "auto")
+        auto = fn()
+        return out["256"], out["128"], auto
+
+    for sizes, n, k in [([64, 1, 0, 128, 129], 1408, 2048), ([300, 0, 513, 90], 512, 1040), ([1, 15], 16, 16),
+                        ([700], 272, 2064), ([137, 401, 59, 403], 256, 512), ([256] * 8, 2048, 4096), ([64], 1536, 80)]:
+        e = len(sizes)
+        a = torch.randn(sum(sizes), k, generator=g, device=dev).to(a_dtype)
+        b = torch.randn(e, n, k, generator=g, device=dev).to(E4M3)
+        b_kn = b.transpose(1, 2).contiguous()
+        sa = torch.rand(e, generator=g, device=dev) + 0.5
+        sb = torch.rand(e, generator=g, device=dev) + 0.5
+        gs = torch.tensor(sizes)
+        big, small, auto = both(lambda: backend.fp8_gmm(a, b, gs, sa, sb, backward=a_dtype == E5M2))
+        assert torch.equal(big.view(torch.int16), small.view(torch.int16)), f"row-major {sizes} {n} {k}"
+        assert torch.equal(big.view(torch.int16), auto.view(torch.int16))
+        big, small, _ = both(lambda: backend.fp8_gmm(a, b_kn, gs, sa, sb, backward=True, b_transposed=True))
+        assert torch.equal(big.view(torch.int16), small.view(torch.int16)), f"b contraction-major {sizes} {n} {k}"
+    # weight gradient: c_i = a_i^T . b_i over ragged row counts
+    for rows, m, n in [([137, 401, 0, 59, 403], 512, 256), ([1, 2, 700], 16, 48), ([100, 30], 1408, 2048)]:
+        total = sum(rows)
+        dy = torch.randn(total, m, generator=g, device=dev).to(a_dtype)
+        x = torch.randn(total, n, generator=g, device=dev).to(E4M3)
+        bounds = [0]
+        for r in rows:
+            bounds.append(bounds[-1] + r)
+        a_list = [dy[bounds[i]: bounds[i + 1]] for i in range(len(rows))]
+        b_list = [x[bounds[i]: bounds[i + 1]] for i in range(len(rows))]
+        ones = torch.ones(len(rows), device=dev)
+
+        def wgrad():
+            out = torch.full((len(rows), m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+            backend.grouped_gemm(a_list, b_list, list(out.unbind(0)), ones, ones, transposed=True)
+            return out
+
+        big, small, _ = both(wgrad)
+        assert torch.equal(big.view(torch.int16), small.view(torch.int16)), f"weight gradient {rows} {m} {n}"
+    # fp8 output with amax, and an output whose pitch and base are not 16-byte aligned (per-group store paths)
+    a = torch.randn(200, 256, generator=g, device=dev).to(a_dtype)
+    b = torch.randn(2, 120, 256, generator=g, device=dev).to(E4M3)
+    ones = torch.ones(2, device=dev)
+
+    def fp8_out():
+        c = torch.zeros(200, 120, device=dev).to(E4M3)
+        amax = torch.zeros(2, device=dev)
+        backend.fp8_gmm(a, b, [150, 50], ones, ones, c, c_scales=torch.full((2,), 0.5, device=dev), c_amaxes=amax,
+                        backward=a_dtype == E5M2)
+        return c, amax
+
+    (cb, ab), (cs, as_), _ = both(fp8_out)
+    assert torch.equal(cb.view(torch.uint8), cs.view(torch.uint8)) and torch.equal(ab, as_)
+    b2 = torch.randn(2, 100, 256, generator=g, device=dev).to(E4M3)   # n = 100: bf16 rows of 200 bytes
+    big, small, _ = both(lambda: backend.fp8_gmm(a, b2, [150, 50], ones, ones, backward=a_dtype == E5M2))
+    assert torch.equal(big.view(torch.int16), small.view(torch.int16))
