@@ -17,6 +17,8 @@
 //     reads its work list, one 64-byte record per tile, and does no scheduling arithmetic of its own
 //     (binary searches over the problem table and integer divisions in the scalar unit cost a tile switch
 //     thousands of cycles, more with every expert).
+//     (Extents below are those of the default tile; the template's TILE = 128 form halves them all, see the
+//     kernel.)
 //   * a workgroup is 4 wavefronts (2 along m x 2 along n), one per SIMD; a wavefront owns a
 //     128 x 128 sub-tile = 4 x 4 MFMA tiles of v_mfma_f32_32x32x64_f8f6f4.  Its 256 accumulators
 //     live in the accumulation registers, the other 256 registers hold fragments and addresses.
