@@ -154,7 +154,9 @@ int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layou
       if (p.k > 0) {  // with k == 0 the operands are never read
         if (p.a == nullptr || p.b == nullptr) return FP8GMM_ERR_NULL_POINTER;
         // a row-major operand is fetched in 16-byte pieces along k, a contraction-major one along its rows
-        if ((!(a_kmajor && b_kmajor) && (p.k & 15)) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
+        // (with b alone contraction-major any k will do: the rows of b past k read as zeros, and the 16-byte piece
+        // of a that straddles k lies inside a's row pitch)
+        if ((!b_kmajor && (p.k & 15)) || (p.lda & 15) || (p.ldb & 15)) return FP8GMM_ERR_ALIGNMENT;
         if ((a_kmajor && (p.m & 15)) || (b_kmajor && (p.n & 15))) return FP8GMM_ERR_ALIGNMENT;
         if ((reinterpret_cast<uintptr_t>(p.a) & 15) || (reinterpret_cast<uintptr_t>(p.b) & 15))
           return FP8GMM_ERR_ALIGNMENT;
@@ -256,7 +258,7 @@ static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int g
       if (pr.k > 0) {
         if (!a_kmajor) {
           o.a = (uint64_t)reinterpret_cast<uintptr_t>(pr.a) + (uint64_t)m0 * (uint64_t)pr.lda;
-          o.a_bytes = (uint32_t)((rows - 1) * pr.lda + pr.k);
+          o.a_bytes = (uint32_t)((rows - 1) * pr.lda + ((pr.k + 15) & ~15));
         } else {
           o.a = (uint64_t)reinterpret_cast<uintptr_t>(pr.a) + (uint64_t)m0;
           o.a_bytes = (uint32_t)((int64_t)(pr.k - 1) * pr.lda + (pr.m - m0));
@@ -374,10 +376,13 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
       const int64_t rows = p.m - it.m0 < BM ? p.m - it.m0 : BM;
       const int64_t cols = p.n - it.n0 < BN ? p.n - it.n0 : BN;
       if (p.k > 0) {
-        // extents: up to the last byte of the tile's last row (row-major) / of the operand's last contraction row
+        // extents: up to the last byte of the tile's last row (row-major) / of the operand's last contraction row.
+        // A row-major a whose k is not a multiple of 16 (allowed next to a contraction-major b) ends inside a
+        // 16-byte piece; the bound includes the whole piece, which lies inside the row's pitch: the hardware
+        // checks the range per dword, and a dword that straddled the bound would lose its valid bytes too.
         if (!a_kmajor) {
           o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0 * (uint64_t)p.lda;
-          o.a_bytes = (uint32_t)((rows - 1) * p.lda + p.k);
+          o.a_bytes = (uint32_t)((rows - 1) * p.lda + ((p.k + 15) & ~15));
         } else {
           o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0;
           o.a_bytes = (uint32_t)((int64_t)(p.k - 1) * p.lda + (p.m - it.m0));

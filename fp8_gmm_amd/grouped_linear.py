@@ -24,7 +24,8 @@ import math
 import numpy as np
 import torch
 
-from .backend import TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize
+from .backend import (TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize,
+                      wgrad_wants_transposed_gradient)
 from .fp8 import Fp8GroupedModuleBase, Fp8WeightCache, get_fp8_te_dtype
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
@@ -200,7 +201,18 @@ class _GroupedLinear(torch.autograd.Function):
         g_scale_invs = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScaleInv)
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
         g_t_views = None
-        if ctx.weight_requires_grad and ctx.reference_layout:
+        # on request (backend.wgrad_wants_transposed_gradient) the weight gradient runs on a transposed copy of the
+        # gradient; the activation is still read where it lies
+        grad_copy = ctx.weight_requires_grad and not ctx.reference_layout and \
+            wgrad_wants_transposed_gradient(cumsums[-1], ctx.num_groups)
+        if grad_copy:
+            _, copy_padded, _, copy_bounds = cumsum_group_sizes(
+                np.diff(np.asarray(cumsums)).tolist(), need_padding=True,
+                pad_multiple=ctx.fp8_meta.get("pad_multiple", PAD_MULTIPLE))
+            _, g_t_views = alloc_transposed(grad_out.size(1), copy_padded, cumsums, copy_bounds, grad_dtype, dev)
+            multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
+                                 g_scales, g_amaxes)
+        elif ctx.weight_requires_grad and ctx.reference_layout:
             _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
                                             dev)
             multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
@@ -223,6 +235,9 @@ class _GroupedLinear(torch.autograd.Function):
             if ctx.reference_layout:
                 x_t_views = transposed_views(input_for_wgrad, padded_cumsums if padded else cumsums)
                 grouped_gemm(g_t_views, x_t_views, TensorBatch.stack_of(grad_weight), g_scale_invs, x_scale_invs)
+            elif grad_copy:
+                grouped_gemm(g_t_views, row_slices(input_for_wgrad, cumsums), TensorBatch.stack_of(grad_weight),
+                             g_scale_invs, x_scale_invs, transposed="b")
             else:  # dW[i] = dY_i^T . X_i on the row-major slices, contraction over the expert's rows
                 grouped_gemm(row_slices(grad_out_fp8, cumsums), row_slices(input_for_wgrad, cumsums),
                              TensorBatch.stack_of(grad_weight), g_scale_invs, x_scale_invs, transposed=True)

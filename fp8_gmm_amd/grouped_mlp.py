@@ -35,6 +35,7 @@ from .backend import (
     multi_cast_transpose_dgelu,
     multi_quantize,
     multi_transpose,
+    wgrad_wants_transposed_gradient,
 )
 from .fp8 import Fp8GroupedModuleBase, Fp8WeightCache, get_fp8_te_dtype
 from .grouped_linear import MODULE_PAD_MULTIPLE, alloc_transposed, row_slices, stage_weight_cast, transposed_views
@@ -184,8 +185,20 @@ class _GroupedMlp(torch.autograd.Function):
         g1_scale_invs = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kScaleInv)
         grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
 
+        # In place, the weight-gradient GEMMs read both operands contraction-major.  On request
+        # (backend.wgrad_wants_transposed_gradient) the casts below also write a transposed copy of the gradient,
+        # zero-padded per expert, and only the activations are read in place.
+        grad_copy = wgrad and in_place and wgrad_wants_transposed_gradient(cumsums[-1], ctx.num_groups)
+        if grad_copy:
+            _, copy_padded, _, copy_bounds = cumsum_group_sizes(
+                np.diff(np.asarray(cumsums)).tolist(), need_padding=True,
+                pad_multiple=ctx.fp8_meta.get("pad_multiple", PAD_MULTIPLE))
         grad_fc2_weight = None
-        if wgrad and not in_place:
+        if grad_copy:
+            _, g_t_views = alloc_transposed(grad_out.size(1), copy_padded, cumsums, copy_bounds, grad_dtype, dev)
+            multi_cast_transpose(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_t_views,
+                                 g1_scales, g1_amaxes)
+        elif wgrad and not in_place:
             _, g_t_views = alloc_transposed(grad_out.size(1), padded, cumsums, padded_cumsums, grad_dtype, dev)
             _, gelu_t_views = alloc_transposed(gelu_out_fp8.size(1), padded, cumsums, padded_cumsums,
                                                gelu_out_fp8.dtype, dev)
@@ -198,7 +211,10 @@ class _GroupedMlp(torch.autograd.Function):
             # fc2 wgrad: dW2[i][H, F] = dY_i^T . gelu_i (reference layout: dY_i^T[H, Mpad] . gelu_i^T[F, Mpad]^T)
             grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev)
             gelu_scale_invs = meta.get_meta_pointers(_T.kForwardInputGroup2, _M.kScaleInv)
-            if in_place:
+            if grad_copy:
+                grouped_gemm(g_t_views, row_slices(gelu_out_fp8, cumsums), TensorBatch.stack_of(grad_fc2_weight),
+                             g1_scale_invs, gelu_scale_invs, transposed="b")
+            elif in_place:
                 grouped_gemm(row_slices(grad_out_fp8, cumsums), row_slices(gelu_out_fp8, cumsums),
                              TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs, gelu_scale_invs, transposed=True)
             else:
@@ -218,9 +234,13 @@ class _GroupedMlp(torch.autograd.Function):
         grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
         g2_scales = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale)
         g2_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax)
-        if wgrad and not in_place:
-            _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums, grad_dtype,
-                                                   dev)
+        if grad_copy or (wgrad and not in_place):
+            if grad_copy:
+                _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), copy_padded, cumsums, copy_bounds,
+                                                       grad_dtype, dev)
+            else:
+                _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), padded, cumsums, padded_cumsums,
+                                                       grad_dtype, dev)
             multi_cast_transpose_dgelu(
                 row_slices(grad_gelu_out, cumsums), row_slices(pre_gelu_out, cumsums),
                 row_slices(grad_pre_fp8, cumsums), grad_pre_t_views, g2_scales, g2_amaxes,
@@ -252,7 +272,10 @@ class _GroupedMlp(torch.autograd.Function):
             # fc1 wgrad: dW1[i][F, H] = d(pre)_i^T[F, Mpad] . X_i^T[H, Mpad]^T
             grad_fc1_weight = torch.empty(ctx.fc1_weight_shape, dtype=torch.bfloat16, device=dev)
             x_scale_invs = meta.get_meta_pointers(_T.kForwardInputGroup1, _M.kScaleInv)
-            if in_place:
+            if grad_copy:
+                grouped_gemm(grad_pre_t_views, row_slices(input_for_wgrad, cumsums),
+                             TensorBatch.stack_of(grad_fc1_weight), g2_scale_invs, x_scale_invs, transposed="b")
+            elif in_place:
                 grouped_gemm(row_slices(grad_pre_fp8, cumsums), row_slices(input_for_wgrad, cumsums),
                              TensorBatch.stack_of(grad_fc1_weight), g2_scale_invs, x_scale_invs, transposed=True)
             else:

@@ -139,7 +139,10 @@ typedef struct fp8gmm_gemm_problem {
  * c[m, n] = epilogue( a[m, k] . b[k, n] ).  This is a forward weight [N_fwd = k, K_fwd = n] as the data-gradient
  * GEMM needs it, read in place: the reference casts a transposed copy of every weight for that GEMM instead
  * (fp8_gmm/grouped_linear.py:69-74,163).  b must be e4m3, n a multiple of 16, (k + 128) * ldb < 2^32.  Plan such tables
- * with fp8gmm_plan_grouped_gemm_layout(..., FP8GMM_GEMM_B_KMAJOR, ...). */
+ * with fp8gmm_plan_grouped_gemm_layout(..., FP8GMM_GEMM_B_KMAJOR, ...).  k need not be a multiple of 16 in this
+ * layout: the rows of b past k read as zeros, so the columns k .. roundup(k, 16) - 1 of a (which must exist: lda is a
+ * multiple of 16) only have to hold finite values - zeros, when a is a padded transposed copy.  That is the
+ * weight-gradient GEMM with a transposed copy of the gradient and the activation read in place. */
 #define FP8GMM_GEMM_B_KMAJOR 2
 /* a is stored contraction-major as well: a[k, m] with m contiguous and lda >= m, i.e.
  * c[m, n] = epilogue( a[k, m]^T . b[k, n] ): the weight-gradient GEMM dW[N, K] = dY[M, N]^T . X[M, K] on the

@@ -732,3 +732,38 @@ def test_small_tile_gives_the_same_bits_as_the_large_tile(dev, a_dtype, monkeypa
     b2 = torch.randn(2, 100, 256, generator=g, device=dev).to(E4M3)   # n = 100: bf16 rows of 200 bytes
     big, small, _ = both(lambda: backend.fp8_gmm(a, b2, [150, 50], ones, ones, backward=a_dtype == E5M2))
     assert torch.equal(big.view(torch.int16), small.view(torch.int16))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tile", ["256", "128"])
+def test_weight_gradient_with_a_transposed_gradient_copy_gives_the_same_bits(dev, tile, monkeypatch):
+    """grouped_gemm(..., transposed="b"): a is a zero-padded transposed copy [m, kpad], b the activation slice
+    [k, n] read in place, k any number.  Must equal transposed=True (both operands in place) bit for bit - in
+    particular in the last row of every tile, whose final 16-byte piece of a ends past k: the load descriptor has to
+    cover the whole piece, or the dword that straddles k is dropped with its valid bytes."""
+    backend = _backend()
+    monkeypatch.setattr(backend, "_TILE", tile)
+    g = torch.Generator(device=dev).manual_seed(77)
+    for rows, m, n in [([669], 512, 256), ([137, 0, 401, 59, 403, 1], 512, 256), ([669, 909], 1408, 2048),
+                       ([1000, 17], 272, 1040)]:
+        total = sum(rows)
+        dy = torch.randn(total, m, generator=g, device=dev).to(E5M2)
+        x = torch.randn(total, n, generator=g, device=dev).to(E4M3)
+        bounds = [0]
+        for r in rows:
+            bounds.append(bounds[-1] + r)
+        a_km = [dy[bounds[i]: bounds[i + 1]] for i in range(len(rows))]
+        b_km = [x[bounds[i]: bounds[i + 1]] for i in range(len(rows))]
+        a_pad = []
+        for t in a_km:
+            r = t.shape[0]
+            buf = torch.zeros(m, (r + 127) // 128 * 128, device=dev).to(E5M2)
+            buf[:, :r] = t.t()
+            a_pad.append(buf)
+        sa = torch.rand(len(rows), generator=g, device=dev) + 0.5
+        sb = torch.rand(len(rows), generator=g, device=dev) + 0.5
+        want = torch.full((len(rows), m, n), float("nan"), dtype=torch.bfloat16, device=dev)
+        got = torch.full_like(want, float("nan"))
+        backend.grouped_gemm(a_km, b_km, list(want.unbind(0)), sa, sb, transposed=True)
+        backend.grouped_gemm(a_pad, b_km, list(got.unbind(0)), sa, sb, transposed="b")
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"rows {rows} m {m} n {n}"

@@ -421,3 +421,41 @@ def test_in_place_gradient_gemms_equal_the_reference_layout(dev, kind):
         for a, b in zip(*res):
             assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}"
         assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", ["linear", "mlp"])
+def test_weight_gradient_on_a_transposed_gradient_copy_gives_the_same_bits(dev, kind, monkeypatch):
+    """FP8GMM_WGRAD=copy: the modules cast a transposed, zero-padded copy of the gradient for the weight-gradient
+    GEMM and read only the activation in place; by default they read both operands in place.  Row counts that are
+    multiples of nothing, an empty expert: the same bits either way - outputs, all gradients, and the backward amax
+    history - over three steps of delayed scaling."""
+    pkg = _pkg()
+    from fp8_gmm_amd import backend
+
+    sizes, h, f = [137, 0, 401, 59, 403, 1], 256, 512
+    e, m = len(sizes), sum(sizes)
+    g = gen(3011)
+    mods = []
+    for _ in range(2):
+        mod = (pkg.GroupedLinear if kind == "linear" else pkg.GroupedMlp)(h, f, e, torch.bfloat16, device=dev)
+        mods.append(mod)
+    mods[1].load_state_dict(mods[0].state_dict())
+    out_cols = f if kind == "linear" else h
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=2)
+    assert not backend.wgrad_wants_transposed_gradient(m, e)   # the default
+    for step in range(3):
+        x = randn_bf16((m, h), g).to(dev)
+        dy = randn_bf16((m, out_cols), g, 1e-2).to(dev)
+        res = []
+        for mod, mode in zip(mods, ("in_place", "copy")):
+            monkeypatch.setattr(backend, "_WGRAD", mode)
+            xd = x.clone().requires_grad_()
+            mod.zero_grad()
+            with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
+                out = mod(xd, torch.tensor(sizes))
+            out.backward(dy)
+            res.append([out, xd.grad] + [p.grad for p in mod.parameters()])
+        for a, b in zip(*res):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}"
+        assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
