@@ -6,6 +6,7 @@ fallback: if the shared library is missing or does not export the expected
 symbols, importing the backend raises.
 """
 import ctypes
+import threading
 import os
 
 import numpy as np
@@ -253,33 +254,53 @@ def plan_grouped_gemm(table, layout=0):
     return total.value
 
 
-def plan_grouped_gemm_launch(table, layout, grid, stream_k):
-    """Validate a host problem table and write the work list of a launch with `grid` workgroups.
-    Returns (GemmPlan, items, fixups): numpy arrays of GEMM_ITEM [rounds * grid] and GEMM_FIXUP [n_fixups]."""
+_plan_scratch = threading.local()   # grow-only output buffers of the launch planner, one set per thread
+
+
+def _plan_into_scratch(table, layout, grid, stream_k):
+    """Plan a launch into this thread's scratch buffers; returns (GemmPlan, items view, fixups view).  The views
+    are overwritten by the thread's next call."""
     L = load()
     plan = GemmPlan()
-    n = len(table)
-    # first guess: striding needs ceil(tiles / grid) records per workgroup, tail sharing a few more
-    tiles = max(1, _tiles_upper_bound(table)) * (4 if layout & GEMM_TILE_128 else 1)
-    guess = (int(np.ceil(tiles / grid)) + 6) * grid
-    items = np.empty(guess, dtype=GEMM_ITEM)
-    fixups = np.empty(grid, dtype=GEMM_FIXUP)
-    rc = L.fp8gmm_plan_grouped_gemm_launch(table.ctypes.data, n, layout, grid, int(bool(stream_k)), items.ctypes.data,
-                                           len(items), fixups.ctypes.data, len(fixups), ctypes.byref(plan))
+    sc = _plan_scratch
+    items = getattr(sc, "items", None)
+    if items is None:
+        items = sc.items = np.empty(8192, dtype=GEMM_ITEM)
+        sc.fixups = np.empty(1024, dtype=GEMM_FIXUP)
+    fixups = sc.fixups
+    args = (table.ctypes.data, len(table), layout, grid, int(bool(stream_k)))
+    rc = L.fp8gmm_plan_grouped_gemm_launch(*args, items.ctypes.data, len(items), fixups.ctypes.data, len(fixups),
+                                           ctypes.byref(plan))
     if rc == -8:  # FP8GMM_ERR_BUFFER_TOO_SMALL: the sizes are in the plan
-        items = np.empty(plan.rounds * plan.grid, dtype=GEMM_ITEM)
-        fixups = np.empty(max(1, plan.n_fixups), dtype=GEMM_FIXUP)
-        rc = L.fp8gmm_plan_grouped_gemm_launch(table.ctypes.data, n, layout, grid, int(bool(stream_k)),
-                                               items.ctypes.data, len(items), fixups.ctypes.data, len(fixups),
+        if plan.rounds * plan.grid > len(items):
+            items = sc.items = np.empty(2 * plan.rounds * plan.grid, dtype=GEMM_ITEM)
+        if plan.n_fixups > len(fixups):
+            fixups = sc.fixups = np.empty(2 * plan.n_fixups, dtype=GEMM_FIXUP)
+        rc = L.fp8gmm_plan_grouped_gemm_launch(*args, items.ctypes.data, len(items), fixups.ctypes.data, len(fixups),
                                                ctypes.byref(plan))
     check(rc)
     return plan, items[: plan.rounds * plan.grid], fixups[: plan.n_fixups]
 
 
-def _tiles_upper_bound(table):
-    m = table["m"].astype(np.int64)
-    n = table["n"].astype(np.int64)
-    return int((((m + 255) // 256) * ((n + 255) // 256)).clip(min=0).sum())
+def plan_grouped_gemm_launch(table, layout, grid, stream_k):
+    """Validate a host problem table and write the work list of a launch with `grid` workgroups.
+    Returns (GemmPlan, items, fixups): numpy arrays of GEMM_ITEM [rounds * grid] and GEMM_FIXUP [n_fixups]."""
+    plan, items, fixups = _plan_into_scratch(table, layout, grid, stream_k)
+    return plan, items.copy(), fixups.copy()
+
+
+def plan_grouped_gemm_blob(table, layout, grid, stream_k):
+    """The same, as the bytes a launch uploads: [problem table | work list | shared tiles], each part on its own
+    cache lines.  Returns (GemmPlan, blob, offset of the work list, offset of the shared-tile records)."""
+    plan, items, fixups = _plan_into_scratch(table, layout, grid, stream_k)
+    off_items = (table.nbytes + 127) // 128 * 128
+    off_fix = off_items + items.nbytes
+    blob = np.empty(off_fix + fixups.nbytes, dtype=np.uint8)
+    blob[: table.nbytes] = table.view(np.uint8).reshape(-1)
+    blob[table.nbytes: off_items] = 0
+    blob[off_items: off_fix] = items.view(np.uint8).reshape(-1)
+    blob[off_fix:] = fixups.view(np.uint8).reshape(-1)
+    return plan, blob, off_items, off_fix
 
 
 _num_cu = {}

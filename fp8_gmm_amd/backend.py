@@ -31,6 +31,24 @@ def _fail(msg):
     raise RuntimeError(msg)
 
 
+class _on_device:
+    """``torch.cuda.device(device)``, entered only when `device` is not the current one already (every launch sits
+    in such a block, and the context manager costs the host several microseconds)."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, device):
+        current = device.index is None or torch.cuda.current_device() == device.index
+        self.guard = None if current else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        return self.guard.__exit__(*exc) if self.guard is not None else False
+
+
 class kernel_timing:
     """Context manager that brackets every kernel launch of this module with HIP events.
 
@@ -206,7 +224,13 @@ def _flush(items):
             launch(base + off)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device):
+    """The HIP stream handle of torch's current stream on `device`."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -244,7 +268,7 @@ def _launch_multi(op, table, out_fmt, device, keep):
     n = len(table)
 
     def launch(dev_ptr):
-        with torch.cuda.device(device), _timed(_OP_NAMES[op], lambda: _algorithmic_bytes(op, table)):
+        with _on_device(device), _timed(_OP_NAMES[op], lambda: _algorithmic_bytes(op, table)):
             s = _stream(device)
             if op == _lib.OP_QUANTIZE:
                 rc = L.fp8gmm_multi_quantize(dev_ptr, n, total, out_fmt, s)
@@ -263,6 +287,16 @@ def _launch_multi(op, table, out_fmt, device, keep):
     _submit(table, device, launch, keep)
 
 
+def _int64_vector(x, n):
+    """x as n int64 values: an array of that shape as it is, a scalar repeated."""
+    if isinstance(x, np.ndarray):
+        if x.dtype == np.int64 and x.shape == (n,):
+            return x
+    elif isinstance(x, int):
+        return np.full(n, x, dtype=np.int64)
+    return np.broadcast_to(np.asarray(x, dtype=np.int64), (n,))
+
+
 class TensorBatch:
     """n row-major 2-D tensors of one dtype on one device, held as arrays (address, rows, columns, row
     pitch in elements) instead of n tensor objects.
@@ -278,9 +312,9 @@ class TensorBatch:
     def __init__(self, ptr, rows, cols, pitch, dtype, device, keep=()):
         n = len(ptr)
         self.ptr = np.asarray(ptr, dtype=np.uint64)
-        self.rows = np.broadcast_to(np.asarray(rows, dtype=np.int64), (n,))
-        self.cols = np.broadcast_to(np.asarray(cols, dtype=np.int64), (n,))
-        self.pitch = np.broadcast_to(np.asarray(pitch, dtype=np.int64), (n,))
+        self.rows = _int64_vector(rows, n)
+        self.cols = _int64_vector(cols, n)
+        self.pitch = _int64_vector(pitch, n)
         self.dtype = dtype
         self.device = device
         self._keep = tuple(keep)  # the tensors whose memory is described stay alive with the batch
@@ -583,24 +617,17 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
     layout = (_lib.GEMM_B_KMAJOR if b_kmajor else 0) | (_lib.GEMM_A_KMAJOR if a_kmajor else 0)
     grid = _lib.gemm_grid(_lib.init(device.index if device.index is not None else torch.cuda.current_device()))
     if not gelu and _small_tiles(table):
-        plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
+        plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
     else:
-        plan, items, fixups = _lib.plan_grouped_gemm_launch(table, layout | (_lib.EPI_GELU if gelu else 0), grid,
-                                                            _STREAM_K)
+        plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | (_lib.EPI_GELU if gelu else 0),
+                                                                     grid, _STREAM_K)
     if plan.total_tiles == 0:
         return
     n = len(table)
     fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], (_lib.EPI_GELU if gelu else 0) | layout)
-    # one upload: [problems | work list | shared tiles], each part on its own cache lines
-    off_items = (table.nbytes + 127) // 128 * 128
-    off_fix = off_items + items.nbytes
-    blob = np.zeros(off_fix + fixups.nbytes, dtype=np.uint8)
-    blob[: table.nbytes] = table.view(np.uint8).reshape(-1)
-    blob[off_items: off_fix] = items.view(np.uint8).reshape(-1)
-    blob[off_fix:] = fixups.view(np.uint8).reshape(-1)
 
     def launch(dev_ptr):
-        with torch.cuda.device(device):
+        with _on_device(device):
             ws = _gemm_workspace(device, plan.n_slots)
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
             probe = _clock_probe.get("counters")
@@ -662,7 +689,7 @@ _workspaces = {}
 def _gemm_workspace(device, n_slots):
     if n_slots == 0:
         return None
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    key = (device, _stream(device))
     ws = _workspaces.get(key)
     need = n_slots * _lib.GEMM_SLOT_BYTES
     if ws is None or ws.numel() < need:
@@ -677,7 +704,7 @@ def warm_up(device=None):
     that none of it falls into a timed or captured region."""
     device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     grid = _lib.gemm_grid(_lib.init(device.index))
-    with torch.cuda.device(device):
+    with _on_device(device):
         _gemm_workspace(device, 2 * grid)
 
 
@@ -706,7 +733,7 @@ def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, mo
     if amax_history.dim() != 2 or scale.numel() != amax_history.shape[1] or scale_inv.numel() != scale.numel():
         _fail("fp8_gmm_amd: amax_history must be [history, slots] and scale / scale_inv [slots]")
     dev = _device_of([amax_history, scale, scale_inv])
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _lib.load().fp8gmm_delayed_scaling_update(
             amax_history.data_ptr(), scale.data_ptr(), scale_inv.data_ptr(), amax_history.shape[0],
             amax_history.shape[1], float(fp8_max), int(margin), int(bool(most_recent)), int(period), int(phase),

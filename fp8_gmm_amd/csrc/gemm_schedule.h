@@ -195,11 +195,18 @@ FP8GMM_HD void cursor_init(const Sched& s, int j, Cursor& c) {
 FP8GMM_HD bool cursor_valid(const Sched& s, int j, const Cursor& c) {
   return (c.dp_i < s.dp_rounds && dp_tile(s, j, c.dp_i) < s.sk_begin) || c.sk_tile >= 0;
 }
-FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c) {
+// `prob_hint`: a problem at or before the one that holds the cursor's tile (a workgroup's tiles come in
+// increasing order, so the previous item's problem will do); negative: search the whole table.
+FP8GMM_HD Item cursor_item(const Sched& s, int xcd, int j, const Cursor& c, int prob_hint = -1) {
   const bool dp = c.dp_i < s.dp_rounds && dp_tile(s, j, c.dp_i) < s.sk_begin;
   Item it;
   it.tile = dp ? dp_tile(s, j, c.dp_i) : c.sk_tile;
-  it.prob = problem_of_tile(s, it.tile);
+  if (prob_hint < 0) {
+    it.prob = problem_of_tile(s, it.tile);
+  } else {
+    it.prob = prob_hint;
+    while (it.prob + 1 < s.nprob && s.probs[it.prob + 1].tile_begin <= it.tile) ++it.prob;
+  }
   tile_origin(s.probs[it.prob].m, s.probs[it.prob].n, it.tile - s.probs[it.prob].tile_begin, &it.m0, &it.n0);
   const int real_nk = (s.probs[it.prob].k + 127) / 128;  // a K tail is zero-filled
   it.k_begin = 0;

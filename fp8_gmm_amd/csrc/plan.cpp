@@ -338,14 +338,89 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
         for (int q = j; q < j + nf; ++q) slot_map[kSlotsPerWg * (x * wgs + q)] = n_slots++;
         fix.push_back(o);
       }
+  const int room = max_items;   // as the caller stated it
+  // One pass over the schedule: the records are written as they are counted, into whatever room the caller gave;
+  // a list that does not fit is only counted, and the call then reports the sizes.
+  if (items == nullptr) max_items = 0;
+  std::vector<int32_t> count(grid, 0);
   int rounds = 0;
+  bool dangling_piece = false;
+  auto write_record = [&](const Item& it, size_t index) {
+    const fp8gmm_gemm_problem& p = probs[it.prob];
+    fp8gmm_gemm_item& o = items[index];
+    o = fp8gmm_gemm_item{};
+    const int64_t rows = p.m - it.m0 < BM ? p.m - it.m0 : BM;
+    const int64_t cols = p.n - it.n0 < BN ? p.n - it.n0 : BN;
+    if (p.k > 0) {
+      // extents: up to the last byte of the tile's last row (row-major) / of the operand's last contraction row.
+      // A row-major a whose k is not a multiple of 16 (allowed next to a contraction-major b) ends inside a
+      // 16-byte piece; the bound includes the whole piece, which lies inside the row's pitch: the hardware
+      // checks the range per dword, and a dword that straddled the bound would lose its valid bytes too.
+      if (!a_kmajor) {
+        o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0 * (uint64_t)p.lda;
+        o.a_bytes = (uint32_t)((rows - 1) * p.lda + ((p.k + 15) & ~15));
+      } else {
+        o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0;
+        o.a_bytes = (uint32_t)((int64_t)(p.k - 1) * p.lda + (p.m - it.m0));
+      }
+      if (!b_kmajor) {
+        o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0 * (uint64_t)p.ldb;
+        o.b_bytes = (uint32_t)((cols - 1) * p.ldb + p.k);
+      } else {
+        o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0;
+        o.b_bytes = (uint32_t)((int64_t)(p.k - 1) * p.ldb + (p.n - it.n0));
+      }
+    }
+    o.lda = p.lda;
+    o.ldb = p.ldb;
+    o.k = p.k;
+    o.k_begin = it.k_begin;
+    o.nk = it.nk;
+    o.m0 = it.m0;
+    o.n0 = it.n0;
+    o.prob = it.prob;
+    o.slot = -1;
+    if (it.slot >= 0) {
+      o.slot = slot_map[it.slot];
+      if (o.slot < 0) dangling_piece = true;  // a partial item that no fix-up record completes
+    }
+  };
   for (int wg = 0; wg < grid; ++wg) {
     const int x = wg % kNumXcd, j = wg / kNumXcd;
+    const Sched& sx = sched[x];
     Cursor c;
-    cursor_init(sched[x], j, c);
-    int count = 0;
-    for (; cursor_valid(sched[x], j, c); cursor_advance(sched[x], j, c)) ++count;
-    if (count > rounds) rounds = count;
+    cursor_init(sx, j, c);
+    int r = 0, prob = 0;
+    // The strided part, which holds nearly all records, without the cursor's repeated index arithmetic: the same
+    // tiles in the same order as cursor_valid / cursor_item / cursor_advance give (dp_tile's position in the
+    // round advances by kRoundRotation, modulo the workgroups of the XCD).
+    for (int pos = j % sx.wgs; c.dp_i < sx.dp_rounds; ++c.dp_i, ++r) {
+      const int tile = sx.range_begin + sx.wgs * c.dp_i + pos;
+      if (tile >= sx.sk_begin) break;
+      pos += kRoundRotation % sx.wgs;
+      if (pos >= sx.wgs) pos -= sx.wgs;
+      const size_t index = (size_t)r * grid + wg;
+      if (index >= (size_t)max_items) continue;
+      while (prob + 1 < n && probs[prob + 1].tile_begin <= tile) ++prob;
+      Item it;
+      it.tile = tile;
+      it.prob = prob;
+      tile_origin(probs[prob].m, probs[prob].n, tile - probs[prob].tile_begin, &it.m0, &it.n0);
+      it.k_begin = 0;
+      it.nk = (probs[prob].k + 127) / 128;
+      it.slot = -1;
+      write_record(it, index);
+    }
+    // what is left: the pieces of the shared remainder
+    for (; cursor_valid(sx, j, c); cursor_advance(sx, j, c), ++r) {
+      const size_t index = (size_t)r * grid + wg;
+      if (index >= (size_t)max_items) continue;
+      const Item it = cursor_item(sx, x, j, c, prob);
+      prob = it.prob;
+      write_record(it, index);
+    }
+    count[wg] = r;
+    if (r > rounds) rounds = r;
   }
   rounds += 1;  // every list ends with a record whose prob is -1
   const int n_fixups = (int)fix.size();
@@ -354,62 +429,15 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   plan->n_fixups = n_fixups;
   plan->n_slots = n_slots;
   if ((int64_t)rounds * grid > INT32_MAX / 64) return FP8GMM_ERR_BAD_SHAPE;
-  if ((int64_t)rounds * grid > max_items || n_fixups > max_fixups) return FP8GMM_ERR_BUFFER_TOO_SMALL;
+  if ((int64_t)rounds * grid > room || n_fixups > max_fixups) return FP8GMM_ERR_BUFFER_TOO_SMALL;
   if (items == nullptr || (n_fixups > 0 && fixups == nullptr)) return FP8GMM_ERR_NULL_POINTER;
-
-  // pass 2: records
+  if (dangling_piece) return FP8GMM_ERR_BAD_ARGUMENT;
   for (int f = 0; f < n_fixups; ++f) fixups[f] = fix[f];
   fp8gmm_gemm_item end_record{};
   end_record.prob = -1;
   end_record.slot = -1;
-  for (int i = 0; i < rounds * grid; ++i) items[i] = end_record;
-  for (int wg = 0; wg < grid; ++wg) {
-    const int x = wg % kNumXcd, j = wg / kNumXcd;
-    Cursor c;
-    cursor_init(sched[x], j, c);
-    int r = 0;
-    for (; cursor_valid(sched[x], j, c); cursor_advance(sched[x], j, c), ++r) {
-      const Item it = cursor_item(sched[x], x, j, c);
-      const fp8gmm_gemm_problem& p = probs[it.prob];
-      fp8gmm_gemm_item& o = items[(size_t)r * grid + wg];
-      o = fp8gmm_gemm_item{};
-      const int64_t rows = p.m - it.m0 < BM ? p.m - it.m0 : BM;
-      const int64_t cols = p.n - it.n0 < BN ? p.n - it.n0 : BN;
-      if (p.k > 0) {
-        // extents: up to the last byte of the tile's last row (row-major) / of the operand's last contraction row.
-        // A row-major a whose k is not a multiple of 16 (allowed next to a contraction-major b) ends inside a
-        // 16-byte piece; the bound includes the whole piece, which lies inside the row's pitch: the hardware
-        // checks the range per dword, and a dword that straddled the bound would lose its valid bytes too.
-        if (!a_kmajor) {
-          o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0 * (uint64_t)p.lda;
-          o.a_bytes = (uint32_t)((rows - 1) * p.lda + ((p.k + 15) & ~15));
-        } else {
-          o.a = (uint64_t)reinterpret_cast<uintptr_t>(p.a) + (uint64_t)it.m0;
-          o.a_bytes = (uint32_t)((int64_t)(p.k - 1) * p.lda + (p.m - it.m0));
-        }
-        if (!b_kmajor) {
-          o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0 * (uint64_t)p.ldb;
-          o.b_bytes = (uint32_t)((cols - 1) * p.ldb + p.k);
-        } else {
-          o.b = (uint64_t)reinterpret_cast<uintptr_t>(p.b) + (uint64_t)it.n0;
-          o.b_bytes = (uint32_t)((int64_t)(p.k - 1) * p.ldb + (p.n - it.n0));
-        }
-      }
-      o.lda = p.lda;
-      o.ldb = p.ldb;
-      o.k = p.k;
-      o.k_begin = it.k_begin;
-      o.nk = it.nk;
-      o.m0 = it.m0;
-      o.n0 = it.n0;
-      o.prob = it.prob;
-      o.slot = -1;
-      if (it.slot >= 0) {
-        o.slot = slot_map[it.slot];
-        if (o.slot < 0) return FP8GMM_ERR_BAD_ARGUMENT;  // a partial item that no fix-up record completes
-      }
-    }
-  }
+  for (int wg = 0; wg < grid; ++wg)
+    for (int r = count[wg]; r < rounds; ++r) items[(size_t)r * grid + wg] = end_record;
   return FP8GMM_OK;
 }
 

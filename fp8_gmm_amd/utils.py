@@ -105,6 +105,7 @@ class Fp8MetaWrapper:
         self._num_groups = num_groups
         self._fp8_meta = fp8_meta
         self._forward_scale_inv_cloned = None
+        self._slot_offsets = {}
 
     def num_groups(self):
         return self._num_groups
@@ -114,15 +115,16 @@ class Fp8MetaWrapper:
 
     def _select(self, fp8_tensor_type, meta_tensor_type):
         """(flat tensor, first index, stride) of the E slots of this tensor type."""
-        fp8_tensor_type = Fp8TensorType(fp8_tensor_type)
-        name = fp8_tensor_type.name
-        if fp8_tensor_type >= Fp8TensorType.kForwardInputGroup1:
+        rule = _SLOT_RULES.get(int(fp8_tensor_type))
+        if rule is None:
+            raise ValueError(f"{fp8_tensor_type} is not a valid Fp8TensorType")
+        forward_copy, backward, stride, second_group, weight = rule
+        if forward_copy:
             assert meta_tensor_type == MetaTensorType.kScaleInv
             assert self._forward_scale_inv_cloned is not None, "forward scale_inv has not been cloned yet"
             flat = self._forward_scale_inv_cloned
         else:
-            key = "scaling_bwd" if fp8_tensor_type >= Fp8TensorType.kGradOutputGroup1 else "scaling_fwd"
-            meta = self._fp8_meta[key]
+            meta = self._fp8_meta["scaling_bwd" if backward else "scaling_fwd"]
             if meta_tensor_type == MetaTensorType.kScale:
                 flat = meta.scale
             elif meta_tensor_type == MetaTensorType.kScaleInv:
@@ -131,8 +133,7 @@ class Fp8MetaWrapper:
                 flat = meta.amax_history[0]
             else:
                 raise ValueError(f"unknown meta tensor type {meta_tensor_type}")
-        stride = self._BACKWARD_OFFSET if "GradOutput" in name else self._FORWARD_OFFSET
-        first = (0 if "Group1" in name else self._num_groups) * stride + (1 if "Weight" in name else 0)
+        first = (self._num_groups if second_group else 0) * stride + weight
         return flat, first, stride
 
     def get_meta_tensors(self, fp8_tensor_type, meta_tensor_type):
@@ -144,5 +145,20 @@ class Fp8MetaWrapper:
         """Device addresses of the same E slots as a uint64 array, without creating E tensor views
         (every backend entry point takes such an array wherever it takes a list of scalars)."""
         flat, first, stride = self._select(fp8_tensor_type, meta_tensor_type)
-        base = flat.data_ptr() + first * flat.element_size()
-        return np.uint64(base) + np.arange(self._num_groups, dtype=np.uint64) * np.uint64(stride * flat.element_size())
+        offsets = self._slot_offsets.get(stride)
+        if offsets is None:
+            offsets = self._slot_offsets[stride] = np.arange(self._num_groups, dtype=np.uint64) * np.uint64(stride * 4)
+        if flat.dim() != 1 or flat.dtype != torch.float32:
+            raise RuntimeError("fp8 meta tensors must be flat fp32 tensors")
+        return np.uint64(flat.data_ptr() + first * 4) + offsets
+
+
+def _slot_rule(t):
+    name = t.name
+    return (t >= Fp8TensorType.kForwardInputGroup1,                  # reads the copy of the forward scale_inv
+            Fp8TensorType.kGradOutputGroup1 <= t < Fp8TensorType.kForwardInputGroup1,   # lives in scaling_bwd
+            Fp8MetaWrapper._BACKWARD_OFFSET if "GradOutput" in name else Fp8MetaWrapper._FORWARD_OFFSET,
+            "Group1" not in name, 1 if "Weight" in name else 0)
+
+
+_SLOT_RULES = {int(t): _slot_rule(t) for t in Fp8TensorType}
