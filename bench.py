@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling|small_tile]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling|lds_rate|small_tile]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -376,6 +376,59 @@ def bench_hbm_ceiling(args):
     }))
 
 
+def bench_lds_rate(args):
+    """lds_rate: how fast one compute unit's LDS serves the fragment reads of the grouped GEMM, measured in isolation
+    (fp8_gmm_amd/csrc/lds_probe.hip): plain 16-byte reads (row-major operands), plain 8-byte reads and transposing
+    8-byte reads (contraction-major operands), 1, 2 and 4 wavefronts per compute unit.  The step arithmetic that
+    follows in `gemm_step` prices one K = 128 step of the 256 x 256 tile (32 MFMAs of 64 cycles per SIMD = 2048
+    cycles) in LDS instruction slots."""
+    import ctypes
+
+    path = os.path.join(ROOT, "fp8_gmm_amd", "libfp8gmm_probe.so")
+    if not os.path.exists(path):
+        sys.exit("bench.py: fp8_gmm_amd/libfp8gmm_probe.so is not built (make -C fp8_gmm_amd/csrc)")
+    probe = ctypes.CDLL(path).fp8gmm_probe_lds
+    probe.restype = ctypes.c_int
+    probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
+                      ctypes.c_void_p]
+    dev = torch.device("cuda:0")
+    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.zeros(blocks * 256, dtype=torch.int32, device=dev)
+    cycles = torch.zeros(blocks, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    iters = 10000
+    names = {0: ("ds_read_b128", 1024), 1: ("ds_read_b64", 512), 2: ("ds_read_b64_tr_b8", 512)}
+    rows = []
+    for waves in (1, 2, 4):
+        for mode, (name, nbytes) in names.items():
+            best = None
+            for _ in range(max(2, args.warmup)):
+                rc = probe(mode, waves, iters, sink.data_ptr(), cycles.data_ptr(), blocks, stream)
+                assert rc == 0, f"probe launch failed: {rc}"
+                torch.cuda.synchronize()
+                c = float(cycles.double().mean().item()) / (iters * 16)
+                best = c if best is None else min(best, c)
+            rows.append({"instruction": name, "wavefronts": waves, "cycles_per_instruction_and_wavefront": round(best, 2),
+                         "cycles_per_instruction_of_the_unit": round(best / waves, 2),
+                         "bytes_per_clock_and_unit": round(nbytes * waves / best, 1)})
+            print(f"# {rows[-1]}", file=sys.stderr, flush=True)
+    at4 = {r["instruction"]: r for r in rows if r["wavefronts"] == 4}
+    b128, tr = at4["ds_read_b128"]["cycles_per_instruction_of_the_unit"], at4["ds_read_b64_tr_b8"]["cycles_per_instruction_of_the_unit"]
+    # one K = 128 step: every wavefront reads 16 KiB of each operand (16 ds_read_b128 or 32 transposing reads)
+    step = {"mfma_cycles": 2048,
+            "read_cycles_both_row_major": round(4 * 32 * b128), "read_cycles_one_contraction_major": round(4 * (16 * b128 + 32 * tr)),
+            "read_cycles_both_contraction_major": round(4 * 64 * tr)}
+    peak = at4["ds_read_b128"]["bytes_per_clock_and_unit"]
+    print(json.dumps({
+        "metric": "LDS read rate of one compute unit, bytes per clock, ds_read_b128 with 4 wavefronts",
+        "value": peak, "unit": "B/clk/CU", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "lds_rate: 16 independent reads per wait, the GEMM's fragment address patterns, one "
+                               "workgroup per compute unit"},
+        "reads": rows, "gemm_step": step, "roofline": None, "cpu_baseline": None,
+    }))
+
+
 def bench_small_tile(args):
     """small_tile: grouped GEMMs that do not fill the machine with full 256 x 256 tiles - few tiles, or problems
     of up to 128 rows - through both tile sizes (FP8GMM_GEMM_TILE_128 against the default), with the choice the
@@ -474,7 +527,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling", "small_tile"])
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling", "lds_rate", "small_tile"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
@@ -491,6 +544,8 @@ def main():
         return bench_cast_pad(args)
     if args.workload == "hbm_ceiling":
         return bench_hbm_ceiling(args)
+    if args.workload == "lds_rate":
+        return bench_lds_rate(args)
     if args.workload == "small_tile":
         return bench_small_tile(args)
 
