@@ -265,8 +265,8 @@ int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_bloc
  * FP8GMM_EPI_GELU, which only weighs the decision below (completing a shared tile costs more with that epilogue).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
  * the last round would otherwise be mostly idle; the launch then needs plan->n_slots workspace slots (never more
  * than 2 * grid).  stream_k == 0: every record is a whole tile, no workspace, no fix-up launch.
- * The sizes are returned in *plan even when max_items / max_fixups are too small (FP8GMM_ERR_BUFFER_TOO_SMALL,
- * nothing written to the arrays): call again with larger arrays.  Host only, no GPU needed.
+ * The sizes are returned in *plan even when max_items / max_fixups are too small (FP8GMM_ERR_BUFFER_TOO_SMALL;
+ * the arrays then hold the part of the list that fitted and are not to be used): call again with larger arrays.  Host only, no GPU needed.
  */
 int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layout, int grid, int stream_k,
                                     fp8gmm_gemm_item* items, int max_items, fp8gmm_gemm_fixup_desc* fixups,

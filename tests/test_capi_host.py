@@ -204,7 +204,7 @@ def test_gemm_grid_is_one_workgroup_per_compute_unit_in_multiples_of_eight():
 
 
 def test_launch_plan_reports_sizes_before_it_writes():
-    """Arrays too small: status -8, the required sizes in the plan, nothing written; then the same call with room."""
+    """Arrays too small: status -8 and the required sizes in the plan; then the same call with room."""
     lib = _lib.load()
     t = _prob([1000, 300], [512, 512], [256, 256])
     plan = _lib.GemmPlan()
@@ -220,5 +220,20 @@ def test_launch_plan_reports_sizes_before_it_writes():
     # a launch never has more workgroups than tiles (rounded up to a multiple of 8) when nothing is shared along K
     p3, it3, _ = _lib.plan_grouped_gemm_launch(_prob([100], [100], [128]), 0, 256, False)
     assert (p3.grid, p3.rounds, p3.total_tiles) == (8, 2, 1) and (it3["prob"] >= 0).sum() == 1
+    # room for part of the list only: the same status and sizes; with exactly the room asked for, the same records
+    # as with room to spare
+    some = np.zeros(20, dtype=_lib.GEMM_ITEM)
+    rc = lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, some.ctypes.data, 20, None, 0,
+                                             ctypes.byref(plan))
+    assert rc == -8 and (plan.grid, plan.rounds) == (16, 2)
+    exact = np.zeros(32, dtype=_lib.GEMM_ITEM)
+    rc = lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, exact.ctypes.data, 32, None, 0,
+                                             ctypes.byref(plan))
+    assert rc == 0 and exact.tobytes() == it.tobytes()
+    # the form the launches upload: [problem table | work list | shared tiles]
+    p4, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(t, 0, 16, False)
+    assert (p4.grid, p4.rounds) == (16, 2) and off_items % 128 == 0 and off_fix == off_items + it.nbytes
+    assert blob[: t.nbytes].tobytes() == t.tobytes() and blob[off_items: off_fix].tobytes() == it.tobytes()
+    assert len(blob) == off_fix
     assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 12, 0, None, 0, None, 0, ctypes.byref(plan)) == -6
     assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, None, 0, None, 0, None) == -1
