@@ -519,6 +519,19 @@ def dense_gemm_comparison(dev, m, n, k, reps=100):
     out["this_kernel_tflops"] = round(flops / min(mine) / 1e12, 1)
     if vendor:
         out["torch_scaled_mm_tflops"] = round(flops / min(vendor) / 1e12, 1)
+    # The same launches on operands that toggle no bits: the board is at its power cap on random data, and what
+    # the kernels gain here is what the cap costs them there.
+    a.view(torch.uint8).zero_()
+    b.view(torch.uint8).zero_()
+    out["all_zero_operands"] = {"this_kernel_tflops": round(
+        flops / timed(lambda: backend.fp8_gmm(a, b.view(1, n, k), sizes, one, one, c)) / 1e12, 1)}
+    if vendor:
+        try:
+            out["all_zero_operands"]["torch_scaled_mm_tflops"] = round(flops / timed(
+                lambda: torch._scaled_mm(a, b.t(), scale_a=one[0], scale_b=one[0], out_dtype=torch.bfloat16,
+                                         out=c)) / 1e12, 1)
+        except Exception as exc:
+            out["vendor_error"] = repr(exc)[:200]
     return out
 
 
