@@ -648,8 +648,8 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
 # Weight-gradient GEMMs contract over an expert's rows, the contiguous index of neither operand.  Both can be read
 # in place (contraction-major), or the gradient can be cast with a transposed, zero-padded copy, as the reference
 # does, and only the activation read in place (grouped_gemm(..., transposed="b")).  A contraction-major operand takes
-# twice the LDS read instructions; on isolated back-to-back launches of config 2's shapes the copy form is 9 - 11 %
-# faster (868 -> 773 us, 855 -> 779 us), inside the step the two weight gradients gain 40 us together and the two casts
+# twice the LDS read instructions; on isolated back-to-back launches of config 2's shapes the copy form is 7 - 15 %
+# faster (900 -> 765 us, 855 -> 795 us), inside the step the two weight gradients gain 40 us together and the two casts
 # that write the copies lose 64 (config 2: 5.79 ms against 5.76 in place; config 4: 1.76 against 1.69).  So the
 # modules read both operands in place; FP8GMM_WGRAD=copy selects the other form.  Same bits either way.
 _WGRAD = os.environ.get("FP8GMM_WGRAD", "in_place")
@@ -758,7 +758,7 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
     ``transposed="b"``: only b is contraction-major, ``a_list[i][m, kpad]`` (a zero-padded transposed copy, kpad >= k a
     multiple of 16) and ``b_list[i][k, n]``, ``c = a[:, :k] . b``: the weight gradient with the reference's transposed
     copy of the gradient and the activation read in place.  A contraction-major operand takes twice the LDS read
-    instructions of a row-major one; as isolated launches with long contractions this form is 9 - 11 % faster than
+    instructions of a row-major one; as isolated launches with long contractions this form is 7 - 15 % faster than
     ``transposed=True``; same bits.
     """
     n = len(a_list)
