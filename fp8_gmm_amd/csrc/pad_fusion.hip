@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(fp8gmm_tensor_des
     if constexpr (OP == OP_TRANSPOSE) {
       u32x2 v[RPT];
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) v[i] = buf_load8(rin, eoff[i]);
+      for (int i = 0; i < RPT; ++i) v[i] = buf_load8_stream(rin, eoff[i]);
 #pragma unroll
       for (int i = 0; i < RPT; ++i) {
         y[i][0] = v[i].x;
@@ -121,11 +121,11 @@ __global__ __launch_bounds__(kPtThreads) void multi_pad_kernel(fp8gmm_tensor_des
       u32x4 xa[RPT];
       u32x4 ga[OP == OP_CAST_DGELU ? RPT : 1];
 #pragma unroll
-      for (int i = 0; i < RPT; ++i) xa[i] = buf_load16(rin, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
+      for (int i = 0; i < RPT; ++i) xa[i] = buf_load16_stream(rin, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
       if constexpr (OP == OP_CAST_DGELU) {
         const __amdgpu_buffer_rsrc_t rpre = make_rsrc(d.in2, in_bytes);
 #pragma unroll
-        for (int i = 0; i < RPT; ++i) ga[i] = buf_load16(rpre, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
+        for (int i = 0; i < RPT; ++i) ga[i] = buf_load16_stream(rpre, eoff[i] == kOobOffset ? kOobOffset : eoff[i] * 2);
       }
       const __amdgpu_buffer_rsrc_t rout = make_rsrc(out, out != nullptr ? in_bytes / 2 : 0u);
 #pragma unroll

@@ -49,8 +49,8 @@ __global__ __launch_bounds__(kPwThreads) void multi_quantize_kernel(fp8gmm_tenso
     for (int it = 0; it < kPwSteps; ++it) {
       const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
       full[it] = off + kPwVec <= numel;
-      a[it] = buf_load16(rin, full[it] ? (uint32_t)(off * 2) : kOobOffset);
-      if constexpr (DGELU) g[it] = buf_load16(rpre, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+      a[it] = buf_load16_stream(rin, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+      if constexpr (DGELU) g[it] = buf_load16_stream(rpre, full[it] ? (uint32_t)(off * 2) : kOobOffset);
     }
 #pragma unroll
     for (int it = 0; it < kPwSteps; ++it) {
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gm
     for (int it = 0; it < kPwSteps; ++it) {
       const int64_t off = base + (int64_t)(it * kPwThreads + threadIdx.x) * kPwVec;
       full[it] = off + kPwVec <= numel;
-      a[it] = buf_load16(rx, full[it] ? (uint32_t)(off * 2) : kOobOffset);
+      a[it] = buf_load16_stream(rx, full[it] ? (uint32_t)(off * 2) : kOobOffset);
     }
 #pragma unroll
     for (int it = 0; it < kPwSteps; ++it) {

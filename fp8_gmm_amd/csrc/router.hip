@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_gather_kernel(const uint16
     for (int c0 = 0; c0 < hidden; c0 += 64 * 8 * 4) {
       u32x4 v[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) v[u] = buf_load16(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+      for (int u = 0; u < 4; ++u) v[u] = buf_load16_stream(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         if (weights != nullptr) {
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_kernel(const uint1
         const __amdgpu_buffer_rsrc_t rs = make_rsrc(x + (size_t)(ok ? p : 0) * hidden, ok ? (uint32_t)hidden * 2u : 0u);
         u32x4 v[kU];
 #pragma unroll
-        for (int u = 0; u < kU; ++u) v[u] = buf_load16(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+        for (int u = 0; u < kU; ++u) v[u] = buf_load16_stream(rs, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
 #pragma unroll
         for (int u = 0; u < kU; ++u) {
           const uint32_t q[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
