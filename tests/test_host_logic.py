@@ -21,7 +21,7 @@ from oracle import modules as orc
 
 
 def test_cumsum_group_sizes_config1():
-    # the worked example of the survey: [137, 401, 59, 403] padded to 16 -> [144, 416, 64, 416]
+    # worked by hand: [137, 401, 59, 403] padded to multiples of 16 -> [144, 416, 64, 416]
     e, padded, cums, pcums = cumsum_group_sizes([137, 401, 59, 403], need_padding=True)
     assert (e, padded) == (4, True)
     assert cums == [0, 137, 538, 597, 1000]
