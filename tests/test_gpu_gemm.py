@@ -457,6 +457,90 @@ def test_random_problem_lists_are_exact(dev):
                     f"trial {trial} problem {i}: shapes {shapes} {a_dtype}"
 
 
+def test_random_launches_of_every_form_are_exact(dev, monkeypatch):
+    """240 random launches over everything a caller can choose: the four operand layouts (row-major, weights read
+    contraction-major, both operands contraction-major, a padded transposed copy with the other operand in place),
+    both gradient formats, the tile size forced either way or left to the launch, tail balancing on and off, bf16
+    and e4m3 outputs, row counts around the tile edges, contractions of any length.  Exactly summable operands
+    ({0, +-0.25 .. +-2}, power-of-two scales): bf16 results must equal torch's fp32 matmul bit for bit, e4m3
+    results its saturating cast, and the recorded amax the exact maximum."""
+    import numpy as np
+
+    backend = _backend()
+    rng = np.random.default_rng(977)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    g = torch.Generator(device=dev).manual_seed(977)
+
+    def exact(shape, dtype):
+        return vals[torch.randint(0, 8, shape, generator=g, device=dev)].to(dtype)
+
+    def rows():
+        if rng.integers(0, 6) == 0:
+            return int(rng.choice([0, 1, 15, 16, 17, 127, 128, 129, 255, 256, 257, 511, 512, 513]))
+        return int(rng.integers(0, 1700))
+
+    def mult16(hi):
+        return int(rng.integers(1, hi // 16 + 1)) * 16
+
+    for trial in range(240):
+        form = int(rng.integers(0, 5))
+        monkeypatch.setattr(backend, "_TILE", str(rng.choice(["auto", "128", "256"])))
+        monkeypatch.setattr(backend, "_STREAM_K", bool(rng.integers(0, 2)))
+        a_dtype = E5M2 if rng.integers(0, 2) else E4M3
+        e = int(rng.integers(1, 12))
+        what = f"trial {trial} form {form} tile {backend._TILE} tail balancing {backend._STREAM_K} {a_dtype}"
+        if form in (0, 1, 2):
+            sizes = [rows() for _ in range(e)]
+            n = mult16(1600) if rng.integers(0, 2) else int(rng.choice([16, 256, 512, 768, 1408, 1536]))
+            k = mult16(4300) if rng.integers(0, 2) else int(rng.choice([16, 128, 256, 768, 1408, 2048, 4096]))
+            what += f" sizes {sizes} n {n} k {k}"
+            a = exact((sum(sizes), k), a_dtype)
+            sa, sb = torch.full((e,), 0.5, device=dev), torch.full((e,), 2.0, device=dev)
+            if form == 1:
+                b = exact((e, k, n), E4M3)
+                c = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, b_transposed=True)
+                weights = [b[i].float() for i in range(e)]
+            else:
+                b = exact((e, n, k), E4M3)
+                weights = [b[i].float().t() for i in range(e)]
+                if form == 0:
+                    c = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, backward=(a_dtype == E5M2))
+                else:
+                    cs, amax = torch.full((e,), 0.25, device=dev), torch.zeros(e, device=dev)
+                    c = backend.fp8_gmm(a, b, torch.tensor(sizes), sa, sb, c_dtype=E4M3, c_scales=cs, c_amaxes=amax)
+            row = 0
+            for i, s in enumerate(sizes):
+                r = a[row: row + s].float() @ weights[i]
+                if form == 2:
+                    want = (r * 0.25).clamp(-448, 448).to(E4M3)
+                    assert torch.equal(c[row: row + s].view(torch.uint8), want.view(torch.uint8)), f"{what} expert {i}"
+                    assert float(amax[i]) == (float(r.abs().max()) if s else 0.0), f"{what} expert {i} amax"
+                else:
+                    want = r.to(torch.bfloat16)
+                    assert torch.equal(c[row: row + s].view(torch.int16), want.view(torch.int16)), f"{what} expert {i}"
+                row += s
+        else:
+            shapes = [(mult16(800), mult16(800), int(rng.integers(0, 1500))) for _ in range(e)]
+            what += f" shapes {shapes}"
+            a_list = [exact((k, m), a_dtype) for m, n, k in shapes]
+            b_list = [exact((k, n), E4M3) for m, n, k in shapes]
+            c_list = [torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev) for m, n, k in shapes]
+            ones = torch.ones(e, device=dev)
+            if form == 3:
+                backend.grouped_gemm(a_list, b_list, c_list, ones, ones, transposed=True)
+            else:
+                copies = []
+                for (m, n, k), a_km in zip(shapes, a_list):
+                    kpad = max((k + 15) // 16 * 16 + 16 * int(rng.integers(0, 2)), 16)
+                    t = torch.zeros(m, kpad, dtype=a_dtype, device=dev)
+                    t[:, :k] = a_km.t()
+                    copies.append(t)
+                backend.grouped_gemm(copies, b_list, c_list, ones, ones, transposed="b")
+            for i, (m, n, k) in enumerate(shapes):
+                want = (a_list[i].float().t() @ b_list[i].float()).to(torch.bfloat16)
+                assert torch.equal(c_list[i].view(torch.int16), want.view(torch.int16)), f"{what} problem {i}"
+
+
 @pytest.mark.parametrize("a_dtype", [E4M3, E5M2])
 def test_contraction_major_b_gives_the_same_bits(dev, a_dtype):
     """fp8_gmm(..., b_transposed=True) reads b[i] as [k, n] in place: for every shape it must return exactly what
