@@ -1,6 +1,6 @@
 """Benchmark of the FP8 grouped-GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example|hbm_ceiling|lds_rate|small_tile]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config1|config5|example]
 
 A step is one GroupedMlp (or GroupedLinear) forward + backward over one batch of synthetic,
 HBM-resident input: casts / transposes / pads, the six (three) grouped GEMMs and the
@@ -17,9 +17,11 @@ delayed-scaling update.  Prints ONE JSON line.
   parity    after the timed passes: sampled rows of every GEMM result of one more step against an fp32
             matmul (torch, on the GPU) of the dequantised fp8 operands, max |err| / max |ref| per result
   also      the step time of a later micro-batch that reuses the first one's fp8 weights (not the headline:
-            the reference casts the weights on every pass)
-  cpu_baseline  the per-expert quantize-dequantize-fp32-matmul loop (oracle/cpu_baseline.py) on
-            a bounded sample, timed on this machine's host cores
+            the reference casts the weights on every pass), the step on the reference's buffers, one dense GEMM
+            of the step's size next to the vendor library's, and - under `configs` - short passes of the other
+            workloads (config 3, 4 and 5) with their own roofline fractions and parity gates
+  cpu_baseline  the per-expert quantize-dequantize-fp32-matmul loop (oracle/cpu_baseline.py) over
+            the workload's own split, timed on this machine's host cores
 """
 import argparse
 import json
@@ -59,7 +61,15 @@ def splits(kind, experts, tokens, seed):
         p /= p.sum()
     else:
         p = np.full(experts, 1.0 / experts)
-    return [int(v) for v in rng.multinomial(tokens, p)]
+    sizes = [int(v) for v in rng.multinomial(tokens, p)]
+    if kind == "zipf":
+        # the workload is defined by having an expert without rows and one with fewer than 16 (a Zipf draw of this
+        # size rarely has either by itself): the two least popular experts hand their rows to the most popular one
+        order = np.argsort(sizes, kind="stable")
+        first, second, top = int(order[0]), int(order[1]), int(order[-1])
+        sizes[top] += sizes[first] + sizes[second] - 7
+        sizes[first], sizes[second] = 0, 7
+    return sizes
 
 
 def gemm_hbm_traffic(workload):
@@ -210,9 +220,10 @@ def sample_shader_clock(work):
     return clocks, watts, cap
 
 
-def bench_cast_pad(args):
+def measure_cast_pad(args):
     """config5: the bandwidth-bound path alone - ONE multi-tensor cast + transpose + amax + pad-to-128 launch over
-    8 bf16 activation tensors [M_i, 4096], M_i uniform in [1, 8191], N(0, 1) values with 0.1 % outliers at +-200."""
+    8 bf16 activation tensors [M_i, 4096], M_i uniform in [1, 8191], N(0, 1) values with 0.1 % outliers at +-200.
+    Returns the JSON line as a dict."""
     import fp8_gmm_amd as pkg  # noqa: F401  (loads the library)
     from fp8_gmm_amd import backend
     from fp8_gmm_amd.backend import kernel_timing
@@ -249,6 +260,14 @@ def bench_cast_pad(args):
     ms_per_step = elapsed / args.steps * 1e3
     d = timing.summary()["multi_pad_cast_transpose"]
     ach = d["work"] / (d["ms"] * 1e-3) / 1e9
+    # correctness gate: the transposed copy is the padded transpose of the row-major copy, both are the bytes torch's
+    # own saturating cast gives, and amax is max|x|, for every tensor
+    ok = True
+    for x, o, t, sc, am in zip(ins, outs, touts, scales, amaxes.tolist()):
+        want = (x.float() * sc).clamp(-448.0, 448.0).to(torch.float8_e4m3fn).view(torch.uint8)
+        m = x.shape[0]
+        ok = ok and torch.equal(o.view(torch.uint8), want) and torch.equal(t.view(torch.uint8)[:, :m], want.t()) \
+            and not bool(t.view(torch.uint8)[:, m:].any()) and am == x.float().abs().max().item()
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import ref
@@ -266,7 +285,7 @@ def bench_cast_pad(args):
         secs = time.perf_counter() - t0
         cpu = {"value": round(reps * cols * (3 * m + t.shape[1]) / secs / 1e9, 3), "unit": "GB/s", "cores": 1,
                "kind": "port", "sample": f"{reps} casts of one [{m}, {cols}] tensor by the scalar C oracle, {secs:.1f} s"}
-    print(json.dumps({
+    return {
         "metric": "cast + transpose + amax + pad GB/s, % of MI355X HBM bandwidth (8 activation tensors)",
         "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
@@ -274,213 +293,14 @@ def bench_cast_pad(args):
         "config": {"workload": "config5: multi_cast_transpose over 8 x [M_i, 4096] bf16, pad 128, e4m3, "
                                "0.1 % outliers at +-200", "rows": rows, "bytes_per_step": nbytes},
         "roofline": {"kernel": "multi_pad_kernel<cast+transpose>", "bound": "hbm", "achieved": round(ach, 1),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None},
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(ach / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel_us": round(d["ms"] * 1e3, 1)},
+        "wall_clock_per_call": {"us": round(ms_per_step * 1e3, 1), "GB/s": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1),
+                                "frac_of_hbm_peak": round(nbytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "parity": {"ok": bool(ok), "checked": "all bytes of both copies against torch's saturating e4m3 cast, zero "
+                                              "padding, amax == max|x|, all 8 tensors"},
         "cpu_baseline": cpu,
-    }))
-
-
-def bench_hbm_ceiling(args):
-    """hbm_ceiling: what this machine's memory system sustains for the read : write mixes of the library's
-    bandwidth-bound kernels, measured with plain streaming kernels (fp8_gmm_amd/csrc/hbm_probe.hip) that do no
-    arithmetic, next to the library's own kernels moving the same bytes.  Every launch moves at least 512 MiB, twice
-    the 256 MB memory-side cache.  Each mix is swept over the grid size (256 ... 16384 workgroups of 256 threads),
-    plain / streaming-hinted accesses and two walks (a trip's accesses a whole grid apart, or 16 KiB contiguous per
-    workgroup); `probes` holds the best launch of each mix and the whole sweep."""
-    import ctypes
-
-    import fp8_gmm_amd as pkg  # noqa: F401
-    from fp8_gmm_amd import backend
-
-    path = os.path.join(ROOT, "fp8_gmm_amd", "libfp8gmm_probe.so")
-    if not os.path.exists(path):
-        sys.exit("bench.py: fp8_gmm_amd/libfp8gmm_probe.so is not built (make -C fp8_gmm_amd/csrc)")
-    probe = ctypes.CDLL(path).fp8gmm_probe_stream
-    probe.restype = ctypes.c_int
-    probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64,
-                      ctypes.c_int, ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    mib = 1 << 20
-    src = torch.empty(1024 * mib, dtype=torch.uint8, device=dev)
-    src.view(torch.int32).random_(0, 2**31 - 1)
-    dst = torch.empty(512 * mib, dtype=torch.uint8, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-
-    def timed(fn):
-        for _ in range(args.warmup):
-            fn()
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-        ev[0].record()
-        for i in range(args.steps):
-            fn()
-            ev[i + 1].record()
-        torch.cuda.synchronize()
-        return min(ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)) * 1e-3   # best launch, seconds
-
-    # (name, input streams, writes, MiB per stream)
-    mixes = [("read only", 1, 0, 1024), ("4 : 1", 4, 1, 256), ("2 : 1", 2, 1, 256), ("1 : 1", 1, 1, 512),
-             ("write only", 0, 1, 512)]
-    rows = []
-    for name, reads, write, per in mixes:
-        best, sweep = None, []
-        for nt in (0, 1, 2, 3):
-            for blocks in (256, 512, 1024, 2048, 4096, 8192, 16384):
-                def fn():
-                    rc = probe(reads, write, nt, src.data_ptr(), dst.data_ptr(), per * mib, blocks, stream)
-                    assert rc == 0, f"probe launch failed: {rc}"
-                secs = timed(fn)
-                gbs = (reads + write) * per * mib / secs / 1e9
-                sweep.append([blocks, nt, round(gbs)])
-                if best is None or gbs > best["GB/s"]:
-                    best = {"mix": name, "MiB_read": reads * per, "MiB_written": write * per, "GB/s": round(gbs, 1),
-                            "us": round(secs * 1e6, 1), "blocks": blocks, "nontemporal": bool(nt & 1),
-                            "blocked": bool(nt & 2)}
-        best["sweep"] = sweep   # [workgroups, flags (1 = streaming hint, 2 = blocked walk), GB/s]
-        rows.append(best)
-        print(f"# probe {name}: {best}", file=sys.stderr, flush=True)
-
-    # the library's kernels on the same bytes: 8 tensors of 32 Mi elements
-    n, numel = 8, 32 * mib
-    x0, g0 = (seeded_normal((numel // 4096, 4096), seed, 1.0, dev) for seed in (7000, 7100))
-    xs, gs = [x0] + [x0.clone() for _ in range(n - 1)], [g0] + [g0.clone() for _ in range(n - 1)]
-    os_ = [torch.empty(numel // 4096, 4096, dtype=torch.float8_e4m3fn, device=dev) for _ in range(n)]
-    ts = [torch.empty(4096, numel // 4096, dtype=torch.float8_e4m3fn, device=dev) for _ in range(n)]
-    scales = [torch.full((1,), 64.0, device=dev) for _ in range(n)]
-    amaxes = torch.zeros(n, device=dev)
-    kernels = []
-    for name, mix, nbytes, fn in (
-            ("multi_quantize (bf16 -> e4m3 + amax)", "2 : 1", 3 * n * numel,
-             lambda: backend.multi_quantize(xs, os_, scales, amaxes)),
-            ("multi_cast_dgelu (bf16 grad, bf16 pre-GELU -> e5m2 + amax)", "4 : 1", 5 * n * numel,
-             lambda: backend.multi_cast_dgelu(xs, gs, [o.view(torch.float8_e5m2) for o in os_], scales, amaxes)),
-            ("multi_cast_transpose (bf16 -> e4m3 + transposed copy + amax)", "1 : 1", 4 * n * numel,
-             lambda: backend.multi_cast_transpose(xs, os_, ts, scales, amaxes))):
-        secs = timed(fn)   # launch + the amax merge that follows it
-        kernels.append({"kernel": name, "mix": mix, "MiB": nbytes // mib, "GB/s": round(nbytes / secs / 1e9, 1),
-                        "us": round(secs * 1e6, 1)})
-        print(f"# library {kernels[-1]}", file=sys.stderr, flush=True)
-    by_mix = {r["mix"]: r["GB/s"] for r in rows}
-    for k in kernels:
-        k["of_probe"] = round(k["GB/s"] / by_mix[k["mix"]], 3)
-    print(json.dumps({
-        "metric": "sustained HBM GB/s of plain streaming kernels by read : write mix (best launch of each sweep)",
-        "value": by_mix["2 : 1"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
-        "data": "synthetic", "config": {"workload": "hbm_ceiling: 512-1280 MiB per launch, grids 256-16384 x 256 "
-                                                    "threads, plain and streaming-hinted accesses, strided and "
-                                                    "blocked walks"},
-        "probes": rows, "library_kernels": kernels,
-        "roofline": {"kernel": "stream_kernel<2 reads, 1 write>", "bound": "hbm", "achieved": by_mix["2 : 1"],
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(by_mix["2 : 1"] / HBM_PEAK_GBS, 4),
-                     "traffic": None},
-        "cpu_baseline": None,
-    }))
-
-
-def bench_lds_rate(args):
-    """lds_rate: how fast one compute unit's LDS serves the fragment reads of the grouped GEMM, measured in isolation
-    (fp8_gmm_amd/csrc/lds_probe.hip): plain 16-byte reads (row-major operands), plain 8-byte reads and transposing
-    8-byte reads (contraction-major operands), 1, 2 and 4 wavefronts per compute unit.  The step arithmetic that
-    follows in `gemm_step` prices one K = 128 step of the 256 x 256 tile (32 MFMAs of 64 cycles per SIMD = 2048
-    cycles) in LDS instruction slots."""
-    import ctypes
-
-    path = os.path.join(ROOT, "fp8_gmm_amd", "libfp8gmm_probe.so")
-    if not os.path.exists(path):
-        sys.exit("bench.py: fp8_gmm_amd/libfp8gmm_probe.so is not built (make -C fp8_gmm_amd/csrc)")
-    probe = ctypes.CDLL(path).fp8gmm_probe_lds
-    probe.restype = ctypes.c_int
-    probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int,
-                      ctypes.c_void_p]
-    dev = torch.device("cuda:0")
-    blocks = torch.cuda.get_device_properties(dev).multi_processor_count
-    sink = torch.zeros(blocks * 256, dtype=torch.int32, device=dev)
-    cycles = torch.zeros(blocks, dtype=torch.int64, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-    iters = 10000
-    names = {0: ("ds_read_b128", 1024), 1: ("ds_read_b64", 512), 2: ("ds_read_b64_tr_b8", 512)}
-    rows = []
-    for waves in (1, 2, 4):
-        for mode, (name, nbytes) in names.items():
-            best = None
-            for _ in range(max(2, args.warmup)):
-                rc = probe(mode, waves, iters, sink.data_ptr(), cycles.data_ptr(), blocks, stream)
-                assert rc == 0, f"probe launch failed: {rc}"
-                torch.cuda.synchronize()
-                c = float(cycles.double().mean().item()) / (iters * 16)
-                best = c if best is None else min(best, c)
-            rows.append({"instruction": name, "wavefronts": waves, "cycles_per_instruction_and_wavefront": round(best, 2),
-                         "cycles_per_instruction_of_the_unit": round(best / waves, 2),
-                         "bytes_per_clock_and_unit": round(nbytes * waves / best, 1)})
-            print(f"# {rows[-1]}", file=sys.stderr, flush=True)
-    at4 = {r["instruction"]: r for r in rows if r["wavefronts"] == 4}
-    b128, tr = at4["ds_read_b128"]["cycles_per_instruction_of_the_unit"], at4["ds_read_b64_tr_b8"]["cycles_per_instruction_of_the_unit"]
-    # one K = 128 step: every wavefront reads 16 KiB of each operand (16 ds_read_b128 or 32 transposing reads)
-    step = {"mfma_cycles": 2048,
-            "read_cycles_both_row_major": round(4 * 32 * b128), "read_cycles_one_contraction_major": round(4 * (16 * b128 + 32 * tr)),
-            "read_cycles_both_contraction_major": round(4 * 64 * tr)}
-    peak = at4["ds_read_b128"]["bytes_per_clock_and_unit"]
-    print(json.dumps({
-        "metric": "LDS read rate of one compute unit, bytes per clock, ds_read_b128 with 4 wavefronts",
-        "value": peak, "unit": "B/clk/CU", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
-        "config": {"workload": "lds_rate: 16 independent reads per wait, the GEMM's fragment address patterns, one "
-                               "workgroup per compute unit"},
-        "reads": rows, "gemm_step": step, "roofline": None, "cpu_baseline": None,
-    }))
-
-
-def bench_small_tile(args):
-    """small_tile: grouped GEMMs that do not fill the machine with full 256 x 256 tiles - few tiles, or problems
-    of up to 128 rows - through both tile sizes (FP8GMM_GEMM_TILE_128 against the default), with the choice the
-    backend makes by itself; HIP events around every launch, mean of `--steps` launches."""
-    import fp8_gmm_amd as pkg  # noqa: F401
-    from fp8_gmm_amd import backend
-    from fp8_gmm_amd.backend import kernel_timing
-
-    dev = torch.device("cuda:0")
-    backend.warm_up(dev)
-    rows = []
-    # experts, rows per expert, n, k
-    shapes = [(8, 64, 2048, 4096), (8, 256, 2048, 4096), (8, 512, 2048, 4096), (8, 1024, 2048, 4096),
-              (8, 2048, 2048, 4096), (16, 128, 4096, 4096), (16, 256, 4096, 4096), (64, 64, 1408, 2048),
-              (64, 128, 1408, 2048), (128, 64, 768, 2048), (128, 128, 2048, 768), (4, 250, 512, 256),
-              (8, 100, 4096, 14336), (8, 300, 14336, 4096)]
-    for e, me, n, k in shapes:
-        m = e * me
-        a = _fp8_cast(seeded_normal((m, k), 9000 + e + me, 1.0, dev), 1.0, torch.float8_e4m3fn)
-        b = _fp8_cast(seeded_normal((e, n, k), 9100 + n, 1.0, dev), 1.0, torch.float8_e4m3fn)
-        ones = torch.ones(e, device=dev)
-        sizes = [me] * e
-        us, outs = {}, {}
-        for tile in ("256", "128", "auto"):
-            backend._TILE = tile
-            c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
-            for _ in range(args.warmup):
-                backend.fp8_gmm(a, b, sizes, ones, ones, c)
-            torch.cuda.synchronize()
-            with kernel_timing() as t:
-                for _ in range(args.steps):
-                    backend.fp8_gmm(a, b, sizes, ones, ones, c)
-                torch.cuda.synchronize()
-            us[tile] = t.summary()["grouped_gemm"]["ms"] * 1e3
-            outs[tile] = c
-        backend._TILE = "auto"
-        large = e * ((me + 255) // 256) * ((n + 255) // 256)
-        small = e * ((me + 127) // 128) * ((n + 127) // 128)
-        rows.append({"experts": e, "rows": me, "n": n, "k": k, "tiles_256": large, "tiles_128": small,
-                     "us_256": round(us["256"], 1), "us_128": round(us["128"], 1), "us_auto": round(us["auto"], 1),
-                     "speedup_128": round(us["256"] / us["128"], 2),
-                     "same_bits": bool(torch.equal(outs["256"].view(torch.int16), outs["128"].view(torch.int16)))})
-        print(f"# {rows[-1]}", file=sys.stderr, flush=True)
-    best = sum(min(r["us_256"], r["us_128"]) for r in rows)
-    auto = sum(r["us_auto"] for r in rows)
-    print(json.dumps({
-        "metric": "grouped GEMM launch time, 128 x 128 against 256 x 256 tiles, launches that do not fill the machine",
-        "value": round(best / auto, 4), "unit": "sum of the better tile's times / sum of the chosen tile's times",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "fp8", "data": "synthetic",
-        "config": {"workload": "small_tile: fp8_gmm forward, bf16 output, equal rows per expert"},
-        "launches": rows, "roofline": None, "cpu_baseline": None}))
+    }
 
 
 def dense_gemm_comparison(dev, m, n, k, reps=100):
@@ -535,33 +355,8 @@ def dense_gemm_comparison(dev, m, n, k, reps=100):
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5", "hbm_ceiling", "lds_rate", "small_tile"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
-    ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
-    ap.add_argument("--headline-only", action="store_true",
-                    help="skip the extra passes after the timed region (clock / power sampling, cached-weights "
-                         "step): what a profiler should see")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run one plain 256 MiB device copy (reads 256 MiB, writes 256 MiB) so that hardware "
-                         "byte counters collected around this command can be scaled against a known transfer")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
-    if args.workload == "config5":
-        return bench_cast_pad(args)
-    if args.workload == "hbm_ceiling":
-        return bench_hbm_ceiling(args)
-    if args.workload == "lds_rate":
-        return bench_lds_rate(args)
-    if args.workload == "small_tile":
-        return bench_small_tile(args)
-
+def measure_module(args):
+    """One module workload (WORKLOADS[args.workload]): returns the JSON line as a dict."""
     import fp8_gmm_amd as pkg
     from fp8_gmm_amd.backend import kernel_timing
 
@@ -638,8 +433,12 @@ def main():
         for name, d in summ.items():
             if name == "grouped_gemm":
                 ach = flops_per_gemm / (d["ms"] * 1e-3) / 1e12
+                alg_gbs = d["bytes"] / (d["ms"] * 1e-3) / 1e9
                 kernels[name] = {"launches_per_step": d["launches"] / args.steps, "ms": round(d["ms"], 4),
-                                 "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4)}
+                                 "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4),
+                                 "algorithmic_bytes_per_launch": round(d["bytes"]),
+                                 "algorithmic_GBps": round(alg_gbs, 1),
+                                 "frac_of_hbm_peak": round(alg_gbs / HBM_PEAK_GBS, 4)}
                 traffic = gemm_hbm_traffic(args.workload)
                 roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
                             "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),
@@ -670,25 +469,6 @@ def main():
                                      "board_power_w_max": max(watts) if watts else None, "board_power_cap_w": cap,
                                      "source": "pp_dpm_sclk and hwmon power1_input (sysfs), 1 ms period, over 40 "
                                                "extra steps"}}
-    # ... and the clock the GEMM launches really ran at: cycles / time counted inside a measurement build of the
-    # kernel by the first workgroup of every XCD (fp8gmm_grouped_gemm_timed), over 5 more steps
-    if roofline is not None and not args.headline_only:
-        counters = torch.zeros(32, dtype=torch.int64, device=dev)
-        with backend.gemm_clock_probe(counters):
-            for _ in range(5):
-                step()
-            torch.cuda.synchronize()
-        c = counters.cpu().reshape(8, 4).to(torch.float64)
-        if (c[:, 3] > 0).all():
-            per_xcd = (c[:, 2] / c[:, 3] * 100.0).tolist()
-            eff = sum(per_xcd) / len(per_xcd)
-            peak_at_clock = 256 * 8192 * eff * 1e6 / 1e12
-            clock = dict(clock or {})
-            clock["counted_in_gemm_kernel"] = {
-                "shader_mhz_mean": round(eff, 1), "per_xcd": [round(v, 1) for v in per_xcd],
-                "mfma_peak_at_that_clock_tflops": round(peak_at_clock, 1),
-                "gemm_frac_of_peak_at_that_clock": round(roofline["achieved"] / peak_at_clock, 4)}
-
     # Not the headline: the same step as a micro-batch after the first of an optimizer step, reusing the fp8
     # weights cast by the first (is_first_microbatch=False), which the reference stubs out.
     also = None
@@ -749,12 +529,15 @@ def main():
         from oracle import cpu_baseline
 
         cores = torch.get_num_threads()
-        sample_tokens = 16384
         cpu_baseline.mlp_step_sample(64, hidden, ffn)  # warm-up of the thread pool
-        secs, fl = cpu_baseline.mlp_step_sample(sample_tokens, hidden, ffn)
+        # the same per-expert loop the reference's test oracle walks, over this workload's split; for workloads
+        # whose split the router decides, or with many experts, one expert's share of the tokens per expert
+        cpu_sizes = sizes if sizes is not None and experts <= 16 else [tokens // 8] * 8
+        secs, fl = cpu_baseline.mlp_step_grouped(cpu_sizes, hidden, ffn)
         cpu = {"value": round(fl / secs / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-               "sample": f"all {sample_tokens} tokens through one expert, {hidden}->{ffn} MLP fwd+bwd (6 GEMMs, "
-                         f"{fl / 1e9:.0f} GFLOP) incl. weight quantisation, {secs:.1f} s"}
+               "sample": f"per-expert loop over the split {cpu_sizes}: quantize -> dequantize -> fp32 matmul, "
+                         f"{hidden}->{ffn} MLP fwd+bwd (6 GEMMs per expert, {fl / 1e9:.0f} GFLOP in all) incl. every "
+                         f"expert's weight quantisation, {secs:.1f} s"}
 
     names = {"mlp": "GroupedMlp", "linear": "GroupedLinear", "routed_mlp": "Fp8MlpModule (router, gather, GroupedMlp, scatter)"}
     line = {
@@ -784,6 +567,54 @@ def main():
         "clock": clock,
         "also": also,
     }
+    return line
+
+
+def short_pass(args, workload):
+    """A short pass of another workload for the `also.configs` record: step time, the GEMM against both roofs, the
+    cast kernels against the HBM roof, and the workload's own parity gate."""
+    import copy
+    import gc
+
+    a = copy.copy(args)
+    a.workload, a.steps, a.warmup = workload, min(args.steps, 10), 3
+    a.no_cpu_baseline, a.headline_only, a.copy_calibration, a.no_kernel_events = True, True, False, False
+    line = measure_cast_pad(a) if workload == "config5" else measure_module(a)
+    gc.collect()
+    torch.cuda.empty_cache()
+    keep = ("value", "unit", "ms_per_step", "steps", "config", "roofline", "kernels", "parity", "wall_clock_per_call")
+    return {k: line[k] for k in keep if line.get(k) is not None}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="config2", choices=sorted(WORKLOADS) + ["config5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-events", action="store_true", help="skip the second pass with per-kernel HIP events")
+    ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate after the timed passes")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="skip the extra passes after the timed region (clock / power sampling, cached-weights "
+                         "step, the other workloads): what a profiler should see")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy (reads 256 MiB, writes 256 MiB) so that hardware "
+                         "byte counters collected around this command can be scaled against a known transfer")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+    if args.workload == "config5":
+        print(json.dumps(measure_cast_pad(args)))
+        return
+    line = measure_module(args)
+    if args.workload == "config2" and not args.headline_only:
+        # every other workload in the same record: short passes, each with its own correctness gate
+        gc_configs = {}
+        for w in ("config3", "config4", "config5"):
+            gc_configs[w] = short_pass(args, w)
+        line["also"] = dict(line.get("also") or {})
+        line["also"]["configs"] = gc_configs
     print(json.dumps(line))
 
 

@@ -120,7 +120,6 @@ EXPORTS = (
     "fp8gmm_init",
     "fp8gmm_gemm_grid",
     "fp8gmm_plan_grouped_gemm_launch",
-    "fp8gmm_grouped_gemm_timed",
     "fp8gmm_grouped_gemm_static",
     "fp8gmm_gemm_tile_shape",
     "fp8gmm_plan_multi_tensor",
@@ -209,8 +208,6 @@ def load():
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp]
     L.fp8gmm_grouped_gemm_static.restype = ci
     L.fp8gmm_grouped_gemm_static.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp]
-    L.fp8gmm_grouped_gemm_timed.restype = ci
-    L.fp8gmm_grouped_gemm_timed.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp, vp]
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t

@@ -10,6 +10,7 @@ descriptor table, has the C library plan it, uploads it through pinned memory on
 the current stream and enqueues ONE kernel.  Nothing here computes on the CPU and
 there is no fallback: without the HIP library the import fails.
 """
+import collections
 import contextlib
 import threading
 
@@ -53,9 +54,10 @@ class kernel_timing:
     """Context manager that brackets every kernel launch of this module with HIP events.
 
     The events are recorded on the stream the kernels are launched on (torch's current
-    stream).  ``records`` holds ``(kernel name, algorithmic work, start event, end event)``;
-    ``summary()`` synchronises and returns per-kernel launch counts, mean duration in ms and
-    the algorithmic work (flops for the GEMM, bytes for the other kernels) per launch.
+    stream).  ``records`` holds ``(kernel name, algorithmic work, algorithmic bytes, start event, end event)``;
+    ``summary()`` synchronises and returns per-kernel launch counts, mean duration in ms, the
+    algorithmic work (flops for the GEMM, bytes for the other kernels) and the algorithmic bytes
+    (every operand read once, every result written once) per launch.
     """
 
     _active = None
@@ -74,22 +76,25 @@ class kernel_timing:
     def summary(self):
         torch.cuda.synchronize()
         out = {}
-        for name, work, start, end in self.records:
-            d = out.setdefault(name, {"launches": 0, "ms": 0.0, "work": 0.0})
+        for name, work, nbytes, start, end in self.records:
+            d = out.setdefault(name, {"launches": 0, "ms": 0.0, "work": 0.0, "bytes": 0.0})
             d["launches"] += 1
             d["ms"] += start.elapsed_time(end)
             d["work"] += work
+            d["bytes"] += nbytes
         for d in out.values():
             d["ms"] /= d["launches"]
             d["work"] /= d["launches"]
+            d["bytes"] /= d["launches"]
         return out
 
 
 class _timed:
-    def __init__(self, name, work_fn):
+    def __init__(self, name, work_fn, bytes_fn=None):
         self.rec = kernel_timing._active
         if self.rec is not None:
             self.name, self.work = name, float(work_fn())
+            self.bytes = float(bytes_fn()) if bytes_fn is not None else self.work
 
     def __enter__(self):
         if self.rec is not None:
@@ -100,7 +105,7 @@ class _timed:
         if self.rec is not None:
             end = torch.cuda.Event(enable_timing=True)
             end.record()
-            self.rec.records.append((self.name, self.work, self.start, end))
+            self.rec.records.append((self.name, self.work, self.bytes, self.start, end))
         return False
 
 
@@ -132,6 +137,13 @@ def _algorithmic_bytes(op, table):
 
 def _algorithmic_flops(table):
     return int((2 * table["m"].astype(np.int64) * table["n"].astype(np.int64) * table["k"].astype(np.int64)).sum())
+
+
+def _algorithmic_gemm_bytes(table, c_bytes):
+    """Both fp8 operands read once, the result (and the bf16 pre-GELU copy, where there is one) written once."""
+    m, n, k = (table[f].astype(np.int64) for f in ("m", "n", "k"))
+    aux = (table["aux"] != 0).astype(np.int64) * 2
+    return int(((m + n) * k + m * n * (c_bytes + aux)).sum())
 
 
 def _device_of(tensors):
@@ -620,7 +632,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
     else:
         plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | (_lib.EPI_GELU if gelu else 0),
-                                                                     grid, _STREAM_K)
+                                                                     grid, options.stream_k)
     if plan.total_tiles == 0:
         return
     n = len(table)
@@ -630,16 +642,11 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         with _on_device(device):
             ws = _gemm_workspace(device, plan.n_slots)
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
-            probe = _clock_probe.get("counters")
-            with _timed("grouped_gemm", lambda: _algorithmic_flops(table)):
-                L = _lib.load()
+            with _timed("grouped_gemm", lambda: _algorithmic_flops(table),
+                        lambda: _algorithmic_gemm_bytes(table, 2 if c_dtype == torch.bfloat16 else 1)):
                 fix_ptr = dev_ptr + off_fix if plan.n_fixups else None
-                if probe is None:
-                    rc = L.fp8gmm_grouped_gemm(dev_ptr, n, dev_ptr + off_items, fix_ptr, plan, *fmts, ws_ptr, ws_bytes,
-                                               _stream(device))
-                else:
-                    rc = L.fp8gmm_grouped_gemm_timed(dev_ptr, n, dev_ptr + off_items, fix_ptr, plan, *fmts, ws_ptr,
-                                                     ws_bytes, probe.data_ptr(), _stream(device))
+                rc = _lib.load().fp8gmm_grouped_gemm(dev_ptr, n, dev_ptr + off_items, fix_ptr, plan, *fmts, ws_ptr,
+                                                     ws_bytes, _stream(device))
         _lib.check(rc)
 
     _submit(blob, device, launch, keep)
@@ -651,25 +658,55 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
 # twice the LDS read instructions; on isolated back-to-back launches of config 2's shapes the copy form is 7 - 15 %
 # faster (900 -> 765 us, 855 -> 795 us), inside the step the two weight gradients gain 40 us together and the two casts
 # that write the copies lose 64 (config 2: 5.79 ms against 5.76 in place; config 4: 1.76 against 1.69).  So the
-# modules read both operands in place; FP8GMM_WGRAD=copy selects the other form.  Same bits either way.
-_WGRAD = os.environ.get("FP8GMM_WGRAD", "in_place")
-
-
-def wgrad_wants_transposed_gradient(total_rows, num_groups):
-    return _WGRAD == "copy" and num_groups > 0 and total_rows > 0
-
-
+# modules read both operands in place; options.wgrad = "copy" selects the other form.  Same bits either way.
+#
 # Tile size of a grouped GEMM.  The 256 x 256 tile is the fast one per flop.  The 128 x 128 tile (two workgroups per
 # compute unit, twice the operand traffic from L2) wins where the large tile leaves the machine idle: launches with
 # fewer large tiles than about half the compute units, and launches whose problems are so short or narrow that the
 # large tiles are mostly padding (measured 1.1 - 1.7 x there, 0.8 - 0.9 x on launches that fill the machine with
-# full tiles; same bits either way).  FP8GMM_TILE=256 / 128 forces one of them.
-_TILE = os.environ.get("FP8GMM_TILE", "auto")
+# full tiles).  Whole tiles get the same bits from either size; a tile that the large-tile launch shares along K is
+# summed from fp32 partial sums, a deterministic but differently associated sum.  options.tile = "256" / "128"
+# forces one size.
+#
+# Tail balancing of the grouped GEMM (the workgroups of an XCD share their range's last tiles along K) needs
+# scratch memory for partial sums and a second, small launch; options.stream_k = False plans every launch without it.
+class GemmOptions:
+    """Launch policy of the grouped GEMMs of this process: ``tile`` "auto" | "256" | "128", ``stream_k`` (share the
+    tail tiles of a launch along K), ``wgrad`` "in_place" | "copy".  The defaults can be preset with the
+    environment variables FP8GMM_TILE, FP8GMM_STREAMK (0 turns sharing off) and FP8GMM_WGRAD, read once when the
+    module is imported; afterwards assign the attributes or use ``gemm_options(...)`` for a block."""
+
+    __slots__ = ("tile", "stream_k", "wgrad")
+
+    def __init__(self, env=os.environ):
+        self.tile = env.get("FP8GMM_TILE", "auto")
+        self.stream_k = env.get("FP8GMM_STREAMK", "1") != "0"
+        self.wgrad = env.get("FP8GMM_WGRAD", "in_place")
+
+
+options = GemmOptions()
+
+
+@contextlib.contextmanager
+def gemm_options(**changes):
+    """Set attributes of ``options`` for the duration of a block."""
+    saved = {k: getattr(options, k) for k in changes}
+    for k, v in changes.items():
+        setattr(options, k, v)
+    try:
+        yield options
+    finally:
+        for k, v in saved.items():
+            setattr(options, k, v)
+
+
+def wgrad_wants_transposed_gradient(total_rows, num_groups):
+    return options.wgrad == "copy" and num_groups > 0 and total_rows > 0
 
 
 def _small_tiles(table):
-    if _TILE != "auto":
-        return _TILE == "128"
+    if options.tile != "auto":
+        return options.tile == "128"
     m, n = table["m"].astype(np.int64), table["n"].astype(np.int64)
     large = int((((m + 255) // 256) * ((n + 255) // 256)).sum())
     if large == 0:
@@ -678,48 +715,46 @@ def _small_tiles(table):
     return large <= 160 or 2 * small <= 5 * large
 
 
-# Tail balancing of the grouped GEMM (the workgroups of an XCD share their range's last tiles along K) needs
-# scratch memory for partial sums; the library takes it from the caller.  One buffer per (device, stream), grown
-# on demand and kept: launches on one stream are ordered and can share it.  FP8GMM_STREAMK=0 plans every launch
-# without tail balancing (no workspace, no second launch).
-_STREAM_K = os.environ.get("FP8GMM_STREAMK", "1") != "0"
-_workspaces = {}
+# The partial sums of tiles shared along K go to a workspace that the library takes from the caller.  One buffer
+# per (device, stream), grown on demand: launches on one stream are ordered and can share it.  The cache keeps the
+# buffers of the few streams used most recently (a program that creates and destroys streams would otherwise leave a
+# buffer behind for each, and a recycled handle would find a stranger's entry - harmless, the contents never
+# matter, but unbounded); release_workspaces() drops them all.
+_MAX_WORKSPACES = 8
+_workspaces = collections.OrderedDict()
 
 
 def _gemm_workspace(device, n_slots):
     if n_slots == 0:
         return None
-    key = (device, _stream(device))
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream(device))
     ws = _workspaces.get(key)
     need = n_slots * _lib.GEMM_SLOT_BYTES
     if ws is None or ws.numel() < need:
         ws = torch.empty(need, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
+    _workspaces.move_to_end(key)
+    while len(_workspaces) > _MAX_WORKSPACES:
+        _workspaces.popitem(last=False)   # queued kernels keep using it: the allocator frees in stream order
     return ws
+
+
+def release_workspaces():
+    """Drop the cached tail-balancing workspaces (they are allocated again on demand)."""
+    _workspaces.clear()
 
 
 def warm_up(device=None):
     """Do everything a first launch on `device` would do besides the launch itself - the library's per-device
-    initialisation and the allocation of a tail-balancing workspace of the largest size a launch can need - so
-    that none of it falls into a timed or captured region."""
-    device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    initialisation and the allocation of a tail-balancing workspace of the largest size a launch can need
+    (2 x grid slots of 256 KB: 128 MiB on 256 compute units) for the current stream - so that none of it falls
+    into a timed or captured region."""
+    device = torch.device("cuda") if device is None else torch.device(device)
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
     grid = _lib.gemm_grid(_lib.init(device.index))
     with _on_device(device):
         _gemm_workspace(device, 2 * grid)
-
-
-# measurement hook of bench.py: while `counters` (8 x 4 int64 on the device) is set, grouped GEMMs are launched
-# through fp8gmm_grouped_gemm_timed
-_clock_probe = {}
-
-
-@contextlib.contextmanager
-def gemm_clock_probe(counters):
-    _clock_probe["counters"] = counters
-    try:
-        yield
-    finally:
-        _clock_probe.pop("counters", None)
 
 
 def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False, keep_scale_inv=None):
@@ -764,6 +799,10 @@ def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_ou
     n = len(a_list)
     if n == 0:
         return
+    if isinstance(transposed, (bool, np.bool_)):
+        transposed = bool(transposed)
+    elif transposed != "b":
+        _fail('fp8_gmm_amd: transposed must be False, True or "b"')
     _check_counts(n, b_list=b_list, c_list=c_list)
     a, b, c = _as_batch(a_list, "a"), _as_batch(b_list, "b"), _as_batch(c_list, "c")
     aux = None if pre_gelu_outs is None else _as_batch(pre_gelu_outs, "pre_gelu_outs")

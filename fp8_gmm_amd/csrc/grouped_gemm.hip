@@ -170,8 +170,7 @@ int scratch_for(int dev, uint8_t** out) {
   return FP8GMM_OK;
 }
 
-typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*, uint64_t*,
-                         hipStream_t);
+typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*, hipStream_t);
 
 // the variant for a format / layout combination, or null when the combination does not exist
 launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor, int tile) {
@@ -185,8 +184,7 @@ launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor, int ti
 
 int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
                    const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
-                   int out_kind, int epilogue, void* workspace, size_t workspace_bytes, uint64_t* counters,
-                   void* stream) {
+                   int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
   if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
   if (n < 0 || plan->total_tiles < 0 || plan->rounds < 0 || plan->n_fixups < 0 || plan->n_slots < 0)
     return FP8GMM_ERR_BAD_ARGUMENT;
@@ -215,7 +213,7 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
     return FP8GMM_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int rc = launch(probs_dev, items_dev, plan->grid, out_kind, epilogue & FP8GMM_EPI_GELU,
-                        static_cast<uint8_t*>(workspace), counters, s);
+                        static_cast<uint8_t*>(workspace), s);
   if (rc != FP8GMM_OK) return rc;
   if (plan->n_fixups > 0) {
     hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups * kFixupSplit), dim3(kFixupThreads), 0, s, probs_dev,
@@ -262,16 +260,7 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gm
                         const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
                         int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
   return fp8gmm::launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
-                                workspace_bytes, nullptr, stream);
-}
-
-int fp8gmm_grouped_gemm_timed(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
-                              const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
-                              int b_fmt, int out_kind, int epilogue, void* workspace, size_t workspace_bytes,
-                              uint64_t* dev_counters, void* stream) {
-  if (dev_counters == nullptr) return FP8GMM_ERR_NULL_POINTER;
-  return fp8gmm::launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
-                                workspace_bytes, dev_counters, stream);
+                                workspace_bytes, stream);
 }
 
 int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
@@ -288,7 +277,7 @@ int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, cons
     if (rc != FP8GMM_OK) return rc;
   }
   return launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, ws,
-                        (size_t)kStaticSlots * FP8GMM_GEMM_SLOT_BYTES, nullptr, stream);
+                        (size_t)kStaticSlots * FP8GMM_GEMM_SLOT_BYTES, stream);
 }
 
 }  // extern "C"

@@ -54,6 +54,7 @@
 
 #include <atomic>
 #include <type_traits>
+#include <utility>
 
 #include "device_utils.h"
 #include "tiling.h"
@@ -87,6 +88,29 @@ constexpr int kFastStores = MT * 8;  // 16-byte stores per wavefront in the stag
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+#define FP8GMM_ALL_ACC_256 \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
+  "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", \
+  "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", \
+  "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", \
+  "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", \
+  "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", \
+  "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", \
+  "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", \
+  "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", \
+  "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", \
+  "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", \
+  "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", \
+  "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", \
+  "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", \
+  "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", \
+  "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
+#define FP8GMM_ALL_ACC_64 \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
+  "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", \
+  "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", \
+  "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63"
+
 #define FP8GMM_SB() __builtin_amdgcn_sched_barrier(0)
 #define FP8GMM_WAIT_VM(n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory")
 #define FP8GMM_WAIT_VM_LGKM(n) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(n) : "memory")
@@ -94,16 +118,41 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define FP8GMM_DMA(lds_addr, voff, rsrc) \
   asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc))
 
-// One MFMA tile's accumulators as ordinary vector registers.  In the main kernel the 256 accumulators of a
-// lane live in the accumulation registers (the other 256 hold fragments and addresses); vector arithmetic
-// cannot read those, and left to itself the register allocator parks them in scratch memory on the way.
-// Reading them 16 at a time, where they are used, keeps the epilogue within the register file.
-__device__ __forceinline__ f32x16 tile_values(const f32x16& a) {
+// The accumulators of a lane are the accumulation registers a0 .. a255 (a0 .. a63 for the small tile), addressed BY
+// NAME in every statement that touches them: MFMA tile (i, j) of a wavefront's sub-tile owns the 16 registers from
+// 16 (NT i + j).  The compiler never sees them as values, so there is nothing for its register allocator to move,
+// split or spill, whatever control flow surrounds the products (with the accumulators as ordinary values and all
+// 512 registers of a lane in use, a second step body or products issued from inside the epilogue end in hundreds
+// of spilled registers).  The statements are volatile and keep their order; what the compiler does not know it
+// cannot protect, so: (1) nothing but these statements may use an accumulation register - every product names the
+// whole file as clobbered, which keeps the compiler from parking spilled values there; (2) the waits the hardware
+// needs between a product and a read of its result are this file's business: results are read tile by tile in the
+// order the products were issued, never sooner than 16 products (a thousand cycles) after the last one into a tile.
+template <int... Is, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F&& f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+#define FP8GMM_ACC_READ(R) asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t[R]) : "n"(BASE + R))
+#define FP8GMM_ACC_ZERO(R) asm volatile("v_accvgpr_write_b32 a[%0], 0" ::"n"(BASE + R))
+#define FP8GMM_16_TIMES(X) X(0); X(1); X(2); X(3); X(4); X(5); X(6); X(7); X(8); X(9); X(10); X(11); X(12); X(13); X(14); X(15)
+template <int BASE>
+__device__ __forceinline__ f32x16 acc_tile() {   // one MFMA tile's accumulators as ordinary vector registers
   f32x16 t;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t[r]) : "a"(a[r]));
+  FP8GMM_16_TIMES(FP8GMM_ACC_READ);
   return t;
 }
+template <int BASE>
+__device__ __forceinline__ void acc_tile_clear() {
+  FP8GMM_16_TIMES(FP8GMM_ACC_ZERO);
+}
+#undef FP8GMM_ACC_READ
+#undef FP8GMM_ACC_ZERO
+#undef FP8GMM_16_TIMES
 
 // Per-problem scalars (scaling factors, the current amax) are read through the scalar unit: they are uniform,
 // and a vector load would have to be waited for with vmcnt(0), i.e. together with every operand load the
@@ -140,14 +189,35 @@ constexpr uint32_t kMaskedOffset = 0x80000000u;  // + any row offset of a tile (
 
 // `s` = a_scale_inv * b_scale_inv and `cs` = c_scale of the problem, read by the caller ahead of time.
 // TILE: 256 (the namespace's constants) or 128 (the small tile: 64 x 64 per wavefront, 16 KB of staging).
+// `released(i, j)` (integral constants) is called right after MFMA tile (i, j) of the staged bf16 path has been read
+// out of its accumulators: from there on they may receive the next tile's products.
+// whether the plain bf16 epilogue through the staging area applies to this tile
 template <int TILE>
-__device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64], const fp8gmm_gemm_problem& pr,
-                                              int m0, int n0, int out_kind, int epilogue, uint8_t* stage,
-                                              bool oob_zero, float s, float cs) {
+__device__ __forceinline__ bool staged_bf16_tile(const fp8gmm_gemm_problem& pr, int m0, int n0, int out_kind,
+                                                 int epilogue) {
+  const int64_t ldc = pr.ldc;
+  const bool interior = (m0 + TILE <= pr.m) && (n0 + TILE <= pr.n);
+  const int cv = pr.n - n0 < TILE ? pr.n - n0 : TILE;
+  const bool desc_ok = ((ldc & 7) == 0) && ldc < (1 << 21) && ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0);
+  return out_kind == FP8GMM_OUT_BF16 && !(epilogue & FP8GMM_EPI_GELU) && desc_ok && (interior || (cv & 7) == 0);
+}
+struct NothingReleased {
+  template <class I, class J>
+  __device__ __forceinline__ void operator()(I, J) const {}
+};
+template <int TILE, class Released = NothingReleased>
+__device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int m0, int n0, int out_kind, int epilogue,
+                                              uint8_t* stage, bool oob_zero, float s, float cs,
+                                              Released released = Released()) {
   constexpr int BM = TILE, BN = TILE, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
   constexpr int kStageBytes = TILE * 32;   // per wavefront: a quarter of one ring unit
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // The lane's offsets into the staging area and the result are formed anew for every tile: computed once per
+  // kernel (they do not depend on the tile) they would occupy a dozen registers all through the main loop, where
+  // there are none to spare.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, khalf = lane >> 5;
   const int M = pr.m, N = pr.n;
@@ -160,7 +230,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
     const int cv = N - n0 < BN ? N - n0 : BN;
     // 16-byte pieces of the tile's rows can be addressed with 32-bit offsets below 2^30
     const bool desc_ok = ((ldc & 7) == 0) && ldc < (1 << 21) && ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0);
-    if (out_kind == FP8GMM_OUT_BF16 && !gelu && desc_ok && (interior || (cv & 7) == 0)) {
+    if (staged_bf16_tile<TILE>(pr, m0, n0, out_kind, epilogue)) {
       // Plain bf16 output: straight-line code with an exact store count.
       // Through LDS, so that a store instruction writes whole lines.  In the MFMA layout a lane holds 4
       // consecutive columns of one row, and a 16-byte store per lane touches 32 rows: 64 separate 32-byte
@@ -187,20 +257,21 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
           buf_store16_stream(v[it], rc, lane_off + row_off);
         }
       };
-#pragma unroll
-      for (int u = 0; u < MT * kUnitsPerRow; ++u) {
-        const int i = u / kUnitsPerRow, jj = u % kUnitsPerRow;
+      static_for<MT * kUnitsPerRow>([&](auto uc) {
+        constexpr int u = decltype(uc)::value;
+        constexpr int i = u / kUnitsPerRow, jj = u % kUnitsPerRow;
         uint8_t* buf = mine + (kStageBytes >= 8192 ? (u & 1) * 4096 : 0);
-#pragma unroll
-        for (int jl = 0; jl < 2; ++jl) {
-          const f32x16 t = tile_values(acc[i][2 * jj + jl]);
+        static_for<2>([&](auto jlc) {
+          constexpr int jl = decltype(jlc)::value;
+          const f32x16 t = acc_tile<16 * (NT * i + 2 * jj + jl)>();
+          released(std::integral_constant<int, i>{}, std::integral_constant<int, 2 * jj + jl>{});
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const u32x2 o = {pack_bf16x2(t[4 * g + 0] * s, t[4 * g + 1] * s),
                              pack_bf16x2(t[4 * g + 2] * s, t[4 * g + 3] * s)};
             *reinterpret_cast<u32x2*>(buf + wr + (((4 * jl + g) ^ ((l32 >> 1) & 7)) << 4)) = o;
           }
-        }
+        });
         // the previous unit's read-back was issued before this unit's conversion: store it now
         if (u > 0) store_unit((u - 1) / kUnitsPerRow, (u - 1) % kUnitsPerRow);
         // only this wavefront touches `mine`, and its LDS operations complete in order
@@ -209,7 +280,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
           const int r = 8 * it + rrow;
           v[it] = *reinterpret_cast<const u32x4*>(buf + r * 128 + ((rchunk ^ ((r >> 1) & 7)) << 4));
         }
-      }
+      });
       store_unit(MT - 1, kUnitsPerRow - 1);
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       fast = true;
@@ -235,13 +306,13 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
       const uint32_t lane_off = col < cv ? (uint32_t)((rrow * (int)ldc + col) * 2) : kMaskedOffset;
       const uint32_t lane_off8 = col8 < cv ? (uint32_t)(rrow8 * (int)ldc + col8) : kMaskedOffset;
       float tile_amax = 0.f;
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
+      static_for<MT>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
         uint32_t f8[NT][4];
         bool any_nan = false;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
+        static_for<NT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          const f32x16 t = acc_tile<16 * (NT * i + j)>();
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             float v[4], x[4];
@@ -263,12 +334,12 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
             f8[j][g] = __builtin_amdgcn_cvt_pk_fp8_f32(x[2], x[3],
                                                        __builtin_amdgcn_cvt_pk_fp8_f32(x[0], x[1], 0u, false), true);
           }
-        }
+        });
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(any_nan) != 0, 0)) {
           // some lane of this block saw a NaN: form the block's bytes again, with 0x7F in place of every NaN
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            const f32x16 t = tile_values(acc[i][j]);
+          static_for<NT>([&](auto jc) {
+            constexpr int j = decltype(jc)::value;
+            const f32x16 t = acc_tile<16 * (NT * i + j)>();
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
               uint32_t nan_bytes = 0;
@@ -279,7 +350,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
               }
               f8[j][g] = (f8[j][g] & ~nan_bytes) | (0x7f7f7f7fu & nan_bytes);
             }
-          }
+          });
         }
         {
           u32x4 rb[8];
@@ -314,7 +385,7 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
             buf_store16_stream(rb[it], rc, lane_off8 + row_off);
           }
         }
-      }
+      });
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       merge_amax(pr.c_amax, wave_max(tile_amax), lane);
     } else if (out_kind == FP8GMM_OUT_BF16) {
@@ -322,12 +393,12 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
       const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) &&
                        (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
+      static_for<MT>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
         const int m = m0 + wave_m * WM + i * 32 + l32;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
+        static_for<NT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          const f32x16 t = acc_tile<16 * (NT * i + j)>();
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -356,19 +427,19 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
               }
             }
           }
-        }
-      }
+        });
+      });
     } else {
       uint8_t* __restrict__ C = static_cast<uint8_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
       const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 3) == 0) &&
                        (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
+      static_for<MT>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
         const int m = m0 + wave_m * WM + i * 32 + l32;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const f32x16 t = tile_values(acc[i][j]);
+        static_for<NT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          const f32x16 t = acc_tile<16 * (NT * i + j)>();
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave_n * WN + j * 32 + g * 8 + khalf * 4;
@@ -403,8 +474,8 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
               }
             }
           }
-        }
-      }
+        });
+      });
       merge_amax(pr.c_amax, wave_max(amax), lane);
     }
     return fast;
@@ -413,40 +484,19 @@ __device__ __forceinline__ bool tile_epilogue(f32x16 (&acc)[TILE / 64][TILE / 64
 // Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
 // (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
 template <int TILE>
-__device__ __forceinline__ void partial_store(f32x16 (&acc)[TILE / 64][TILE / 64], uint8_t* slot) {
+__device__ __forceinline__ void partial_store(uint8_t* slot) {
   constexpr int MT = TILE / 64, NT = TILE / 64;
   float* base = reinterpret_cast<float*>(slot) + threadIdx.x * 4;
+  static_for<MT * NT>([&](auto tc) {
+    constexpr int ij = decltype(tc)::value;
+    const f32x16 t = acc_tile<16 * ij>();
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const f32x16 t = tile_values(acc[i][j]);
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
-        global_store(base + ((i * NT + j) * 4 + g) * (NTHREADS * 4), v);
-      }
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
+      global_store(base + (ij * 4 + g) * (NTHREADS * 4), v);
     }
+  });
 }
-// Measurement on the side (fp8gmm_grouped_gemm_timed): when `counters` (8 x 4 uint64 of device memory) is not
-// null, the first workgroup of every XCD writes its shader-cycle counter and the constant 100 MHz counter when it
-// starts and adds the differences to two running totals when it ends, so that the caller can derive the clock
-// the launch really ran at (the counters of different compute units are not comparable, hence the same
-// workgroup takes both readings).  Two uniform branches per launch otherwise.
-__device__ __forceinline__ void clock_probe_mark(uint64_t* counters, int which) {
-  if (counters != nullptr && blockIdx.x < kNumXcd && threadIdx.x == 0) {
-    volatile uint64_t* const q = counters + 4 * blockIdx.x;
-    const uint64_t cycles = (uint64_t)clock64(), ticks = (uint64_t)wall_clock64();
-    if (which == 0) {
-      q[0] = cycles;
-      q[1] = ticks;
-    } else {  // totals over all launches since the counters were cleared
-      q[2] += cycles - q[0];
-      q[3] += ticks - q[1];
-    }
-  }
-}
-
 // The half of a work-list record (fp8gmm_gemm_item) that a side of the kernel needs, as scalar loads.
 struct ItemLoad {   // bytes 0..31: what the load stream needs besides ItemTile
   uint64_t a, b;
@@ -480,7 +530,7 @@ static_assert(offsetof(fp8gmm_gemm_item, k) == 32 && offsetof(fp8gmm_gemm_item, 
 template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_kernel(
     const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items, int out_kind,
-    int epilogue, uint8_t* __restrict__ workspace, uint64_t* __restrict__ counters) {
+    int epilogue, uint8_t* __restrict__ workspace) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   // the tile's extents shadow the namespace's (which are those of the 256 x 256 tile)
   [[maybe_unused]] constexpr int BM = TILE;
@@ -489,7 +539,6 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   constexpr int kFastStores = MT * (NT / 2) * 4;    // stores per wavefront in the staged bf16 epilogue
   static_assert(TILE == 256 || TILE == 128, "tile sizes with a step sequence below");
 
-  clock_probe_mark(counters, 0);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: what depends on it stays in scalar registers
@@ -734,13 +783,48 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   // LDS depends on: at the first barrier after it they may stay in flight.
   bool relaxed = false;
 
-// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp)
-#define FP8GMM_MF0(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb0[j], fa0[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
-#define FP8GMM_MF1(i, j) \
-  acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb1[j], fa1[i], acc[i][j], B_FMT, A_FMT, 0, 0, 0, 0)
+  // The accumulation registers belong to the statements below (see acc_tile): named as clobbered once, they count
+  // as used everywhere, and the compiler keeps out of them.
+  if constexpr (TILE == 256) {
+    asm volatile("" ::: FP8GMM_ALL_ACC_256);
+  } else {
+    asm volatile("" ::: FP8GMM_ALL_ACC_64);
+  }
+// source 0 = weights (format B_FMT -> cbsz), source 1 = tokens (format A_FMT -> blgp); MFMA tile (i, j) accumulates
+// in a[16 (NT i + j) ..+15]
+#if defined(__HIP_DEVICE_COMPILE__)
+#define FP8GMM_MFMA(i, j, FB, FA)                                                                      \
+  asm volatile("v_mfma_f32_32x32x64_f8f6f4 a[%2:%3], %0, %1, a[%2:%3] cbsz:%4 blgp:%5" ::"v"(FB), "v"(FA), \
+               "n"(16 * (NT * (i) + (j))), "n"(16 * (NT * (i) + (j)) + 15), "n"(B_FMT), "n"(A_FMT))
+// ... starting from zero: the first product into a tile's accumulators
+#define FP8GMM_MFMA_Z(i, j, FB, FA)                                                                    \
+  asm volatile("v_mfma_f32_32x32x64_f8f6f4 a[%2:%3], %0, %1, 0 cbsz:%4 blgp:%5" ::"v"(FB), "v"(FA),      \
+               "n"(16 * (NT * (i) + (j))), "n"(16 * (NT * (i) + (j)) + 15), "n"(B_FMT), "n"(A_FMT))
+#else  // the host pass only needs the kernel's signature (and cannot take 32-byte vectors as "v" operands)
+#define FP8GMM_MFMA(i, j, FB, FA) (void)0
+#define FP8GMM_MFMA_Z(i, j, FB, FA) (void)0
+#endif
+// FIRST (of the enclosing step): the first step of a tile, whose low-half products have been issued already - from
+// inside the previous tile's epilogue, or by start_tile
+#define FP8GMM_MF0(i, j)                                    \
+  do {                                                      \
+    if constexpr (!FIRST) FP8GMM_MFMA(i, j, fb0[j], fa0[i]); \
+  } while (0)
+#define FP8GMM_MF1(i, j) FP8GMM_MFMA(i, j, fb1[j], fa1[i])
 
   ItemTile cp_next = item_tile(0);  // the compute side's next record, fetched ahead like the load side's
+  // The first 16 products of a tile (the low K half of its first step) start its accumulators from zero and need
+  // registers only - the fragments are read a half-step ahead.  They are issued as soon as the accumulators are
+  // free: from inside the previous tile's epilogue where that is the staged bf16 form, right after it otherwise.
+  // Invariant at the top of the item loop: if the item has K work, those products are under way.
+  auto start_tile = [&fb0, &fa0]() {
+    static_for<MT * NT>([&](auto tc) {
+      constexpr int i = decltype(tc)::value / NT, j = decltype(tc)::value % NT;
+      const i32x8 wf = fb0[j], tf = fa0[i];
+      FP8GMM_MFMA_Z(i, j, wf, tf);
+    });
+  };
+  if (cp_next.nk > 0) start_tile();
   for (int r_cp = 0;; ++r_cp) {
     const ItemTile g = cp_next;
     if (g.prob < 0) break;
@@ -751,17 +835,10 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
     const float scale_c = load_scale(pr.c_scale);
     const int m0 = g.m0, n0 = g.n0;
 
-    f32x16 acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
     // One K = 128 step.  `same_item`: the load cursor stays inside its current item after this step (the caller
     // knows), so advancing it is three additions; otherwise the general advance, which may switch items.
-    auto k_step = [&](auto same_item) {
+    auto k_step = [&](auto same_item, auto first) {
+      constexpr bool FIRST = decltype(first)::value;
       // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
       // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
       // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
@@ -916,22 +993,38 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
     // The load cursor runs two steps ahead of this loop: while at least three steps of the item remain, its
     // next step lies in the same item.
     int kt = 0;
-    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{});
-    for (; kt < g.nk; ++kt) k_step(std::false_type{});
+    if (g.nk > 0) {
+      k_step(std::false_type{}, std::true_type{});
+      kt = 1;
+    } else {
+      static_for<MT * NT>([&](auto tc) { acc_tile_clear<16 * decltype(tc)::value>(); });
+    }
+    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{}, std::false_type{});
+    for (; kt < g.nk; ++kt) k_step(std::false_type{}, std::false_type{});
     // ---- epilogue ----
+    uint8_t* const stage = lds + ((ua + 4) % RING) * US;  // free until the next step's token loads
+    const bool more = cp_next.prob >= 0 && cp_next.nk > 0;  // the fragments in fa0 / fb0 open another tile
     if (g.slot >= 0) {
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
-      partial_store<TILE>(acc, workspace + (size_t)g.slot * kPartialBytes);
+      partial_store<TILE>(workspace + (size_t)g.slot * kPartialBytes);
       relaxed = false;
+      if (more) start_tile();
+    } else if (more && staged_bf16_tile<TILE>(pr, m0, n0, out_kind, epilogue)) {
+      // the next tile's first products go out as the accumulators they overwrite are read out, in the shadow of
+      // the epilogue's vector arithmetic
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, scale_ab, scale_c,
+                                    [&fb0, &fa0](auto ic, auto jc) {
+                                      constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+                                      const i32x8 wf = fb0[j], tf = fa0[i];
+                                      FP8GMM_MFMA_Z(i, j, wf, tf);
+                                    });
     } else {
-      // free until the next step's token loads: the unit that held the last step's weights
-      relaxed = tile_epilogue<TILE>(acc, pr, m0, n0, out_kind, epilogue, lds + ((ua + 4) % RING) * US, !A_TR && !B_TR, scale_ab,
-                              scale_c);
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, scale_ab, scale_c);
+      if (more) start_tile();
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS
   FP8GMM_WAIT_VM(0);
-  clock_probe_mark(counters, 1);
 }
 
 
@@ -958,13 +1051,13 @@ int prepare_variant(int dev) {
 
 template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item* items_dev, int grid, int out_kind,
-                   int epilogue, uint8_t* workspace, uint64_t* counters, hipStream_t stream) {
+                   int epilogue, uint8_t* workspace, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
   const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR, TILE>(dev);
   if (rc != FP8GMM_OK) return rc;
   hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>), dim3(grid), dim3(NTHREADS),
-                     RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace, counters);
+                     RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
@@ -989,7 +1082,7 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item*
 #define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT, TL)                                                                     \
   extern template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                        \
   extern template int launch_variant<AF, BF, AT, BT, TL>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, \
-                                                         int, uint8_t*, uint64_t*, hipStream_t);
+                                                         int, uint8_t*, hipStream_t);
 #ifndef FP8GMM_VARIANT_INDEX
 FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_DECLARE_VARIANT)
 #endif

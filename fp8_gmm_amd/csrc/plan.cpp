@@ -297,6 +297,7 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
     return plan_small_tiles(probs, n, layout & ~FP8GMM_GEMM_TILE_128, grid, items, max_items, plan);
   }
   plan->tile = kGemmTileM;
+  const int layout_given = layout, grid_given = grid;
   const bool gelu = (layout & FP8GMM_EPI_GELU) != 0;  // only weighs the decision to share tiles along K
   layout &= ~FP8GMM_EPI_GELU;
   int total_tiles = 0;
@@ -338,6 +339,10 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
         for (int q = j; q < j + nf; ++q) slot_map[kSlotsPerWg * (x * wgs + q)] = n_slots++;
         fix.push_back(o);
       }
+  // a caller with a fixed amount of workspace (stream_k > 1 = its slots): whole tiles when sharing needs more
+  if (sk && stream_k > 1 && n_slots > stream_k)
+    return fp8gmm_plan_grouped_gemm_launch(probs, n, layout_given, grid_given, 0, items, max_items, fixups, max_fixups,
+                                           plan);
   const int room = max_items;   // as the caller stated it
   // One pass over the schedule: the records are written as they are counted, into whatever room the caller gave;
   // a list that does not fit is only counted, and the call then reports the sizes.

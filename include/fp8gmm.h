@@ -264,7 +264,9 @@ int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_bloc
  * fixups[0 .. n_fixups).  `layout` takes the launch's flags: the KMAJOR flags as for the plain plan, and
  * FP8GMM_EPI_GELU, which only weighs the decision below (completing a shared tile costs more with that epilogue).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
  * the last round would otherwise be mostly idle; the launch then needs plan->n_slots workspace slots (never more
- * than 2 * grid).  stream_k == 0: every record is a whole tile, no workspace, no fix-up launch.
+ * than 2 * grid).  stream_k > 1: the same, but with at most stream_k slots - a launch whose sharing would need more
+ * is planned with whole tiles instead (callers of fp8gmm_grouped_gemm_static pass FP8GMM_GEMM_STATIC_SLOTS and never
+ * see FP8GMM_ERR_WORKSPACE).  stream_k == 0: every record is a whole tile, no workspace, no fix-up launch.
  * The sizes are returned in *plan even when max_items / max_fixups are too small (FP8GMM_ERR_BUFFER_TOO_SMALL;
  * the arrays then hold the part of the list that fitted and are not to be used): call again with larger arrays.  Host only, no GPU needed.
  */
@@ -303,18 +305,6 @@ int fp8gmm_grouped_gemm(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gm
 int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
                                const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
                                int b_fmt, int out_kind, int epilogue, void* stream);
-
-/*
- * The same launch with a measurement on the side, no counterpart in the reference: `dev_counters` (device memory,
- * 8 x 4 uint64, one group of four per XCD, cleared by the caller) receives from the first workgroup of every XCD
- * {shader-cycle counter, 100 MHz counter} when it starts ([0], [1]) and the elapsed cycles and ticks added to
- * [2], [3] when it ends: [2] / [3] * 100 MHz is the clock the launch really ran at, which the clock the driver
- * reports overstates while the chip is power-limited.  Same kernel, same results; bench.py reports the figure.
- */
-int fp8gmm_grouped_gemm_timed(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
-                              const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
-                              int b_fmt, int out_kind, int epilogue, void* workspace, size_t workspace_bytes,
-                              uint64_t* dev_counters, void* stream);
 
 /*
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:

@@ -154,7 +154,6 @@ def test_launch_entry_points_validate_before_touching_the_gpu():
     assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, None, 0, None) == -9
     assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake, 2 * 262144 - 1, None) == -9
     assert lib.fp8gmm_grouped_gemm(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake + 8, 2 * 262144, None) == -9
-    assert lib.fp8gmm_grouped_gemm_timed(fake, 1, fake, fake, sk, 0, 0, 2, 0, fake, 2 * 262144, None, None) == -1
     assert b"workspace" in lib.fp8gmm_status_string(-9)
 
 

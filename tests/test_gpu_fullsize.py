@@ -160,14 +160,16 @@ def test_grouped_mlp_full_size_step(dev):
 
 
 def _bench_splits(kind, experts, tokens, seed):
-    """The split bench.py draws for its workloads (same generator, same seed)."""
-    rng = np.random.default_rng(seed)
-    if kind == "zipf":
-        p = 1.0 / np.arange(1, experts + 1) ** 1.1
-        p /= p.sum()
-    else:
-        p = np.full(experts, 1.0 / experts)
-    return [int(v) for v in rng.multinomial(tokens, p)]
+    """The split bench.py draws for its workloads (its own function: same generator, same seed, and for the Zipf
+    workload the same empty and tiny expert)."""
+    import importlib.util
+    import os
+
+    spec = importlib.util.spec_from_file_location(
+        "bench_for_splits", os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    return bench.splits(kind, experts, tokens, seed)
 
 
 def _slice_amax(t, bounds):
@@ -191,11 +193,7 @@ def test_config3_grouped_linear_seventeen_steps(dev):
     e, k, n, tokens, hist, steps = 64, 2048, 1408, 24576, 16, 18
     sizes = _bench_splits("zipf", e, tokens, 1003)
     assert sum(sizes) == tokens and len(sizes) == e
-    # the split bench.py uses has no empty expert and none under 16 rows by itself; this workload is defined
-    # by having both, so the two least popular experts hand their rows to the first
-    order = np.argsort(sizes)
-    sizes[0] += sizes[order[0]] + sizes[order[1]] - 7
-    sizes[order[0]], sizes[order[1]] = 0, 7
+    # this workload is defined by having an expert without rows and one with fewer than 16
     assert sum(sizes) == tokens and 0 in sizes and any(0 < s < 16 for s in sizes)
     bounds = _bounds(sizes)
     g = torch.Generator(device=dev).manual_seed(1003)

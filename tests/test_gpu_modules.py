@@ -449,7 +449,7 @@ def test_weight_gradient_on_a_transposed_gradient_copy_gives_the_same_bits(dev, 
         dy = randn_bf16((m, out_cols), g, 1e-2).to(dev)
         res = []
         for mod, mode in zip(mods, ("in_place", "copy")):
-            monkeypatch.setattr(backend, "_WGRAD", mode)
+            monkeypatch.setattr(backend.options, "wgrad", mode)
             xd = x.clone().requires_grad_()
             mod.zero_grad()
             with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
