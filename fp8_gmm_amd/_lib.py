@@ -111,6 +111,42 @@ class GemmPlan(ctypes.Structure):
                 ("reserved", ctypes.c_int32 * 2)]
 
 
+class LinearPass(ctypes.Structure):
+    """struct fp8gmm_linear_pass: one pass of a grouped linear layer, as the pass planner takes it"""
+
+    _fields_ = [("experts", ctypes.c_int32), ("in_features", ctypes.c_int32), ("out_features", ctypes.c_int32),
+                ("fwd_fmt", ctypes.c_int32), ("bwd_fmt", ctypes.c_int32), ("cast_weights", ctypes.c_int32),
+                ("dgrad", ctypes.c_int32), ("wgrad", ctypes.c_int32), ("grid", ctypes.c_int32),
+                ("stream_k", ctypes.c_int32), ("tile_policy", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("tokens", ctypes.c_int64), ("group_sizes", ctypes.c_void_p),
+                ("x", ctypes.c_void_p), ("x_fp8", ctypes.c_void_p), ("w", ctypes.c_void_p), ("w_fp8", ctypes.c_void_p),
+                ("y", ctypes.c_void_p), ("dy", ctypes.c_void_p), ("dy_fp8", ctypes.c_void_p), ("dx", ctypes.c_void_p),
+                ("dw", ctypes.c_void_p), ("fwd_scale", ctypes.c_void_p), ("fwd_scale_inv", ctypes.c_void_p),
+                ("fwd_amax", ctypes.c_void_p), ("bwd_scale", ctypes.c_void_p), ("bwd_scale_inv", ctypes.c_void_p),
+                ("bwd_amax", ctypes.c_void_p)]
+
+
+class PassLaunch(ctypes.Structure):
+    """struct fp8gmm_pass_launch"""
+
+    _fields_ = [("kind", ctypes.c_int32), ("op", ctypes.c_int32), ("n", ctypes.c_int32),
+                ("total_blocks", ctypes.c_int32), ("out_fmt", ctypes.c_int32), ("a_fmt", ctypes.c_int32),
+                ("b_fmt", ctypes.c_int32), ("out_kind", ctypes.c_int32), ("epilogue", ctypes.c_int32),
+                ("reserved", ctypes.c_int32), ("table_offset", ctypes.c_int64), ("items_offset", ctypes.c_int64),
+                ("fixups_offset", ctypes.c_int64), ("plan", GemmPlan), ("work", ctypes.c_double),
+                ("bytes", ctypes.c_double)]
+
+
+class PassPlan(ctypes.Structure):
+    """struct fp8gmm_pass_plan"""
+
+    _fields_ = [("n_launches", ctypes.c_int32), ("reserved", ctypes.c_int32), ("blob_bytes", ctypes.c_int64),
+                ("launch", PassLaunch * 4)]
+
+
+PASS_CAST = 1
+PASS_GEMM = 2
+
 EXPORTS = (
     "fp8gmm_version",
     "fp8gmm_status_string",
@@ -121,6 +157,11 @@ EXPORTS = (
     "fp8gmm_gemm_grid",
     "fp8gmm_plan_grouped_gemm_launch",
     "fp8gmm_grouped_gemm_static",
+    "fp8gmm_plan_linear_forward",
+    "fp8gmm_plan_linear_backward",
+    "fp8gmm_run_planned",
+    "fp8gmm_sizeof_linear_pass",
+    "fp8gmm_sizeof_pass_plan",
     "fp8gmm_gemm_tile_shape",
     "fp8gmm_plan_multi_tensor",
     "fp8gmm_plan_grouped_gemm",
@@ -208,6 +249,15 @@ def load():
     L.fp8gmm_grouped_gemm.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp, ctypes.c_size_t, vp]
     L.fp8gmm_grouped_gemm_static.restype = ci
     L.fp8gmm_grouped_gemm_static.argtypes = [vp, ci, vp, vp, pp, ci, ci, ci, ci, vp]
+    for fn in (L.fp8gmm_plan_linear_forward, L.fp8gmm_plan_linear_backward):
+        fn.restype = ci
+        fn.argtypes = [ctypes.POINTER(LinearPass), vp, ctypes.c_size_t, ctypes.POINTER(PassPlan)]
+    L.fp8gmm_run_planned.restype = ci
+    L.fp8gmm_run_planned.argtypes = [vp, ctypes.POINTER(PassLaunch), vp, ctypes.c_size_t, vp]
+    L.fp8gmm_sizeof_linear_pass.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_linear_pass.argtypes = []
+    L.fp8gmm_sizeof_pass_plan.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_pass_plan.argtypes = []
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t
@@ -227,7 +277,9 @@ def load():
     L.fp8gmm_gemm_fixup.restype = ci
     L.fp8gmm_gemm_fixup.argtypes = [vp, ci, ci, ci, ci, ip, vp, ci]
     if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize \
-            or L.fp8gmm_sizeof_gemm_item() != GEMM_ITEM.itemsize or ctypes.sizeof(GemmPlan) != 32:
+            or L.fp8gmm_sizeof_gemm_item() != GEMM_ITEM.itemsize or ctypes.sizeof(GemmPlan) != 32 \
+            or L.fp8gmm_sizeof_linear_pass() != ctypes.sizeof(LinearPass) \
+            or L.fp8gmm_sizeof_pass_plan() != ctypes.sizeof(PassPlan):
         raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
     _lib = L
     return L

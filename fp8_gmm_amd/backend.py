@@ -12,6 +12,7 @@ there is no fallback: without the HIP library the import fails.
 """
 import collections
 import contextlib
+import ctypes
 import threading
 
 import numpy as np
@@ -755,6 +756,65 @@ def warm_up(device=None):
     grid = _lib.gemm_grid(_lib.init(device.index))
     with _on_device(device):
         _gemm_workspace(device, 2 * grid)
+
+
+# ------------------------------------------------------------------------------------------------
+# a whole pass of a grouped linear layer, planned by one library call
+# ------------------------------------------------------------------------------------------------
+_PASS_KERNEL_NAMES = {_lib.PASS_CAST: "multi_quantize", _lib.PASS_GEMM: "grouped_gemm"}
+
+
+def linear_pass(device, backward=False, **fields):
+    """Plans one pass of a grouped linear layer with ONE library call (fp8gmm_plan_linear_forward / _backward),
+    uploads its tables with one copy and enqueues its launches.  ``fields`` are the members of
+    ``fp8gmm_linear_pass`` (include/fp8gmm.h): tensors are given as tensors (their addresses are taken here),
+    ``group_sizes`` as an int64 numpy array.  The tables are the ones the per-launch entry points of this module
+    build for the same tensors; what this call saves is the host time of building them in Python."""
+    L = _lib.load()
+    flush_uploads()   # launches queued before this pass come first
+    keep = []
+    desc = _lib.LinearPass()
+    for name, value in fields.items():
+        if isinstance(value, torch.Tensor):
+            keep.append(value)
+            value = value.data_ptr()
+        elif isinstance(value, np.ndarray):
+            keep.append(value)
+            value = value.ctypes.data
+        setattr(desc, name, value)
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    grid = _lib.gemm_grid(_lib.init(index))
+    desc.grid = grid
+    desc.stream_k = int(bool(options.stream_k))
+    desc.tile_policy = {"auto": 0, "256": 256, "128": 128}[options.tile]
+    # room for the tables: descriptors, problem tables and, per GEMM, a work list of at most one record per
+    # 128 x 128 tile plus a few rounds of end records
+    widest = max(desc.in_features, desc.out_features)
+    tiles = (desc.tokens // 128 + desc.experts) * ((widest + 127) // 128) + \
+        desc.experts * ((desc.in_features + 127) // 128) * ((desc.out_features + 127) // 128)
+    bound = 4096 + desc.experts * (2 * 128 + 3 * 96) + 3 * (tiles + 8 * grid) * 64 + 3 * 32 * 2 * grid
+    plan = _lib.PassPlan()
+    fn = L.fp8gmm_plan_linear_backward if backward else L.fp8gmm_plan_linear_forward
+    pinned = torch.empty(bound, dtype=torch.uint8, pin_memory=True)
+    rc = fn(ctypes.byref(desc), pinned.data_ptr(), bound, ctypes.byref(plan))
+    if rc == -8:   # FP8GMM_ERR_BUFFER_TOO_SMALL: the plan says how much room it needs
+        bound = int(plan.blob_bytes)
+        pinned = torch.empty(bound, dtype=torch.uint8, pin_memory=True)
+        rc = fn(ctypes.byref(desc), pinned.data_ptr(), bound, ctypes.byref(plan))
+    _lib.check(rc)
+    with _on_device(device):
+        blob = pinned[: plan.blob_bytes].to(device, non_blocking=True)
+        base, stream = blob.data_ptr(), _stream(device)
+        for i in range(plan.n_launches):
+            rec = plan.launch[i]
+            if rec.kind == 0:
+                continue
+            ws = _gemm_workspace(device, rec.plan.n_slots) if rec.kind == _lib.PASS_GEMM else None
+            ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
+            with _timed(_PASS_KERNEL_NAMES[rec.kind], lambda: rec.work, lambda: rec.bytes):
+                rc = L.fp8gmm_run_planned(base, ctypes.byref(rec), ws_ptr, ws_bytes, stream)
+            _lib.check(rc)
+    return plan, pinned
 
 
 def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False, keep_scale_inv=None):

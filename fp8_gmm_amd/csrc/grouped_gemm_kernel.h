@@ -801,8 +801,8 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   asm volatile("v_mfma_f32_32x32x64_f8f6f4 a[%2:%3], %0, %1, 0 cbsz:%4 blgp:%5" ::"v"(FB), "v"(FA),      \
                "n"(16 * (NT * (i) + (j))), "n"(16 * (NT * (i) + (j)) + 15), "n"(B_FMT), "n"(A_FMT))
 #else  // the host pass only needs the kernel's signature (and cannot take 32-byte vectors as "v" operands)
-#define FP8GMM_MFMA(i, j, FB, FA) (void)0
-#define FP8GMM_MFMA_Z(i, j, FB, FA) (void)0
+#define FP8GMM_MFMA(i, j, FB, FA) ((void)(FB), (void)(FA))
+#define FP8GMM_MFMA_Z(i, j, FB, FA) ((void)(FB), (void)(FA))
 #endif
 // FIRST (of the enclosing step): the first step of a tile, whose low-half products have been issued already - from
 // inside the previous tile's epilogue, or by start_tile

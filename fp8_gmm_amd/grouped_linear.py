@@ -24,8 +24,9 @@ import math
 import numpy as np
 import torch
 
-from .backend import (TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, multi_cast_transpose, multi_quantize,
-                      wgrad_wants_transposed_gradient)
+from . import _lib
+from .backend import (TensorBatch, batched_uploads, fp8_gmm, grouped_gemm, linear_pass, multi_cast_transpose,
+                      multi_quantize, wgrad_wants_transposed_gradient)
 from .fp8 import Fp8GroupedModuleBase, Fp8WeightCache, get_fp8_te_dtype
 from .utils import PAD_MULTIPLE, Fp8MetaWrapper, Fp8TensorType, MetaTensorType, cumsum_group_sizes, to_torch_dtype
 
@@ -129,6 +130,46 @@ class _GroupedLinear(torch.autograd.Function):
         fp8_dtype = to_torch_dtype(fwd_dtype)
         dev = input.device
 
+        if fp8_meta.get("planned_passes", True) and not reference_layout and not cutlass and input.is_cuda and input.is_contiguous() and weight.is_contiguous() \
+                and input.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
+            # The default data flow as one planned pass: every table of the cast launch and of the GEMM comes out of
+            # one library call (with 64 experts the array arithmetic below costs more host time than the kernels run).
+            sizes = np.diff(np.asarray(cumsums, dtype=np.int64))
+            input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
+            if weight_cache is None:
+                weight_fp8, cast_weights = torch.empty(weight.shape, dtype=fp8_dtype, device=dev), True
+            else:
+                weight_fp8, _ = weight_cache.buffers(weight, fp8_dtype, False)
+                cast_weights = bool(update_fp8_weights)
+                if cast_weights:
+                    weight_cache.valid, weight_cache.valid_t = True, False
+                else:
+                    weight_cache.require(False)
+            out = torch.empty(input.size(0), weight.size(1), dtype=torch.bfloat16, device=dev)
+            fwd = fp8_meta["scaling_fwd"]
+            linear_pass(dev, False, experts=num_groups, in_features=weight.size(2), out_features=weight.size(1),
+                        fwd_fmt=_lib.E4M3 if fp8_dtype == torch.float8_e4m3fn else _lib.E5M2, cast_weights=cast_weights,
+                        tokens=input.size(0), group_sizes=sizes, x=input, x_fp8=input_fp8, w=weight, w_fp8=weight_fp8,
+                        y=out, fwd_scale=fwd.scale, fwd_scale_inv=fwd.scale_inv, fwd_amax=fwd.amax_history)
+            if is_grad_enabled:
+                ctx.save_for_backward(input_fp8 if wgrad_needed else None, weight_fp8 if dgrad_needed else None)
+                ctx.reference_layout = False
+                ctx.planned = True
+                ctx.sizes = sizes
+                ctx.group_sizes = group_sizes
+                meta.set_forward_scale_inv_cloned()
+                ctx.meta = meta
+                ctx.num_groups = num_groups
+                ctx.padded = padded
+                ctx.cumsums = cumsums
+                ctx.padded_cumsums = padded_cumsums
+                ctx.fp8_meta = fp8_meta
+                ctx.weight_shape = weight.shape
+                ctx.input_requires_grad = input.requires_grad
+                ctx.weight_requires_grad = weight.requires_grad
+                ctx.cutlass = cutlass
+            return out
+
         plain = ([], [], [], [])            # inputs, outputs, scales, amaxes for cast only
         with_t = ([], [], [], [], [])       # inputs, outputs, transposes, scales, amaxes
 
@@ -173,6 +214,7 @@ class _GroupedLinear(torch.autograd.Function):
             else:
                 ctx.save_for_backward(input_fp8 if wgrad_needed else None, weight_fp8 if dgrad_needed else None)
             ctx.reference_layout = reference_layout
+            ctx.planned = False
             ctx.group_sizes = group_sizes
             meta.set_forward_scale_inv_cloned()
             ctx.meta = meta
@@ -195,6 +237,26 @@ class _GroupedLinear(torch.autograd.Function):
         grad_dtype = to_torch_dtype(get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=False))
         grad_out = grad_out.contiguous()
         dev = grad_out.device
+
+        if ctx.planned and not wgrad_wants_transposed_gradient(cumsums[-1], ctx.num_groups) \
+                and grad_out.dtype == torch.bfloat16 and (ctx.input_requires_grad or ctx.weight_requires_grad):
+            e, n, k = ctx.weight_shape
+            grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
+            grad_input = torch.empty(grad_out.size(0), k, dtype=torch.bfloat16, device=dev) \
+                if ctx.input_requires_grad else None
+            grad_weight = torch.empty(ctx.weight_shape, dtype=torch.bfloat16, device=dev) \
+                if ctx.weight_requires_grad else None
+            bwd = ctx.fp8_meta["scaling_bwd"]
+            fwd_fmt = get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=True)
+            linear_pass(dev, True, experts=e, in_features=k, out_features=n,
+                        fwd_fmt=_lib.E4M3 if to_torch_dtype(fwd_fmt) == torch.float8_e4m3fn else _lib.E5M2,
+                        bwd_fmt=_lib.E4M3 if grad_dtype == torch.float8_e4m3fn else _lib.E5M2,
+                        dgrad=int(ctx.input_requires_grad), wgrad=int(ctx.weight_requires_grad),
+                        tokens=grad_out.size(0), group_sizes=ctx.sizes, dy=grad_out, dy_fp8=grad_out_fp8,
+                        x_fp8=input_for_wgrad, w_fp8=weight_for_dgrad, dx=grad_input, dw=grad_weight,
+                        fwd_scale_inv=meta._forward_scale_inv_cloned, bwd_scale=bwd.scale,
+                        bwd_scale_inv=bwd.scale_inv, bwd_amax=bwd.amax_history)
+            return grad_input, grad_weight, None, None, None, None, None, None
 
         g_scales = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kScale)
         g_amaxes = meta.get_meta_pointers(Fp8TensorType.kGradOutputGroup1, MetaTensorType.kAmax)
@@ -253,15 +315,18 @@ class GroupedLinear(Fp8GroupedModuleBase):
     data-gradient GEMM and zero-padded transposed fp8 activations / gradients for the weight-gradient GEMM.  By
     default those GEMMs read the row-major fp8 tensors in place and none of the copies is cast: same results bit
     for bit, less memory traffic, no padding.
+    ``planned_passes=False`` builds the tables of every launch in Python through the per-launch entry points of
+    ``backend`` (the same tables, several times the host time).
     ``is_first_microbatch``: None casts the weights to fp8 on every pass; True casts them into buffers the
     module keeps; False reuses those buffers (gradient accumulation over micro-batches of one optimizer step).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda", cutlass=False,
-                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False):
+                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False, planned_passes=True):
         super().__init__()
         self.fp8_meta["pad_multiple"] = pad_multiple
         self.fp8_meta["reference_layout"] = reference_layout
+        self.fp8_meta["planned_passes"] = planned_passes
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.in_features = in_features
         self.out_features = out_features

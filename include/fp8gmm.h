@@ -306,6 +306,89 @@ int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, cons
                                const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt,
                                int b_fmt, int out_kind, int epilogue, void* stream);
 
+/* ---- a whole pass of a grouped linear layer, planned by one call ---------------------------- */
+/*
+ * The launches of one pass of a grouped linear layer (E experts, in_features -> out_features, token-sorted rows) in
+ * the default data flow: activations, gradients and weights are cast to fp8 once, row-major, and every GEMM reads
+ * them in place.
+ *   forward : cast x (and, unless cast_weights == 0, the weights) ; y[rows_i] = x_fp8[rows_i] . w_fp8[i]^T
+ *   backward: cast dy ; dx[rows_i] = dy_fp8[rows_i] . w_fp8[i]  (dgrad != 0) ; dw[i] = dy_fp8[rows_i]^T . x_fp8[rows_i]
+ *             (wgrad != 0)
+ * replaces, for that data flow, the per-expert host loops of fp8_gmm/grouped_linear.py:109-188 and the argument
+ * packing of csrc/fp8_gmm.cu:115-135 and csrc/multi_pad_fusion.cu:455-502.  The scaling metadata is addressed
+ * through the bases of the flat fp32 arrays in TransformerEngine's slot layout, which the reference indexes in
+ * fp8_gmm/utils.py:98-103: forward slots 3 i (input of expert i) and 3 i + 1 (its weight), backward slot 2 i (its
+ * output gradient).  For the backward pass fwd_scale_inv is the copy of the forward scale_inv taken after the
+ * forward pass.  All data pointers are device pointers that are only stored, never dereferenced, by the planner.
+ */
+typedef struct fp8gmm_linear_pass {
+  int32_t experts, in_features, out_features;
+  int32_t fwd_fmt, bwd_fmt;          /* FP8GMM_E4M3 / FP8GMM_E5M2 of forward tensors and of gradients */
+  int32_t cast_weights;              /* forward: 0 when w_fp8 already holds the cast weights (cached) */
+  int32_t dgrad, wgrad;              /* backward: which gradients are wanted */
+  int32_t grid;                      /* fp8gmm_gemm_grid() of the device */
+  int32_t stream_k;                  /* as for fp8gmm_plan_grouped_gemm_launch */
+  int32_t tile_policy;               /* 0: the library chooses per launch; 256 or 128: that tile for every launch */
+  int32_t reserved;
+  int64_t tokens;                    /* rows of x / dy: must equal the sum of group_sizes */
+  const int64_t* group_sizes;        /* HOST array [experts] */
+  const void* x;                     /* bf16 [tokens, in_features] */
+  void* x_fp8;                       /* fp8  [tokens, in_features] */
+  const void* w;                     /* bf16 [experts, out_features, in_features] */
+  void* w_fp8;                       /* fp8, same shape */
+  void* y;                           /* bf16 [tokens, out_features] */
+  const void* dy;                    /* bf16 [tokens, out_features] */
+  void* dy_fp8;                      /* fp8, same shape */
+  void* dx;                          /* bf16 [tokens, in_features] */
+  void* dw;                          /* bf16 [experts, out_features, in_features] */
+  const float* fwd_scale;
+  const float* fwd_scale_inv;
+  float* fwd_amax;                   /* row 0 of the forward amax history */
+  const float* bwd_scale;
+  const float* bwd_scale_inv;
+  float* bwd_amax;
+} fp8gmm_linear_pass;
+
+#define FP8GMM_PASS_NOTHING 0   /* a launch that turned out empty (no rows at all) */
+#define FP8GMM_PASS_CAST 1
+#define FP8GMM_PASS_GEMM 2
+/* One launch of a planned pass; offsets are bytes from the start of the blob. */
+typedef struct fp8gmm_pass_launch {
+  int32_t kind;                  /* FP8GMM_PASS_* */
+  int32_t op;                    /* cast: FP8GMM_OP_* */
+  int32_t n;                     /* descriptors / problems */
+  int32_t total_blocks;          /* cast: workgroups */
+  int32_t out_fmt;               /* cast: fp8 format written */
+  int32_t a_fmt, b_fmt, out_kind, epilogue;   /* GEMM: the arguments of fp8gmm_grouped_gemm */
+  int32_t reserved;
+  int64_t table_offset;          /* descriptors / problem table */
+  int64_t items_offset;          /* GEMM: work list */
+  int64_t fixups_offset;         /* GEMM: shared-tile records */
+  fp8gmm_gemm_plan plan;         /* GEMM */
+  double work;                   /* algorithmic flops (GEMM) or bytes (cast) of the launch */
+  double bytes;                  /* algorithmic bytes: every operand read once, every result written once */
+} fp8gmm_pass_launch;
+typedef struct fp8gmm_pass_plan {
+  int32_t n_launches;
+  int32_t reserved;
+  int64_t blob_bytes;            /* bytes of the blob in use: what has to be uploaded */
+  fp8gmm_pass_launch launch[4];
+} fp8gmm_pass_plan;
+size_t fp8gmm_sizeof_linear_pass(void);
+size_t fp8gmm_sizeof_pass_plan(void);
+/*
+ * Write every table of the pass into `blob` (host memory, preferably pinned, 128-byte aligned; blob_bytes its
+ * capacity) and describe the launches in *out.  FP8GMM_ERR_BUFFER_TOO_SMALL: out->blob_bytes says how much room the
+ * pass needs; call again.  The tables are those that the per-launch planning calls produce for the same tensors.
+ * Host only, no GPU needed.
+ */
+int fp8gmm_plan_linear_forward(const fp8gmm_linear_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
+int fp8gmm_plan_linear_backward(const fp8gmm_linear_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
+/* Enqueue one launch of a planned pass; blob_dev is the DEVICE copy of the blob (the cast launch writes into its
+ * descriptors, so every pass uploads afresh); workspace as for fp8gmm_grouped_gemm. */
+int fp8gmm_run_planned(const void* blob_dev, const fp8gmm_pass_launch* launch, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
 /*
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:
  *   amax = max over the `history_len` rows of amax_history[history_len, slots] (most_recent != 0: row 0)

@@ -459,3 +459,110 @@ def test_weight_gradient_on_a_transposed_gradient_copy_gives_the_same_bits(dev, 
         for a, b in zip(*res):
             assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}"
         assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("sizes", [[137, 0, 59, 403, 1, 700], [0, 0, 16], [300] * 9])
+def test_planned_passes_equal_the_per_launch_path(dev, sizes):
+    """GroupedLinear plans a whole pass with one library call (fp8gmm_plan_linear_forward / _backward).  Outputs,
+    gradients, fp8 scaling state and amax history must equal, bit for bit, what the per-launch entry points give
+    over three steps (ragged, empty and equal experts; with cached fp8 weights on the last step)."""
+    import fp8_gmm_amd as pkg
+
+    e, k, n = len(sizes), 256, 384
+    g = torch.Generator(device=dev).manual_seed(5)
+    w = (torch.randn(e, n, k, generator=g, device=dev) * 0.02).to(torch.bfloat16)
+    xs = [torch.randn(sum(sizes), k, generator=g, device=dev).to(torch.bfloat16) for _ in range(3)]
+    dys = [(torch.randn(sum(sizes), n, generator=g, device=dev) * 1e-2).to(torch.bfloat16) for _ in range(3)]
+    results = []
+    for planned in (True, False):
+        module = pkg.GroupedLinear(k, n, e, torch.bfloat16, device=dev, planned_passes=planned)
+        module.weight_tensor.data.copy_(w)
+        recipe = pkg.DelayedScaling(amax_history_len=2)
+        trace = []
+        for step, first in enumerate((None, True, False)):
+            x = xs[step].clone().requires_grad_()
+            module.zero_grad(set_to_none=True)
+            with pkg.fp8_autocast(enabled=True, fp8_recipe=recipe):
+                out = module(x, torch.tensor(sizes), is_first_microbatch=first)
+            out.backward(dys[step])
+            torch.cuda.synchronize()
+            fwd, bwd = module.fp8_meta["scaling_fwd"], module.fp8_meta["scaling_bwd"]
+            trace.append([out.detach().clone(), x.grad.clone(), module.weight_tensor.grad.clone(), fwd.scale.clone(),
+                          fwd.amax_history.clone(), bwd.scale.clone(), bwd.amax_history.clone()])
+        results.append(trace)
+    names = ["out", "grad_input", "grad_weight", "fwd scale", "fwd amax history", "bwd scale", "bwd amax history"]
+    for step, (a, b) in enumerate(zip(*results)):
+        for name, ta, tb in zip(names, a, b):
+            assert torch.equal(ta.view(torch.int16) if ta.dtype == torch.bfloat16 else ta,
+                               tb.view(torch.int16) if tb.dtype == torch.bfloat16 else tb), f"step {step}: {name}"
+
+
+@pytest.mark.gpu
+def test_planned_pass_tables_are_those_of_the_per_launch_entry_points(dev, monkeypatch):
+    """The tables fp8gmm_plan_linear_forward / _backward write for given buffers must be, byte for byte, the tensor
+    descriptors, problem tables, work lists and shared-tile records that backend.multi_quantize / fp8_gmm /
+    grouped_gemm build for the same buffers (captured here without launching anything)."""
+    import ctypes
+
+    import numpy as np
+
+    from fp8_gmm_amd import _lib, backend
+
+    sizes = [700, 0, 33, 1291, 5, 256]
+    e, k, n, tokens = len(sizes), 512, 768, sum(sizes)
+    E4, E5 = torch.float8_e4m3fn, torch.float8_e5m2
+    x = torch.zeros(tokens, k, dtype=torch.bfloat16, device=dev)
+    w = torch.zeros(e, n, k, dtype=torch.bfloat16, device=dev)
+    x8, w8 = torch.zeros(tokens, k, dtype=E4, device=dev), torch.zeros(e, n, k, dtype=E4, device=dev)
+    y = torch.zeros(tokens, n, dtype=torch.bfloat16, device=dev)
+    dy, dy8 = torch.zeros(tokens, n, dtype=torch.bfloat16, device=dev), torch.zeros(tokens, n, dtype=E5, device=dev)
+    dx, dw = torch.zeros(tokens, k, dtype=torch.bfloat16, device=dev), torch.zeros(e, n, k, dtype=torch.bfloat16, device=dev)
+    fs, fsi, fa = (torch.ones(3 * e, device=dev) for _ in range(3))
+    bs, bsi, ba = (torch.ones(2 * e, device=dev) for _ in range(3))
+    bounds = np.concatenate([[0], np.cumsum(sizes)])
+    ptr = lambda t, first, stride: np.uint64(t.data_ptr() + 4 * first) + np.arange(e, dtype=np.uint64) * np.uint64(4 * stride)
+    rows, stack = backend.TensorBatch.rows_of, backend.TensorBatch.stack_of
+
+    captured = []
+    monkeypatch.setattr(backend, "_flush", lambda items: captured.extend(bytes(it[0].view(np.uint8).reshape(-1)) for it in items))
+    with backend.batched_uploads():
+        backend.multi_quantize(rows(x, bounds) + stack(w), rows(x8, bounds) + stack(w8),
+                               np.concatenate([ptr(fs, 0, 3), ptr(fs, 1, 3)]), np.concatenate([ptr(fa, 0, 3), ptr(fa, 1, 3)]))
+        backend.fp8_gmm(x8, w8, sizes, ptr(fsi, 0, 3), ptr(fsi, 1, 3), c=y)
+        backend.multi_quantize(rows(dy, bounds), rows(dy8, bounds), ptr(bs, 0, 2), ptr(ba, 0, 2))
+        backend.fp8_gmm(dy8, w8, sizes, ptr(bsi, 0, 2), ptr(fsi, 1, 3), c=dx, backward=True, b_transposed=True)
+        backend.grouped_gemm(rows(dy8, bounds), rows(x8, bounds), stack(dw), ptr(bsi, 0, 2), ptr(fsi, 0, 3), transposed=True)
+    assert len(captured) == 5
+
+    grid = _lib.gemm_grid(_lib.init(torch.cuda.current_device()))
+    gs = np.asarray(sizes, dtype=np.int64)
+    desc = _lib.LinearPass(experts=e, in_features=k, out_features=n, fwd_fmt=_lib.E4M3, bwd_fmt=_lib.E5M2, cast_weights=1,
+                           dgrad=1, wgrad=1, grid=grid, stream_k=int(backend.options.stream_k), tile_policy=0, tokens=tokens,
+                           group_sizes=gs.ctypes.data, x=x.data_ptr(), x_fp8=x8.data_ptr(), w=w.data_ptr(),
+                           w_fp8=w8.data_ptr(), y=y.data_ptr(), dy=dy.data_ptr(), dy_fp8=dy8.data_ptr(), dx=dx.data_ptr(),
+                           dw=dw.data_ptr(), fwd_scale=fs.data_ptr(), fwd_scale_inv=fsi.data_ptr(), fwd_amax=fa.data_ptr(),
+                           bwd_scale=bs.data_ptr(), bwd_scale_inv=bsi.data_ptr(), bwd_amax=ba.data_ptr())
+    L = _lib.load()
+    blob = np.zeros(1 << 22, dtype=np.uint8)
+    want = iter(captured)
+    for fn in (L.fp8gmm_plan_linear_forward, L.fp8gmm_plan_linear_backward):
+        plan = _lib.PassPlan()
+        # a blob that is too small reports the size the pass needs
+        assert fn(ctypes.byref(desc), blob.ctypes.data, 1024, ctypes.byref(plan)) == -8
+        need = plan.blob_bytes
+        _lib.check(fn(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+        assert plan.blob_bytes == need
+        for i in range(plan.n_launches):
+            rec, ref = plan.launch[i], next(want)
+            if rec.kind == _lib.PASS_CAST:
+                got = bytes(blob[rec.table_offset: rec.table_offset + rec.n * 128])
+                assert got == ref, "tensor descriptors differ"
+            else:
+                probs = bytes(blob[rec.table_offset: rec.table_offset + rec.n * 96])
+                items = bytes(blob[rec.items_offset: rec.items_offset + rec.plan.rounds * rec.plan.grid * 64])
+                fix = bytes(blob[rec.fixups_offset: rec.fixups_offset + rec.plan.n_fixups * 32])
+                off_items = (rec.n * 96 + 127) // 128 * 128
+                assert probs == ref[: rec.n * 96], "problem table differs"
+                assert items == ref[off_items: off_items + len(items)], "work list differs"
+                assert fix == ref[off_items + len(items):], "shared-tile records differ"
