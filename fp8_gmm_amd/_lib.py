@@ -18,6 +18,7 @@ E4M3 = 0
 E5M2 = 1
 OUT_BF16 = 2
 EPI_GELU = 1
+EPI_DGELU = 8
 GEMM_B_KMAJOR = 2
 GEMM_A_KMAJOR = 4
 GEMM_TILE_128 = 0x100   # planning flag: 128 x 128 tiles, two workgroups per compute unit

@@ -618,7 +618,7 @@ def multi_cast_dgelu(inputs, gelu_inputs, outputs, scales, amaxes):
 # ------------------------------------------------------------------------------------------------
 # GEMMs
 # ------------------------------------------------------------------------------------------------
-def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=False, a_kmajor=False):
+def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=False, a_kmajor=False, dgelu=False):
     if a_dtype not in _FP8_DTYPES or b_dtype not in _FP8_DTYPES:
         _fail("fp8_gmm_amd: GEMM operands must be fp8")
     if a_dtype == torch.float8_e5m2 and b_dtype == torch.float8_e5m2:
@@ -629,15 +629,15 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
         _fail("fp8_gmm_amd: a contraction-major b must be float8_e4m3fn")
     layout = (_lib.GEMM_B_KMAJOR if b_kmajor else 0) | (_lib.GEMM_A_KMAJOR if a_kmajor else 0)
     grid = _lib.gemm_grid(_lib.init(device.index if device.index is not None else torch.cuda.current_device()))
-    if not gelu and _small_tiles(table):
+    epi = _lib.EPI_GELU if gelu else _lib.EPI_DGELU if dgelu else 0
+    if not epi and _small_tiles(table):
         plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
     else:
-        plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | (_lib.EPI_GELU if gelu else 0),
-                                                                     grid, options.stream_k)
+        plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | epi, grid, options.stream_k)
     if plan.total_tiles == 0:
         return
     n = len(table)
-    fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], (_lib.EPI_GELU if gelu else 0) | layout)
+    fmts = (_FMT[a_dtype], _FMT[b_dtype], _OUT_KIND[c_dtype], epi | layout)
 
     def launch(dev_ptr):
         with _on_device(device):
@@ -929,7 +929,7 @@ def _group_sizes_list(group_sizes):
 
 
 def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch.bfloat16, pre_gelu_out=None,
-            c_scales=None, c_amaxes=None, backward=False, cutlass=False, b_transposed=False):
+            c_scales=None, c_amaxes=None, backward=False, cutlass=False, b_transposed=False, dgelu_pre=None):
     """Grouped GEMM over row slices of ``a``: expert i multiplies rows
     ``[sum(group_sizes[:i]), sum(group_sizes[:i+1]))`` of ``a[tokens, k]`` with ``b[i][n, k]^T``.
 
@@ -942,6 +942,12 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     ``b_transposed=True`` (not in the reference): ``b`` is ``[experts, k, n]`` and expert i multiplies with
     ``b[i]`` as it stands.  That is a forward weight stack used by the data-gradient GEMM without the transposed
     copy the reference casts for it (grouped_linear.py:69-74,163); same results, bit for bit.
+
+    ``dgelu_pre`` (not in the reference, which notes the missing fusion at grouped_mlp.py:252-253): a bf16
+    ``[tokens, n]`` pre-GELU activation; the result is multiplied by ``dgelu_tanh(dgelu_pre)`` in the GEMM's epilogue
+    before the one rounding to ``c``'s type.  With an fp8 ``c`` this is the fc2 data-gradient GEMM and the
+    cast + dGELU pass behind it in one kernel; the product is formed from the fp32 accumulator, where the separate
+    pass starts from the bf16-rounded gradient.
     """
     sizes = _group_sizes_list(group_sizes)
     e = len(sizes)
@@ -969,7 +975,12 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
         or not pre_gelu_out.is_contiguous()
     ):
         _fail("fp8_gmm_amd: pre_gelu_out must be a contiguous bf16 [tokens, n] tensor")
-    dev = _device_of([a, b, c, pre_gelu_out])
+    if dgelu_pre is not None:
+        if pre_gelu_out is not None or cutlass:
+            _fail("fp8_gmm_amd: dgelu_pre excludes pre_gelu_out and cutlass=True")
+        if dgelu_pre.dtype != torch.bfloat16 or tuple(dgelu_pre.shape) != (tokens, nn) or not dgelu_pre.is_contiguous():
+            _fail("fp8_gmm_amd: dgelu_pre must be a contiguous bf16 [tokens, n] tensor")
+    dev = _device_of([a, b, c, pre_gelu_out, dgelu_pre])
 
     starts = np.zeros(e + 1, dtype=np.int64)
     np.cumsum(np.asarray(sizes, dtype=np.int64), out=starts[1:])
@@ -980,6 +991,8 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
     table["c"] = c.data_ptr() + row0 * np.uint64(nn * c.element_size())
     if pre_gelu_out is not None:
         table["aux"] = pre_gelu_out.data_ptr() + row0 * np.uint64(nn * 2)
+    if dgelu_pre is not None:
+        table["aux"] = dgelu_pre.data_ptr() + row0 * np.uint64(nn * 2)
     table["m"] = np.asarray(sizes, dtype=np.int32)
     table["n"] = nn
     table["k"] = k
@@ -993,7 +1006,8 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
         table["c_scale"] = _scalar_ptrs(c_scales, e, "c_scales")
         table["c_amax"] = _scalar_ptrs(c_amaxes, e, "c_amaxes")
     _launch_gemm(table, a.dtype, b.dtype, c.dtype, pre_gelu_out is not None, dev,
-                 (a, b, c, pre_gelu_out, a_scale_invs, b_scale_invs, c_scales, c_amaxes), b_kmajor=b_transposed)
+                 (a, b, c, pre_gelu_out, dgelu_pre, a_scale_invs, b_scale_invs, c_scales, c_amaxes),
+                 b_kmajor=b_transposed, dgelu=dgelu_pre is not None)
     if cutlass:
         multi_scale_mul(TensorBatch.rows_of(c, starts), a_scale_invs, b_scale_invs)
     return c

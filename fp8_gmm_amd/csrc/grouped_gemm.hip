@@ -63,6 +63,7 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
   const float sb_inv = pr.b_scale_inv ? *pr.b_scale_inv : 1.f;
   const float s = sa_inv * sb_inv;
   const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
+  const bool dgelu_in = (epilogue & FP8GMM_EPI_DGELU) != 0 && pr.aux != nullptr;   // aux is then an input
   const int64_t ldc = pr.ldc;
   uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
   const bool aux_ok = AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0;
@@ -81,6 +82,11 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
       r[e] = gelu ? gelu_tanh_fast(v[e]) : v[e];
     }
     const int64_t off = (int64_t)m * ldc + n;
+    if (dgelu_in) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < N) r[e] = v[e] * dgelu(bf16_to_f32(AUX[off + e]));
+    }
     if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       const bool vec = ((ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(C) & 7) == 0) && aux_ok;
@@ -189,7 +195,9 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
   if (n < 0 || plan->total_tiles < 0 || plan->rounds < 0 || plan->n_fixups < 0 || plan->n_slots < 0)
     return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_kind != FP8GMM_OUT_BF16 && out_kind != FP8GMM_E4M3 && out_kind != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
-  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR)) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (epilogue & ~(FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU | FP8GMM_GEMM_A_KMAJOR | FP8GMM_GEMM_B_KMAJOR))
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if ((epilogue & FP8GMM_EPI_GELU) && (epilogue & FP8GMM_EPI_DGELU)) return FP8GMM_ERR_BAD_ARGUMENT;
   const bool a_kmajor = (epilogue & FP8GMM_GEMM_A_KMAJOR) != 0;
   const bool b_kmajor = (epilogue & FP8GMM_GEMM_B_KMAJOR) != 0;
   if (a_kmajor && !b_kmajor) return FP8GMM_ERR_BAD_ARGUMENT;
@@ -200,7 +208,8 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
   const int tile = plan->tile == 0 ? kGemmTileM : plan->tile;
   if (tile != kGemmTileM && tile != FP8GMM_GEMM_SMALL_TILE) return FP8GMM_ERR_BAD_ARGUMENT;
   // the small tile is never shared along K and has no fused GELU epilogue
-  if (tile != kGemmTileM && (plan->n_slots != 0 || plan->n_fixups != 0 || (epilogue & FP8GMM_EPI_GELU)))
+  if (tile != kGemmTileM &&
+      (plan->n_slots != 0 || plan->n_fixups != 0 || (epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU))))
     return FP8GMM_ERR_BAD_ARGUMENT;
   const launch_fn launch = variant_for(a_fmt, b_fmt, a_kmajor, b_kmajor, tile);
   if (launch == nullptr) return FP8GMM_ERR_BAD_FORMAT;
@@ -212,12 +221,13 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
                             (reinterpret_cast<uintptr_t>(workspace) & 255) != 0))
     return FP8GMM_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int rc = launch(probs_dev, items_dev, plan->grid, out_kind, epilogue & FP8GMM_EPI_GELU,
+  const int rc = launch(probs_dev, items_dev, plan->grid, out_kind, epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU),
                         static_cast<uint8_t*>(workspace), s);
   if (rc != FP8GMM_OK) return rc;
   if (plan->n_fixups > 0) {
     hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups * kFixupSplit), dim3(kFixupThreads), 0, s, probs_dev,
-                       fixups_dev, out_kind, epilogue & FP8GMM_EPI_GELU, static_cast<const uint8_t*>(workspace));
+                       fixups_dev, out_kind, epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU),
+                       static_cast<const uint8_t*>(workspace));
     if (hipGetLastError() != hipSuccess) return FP8GMM_ERR_LAUNCH;
   }
   return FP8GMM_OK;

@@ -178,7 +178,8 @@ __device__ __forceinline__ void merge_amax(float* slot, float wave_amax, int lan
 // stores, amax.  Returns true when the staged bf16 path ran (exactly kFastStores stores per wavefront).
 // `stage`: 32 KB of LDS that no wavefront reads or loads into until the barrier at the end of the staged path.
 // `oob_zero`: accumulators of rows past m and columns past n are exactly zero (both operands row-major: what
-// lies outside the tile's rows is outside the load descriptors).
+// lies outside the tile's rows is outside the load descriptors); `oob_rows_zero`: those of rows past m are
+// (operand a row-major).
 //
 // The staged paths store through a buffer descriptor that spans the tile's valid rows: rows past m fall outside
 // it and are dropped by the hardware, lanes whose columns lie past n carry an offset beyond any descriptor.
@@ -199,7 +200,8 @@ __device__ __forceinline__ bool staged_bf16_tile(const fp8gmm_gemm_problem& pr, 
   const bool interior = (m0 + TILE <= pr.m) && (n0 + TILE <= pr.n);
   const int cv = pr.n - n0 < TILE ? pr.n - n0 : TILE;
   const bool desc_ok = ((ldc & 7) == 0) && ldc < (1 << 21) && ((reinterpret_cast<uintptr_t>(pr.c) & 15) == 0);
-  return out_kind == FP8GMM_OUT_BF16 && !(epilogue & FP8GMM_EPI_GELU) && desc_ok && (interior || (cv & 7) == 0);
+  return out_kind == FP8GMM_OUT_BF16 && !(epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU)) && desc_ok &&
+         (interior || (cv & 7) == 0);
 }
 struct NothingReleased {
   template <class I, class J>
@@ -207,7 +209,7 @@ struct NothingReleased {
 };
 template <int TILE, class Released = NothingReleased>
 __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int m0, int n0, int out_kind, int epilogue,
-                                              uint8_t* stage, bool oob_zero, float s, float cs,
+                                              uint8_t* stage, bool oob_zero, bool oob_rows_zero, float s, float cs,
                                               Released released = Released()) {
   constexpr int BM = TILE, BN = TILE, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
   constexpr int kStageBytes = TILE * 32;   // per wavefront: a quarter of one ring unit
@@ -223,6 +225,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
   const int M = pr.m, N = pr.n;
   bool fast = false;
     const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
+    const bool dgelu_in = (epilogue & FP8GMM_EPI_DGELU) != 0 && pr.aux != nullptr;   // aux is then an INPUT
     const int64_t ldc = pr.ldc;
     float amax = 0.f;
     const bool interior = (m0 + BM <= M) && (n0 + BN <= N);
@@ -388,6 +391,75 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
       });
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
       merge_amax(pr.c_amax, wave_max(tile_amax), lane);
+    } else if (TILE == 256 && out_kind != FP8GMM_OUT_BF16 && dgelu_in && desc_ok && ((ldc & 15) == 0) &&
+               ((reinterpret_cast<uintptr_t>(pr.aux) & 7) == 0) && n0 + BN <= N && (interior || oob_rows_zero)) {
+      // The data gradient with the GELU's derivative folded in: x = v * dgelu(pre), fp8(x * c_scale), amax of x.
+      // `pre` (bf16, the layout of c) is read in the MFMA layout, 8 bytes per lane and piece, one 32-row block
+      // ahead of the arithmetic; the fp8 bytes of a block go through the staging area (32 rows x 128 B, chunk c of
+      // row r at chunk c ^ ((r >> 1) & 7)) so that every store instruction writes whole lines.  Rows past m hold
+      // zero accumulators (oob_rows_zero) and read pre = 0 through the descriptor: x = 0 there, the amax is left
+      // alone and the stores fall outside the result's descriptor.
+      uint8_t* const C = static_cast<uint8_t*>(pr.c) + (int64_t)m0 * ldc + n0;
+      const uint16_t* const PRE = static_cast<const uint16_t*>(pr.aux) + (int64_t)m0 * ldc + n0;
+      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
+      const __amdgpu_buffer_rsrc_t rp = make_rsrc(PRE, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
+      uint8_t* mine = stage + wave * 8192;
+      const int wr8 = l32 * 128 + khalf * 4;  // + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
+      const int rrow8 = lane >> 3, rchunk8 = lane & 7;
+      const uint32_t lane_off8 = (uint32_t)(rrow8 * (int)ldc + wave_n * WN + rchunk8 * 16);
+      const uint32_t pre_lane = (uint32_t)(((wave_m * WM + l32) * (int)ldc + wave_n * WN + khalf * 4) * 2);
+      float tile_amax = 0.f;
+      u32x2 pre[2][NT * 4];
+      auto fetch = [&](int i, u32x2 (&dst)[NT * 4]) {
+        const uint32_t row_off = (uint32_t)(i * 32 * (int)ldc * 2);
+#pragma unroll
+        for (int jg = 0; jg < NT * 4; ++jg) dst[jg] = buf_load8_stream(rp, pre_lane + row_off + (uint32_t)(jg * 16));
+      };
+      fetch(0, pre[0]);
+      static_for<MT>([&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        if constexpr (i + 1 < MT) fetch(i + 1, pre[(i + 1) & 1]);
+        uint32_t f8[NT][4];
+        static_for<NT>([&](auto jc) {
+          constexpr int j = decltype(jc)::value;
+          const f32x16 t = acc_tile<16 * (NT * i + j)>();
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const u32x2 pw = pre[i & 1][j * 4 + g];
+            float x[4];
+            x[0] = (t[g * 4 + 0] * s) * dgelu(bf16_lo_to_f32(pw.x));
+            x[1] = (t[g * 4 + 1] * s) * dgelu(bf16_hi_to_f32(pw.x));
+            x[2] = (t[g * 4 + 2] * s) * dgelu(bf16_lo_to_f32(pw.y));
+            x[3] = (t[g * 4 + 3] * s) * dgelu(bf16_hi_to_f32(pw.y));
+            // a pinned chain of hardware max operations, as in the GELU form: x is computed, hence never a
+            // signalling NaN, and a quiet NaN loses against the running maximum
+#pragma unroll
+            for (int q = 0; q < 4; ++q) asm volatile("v_max_f32 %0, %0, |%1|" : "+v"(tile_amax) : "v"(x[q]));
+            f8[j][g] = out_kind == FP8GMM_E4M3 ? cvt4_fp8<FP8GMM_E4M3>(x[0] * cs, x[1] * cs, x[2] * cs, x[3] * cs)
+                                               : cvt4_fp8<FP8GMM_E5M2>(x[0] * cs, x[1] * cs, x[2] * cs, x[3] * cs);
+          }
+        });
+        // only this wavefront touches `mine`, and its LDS operations complete in order
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<uint32_t*>(mine + wr8 + (((2 * j + (g >> 1)) ^ ((l32 >> 1) & 7)) << 4) + (g & 1) * 8) =
+                f8[j][g];
+        u32x4 rb[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const int r = 8 * it + rrow8;
+          rb[it] = *reinterpret_cast<const u32x4*>(mine + r * 128 + ((rchunk8 ^ ((r >> 1) & 7)) << 4));
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+          const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 8 * it) * (int)ldc);
+          buf_store16_stream(rb[it], rc, lane_off8 + row_off);
+        }
+      });
+      __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
+      merge_amax(pr.c_amax, wave_max(tile_amax), lane);
     } else if (out_kind == FP8GMM_OUT_BF16) {
       uint16_t* __restrict__ C = static_cast<uint16_t*>(pr.c);
       uint16_t* __restrict__ AUX = static_cast<uint16_t*>(pr.aux);
@@ -410,6 +482,11 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
               r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
             }
             const int64_t off = (int64_t)m * ldc + n;
+            if (dgelu_in) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                if (n + q < N) r[q] = v[q] * dgelu(bf16_to_f32(AUX[off + q]));
+            }
             if (vec && n + 3 < N) {
               u32x2 o = {pack_bf16x2(r[0], r[1]), pack_bf16x2(r[2], r[3])};
               global_store(C + off, o);
@@ -449,6 +526,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
             for (int q = 0; q < 4; ++q) {
               v[q] = t[g * 4 + q] * s;
               r[q] = gelu ? gelu_tanh_fast(v[q]) : v[q];
+              if (dgelu_in && n + q < N) r[q] = v[q] * dgelu(bf16_to_f32(AUX[(int64_t)m * ldc + n + q]));
               if (n + q < N) amax = amax_step(amax, r[q]);
             }
             uint32_t w;
@@ -825,6 +903,16 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
     });
   };
   if (cp_next.nk > 0) start_tile();
+  // Where an epilogue cannot take the next tile's products in (every form but the staged bf16 one), it does not
+  // have to carry that tile's first fragments through its arithmetic either: they are fetched again afterwards,
+  // from the ring units that still hold them, which leaves the epilogue 64 more registers.
+  auto refetch_first_fragments = [&](int unit_a) {
+    const int unit_b = ring_inc(unit_a);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + unit_b * US, j, 0);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds + unit_a * US, i, 0);
+  };
   for (int r_cp = 0;; ++r_cp) {
     const ItemTile g = cp_next;
     if (g.prob < 0) break;
@@ -1008,19 +1096,25 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
       partial_store<TILE>(workspace + (size_t)g.slot * kPartialBytes);
       relaxed = false;
-      if (more) start_tile();
+      if (more) {
+        refetch_first_fragments(ua);
+        start_tile();
+      }
     } else if (more && staged_bf16_tile<TILE>(pr, m0, n0, out_kind, epilogue)) {
       // the next tile's first products go out as the accumulators they overwrite are read out, in the shadow of
       // the epilogue's vector arithmetic
-      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, scale_ab, scale_c,
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, !A_TR, scale_ab, scale_c,
                                     [&fb0, &fa0](auto ic, auto jc) {
                                       constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
                                       const i32x8 wf = fb0[j], tf = fa0[i];
                                       FP8GMM_MFMA_Z(i, j, wf, tf);
                                     });
     } else {
-      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, scale_ab, scale_c);
-      if (more) start_tile();
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, !A_TR, scale_ab, scale_c);
+      if (more) {
+        refetch_first_fragments(ua);
+        start_tile();
+      }
     }
   }
   // zero-fill loads issued past the end of the stream still target this workgroup's LDS

@@ -293,13 +293,14 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   *plan = fp8gmm_gemm_plan{};
   if (grid <= 0 || (grid % kNumXcd) != 0 || max_items < 0 || max_fixups < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (layout & FP8GMM_GEMM_TILE_128) {
-    if (layout & FP8GMM_EPI_GELU) return FP8GMM_ERR_BAD_ARGUMENT;
+    if (layout & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU)) return FP8GMM_ERR_BAD_ARGUMENT;
     return plan_small_tiles(probs, n, layout & ~FP8GMM_GEMM_TILE_128, grid, items, max_items, plan);
   }
   plan->tile = kGemmTileM;
   const int layout_given = layout, grid_given = grid;
-  const bool gelu = (layout & FP8GMM_EPI_GELU) != 0;  // only weighs the decision to share tiles along K
-  layout &= ~FP8GMM_EPI_GELU;
+  // the epilogue flags only weigh the decision to share tiles along K (completing a tile costs more with them)
+  const bool gelu = (layout & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU)) != 0;
+  layout &= ~(FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU);
   int total_tiles = 0;
   const int rc = fp8gmm_plan_grouped_gemm_layout(probs, n, layout, &total_tiles);
   if (rc != FP8GMM_OK) return rc;

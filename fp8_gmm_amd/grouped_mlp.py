@@ -221,20 +221,31 @@ class _GroupedMlp(torch.autograd.Function):
                 grouped_gemm(g_t_views, gelu_t_views, TensorBatch.stack_of(grad_fc2_weight), g1_scale_invs,
                              gelu_scale_invs)
 
-        # fc2 dgrad: d(gelu_out)[tokens, F]
-        grad_gelu_out = fp8_gmm(
-            grad_out_fp8, fc2_weight_dgrad, ctx.group_sizes, g1_scale_invs,
-            meta.get_meta_pointers(_T.kForwardWeightGroup2, _M.kScaleInv),
-            backward=True, cutlass=False, b_transposed=b_transposed,
-        )
+        grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
+        g2_scales = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale)
+        g2_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax)
+        fused = bool(ctx.fp8_meta.get("fused_dgelu", False)) and in_place and not grad_copy
+        grad_gelu_out = None
+        if fused:
+            # fc2 dgrad with the GELU's derivative and the cast in its epilogue: d(pre_gelu) in fp8 straight from the
+            # fp32 accumulators; no bf16 d(gelu_out), no separate pass over [tokens, F]
+            fp8_gmm(grad_out_fp8, fc2_weight_dgrad, ctx.group_sizes, g1_scale_invs,
+                    meta.get_meta_pointers(_T.kForwardWeightGroup2, _M.kScaleInv), c=grad_pre_fp8,
+                    c_scales=g2_scales, c_amaxes=g2_amaxes, backward=True, b_transposed=True, dgelu_pre=pre_gelu_out)
+        else:
+            # fc2 dgrad: d(gelu_out)[tokens, F]
+            grad_gelu_out = fp8_gmm(
+                grad_out_fp8, fc2_weight_dgrad, ctx.group_sizes, g1_scale_invs,
+                meta.get_meta_pointers(_T.kForwardWeightGroup2, _M.kScaleInv),
+                backward=True, cutlass=False, b_transposed=b_transposed,
+            )
 
         # d(pre_gelu) = d(gelu_out) * dgelu(pre_gelu), cast to fp8; the padded transpose only feeds fc1 wgrad in
         # the reference's layout (the reference always transposes and notes the missing cast-only kernel,
         # grouped_mlp.py:252-253)
-        grad_pre_fp8 = torch.empty(pre_gelu_out.shape, dtype=grad_dtype, device=dev)
-        g2_scales = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kScale)
-        g2_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup2, _M.kAmax)
-        if grad_copy or (wgrad and not in_place):
+        if fused:
+            pass
+        elif grad_copy or (wgrad and not in_place):
             if grad_copy:
                 _, grad_pre_t_views = alloc_transposed(pre_gelu_out.size(1), copy_padded, cumsums, copy_bounds,
                                                        grad_dtype, dev)
@@ -292,13 +303,19 @@ class GroupedMlp(Fp8GroupedModuleBase):
     ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None, is_first_microbatch=None)``;
     ``reference_layout`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
     the module's fp8 weight buffers).
+    ``fused_dgelu=True`` (default layout only): the fc2 data-gradient GEMM applies the GELU's derivative and the cast to
+    fp8 in its epilogue, from the fp32 accumulators (one rounding, where the separate pass rounds to bf16 first), and
+    the pass over ``[tokens, out_features]`` that the reference runs behind that GEMM (grouped_mlp.py:243-287) is gone.
+    Off by default: with one wavefront per SIMD the epilogue's arithmetic costs the GEMM more than the pass it
+    replaces.
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
-                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False):
+                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False, fused_dgelu=False):
         super().__init__()
         self.fp8_meta["pad_multiple"] = pad_multiple
         self.fp8_meta["reference_layout"] = reference_layout
+        self.fp8_meta["fused_dgelu"] = fused_dgelu
         assert dtype == torch.bfloat16, "bfloat16 parameters only"
         self.num_groups = num_groups
         self.fc1_weight = torch.nn.Parameter(

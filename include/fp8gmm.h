@@ -135,6 +135,14 @@ typedef struct fp8gmm_gemm_problem {
 
 /* flags of fp8gmm_grouped_gemm (its `epilogue` argument) */
 #define FP8GMM_EPI_GELU 1
+/* The derivative of the GELU folded into a data-gradient GEMM: `aux` is an INPUT, the bf16 pre-GELU activation
+ * [m, n] (pitch ldc) that the forward GELU-aux epilogue wrote, and
+ *   x = v * dgelu_tanh(aux);   out fp8: c = fp8_saturate(x * *c_scale), *c_amax = max(*c_amax, max|x|);   out bf16: c = bf16(x)
+ * The reference forms x from the bf16-rounded v in a pass of its own (MultiPadCastTransposeDgelu,
+ * csrc/multi_pad_fusion.cu:587, after the fc2 data-gradient GEMM, fp8_gmm/grouped_mlp.py:243-287) and notes the
+ * missing fusion (:252-253); here v stays in fp32 until the one rounding to fp8.  Not together with
+ * FP8GMM_EPI_GELU. */
+#define FP8GMM_EPI_DGELU 8
 /* b is stored contraction-major: b[k, n] with n contiguous and ldb >= n its row pitch, i.e.
  * c[m, n] = epilogue( a[m, k] . b[k, n] ).  This is a forward weight [N_fwd = k, K_fwd = n] as the data-gradient
  * GEMM needs it, read in place: the reference casts a transposed copy of every weight for that GEMM instead
@@ -262,7 +270,7 @@ int fp8gmm_multi_cast_dgelu(fp8gmm_tensor_desc* descs_dev, int n, int total_bloc
  * Validates `probs[0..n)` like fp8gmm_plan_grouped_gemm_layout, fills tile_begin / cost_begin, and writes the work
  * list of a launch with `grid` workgroups (fp8gmm_gemm_grid) into items[0 .. rounds * grid) and
  * fixups[0 .. n_fixups).  `layout` takes the launch's flags: the KMAJOR flags as for the plain plan, and
- * FP8GMM_EPI_GELU, which only weighs the decision below (completing a shared tile costs more with that epilogue).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
+ * FP8GMM_EPI_GELU / FP8GMM_EPI_DGELU, which only weigh the decision below (completing a shared tile costs more with that epilogue).  stream_k != 0: the workgroups of an XCD share the tail tiles of their range along K when
  * the last round would otherwise be mostly idle; the launch then needs plan->n_slots workspace slots (never more
  * than 2 * grid).  stream_k > 1: the same, but with at most stream_k slots - a launch whose sharing would need more
  * is planned with whole tiles instead (callers of fp8gmm_grouped_gemm_static pass FP8GMM_GEMM_STATIC_SLOTS and never
@@ -282,7 +290,7 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
  *   plan         : the host struct fp8gmm_plan_grouped_gemm_launch filled
  *   a_fmt, b_fmt : FP8GMM_E4M3 / FP8GMM_E5M2 (e5m2 x e5m2 is rejected, as cuBLASLt does)
  *   out_kind     : FP8GMM_OUT_BF16, or FP8GMM_E4M3 / FP8GMM_E5M2 for an fp8 `c`
- *   epilogue     : FP8GMM_EPI_GELU and the layout flags the table was planned with
+ *   epilogue     : FP8GMM_EPI_GELU or FP8GMM_EPI_DGELU, and the layout flags the table was planned with
  *   workspace    : device memory, workspace_bytes >= plan->n_slots * FP8GMM_GEMM_SLOT_BYTES, 256-byte aligned,
  *                  contents irrelevant; may be NULL when n_slots == 0.  Launches that overlap in time (different
  *                  streams) need different workspaces.  Too small: FP8GMM_ERR_WORKSPACE, nothing is launched.

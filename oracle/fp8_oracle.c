@@ -366,3 +366,23 @@ void orc_epilogue_gelu_fp8(const float* acc, int64_t n, float sa, float sb, cons
     if ((int32_t)f2u(mx) > (int32_t)f2u(*amax)) *amax = mx;
   }
 }
+
+/* The data-gradient epilogue with the GELU's derivative folded in (no reference kernel: the reference forms the
+ * product in a separate pass from the bf16-rounded GEMM result, fp8_gmm/grouped_mlp.py:243-287, and notes the missing
+ * fusion at :252-253):  v = acc * (sa * sb);  x = v * dgelu(pre);  c = fp8(x * c_scale);  amax = max|x|.
+ * dgelu is the function of the cast kernels (multi_pad_fusion.cu:39-44), v is NOT rounded to bf16 first. */
+void orc_epilogue_dgelu_fp8(const float* acc, int64_t n, float sa, float sb, const float* c_scale, int fmt,
+                            const uint16_t* pre, uint8_t* c, float* amax) {
+  float s = sa * sb;
+  float cs = c_scale ? *c_scale : 1.0f;
+  float mx = 0.0f;
+  for (int64_t i = 0; i < n; ++i) {
+    float v = acc[i] * s;
+    float x = v * orc_dgelu(orc_bf16_to_f32(pre[i]));
+    mx = amax_step(mx, x);
+    c[i] = orc_f32_to_fp8(x * cs, fmt);
+  }
+  if (amax) {
+    if ((int32_t)f2u(mx) > (int32_t)f2u(*amax)) *amax = mx;
+  }
+}

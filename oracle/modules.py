@@ -120,14 +120,17 @@ def grouped_linear_step(x, w, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn
 
 
 def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3fn, bwd_dtype=torch.float8_e5m2,
-                     cached=None, given=None):
+                     cached=None, given=None, fused_dgelu=False):
     """One forward + backward of GroupedMlp. x [M, H], w1 [E, F, H], w2 [E, H, F], dy [M, H].
     ``cached``: the result of an earlier step whose fp8 weights are reused.
 
     ``given``: intermediates of another implementation's run of the same step (any of ``pre``, ``gelu_fp8``,
     ``grad_gelu``, ``dpre_fp8``).  A given tensor replaces this function's own from the point where it is
     produced, so that everything downstream is computed from identical bytes and can be compared GEMM by GEMM;
-    this function's own values are returned beside them under ``own_*`` (the amax it records stays its own)."""
+    this function's own values are returned beside them under ``own_*`` (the amax it records stays its own).
+
+    ``fused_dgelu``: d(pre-GELU) is formed in the epilogue of the fc2 data-gradient GEMM, from the fp32 result
+    (no bf16 d(GELU output): ``grad_gelu`` is None), as GroupedMlp(fused_dgelu=True) does."""
     given = given or {}
     e = len(sizes)
     b = _bounds(sizes)
@@ -164,20 +167,28 @@ def grouped_mlp_step(x, w1, w2, sizes, dy, fwd, bwd, fwd_dtype=torch.float8_e4m3
         ref.multi_transpose([gelu_fp8[b[i]: b[i + 1]].contiguous()], [t])
         gelu_ts.append(t)
     grad_w2 = _wgrad(dy_ts, gelu_ts, g1_inv, [fwd_inv[s] for s in x2])
-    grad_gelu = _gmm_bf16(dy_fp8, w2_t, sizes, g1_inv, [fwd_inv[s] for s in w2s])
-    own["own_grad_gelu"] = grad_gelu
-    grad_gelu = given.get("grad_gelu", grad_gelu)
-
     dpre_fp8 = torch.empty(m, ffn, dtype=bwd_dtype)
     dpre_ts = []
-    for i, s in enumerate(sizes):
-        mp = (s + 15) // 16 * 16
-        t = torch.empty(ffn, mp, dtype=bwd_dtype)
-        o = torch.empty(s, ffn, dtype=bwd_dtype)
-        ref.multi_cast_transpose_dgelu([grad_gelu[b[i]: b[i + 1]].contiguous()], [pre[b[i]: b[i + 1]].contiguous()],
-                                       [o], [t], [bwd.scale[g2[i]: g2[i] + 1]], [bwd.amax(g2[i])])
-        dpre_fp8[b[i]: b[i + 1]] = o
-        dpre_ts.append(t)
+    if fused_dgelu:
+        grad_gelu = None
+        ref.fp8_gmm(dy_fp8, w2_t, sizes, g1_inv, [fwd_inv[s] for s in w2s], dpre_fp8, bwd_dtype, None,
+                    [bwd.scale[s: s + 1] for s in g2], [bwd.amax(s) for s in g2], dgelu_pre=pre)
+        for i, s in enumerate(sizes):
+            t = torch.empty(ffn, (s + 15) // 16 * 16, dtype=bwd_dtype)
+            ref.multi_transpose([dpre_fp8[b[i]: b[i + 1]].contiguous()], [t])
+            dpre_ts.append(t)
+    else:
+        grad_gelu = _gmm_bf16(dy_fp8, w2_t, sizes, g1_inv, [fwd_inv[s] for s in w2s])
+        own["own_grad_gelu"] = grad_gelu
+        grad_gelu = given.get("grad_gelu", grad_gelu)
+        for i, s in enumerate(sizes):
+            mp = (s + 15) // 16 * 16
+            t = torch.empty(ffn, mp, dtype=bwd_dtype)
+            o = torch.empty(s, ffn, dtype=bwd_dtype)
+            ref.multi_cast_transpose_dgelu([grad_gelu[b[i]: b[i + 1]].contiguous()], [pre[b[i]: b[i + 1]].contiguous()],
+                                           [o], [t], [bwd.scale[g2[i]: g2[i] + 1]], [bwd.amax(g2[i])])
+            dpre_fp8[b[i]: b[i + 1]] = o
+            dpre_ts.append(t)
     own["own_dpre_fp8"] = dpre_fp8
     if "dpre_fp8" in given:
         dpre_fp8 = given["dpre_fp8"]

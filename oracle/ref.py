@@ -76,6 +76,7 @@ def lib():
             "orc_gemm_f32": [vp, i32, vp, i32, i64, i64, i64, i64, i64, vp],
             "orc_epilogue_bf16": [vp, i64, ctypes.c_float, ctypes.c_float, vp],
             "orc_epilogue_gelu_fp8": [vp, i64, ctypes.c_float, ctypes.c_float, vp, i32, vp, vp, vp],
+            "orc_epilogue_dgelu_fp8": [vp, i64, ctypes.c_float, ctypes.c_float, vp, i32, vp, vp, vp],
         }.items():
             fn = getattr(L, name)
             fn.restype = None
@@ -228,12 +229,18 @@ def gemm_acc(a, b):
 
 
 def cublas_fp8_gemm(a, b, c, a_scale_inv, b_scale_inv, pre_gelu_out=None, c_scale=None, c_amax=None,
-                    backward=False, naive=False):
-    """c[m, n] = epilogue((a[m, k] . b[n, k]^T) * a_scale_inv * b_scale_inv), see orc_epilogue_*."""
+                    backward=False, naive=False, dgelu_pre=None):
+    """c[m, n] = epilogue((a[m, k] . b[n, k]^T) * a_scale_inv * b_scale_inv), see orc_epilogue_*.
+    ``dgelu_pre`` (bf16 [m, n], an input): the result times dgelu(dgelu_pre) before the rounding to fp8."""
     acc = (gemm_acc_naive if naive else gemm_acc)(a.contiguous(), b.contiguous()).contiguous()
     sa, sb = float(a_scale_inv), float(b_scale_inv)
     _cpu_contig(c)
-    if c.dtype == torch.bfloat16:
+    if dgelu_pre is not None:
+        assert pre_gelu_out is None and c.dtype != torch.bfloat16 and c_scale is not None and c_amax is not None
+        _cpu_contig(dgelu_pre, torch.bfloat16)
+        lib().orc_epilogue_dgelu_fp8(_ptr(acc), acc.numel(), sa, sb, _ptr(c_scale), fmt_of(c.dtype), _ptr(dgelu_pre),
+                                     _ptr(c), _ptr(c_amax))
+    elif c.dtype == torch.bfloat16:
         assert pre_gelu_out is None
         lib().orc_epilogue_bf16(_ptr(acc), acc.numel(), sa, sb, _ptr(c))
     else:
@@ -247,7 +254,7 @@ def cublas_fp8_gemm(a, b, c, a_scale_inv, b_scale_inv, pre_gelu_out=None, c_scal
 
 
 def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch.bfloat16, pre_gelu_out=None,
-            c_scales=None, c_amaxes=None, backward=False, cutlass=False, naive=False):
+            c_scales=None, c_amaxes=None, backward=False, cutlass=False, naive=False, dgelu_pre=None):
     """Per-expert loop of the reference (fp8_gmm/backend.py:84-96; oracle form fp8_gmm/test.py:209-214)."""
     if c is None:
         c = torch.empty(a.shape[0], b.shape[1], dtype=c_dtype)
@@ -262,6 +269,7 @@ def fp8_gmm(a, b, group_sizes, a_scale_invs, b_scale_invs, c=None, c_dtype=torch
                 c_scale=c_scales[i] if c_scales is not None else None,
                 c_amax=c_amaxes[i] if c_amaxes is not None else None,
                 backward=backward, naive=naive,
+                dgelu_pre=dgelu_pre[start:end].contiguous() if dgelu_pre is not None else None,
             )
         start = end
     return c

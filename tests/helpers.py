@@ -138,6 +138,21 @@ def fp8_code_distance(a, b):
     return (sa - sb).abs()
 
 
+def assert_fp8_codes_close(got, want, what, max_fraction_off=0.01):
+    """Two fp8 tensors whose values come from contractions summed in different orders: at most one code step apart
+    wherever the value is not tiny, on at most `max_fraction_off` of the elements.  A sum of thousands of terms that
+    cancels to under a hundredth of the tensor's typical size carries the summation-order noise at full weight, and
+    the fp8 codes are dense around zero: there the VALUES must agree to a hundredth of the typical size instead."""
+    dist = fp8_code_distance(got, want)
+    wv, gv = want.float(), got.float()
+    rms = wv.pow(2).mean().sqrt()
+    big = wv.abs() > 1e-2 * rms
+    assert (dist[big] <= 1).all(), f"{what}: {int((dist[big] > 1).sum())} values more than one code step apart"
+    assert ((gv - wv).abs()[~big] <= 1e-2 * rms).all(), f"{what}: small values differ by more than 1e-2 of the rms"
+    off = (dist != 0).float().mean().item()
+    assert off <= max_fraction_off, f"{what}: {off:.4f} of the bytes differ"
+
+
 def _mini_meta(gpu_meta, slots):
     """The scaling state of `slots` of a module's GPU meta as an oracle Meta with history length 1 (amax row
     cleared: the oracle records its own)."""

@@ -142,7 +142,8 @@ def test_launch_entry_points_validate_before_touching_the_gpu():
 
     assert gemm(1, 1, 1, 2, 0) == -3  # e5m2 x e5m2
     assert gemm(1, 0, 0, 9, 0) == -3  # unknown output kind
-    assert gemm(1, 0, 0, 2, 8) == -6  # unknown epilogue flag
+    assert gemm(1, 0, 0, 2, 16) == -6  # unknown epilogue flag
+    assert gemm(1, 0, 0, 2, 1 | 8) == -6  # GELU and its derivative exclude each other
     assert gemm(1, 0, 0, 2, 0) == -1  # tables missing
     assert gemm(0, 0, 0, 2, 0) == 0   # nothing to do
     assert gemm(1, 0, 0, 2, 0, plan=_lib.GemmPlan()) == 0   # a plan without tiles

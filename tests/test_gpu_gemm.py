@@ -8,8 +8,8 @@ and exact equality wherever the arithmetic is exact (power-of-two data, identity
 import pytest
 import torch
 
-from helpers import (assert_bytes_equal, assert_gemm_close, assert_scalar_bits_equal, fp8_code_distance, gen,
-                     randn_bf16)
+from helpers import (assert_bytes_equal, assert_fp8_codes_close, assert_gemm_close, assert_scalar_bits_equal,
+                     fp8_code_distance, gen, randn_bf16)
 from oracle import ref
 
 pytestmark = pytest.mark.gpu
@@ -827,3 +827,71 @@ def test_weight_gradient_with_a_transposed_gradient_copy_gives_the_same_bits(dev
         backend.grouped_gemm(a_km, b_km, list(want.unbind(0)), sa, sb, transposed=True)
         backend.grouped_gemm(a_pad, b_km, list(got.unbind(0)), sa, sb, transposed="b")
         assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"rows {rows} m {m} n {n}"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("out_dtype", [E5M2, E4M3], ids=["e5m2", "e4m3"])
+@pytest.mark.parametrize("sizes,n,k,b_kn", [
+    ([300, 0, 513, 90], 512, 256, True),     # whole tiles in n, ragged rows: the staged form, rows past m
+    ([256], 256, 4096, True),                # few tiles, long K: shared along K, completed by the fix-up launch
+    ([137, 401, 59], 528, 272, True),        # n not a tile multiple: the per-group form
+    ([64, 700], 768, 512, False),            # row-major weights
+])
+def test_dgelu_epilogue_is_exact_on_exact_operands(dev, out_dtype, sizes, n, k, b_kn, monkeypatch):
+    """fp8_gmm(..., dgelu_pre=pre): c = fp8((a . b) * scales * dgelu(pre) * c_scale), amax = max |(a . b) * scales *
+    dgelu(pre)|.  Operands from {0, +-0.25 .. +-2} and power-of-two scales make the accumulator exact, and dgelu is a
+    fixed sequence of IEEE operations that the C oracle repeats, so bytes and amax must equal the oracle's bit for
+    bit - through the staged form, the per-group form and the fix-up launch alike.  A wrong lane-to-element map of
+    the pre-activation reads, a dropped row block or a product formed in another order cannot pass."""
+    backend = _backend()
+    monkeypatch.setattr(backend.options, "tile", "256")
+    g = gen(900 + n + k)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25])
+    e, m = len(sizes), sum(sizes)
+    a = _q(vals[torch.randint(0, 8, (m, k), generator=g)].to(torch.bfloat16), E5M2)
+    b = _q(vals[torch.randint(0, 8, (e, n, k), generator=g)].to(torch.bfloat16), E4M3)
+    pre = (torch.randn(m, n, generator=g) * 2.0).to(torch.bfloat16)
+    pre[0, :8] = torch.tensor([0.0, -0.0, 30.0, -30.0, float("inf"), float("-inf"), 1e-30, -1e-30]).to(torch.bfloat16)
+    sa, sb = [0.5] * e, [2.0 ** -(i % 3) for i in range(e)]
+    cs = [2.0 ** (3 + i % 2) for i in range(e)]
+    want = torch.zeros(m, n, dtype=out_dtype)
+    want_amax = [torch.zeros(1) for _ in range(e)]
+    ref.fp8_gmm(a, b, sizes, _scalars(sa), _scalars(sb), want, out_dtype, None, _scalars(cs), want_amax, dgelu_pre=pre)
+    got = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=dev).view(torch.uint8)[:, :n].contiguous().view(out_dtype)
+    got.view(torch.uint8).fill_(0x55)
+    amax = torch.zeros(e, device=dev)
+    bd = b.to(dev).transpose(1, 2).contiguous() if b_kn else b.to(dev)
+    backend.fp8_gmm(a.to(dev), bd, torch.tensor(sizes), _scalars(sa, dev), _scalars(sb, dev), got, out_dtype, None,
+                    _scalars(cs, dev), list(amax.unbind(0)), True, False, b_transposed=b_kn, dgelu_pre=pre.to(dev))
+    torch.cuda.synchronize()
+    assert_bytes_equal(got.cpu(), want, "fused dgelu fp8 bytes")
+    assert_scalar_bits_equal(amax.cpu(), torch.cat(want_amax), "fused dgelu amax")
+    assert torch.cat(want_amax).max() > 0
+
+
+@pytest.mark.gpu
+def test_dgelu_epilogue_on_random_operands(dev):
+    """The same call on Gaussian operands at the fc2 data-gradient shape of a small MLP: the MFMA's summation order
+    differs from the oracle's, so bytes are held to one fp8 code step (and nearly all must be equal), amax to 1e-3."""
+    backend = _backend()
+    g = gen(77)
+    sizes, n, k = [700, 33, 0, 291], 1024, 512
+    e, m = len(sizes), sum(sizes)
+    a = _q(randn_bf16((m, k), g), E5M2)
+    b = _q(randn_bf16((e, k, n), g), E4M3)          # [E, k, n]: a forward weight stack read in place
+    pre = randn_bf16((m, n), g)
+    sa, sb, cs = [0.01] * e, [0.5] * e, [300.0] * e
+    want = torch.zeros(m, n, dtype=E5M2)
+    want_amax = [torch.zeros(1) for _ in range(e)]
+    ref.fp8_gmm(a, b.transpose(1, 2).contiguous(), sizes, _scalars(sa), _scalars(sb), want, E5M2, None, _scalars(cs),
+                want_amax, dgelu_pre=pre)
+    got = torch.zeros(m, n, dtype=torch.uint8, device=dev).view(E5M2)
+    amax = torch.zeros(e, device=dev)
+    backend.fp8_gmm(a.to(dev), b.to(dev), torch.tensor(sizes), _scalars(sa, dev), _scalars(sb, dev), got, E5M2, None,
+                    _scalars(cs, dev), list(amax.unbind(0)), True, False, b_transposed=True, dgelu_pre=pre.to(dev))
+    torch.cuda.synchronize()
+    assert_fp8_codes_close(got.cpu(), want, "fused dgelu bytes")
+    ref_amax = torch.cat(want_amax)
+    live = ref_amax > 0
+    assert torch.allclose(amax.cpu()[live], ref_amax[live], rtol=1e-3, atol=0)
+    assert (amax.cpu()[~live] == 0).all()

@@ -339,3 +339,85 @@ def test_meta_update_hand_worked_keep_scale_inv():
     assert m.scale.tolist() == [448.0, 224.0, 112.0, 56.0, 28.0, 14.0]   # every scale moves ...
     assert torch.equal(m.scale_inv, torch.tensor([1.0 / 448.0, 3.0, 1.0 / 112.0, 1.0 / 56.0, 3.0, 1.0 / 14.0],
                                                  dtype=torch.float32))                    # ... kept slots do not
+
+
+def _dgelu_f64(c):
+    """d/dc of 0.5 c (1 + tanh(0.79788456 c (1 + 0.044715 c^2))) in double precision (the closed form of
+    fp8_gmm/test.py:32-34 and csrc/multi_pad_fusion.cu:39-44)."""
+    c = c.double()
+    t = torch.tanh(0.79788456 * c * (1 + 0.044715 * c * c))
+    return 0.5 * c * ((1 - t * t) * (0.79788456 + 0.1070322243 * c * c)) + 0.5 * (1 + t)
+
+
+def _bf16_sweep():
+    """Every bf16 value up to 5e10 in magnitude.  That is the domain on which this build's 21-operation dGELU stays
+    within 3e-6 of the formula: its exp(-2|u|) is floored at 2^-125 while the factor c (1.5958 + 0.2141 c^2) next to
+    it keeps growing, so the error passes 3e-6 at |c| = 8e10 and an fp8 code step of the values 0 / 1 at 3.5e12.
+    (The reference's single-precision expression, csrc/multi_pad_fusion.cu:39-44, is exact up to 1.8e19 and 0 * inf
+    beyond, where the square overflows.)  Pre-GELU activations of that size do not occur."""
+    bits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16)
+    x = bits.view(torch.bfloat16)
+    return x[x.float().abs() <= 5e10]
+
+
+def _signed_codes(t):
+    c = t.view(torch.uint8).to(torch.int32)
+    return torch.where(c >= 128, -(c - 128), c)
+
+
+@pytest.mark.parametrize("dtype", [torch.float8_e5m2, torch.float8_e4m3fn])
+def test_dgelu_cast_codes_against_double_precision(dtype):
+    """The fp8 CODES that the cast + dGELU functions write (not only the dGELU values) against a double-precision
+    dGELU.  Over every bf16 pre-activation of the domain, with three gradients each: the byte written for
+    x = dy * dgelu(pre) must lie between the bytes that torch's saturating cast gives for x - d and x + d, where x is
+    formed in double precision and d = 3e-6 |dy| is the error bound of this build's dGELU (so the byte is the
+    correctly rounded code of a value that close to the closed form); on 99 % of the inputs it must be the code of
+    x itself; amax within 1e-5.  This ties the bytes of multi_cast_transpose_dgelu / multi_cast_dgelu to the
+    reference's formula independently of the kernel that shares the oracle's operation sequence."""
+    pre = _bf16_sweep()
+    fmax = 448.0 if dtype == torch.float8_e4m3fn else 57344.0
+
+    def cast(v):
+        return _signed_codes((v * scale).clamp(-fmax, fmax).float().to(dtype))
+
+    for dy_val, scale in ((1.0, 16.0), (-0.37109375, 64.0), (0.0072021484375, 4096.0)):
+        dy = torch.full(pre.shape, dy_val).to(torch.bfloat16)
+        n = pre.numel()
+        out = torch.empty(1, n, dtype=dtype)
+        t = torch.empty(n, 16, dtype=dtype)
+        amax = torch.zeros(1)
+        ref.multi_cast_transpose_dgelu([dy.view(1, n)], [pre.view(1, n)], [out], [t], [torch.tensor([scale])], [amax])
+        x64 = dy.double() * _dgelu_f64(pre)
+        d = 3e-6 * abs(dy_val)
+        got = _signed_codes(out).view(-1)
+        lo, hi = torch.minimum(cast(x64 - d), cast(x64 + d)), torch.maximum(cast(x64 - d), cast(x64 + d))
+        assert ((got >= lo) & (got <= hi)).all(), (dy_val, int(((got < lo) | (got > hi)).sum()))
+        assert (got != cast(x64)).float().mean() < 0.01
+        assert abs(amax.item() - x64.abs().max().item()) <= 1e-5 * x64.abs().max().item()
+
+
+def test_fused_dgelu_epilogue_against_double_precision():
+    """orc_epilogue_dgelu_fp8 (the data-gradient epilogue with the GELU's derivative folded in): bytes within one
+    code step of fp8((acc * sa * sb) * dgelu_f64(pre) * c_scale) formed in double precision, amax within 1e-5, and
+    the merge with a larger previous amax leaves it alone."""
+    from helpers import fp8_code_distance
+
+    g = torch.Generator().manual_seed(11)
+    acc = (torch.randn(4096, generator=g) * 37.0).contiguous()
+    pre = (torch.randn(4096, generator=g) * 2.5).to(torch.bfloat16).contiguous()
+    sa, sb, cs = 0.03125, 0.75, 40.0
+    for dtype, fmax in ((torch.float8_e5m2, 57344.0), (torch.float8_e4m3fn, 448.0)):
+        out = torch.empty(4096, dtype=dtype)
+        amax = torch.zeros(1)
+        scale = torch.tensor([cs])
+        ref.lib().orc_epilogue_dgelu_fp8(acc.data_ptr(), 4096, sa, sb, scale.data_ptr(), ref.fmt_of(dtype),
+                                         pre.data_ptr(), out.data_ptr(), amax.data_ptr())
+        x64 = acc.double() * (sa * sb) * _dgelu_f64(pre)
+        want = (x64 * cs).clamp(-fmax, fmax).float().to(dtype)
+        dist = fp8_code_distance(out, want)
+        assert dist.max() <= 1 and (dist != 0).float().mean() < 0.01
+        assert abs(amax.item() - x64.abs().max().item()) <= 1e-5 * x64.abs().max().item()
+        big = torch.tensor([1e9])
+        ref.lib().orc_epilogue_dgelu_fp8(acc.data_ptr(), 4096, sa, sb, scale.data_ptr(), ref.fmt_of(dtype),
+                                         pre.data_ptr(), out.data_ptr(), big.data_ptr())
+        assert big.item() == 1e9
