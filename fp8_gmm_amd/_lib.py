@@ -88,7 +88,7 @@ GEMM_ITEM = np.dtype(
         ("n0", "<i4"),
         ("prob", "<i4"),
         ("slot", "<i4"),
-        ("reserved", "<i4"),
+        ("flags", "<i4"),
     ],
     align=False,
 )
@@ -318,7 +318,7 @@ def _plan_into_scratch(table, layout, grid, stream_k):
         items = sc.items = np.empty(8192, dtype=GEMM_ITEM)
         sc.fixups = np.empty(1024, dtype=GEMM_FIXUP)
     fixups = sc.fixups
-    args = (table.ctypes.data, len(table), layout, grid, int(bool(stream_k)))
+    args = (table.ctypes.data, len(table), layout, grid, int(stream_k))   # 0 off, 1 on, > 1 on with that many slots
     rc = L.fp8gmm_plan_grouped_gemm_launch(*args, items.ctypes.data, len(items), fixups.ctypes.data, len(fixups),
                                            ctypes.byref(plan))
     if rc == -8:  # FP8GMM_ERR_BUFFER_TOO_SMALL: the sizes are in the plan

@@ -207,11 +207,14 @@ struct NothingReleased {
   template <class I, class J>
   __device__ __forceinline__ void operator()(I, J) const {}
 };
+// `mt`: 32-row blocks per wavefront: MT, or MT / 2 for a tile of half height, whose wavefronts stand on rows
+// wave_m * 64 + 32 i.  Returns the number of stores per wavefront that the staged bf16 form left in flight (0: another form ran).
 template <int TILE, class Released = NothingReleased>
-__device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int m0, int n0, int out_kind, int epilogue,
-                                              uint8_t* stage, bool oob_zero, bool oob_rows_zero, float s, float cs,
-                                              Released released = Released()) {
-  constexpr int BM = TILE, BN = TILE, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
+__device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int m0, int n0, int out_kind, int epilogue,
+                                             uint8_t* stage, int mt, bool oob_zero, bool oob_rows_zero, float s, float cs,
+                                             Released released = Released()) {
+  constexpr int BM = TILE, BN = TILE, WN = TILE / 2, MT = TILE / 64, NT = WN / 32;
+  const int WM = mt * 32;   // rows of a wavefront's sub-tile
   constexpr int kStageBytes = TILE * 32;   // per wavefront: a quarter of one ring unit
   // The lane's offsets into the staging area and the result are formed anew for every tile: computed once per
   // kernel (they do not depend on the tile) they would occupy a dozen registers all through the main loop, where
@@ -223,7 +226,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
   const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
   const int l32 = lane & 31, khalf = lane >> 5;
   const int M = pr.m, N = pr.n;
-  bool fast = false;
+  int fast = 0;
     const bool gelu = (epilogue & FP8GMM_EPI_GELU) != 0;
     const bool dgelu_in = (epilogue & FP8GMM_EPI_DGELU) != 0 && pr.aux != nullptr;   // aux is then an INPUT
     const int64_t ldc = pr.ldc;
@@ -263,6 +266,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
       static_for<MT * kUnitsPerRow>([&](auto uc) {
         constexpr int u = decltype(uc)::value;
         constexpr int i = u / kUnitsPerRow, jj = u % kUnitsPerRow;
+        if (i >= mt) return;
         uint8_t* buf = mine + (kStageBytes >= 8192 ? (u & 1) * 4096 : 0);
         static_for<2>([&](auto jlc) {
           constexpr int jl = decltype(jlc)::value;
@@ -284,9 +288,9 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
           v[it] = *reinterpret_cast<const u32x4*>(buf + r * 128 + ((rchunk ^ ((r >> 1) & 7)) << 4));
         }
       });
-      store_unit(MT - 1, kUnitsPerRow - 1);
+      store_unit(mt - 1, kUnitsPerRow - 1);
       __builtin_amdgcn_s_barrier();  // the staging area goes back to the operand ring
-      fast = true;
+      fast = mt * kUnitsPerRow * 4;
     } else if (TILE == 256 && out_kind == FP8GMM_E4M3 && gelu && pr.aux != nullptr && desc_ok && ((ldc & 15) == 0) &&
                ((reinterpret_cast<uintptr_t>(pr.aux) & 15) == 0) && (interior || (oob_zero && (cv & 15) == 0))) {
       // The fused GELU form (e4m3 gelu(v) * c_scale, bf16 v on the side, amax of gelu(v)): both outputs go
@@ -311,6 +315,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
       float tile_amax = 0.f;
       static_for<MT>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
+        if (i >= mt) return;
         uint32_t f8[NT][4];
         bool any_nan = false;
         static_for<NT>([&](auto jc) {
@@ -418,7 +423,10 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
       fetch(0, pre[0]);
       static_for<MT>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
-        if constexpr (i + 1 < MT) fetch(i + 1, pre[(i + 1) & 1]);
+        if (i >= mt) return;
+        if constexpr (i + 1 < MT) {
+          if (i + 1 < mt) fetch(i + 1, pre[(i + 1) & 1]);
+        }
         uint32_t f8[NT][4];
         static_for<NT>([&](auto jc) {
           constexpr int j = decltype(jc)::value;
@@ -467,6 +475,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
                        (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
       static_for<MT>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
+        if (i >= mt) return;
         const int m = m0 + wave_m * WM + i * 32 + l32;
         static_for<NT>([&](auto jc) {
           constexpr int j = decltype(jc)::value;
@@ -513,6 +522,7 @@ __device__ __forceinline__ bool tile_epilogue(const fp8gmm_gemm_problem& pr, int
                        (AUX == nullptr || (reinterpret_cast<uintptr_t>(AUX) & 7) == 0);
       static_for<MT>([&](auto ic) {
         constexpr int i = decltype(ic)::value;
+        if (i >= mt) return;
         const int m = m0 + wave_m * WM + i * 32 + l32;
         static_for<NT>([&](auto jc) {
           constexpr int j = decltype(jc)::value;
@@ -582,7 +592,7 @@ struct ItemLoad {   // bytes 0..31: what the load stream needs besides ItemTile
   int32_t lda, ldb;
 };
 struct ItemTile {   // bytes 32..63
-  int32_t k, k_begin, nk, m0, n0, prob, slot, reserved;
+  int32_t k, k_begin, nk, m0, n0, prob, slot, flags;
 };
 static_assert(sizeof(fp8gmm_gemm_item) == 64 && sizeof(ItemLoad) == 32 && sizeof(ItemTile) == 32, "record layout");
 static_assert(offsetof(fp8gmm_gemm_item, k) == 32 && offsetof(fp8gmm_gemm_item, lda) == 24, "record layout");
@@ -656,6 +666,15 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   int fat_off[MT];
 #pragma unroll
   for (int i = 0; i < MT; ++i) fat_off[i] = tr_row + (((wave_m * (WM / 16) + 2 * i + tr_g) ^ tr_swz) << 4);
+  // Tiles of half height (FP8GMM_ITEM_HALF_HEIGHT: at most 128 valid rows): the wavefronts stand two by two on
+  // rows wave_m * 64 + 32 i, i < 2, and issue half the products.  Row-major tokens: the fragment addresses move
+  // down by wave_m * 64 rows, a uniform amount that goes into the unit's base address (half_rows_back).
+  // Contraction-major: the 16-byte chunk of fragment i is chunk wave_m * 4 + 2 i + tr_g (fat_half).
+  [[maybe_unused]] const int half_rows_back = wave_m * 64 * BK;
+  [[maybe_unused]] int fat_half[MT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+    fat_half[i] = tr_row + (((wave_m * (WM / 32) + 2 * (i & 1) + tr_g) ^ tr_swz) << 4);
 
   // ---- this workgroup's work list (uniform): records blockIdx.x, blockIdx.x + grid, ... up to the end record.
   // Both sides of the kernel walk it, the load side ahead of the compute side, and both read a record one item
@@ -813,11 +832,12 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
       read_half_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * kTrPitch), h);
     }
   };
-  [[maybe_unused]] auto half_a = [&](i32x8& f, const uint8_t* unit, int i, int hh, int h) {
+  // (token fragments: `half` = the tile they are read for is of half height)
+  [[maybe_unused]] auto half_a = [&](i32x8& f, const uint8_t* unit, int i, int hh, int h, bool half = false) {
     if constexpr (!A_TR) {
-      read_half(f, unit + fa_off + i * 32 * BK, hh, h);
+      read_half(f, unit - (half ? half_rows_back : 0) + fa_off + i * 32 * BK, hh, h);
     } else {
-      read_half_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * kTrPitch), h);
+      read_half_tr(f, (uint32_t)(uintptr_t)unit + (half ? fat_half[i] : fat_off[i]) + hh * (64 * kTrPitch), h);
     }
   };
   // weight fragment j / token fragment i, K half hh, of the unit at `unit`
@@ -828,11 +848,11 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
       read_frag_tr(f, (uint32_t)(uintptr_t)unit + fbt_off[j] + hh * (64 * kTrPitch));
     }
   };
-  auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh) {
+  auto read_frag_a = [&](i32x8& f, const uint8_t* unit, int i, int hh, bool half = false) {
     if constexpr (!A_TR) {
-      read_frag(f, unit + fa_off + i * 32 * BK, hh);
+      read_frag(f, unit - (half ? half_rows_back : 0) + fa_off + i * 32 * BK, hh);
     } else {
-      read_frag_tr(f, (uint32_t)(uintptr_t)unit + fat_off[i] + hh * (64 * kTrPitch));
+      read_frag_tr(f, (uint32_t)(uintptr_t)unit + (half ? fat_half[i] : fat_off[i]) + hh * (64 * kTrPitch));
     }
   };
 
@@ -852,14 +872,22 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   __builtin_amdgcn_s_barrier();
 #pragma unroll
   for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + US, j, 0);
+  // height of the tile that a record's K steps belong to - for a record without K steps, of the next record with
+  // some (the planner notes it there): the load stream skips records without K steps, so the fragments read at
+  // the end of a tile are those of the next tile that has any
+  auto half_height = [](const ItemTile& t) {
+    return TILE == 256 && ((t.nk > 0 ? t.flags : t.flags >> 1) & FP8GMM_ITEM_HALF_HEIGHT) != 0;
+  };
+  ItemTile cp_next = item_tile(0);  // the compute side's next record, fetched ahead like the load side's
+  bool nxt_half = half_height(cp_next);   // height of the tile whose first fragments are in fa0 / fb0
 #pragma unroll
-  for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds, i, 0);
+  for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds, i, 0, nxt_half);
   int ua = 0;  // ring unit of the current step's token rows; its weight rows are in the next unit
   // vmcnt counts loads and stores in issue order.  The barrier of a step needs the next step's units, which are
   // older than the token loads issued during the low half-step: "all but the newest kParts".  Right after an
   // interior epilogue the newest operations also include that epilogue's kFastStores stores, which nothing in
   // LDS depends on: at the first barrier after it they may stay in flight.
-  bool relaxed = false;
+  int relaxed = 0;   // stores of the epilogue just before that may stay in flight at the next barrier
 
   // The accumulation registers belong to the statements below (see acc_tile): named as clobbered once, they count
   // as used everywhere, and the compiler keeps out of them.
@@ -890,28 +918,29 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
   } while (0)
 #define FP8GMM_MF1(i, j) FP8GMM_MFMA(i, j, fb1[j], fa1[i])
 
-  ItemTile cp_next = item_tile(0);  // the compute side's next record, fetched ahead like the load side's
   // The first 16 products of a tile (the low K half of its first step) start its accumulators from zero and need
   // registers only - the fragments are read a half-step ahead.  They are issued as soon as the accumulators are
   // free: from inside the previous tile's epilogue where that is the staged bf16 form, right after it otherwise.
   // Invariant at the top of the item loop: if the item has K work, those products are under way.
-  auto start_tile = [&fb0, &fa0]() {
+  // (a tile of half height has the products i < MT / 2 only)
+  auto start_tile = [&fb0, &fa0](bool half, bool upper_only = false) {
     static_for<MT * NT>([&](auto tc) {
       constexpr int i = decltype(tc)::value / NT, j = decltype(tc)::value % NT;
+      if ((i >= MT / 2 && half) || (i < MT / 2 && upper_only)) return;
       const i32x8 wf = fb0[j], tf = fa0[i];
       FP8GMM_MFMA_Z(i, j, wf, tf);
     });
   };
-  if (cp_next.nk > 0) start_tile();
+  if (cp_next.nk > 0) start_tile(nxt_half);
   // Where an epilogue cannot take the next tile's products in (every form but the staged bf16 one), it does not
   // have to carry that tile's first fragments through its arithmetic either: they are fetched again afterwards,
   // from the ring units that still hold them, which leaves the epilogue 64 more registers.
-  auto refetch_first_fragments = [&](int unit_a) {
+  auto refetch_first_fragments = [&](int unit_a, bool half) {
     const int unit_b = ring_inc(unit_a);
 #pragma unroll
     for (int j = 0; j < NT; ++j) read_frag_b(fb0[j], lds + unit_b * US, j, 0);
 #pragma unroll
-    for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds + unit_a * US, i, 0);
+    for (int i = 0; i < MT; ++i) read_frag_a(fa0[i], lds + unit_a * US, i, 0, half);
   };
   for (int r_cp = 0;; ++r_cp) {
     const ItemTile g = cp_next;
@@ -922,11 +951,18 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
     const float scale_ab = load_scale(pr.a_scale_inv) * load_scale(pr.b_scale_inv);
     const float scale_c = load_scale(pr.c_scale);
     const int m0 = g.m0, n0 = g.n0;
+    const bool cur_half = TILE == 256 && (g.flags & FP8GMM_ITEM_HALF_HEIGHT) != 0;   // this tile's height
+    bool read_half_next = cur_half;   // height of the tile that the NEXT step belongs to
 
     // One K = 128 step.  `same_item`: the load cursor stays inside its current item after this step (the caller
     // knows), so advancing it is three additions; otherwise the general advance, which may switch items.
-    auto k_step = [&](auto same_item, auto first) {
+    // `half_height_tile`: the sequence for a tile of half height.  The two heights are two kinds of step, each
+    // straight-line code: with both sequences inside one step behind a uniform branch, every wait for a fragment
+    // after the join becomes a wait for all of them (6 % of a launch).
+    auto k_step = [&](auto same_item, auto first, auto half_height_tile) {
       constexpr bool FIRST = decltype(first)::value;
+      constexpr bool SAME = decltype(same_item)::value;
+      constexpr bool HALF = decltype(half_height_tile)::value;
       // ring: [ua] tokens of this step, [ub] its weights, [na], [nb] the next step's, [fa] free since the
       // previous step's barrier: it receives the tokens of step + 2 during the low half-step.  The weights of
       // step + 2 go where this step's tokens are, once this step's barrier has shown that every wavefront
@@ -937,7 +973,38 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
       const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
       // ---- low K half: fragments in fa0 / fb0; fetch the high half's from the same units.  No barrier:
       // nothing written since the last one is read here.
-      if constexpr (TILE == 128) {
+      if constexpr (HALF) {
+        // a tile of half height: 8 products per K half, the same loads, three quarters of the fragment reads
+        const uint8_t* qa = lds + ua * US;
+        const uint8_t* qb = lds + ub * US;
+        dma_a(fa, 0);
+        half_b(fb1[0], qb, 0, 1, 0);
+        half_b(fb1[0], qb, 0, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 1); FP8GMM_SB();
+        dma_a(fa, 1);
+        half_b(fb1[1], qb, 1, 1, 0);
+        half_b(fb1[1], qb, 1, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 2); FP8GMM_SB();
+        dma_a(fa, 2);
+        half_b(fb1[2], qb, 2, 1, 0);
+        half_b(fb1[2], qb, 2, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(0, 3); FP8GMM_SB();
+        dma_a(fa, 3);
+        half_b(fb1[3], qb, 3, 1, 0);
+        half_b(fb1[3], qb, 3, 1, 1);
+        FP8GMM_SB(); FP8GMM_MF0(1, 0); FP8GMM_SB();
+        dma_a(fa, 4);
+        half_a(fa1[0], qa, 0, 1, 0, true);
+        half_a(fa1[0], qa, 0, 1, 1, true);
+        FP8GMM_SB(); FP8GMM_MF0(1, 1); FP8GMM_SB();
+        dma_a(fa, 5);
+        half_a(fa1[1], qa, 1, 1, 0, true);
+        half_a(fa1[1], qa, 1, 1, 1, true);
+        FP8GMM_SB(); FP8GMM_MF0(1, 2); FP8GMM_SB();
+        dma_a(fa, 6);
+        dma_a(fa, 7);
+        FP8GMM_SB(); FP8GMM_MF0(1, 3); FP8GMM_SB();
+      } else if constexpr (TILE == 128) {
         const uint8_t* qa = lds + ua * US;
         const uint8_t* qb = lds + ub * US;
         dma_a(fa, 0);
@@ -999,14 +1066,57 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
       }
       // ---- high K half: fragments in fa1 / fb1.  The barrier proves that every wavefront has read this
       // step's units (lgkmcnt(0)) and that the next step's units have landed for all of them.
-      if (relaxed) {
+      if (relaxed == kFastStores) {
         FP8GMM_WAIT_VM_LGKM(kParts + kFastStores);
-        relaxed = false;
+      } else if (relaxed == kFastStores / 2) {
+        FP8GMM_WAIT_VM_LGKM(kParts + kFastStores / 2);
       } else {
         FP8GMM_WAIT_VM_LGKM(kParts);
       }
+      relaxed = 0;
       __builtin_amdgcn_s_barrier();
-      if constexpr (TILE == 128) {
+      if constexpr (HALF) {
+        // the next step's fragments: in a step after which the load cursor may change items, all four token
+        // fragments, addressed as the tile of that step wants them (a tile of full height may follow)
+        const uint8_t* qa = lds + na * US;
+        const uint8_t* qb = lds + nb * US;
+        const bool nh = SAME ? true : read_half_next;
+        FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
+        dma_b(ua, 0);
+        half_b(fb0[0], qb, 0, 0, 0);
+        half_b(fb0[0], qb, 0, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF1(0, 1); FP8GMM_SB();
+        dma_b(ua, 1);
+        half_b(fb0[1], qb, 1, 0, 0);
+        half_b(fb0[1], qb, 1, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF1(0, 2); FP8GMM_SB();
+        dma_b(ua, 2);
+        half_b(fb0[2], qb, 2, 0, 0);
+        half_b(fb0[2], qb, 2, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF1(0, 3); FP8GMM_SB();
+        dma_b(ua, 3);
+        half_b(fb0[3], qb, 3, 0, 0);
+        half_b(fb0[3], qb, 3, 0, 1);
+        FP8GMM_SB(); FP8GMM_MF1(1, 0); FP8GMM_SB();
+        dma_b(ua, 4);
+        half_a(fa0[0], qa, 0, 0, 0, nh);
+        half_a(fa0[0], qa, 0, 0, 1, nh);
+        FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
+        dma_b(ua, 5);
+        half_a(fa0[1], qa, 1, 0, 0, nh);
+        half_a(fa0[1], qa, 1, 0, 1, nh);
+        FP8GMM_SB(); FP8GMM_MF1(1, 2); FP8GMM_SB();
+        dma_b(ua, 6);
+        if constexpr (!SAME) {
+          half_a(fa0[2], qa, 2, 0, 0, nh);
+          half_a(fa0[2], qa, 2, 0, 1, nh);
+        }
+        dma_b(ua, 7);
+        if constexpr (!SAME) {
+          half_a(fa0[3], qa, 3, 0, 0, nh);
+          half_a(fa0[3], qa, 3, 0, 1, nh);
+        }
+      } else if constexpr (TILE == 128) {
         const uint8_t* qa = lds + na * US;
         const uint8_t* qb = lds + nb * US;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
@@ -1021,15 +1131,11 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
         FP8GMM_SB(); FP8GMM_MF1(1, 1); FP8GMM_SB();
         dma_b(ua, 3);
         read_frag_a(fa0[1], qa, 1, 0);
-        if constexpr (decltype(same_item)::value) {
-          ++ld_kt;
-          step_setup();
-        } else {
-          dma_advance();
-        }
       } else {
         const uint8_t* qa = lds + na * US;
         const uint8_t* qb = lds + nb * US;
+        // (after a step that may end its item, the next step's tile may be of half height)
+        const bool nh = decltype(same_item)::value ? false : read_half_next;
         FP8GMM_SB(); FP8GMM_MF1(0, 0); FP8GMM_SB();
         dma_b(ua, 0);
         half_b(fb0[0], qb, 0, 0, 0);
@@ -1049,71 +1155,93 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
         half_b(fb0[3], qb, 3, 0, 1);
         FP8GMM_SB(); FP8GMM_MF1(1, 2); FP8GMM_SB();
         dma_b(ua, 3);
-        half_a(fa0[0], qa, 0, 0, 0);
+        half_a(fa0[0], qa, 0, 0, 0, nh);
         FP8GMM_SB(); FP8GMM_MF1(1, 3); FP8GMM_SB();
-        half_a(fa0[0], qa, 0, 0, 1);
+        half_a(fa0[0], qa, 0, 0, 1, nh);
         FP8GMM_SB(); FP8GMM_MF1(2, 0); FP8GMM_SB();
         dma_b(ua, 4);
-        half_a(fa0[1], qa, 1, 0, 0);
+        half_a(fa0[1], qa, 1, 0, 0, nh);
         FP8GMM_SB(); FP8GMM_MF1(2, 1); FP8GMM_SB();
-        half_a(fa0[1], qa, 1, 0, 1);
+        half_a(fa0[1], qa, 1, 0, 1, nh);
         FP8GMM_SB(); FP8GMM_MF1(2, 2); FP8GMM_SB();
         dma_b(ua, 5);
-        half_a(fa0[2], qa, 2, 0, 0);
+        half_a(fa0[2], qa, 2, 0, 0, nh);
         FP8GMM_SB(); FP8GMM_MF1(2, 3); FP8GMM_SB();
-        half_a(fa0[2], qa, 2, 0, 1);
+        half_a(fa0[2], qa, 2, 0, 1, nh);
         FP8GMM_SB(); FP8GMM_MF1(3, 0); FP8GMM_SB();
         dma_b(ua, 6);
-        half_a(fa0[3], qa, 3, 0, 0);
+        half_a(fa0[3], qa, 3, 0, 0, nh);
         FP8GMM_SB(); FP8GMM_MF1(3, 1); FP8GMM_SB();
         dma_b(ua, 7);
-        half_a(fa0[3], qa, 3, 0, 1);
-        if constexpr (decltype(same_item)::value) {
-          ++ld_kt;
-          step_setup();
-        } else {
-          dma_advance();
-        }
+        half_a(fa0[3], qa, 3, 0, 1, nh);
+      }
+      // common to every sequence: the load cursor moves on (in the shadow of the step's last products)
+      if constexpr (SAME) {
+        ++ld_kt;
+        step_setup();
+      } else {
+        dma_advance();
+      }
+      if constexpr (HALF) {
+        FP8GMM_SB(); FP8GMM_MF1(1, 3); FP8GMM_SB();
+      } else if constexpr (TILE == 256) {
         FP8GMM_SB(); FP8GMM_MF1(3, 2); FP8GMM_MF1(3, 3); FP8GMM_SB();
       }
       ua = na;
     };
     // The load cursor runs two steps ahead of this loop: while at least three steps of the item remain, its
     // next step lies in the same item.
-    int kt = 0;
-    if (g.nk > 0) {
-      k_step(std::false_type{}, std::true_type{});
-      kt = 1;
-    } else {
-      static_for<MT * NT>([&](auto tc) { acc_tile_clear<16 * decltype(tc)::value>(); });
-    }
-    for (; kt + 3 < g.nk; ++kt) k_step(std::true_type{}, std::false_type{});
-    for (; kt < g.nk; ++kt) k_step(std::false_type{}, std::false_type{});
+    // The token fragments that a tile's LAST step reads belong to the next tile with K steps, and are addressed by
+    // that tile's height.
+    const bool after_half = half_height(cp_next);
+    // One run of steps per height, one after the other, the run of the other height with no steps: as alternatives
+    // behind a branch, the compiler carries the load cursor's scalar state (descriptors, LDS addresses) through the
+    // join in vector registers, which the LDS-DMA statements cannot take.
+    auto steps = [&](int nk, auto half_c) {
+      int kt = 0;
+      if (nk > 0) {
+        if (nk == 1) read_half_next = after_half;
+        k_step(std::false_type{}, std::true_type{}, half_c);
+        kt = 1;
+      }
+      for (; kt + 3 < nk; ++kt) k_step(std::true_type{}, std::false_type{}, half_c);
+      for (; kt < nk; ++kt) {
+        if (kt == nk - 1) read_half_next = after_half;
+        k_step(std::false_type{}, std::false_type{}, half_c);
+      }
+    };
+    if (g.nk == 0) static_for<MT * NT>([&](auto tc) { acc_tile_clear<16 * decltype(tc)::value>(); });
+    steps(cur_half ? 0 : g.nk, std::false_type{});
+    if constexpr (TILE == 256) steps(cur_half ? g.nk : 0, std::true_type{});
     // ---- epilogue ----
     uint8_t* const stage = lds + ((ua + 4) % RING) * US;  // free until the next step's token loads
     const bool more = cp_next.prob >= 0 && cp_next.nk > 0;  // the fragments in fa0 / fb0 open another tile
+    const int mt = cur_half ? MT / 2 : MT;                  // 32-row blocks of this tile per wavefront
     if (g.slot >= 0) {
       // a piece of a tile that is shared along K: leave the accumulators for the fix-up kernel
       partial_store<TILE>(workspace + (size_t)g.slot * kPartialBytes);
-      relaxed = false;
+      relaxed = 0;
       if (more) {
-        refetch_first_fragments(ua);
-        start_tile();
+        refetch_first_fragments(ua, after_half);
+        start_tile(after_half);
       }
     } else if (more && staged_bf16_tile<TILE>(pr, m0, n0, out_kind, epilogue)) {
       // the next tile's first products go out as the accumulators they overwrite are read out, in the shadow of
       // the epilogue's vector arithmetic
-      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, !A_TR, scale_ab, scale_c,
-                                    [&fb0, &fa0](auto ic, auto jc) {
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, mt, !A_TR && !B_TR, !A_TR, scale_ab, scale_c,
+                                    [&fb0, &fa0, after_half](auto ic, auto jc) {
                                       constexpr int i = decltype(ic)::value, j = decltype(jc)::value;
+                                      if (i >= MT / 2 && after_half) return;
                                       const i32x8 wf = fb0[j], tf = fa0[i];
                                       FP8GMM_MFMA_Z(i, j, wf, tf);
                                     });
+      // a tile of half height released the lower blocks only
+      if (cur_half && !after_half) start_tile(false, true);
     } else {
-      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, !A_TR && !B_TR, !A_TR, scale_ab, scale_c);
+      relaxed = tile_epilogue<TILE>(pr, m0, n0, out_kind, epilogue, stage, mt, !A_TR && !B_TR, !A_TR, scale_ab, scale_c);
       if (more) {
-        refetch_first_fragments(ua);
-        start_tile();
+        refetch_first_fragments(ua, after_half);
+        start_tile(after_half);
       }
     }
   }

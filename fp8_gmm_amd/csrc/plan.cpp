@@ -389,6 +389,8 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
     if (it.slot >= 0) {
       o.slot = slot_map[it.slot];
       if (o.slot < 0) dangling_piece = true;  // a partial item that no fix-up record completes
+    } else if (rows <= BM / 2) {
+      o.flags = FP8GMM_ITEM_HALF_HEIGHT;      // a whole tile with at most 128 valid rows
     }
   };
   for (int wg = 0; wg < grid; ++wg) {
@@ -427,6 +429,18 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
     }
     count[wg] = r;
     if (r > rounds) rounds = r;
+    // records without K steps repeat the height of the next record that has some (see FP8GMM_ITEM_HALF_HEIGHT)
+    int next_height = 0;
+    for (int q = r - 1; q >= 0; --q) {
+      const size_t index = (size_t)q * grid + wg;
+      if (index >= (size_t)max_items) continue;
+      fp8gmm_gemm_item& o = items[index];
+      if (o.nk == 0) {
+        o.flags |= next_height << 1;
+      } else {
+        next_height = o.flags & FP8GMM_ITEM_HALF_HEIGHT;
+      }
+    }
   }
   rounds += 1;  // every list ends with a record whose prob is -1
   const int n_fixups = (int)fix.size();

@@ -191,8 +191,14 @@ typedef struct fp8gmm_gemm_item {
   int32_t m0, n0;      /* origin of the tile in c */
   int32_t prob;        /* index into the problem table; -1 ends a workgroup's list */
   int32_t slot;        /* -1: whole tile, the epilogue runs; else the workspace slot that receives the partial sums */
-  int32_t reserved;
+  int32_t flags;       /* FP8GMM_ITEM_* */
 } fp8gmm_gemm_item;    /* 64 bytes */
+/* The tile holds at most 128 valid rows (the last row of tiles of a ragged problem): the kernel runs it at half
+ * height - its wavefronts stand on rows 64 w + 32 i, i < 2, and issue half the products; same loads, same bits.
+ * Whole 256 x 256 tiles only (never a piece of a tile shared along K).  In a record without K steps (nk == 0) the
+ * bit one position up repeats this flag of the workgroup's next record that has K steps: the kernel's load stream
+ * skips records without K steps, and what it fetches at the end of a tile is laid out for the tile that follows. */
+#define FP8GMM_ITEM_HALF_HEIGHT 1
 
 /* One tile that was shared along K: the fix-up launch adds the partial sums of the workspace slots first_slot,
  * first_slot + 1, ..., first_slot + n_pieces - 1 (the tile's pieces in K order) and runs the epilogue. */

@@ -142,6 +142,16 @@ def check_launch_plan(shapes, table, total, grid, stream_k):
                 assert 0 <= rec["slot"] < plan.n_slots and slot not in slot_name
                 slot_name[slot] = int(rec["slot"])
                 pieces_of.setdefault((prob, m0, n0), []).append((k_begin, int(rec["slot"])))
+        # height: whole tiles with at most 128 valid rows are flagged; a record without K steps repeats, one bit
+        # up, the flag of the workgroup's next record that has some
+        following = 0
+        for rec, (tile, prob, m0, n0, k_begin, nk, slot) in reversed(list(zip(col, want))):
+            half = int(slot < 0 and shapes[prob][0] - m0 <= TILE // 2)
+            if nk == 0:
+                assert rec["flags"] == half | following << 1
+            else:
+                assert rec["flags"] == half
+                following = half
     assert plan.rounds == longest + 1
     assert sorted(slot_name.values()) == list(range(plan.n_slots))   # renumbered from 0 without gaps
     assert plan.n_fixups == len(fixups) == len(pieces_of)
@@ -324,3 +334,37 @@ def test_small_tile_plan():
     plan = _lib.GemmPlan()
     assert _lib.load().fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 1, _lib.GEMM_TILE_128 | _lib.EPI_GELU, 16, 0,
                                                        None, 0, None, 0, ctypes.byref(plan)) < 0
+
+
+def test_half_height_flag_marks_the_ragged_last_row_of_tiles():
+    """FP8GMM_ITEM_HALF_HEIGHT: the one tile row of a 100-row problem and the last of a 300-row problem (44 rows),
+    not the 129 valid rows of a 385-row problem; never a piece of a tile shared along K; never a 128 x 128 tile."""
+    shapes = [(100, 512, 256), (300, 512, 256), (385, 256, 256), (128, 256, 256)]
+    table, total = make_table(shapes)
+    plan, items, _ = _lib.plan_grouped_gemm_launch(table.copy(), 0, 8, False)
+    recs = items[items["prob"] >= 0]
+    assert len(recs) == total == 2 + 4 + 2 + 1
+    flagged = sorted((int(r["prob"]), int(r["m0"]), int(r["n0"])) for r in recs if r["flags"] & 1)
+    assert flagged == [(0, 0, 0), (0, 0, 256), (1, 256, 0), (1, 256, 256), (3, 0, 0)]
+    assert (items["flags"][items["prob"] < 0] == 0).all()
+    # a single short tile, shared along K between the workgroups: pieces run at full height
+    table, total = make_table([(100, 256, 8192)])
+    plan, items, fixups = _lib.plan_grouped_gemm_launch(table.copy(), 0, 64, True)
+    assert plan.n_slots > 1 and len(fixups) == 1 and (items["flags"] == 0).all()
+    plan, items, _ = _lib.plan_grouped_gemm_launch(table.copy(), _lib.GEMM_TILE_128, 64, False)
+    assert plan.tile == 128 and (items["flags"] == 0).all()
+
+
+def test_slot_cap_falls_back_to_whole_tiles():
+    """stream_k > 1 states how many workspace slots the caller has: a plan that would need more shares nothing."""
+    fc2 = [(m, 4096, 14336) for m in MLP]
+    table, total = make_table(fc2)
+    free, items_free, fix_free = _lib.plan_grouped_gemm_launch(table.copy(), 0, 256, True)
+    assert free.n_slots > 2 and free.n_fixups > 0
+    enough, items_enough, fix_enough = _lib.plan_grouped_gemm_launch(table.copy(), 0, 256, free.n_slots)
+    assert (enough.n_slots, enough.n_fixups, enough.rounds) == (free.n_slots, free.n_fixups, free.rounds)
+    assert items_enough.tobytes() == items_free.tobytes() and fix_enough.tobytes() == fix_free.tobytes()
+    whole, items_whole, _ = _lib.plan_grouped_gemm_launch(table.copy(), 0, 256, False)
+    short, items_short, fix_short = _lib.plan_grouped_gemm_launch(table.copy(), 0, 256, free.n_slots - 1)
+    assert (short.n_slots, short.n_fixups, len(fix_short)) == (0, 0, 0) and short.rounds == whole.rounds
+    assert items_short.tobytes() == items_whole.tobytes()
