@@ -438,7 +438,12 @@ def measure_module(args):
                                  "tflops": round(ach, 1), "frac_of_mfma_peak": round(ach / FP8_PEAK_TFLOPS, 4),
                                  "algorithmic_bytes_per_launch": round(d["bytes"]),
                                  "algorithmic_GBps": round(alg_gbs, 1),
-                                 "frac_of_hbm_peak": round(alg_gbs / HBM_PEAK_GBS, 4)}
+                                 "frac_of_hbm_peak": round(alg_gbs / HBM_PEAK_GBS, 4),
+                                 "by_form": {form: {
+                                     "launches_per_step": c["launches"] / args.steps, "ms": round(c["ms"], 4),
+                                     "frac_of_mfma_peak": round(c["work"] / (c["ms"] * 1e-3) / 1e12 / FP8_PEAK_TFLOPS, 4),
+                                     "frac_of_hbm_peak": round(c["bytes"] / (c["ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                                     for form, c in sorted(d.get("forms", {}).items())}}
                 traffic = gemm_hbm_traffic(args.workload)
                 roofline = {"kernel": "grouped_gemm_kernel", "bound": "mfma", "achieved": round(ach, 1),
                             "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / FP8_PEAK_TFLOPS, 4),

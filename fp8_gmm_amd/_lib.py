@@ -175,6 +175,7 @@ EXPORTS = (
     "fp8gmm_multi_cast_dgelu",
     "fp8gmm_grouped_gemm",
     "fp8gmm_delayed_scaling_update",
+    "fp8gmm_upload",
     "fp8gmm_route_workspace_bytes",
     "fp8gmm_route_sort",
     "fp8gmm_route_invert",
@@ -261,6 +262,8 @@ def load():
     L.fp8gmm_sizeof_pass_plan.argtypes = []
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
+    L.fp8gmm_upload.restype = ci
+    L.fp8gmm_upload.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t
     L.fp8gmm_route_workspace_bytes.argtypes = [ci, ci]
     L.fp8gmm_route_sort.restype = ci

@@ -55,10 +55,11 @@ class kernel_timing:
     """Context manager that brackets every kernel launch of this module with HIP events.
 
     The events are recorded on the stream the kernels are launched on (torch's current
-    stream).  ``records`` holds ``(kernel name, algorithmic work, algorithmic bytes, start event, end event)``;
-    ``summary()`` synchronises and returns per-kernel launch counts, mean duration in ms, the
+    stream).  ``records`` holds ``(kernel name, algorithmic work, algorithmic bytes, start event, end event,
+    form)``; ``summary()`` synchronises and returns per-kernel launch counts, mean duration in ms, the
     algorithmic work (flops for the GEMM, bytes for the other kernels) and the algorithmic bytes
-    (every operand read once, every result written once) per launch.
+    (every operand read once, every result written once) per launch; for the grouped GEMM also the same four
+    figures per operand form under ``"forms"`` (``gemm_form``).
     """
 
     _active = None
@@ -77,25 +78,43 @@ class kernel_timing:
     def summary(self):
         torch.cuda.synchronize()
         out = {}
-        for name, work, nbytes, start, end in self.records:
+        for name, work, nbytes, start, end, form in self.records:
+            ms = start.elapsed_time(end)
             d = out.setdefault(name, {"launches": 0, "ms": 0.0, "work": 0.0, "bytes": 0.0})
-            d["launches"] += 1
-            d["ms"] += start.elapsed_time(end)
-            d["work"] += work
-            d["bytes"] += nbytes
+            cells = [d]
+            if form is not None:
+                cells.append(d.setdefault("forms", {}).setdefault(form, {"launches": 0, "ms": 0.0, "work": 0.0,
+                                                                         "bytes": 0.0}))
+            for c in cells:
+                c["launches"] += 1
+                c["ms"] += ms
+                c["work"] += work
+                c["bytes"] += nbytes
         for d in out.values():
-            d["ms"] /= d["launches"]
-            d["work"] /= d["launches"]
-            d["bytes"] /= d["launches"]
+            for c in [d] + list(d.get("forms", {}).values()):
+                for key in ("ms", "work", "bytes"):
+                    c[key] /= c["launches"]
         return out
 
 
+def gemm_form(a_fmt, flags):
+    """Name of a grouped-GEMM launch by what it reads: the format of operand a (0 = e4m3, 1 = e5m2: a gradient) and
+    which operands are stored contraction-major (the launch's FP8GMM_GEMM_*_KMAJOR flags)."""
+    fmt = "e5m2" if a_fmt == _lib.E5M2 else "e4m3"
+    if flags & _lib.GEMM_A_KMAJOR:
+        return f"{fmt} a and b contraction-major (weight gradient in place)"
+    if flags & _lib.GEMM_B_KMAJOR:
+        return f"{fmt} a row-major, b contraction-major"
+    return f"{fmt} a and b row-major" + (", GELU epilogue" if flags & _lib.EPI_GELU else "")
+
+
 class _timed:
-    def __init__(self, name, work_fn, bytes_fn=None):
+    def __init__(self, name, work_fn, bytes_fn=None, form=None):
         self.rec = kernel_timing._active
         if self.rec is not None:
             self.name, self.work = name, float(work_fn())
             self.bytes = float(bytes_fn()) if bytes_fn is not None else self.work
+            self.form = form() if callable(form) else form
 
     def __enter__(self):
         if self.rec is not None:
@@ -106,7 +125,7 @@ class _timed:
         if self.rec is not None:
             end = torch.cuda.Event(enable_timing=True)
             end.record()
-            self.rec.records.append((self.name, self.work, self.bytes, self.start, end))
+            self.rec.records.append((self.name, self.work, self.bytes, self.start, end, self.form))
         return False
 
 
@@ -161,18 +180,110 @@ def _device_of(tensors):
     return dev
 
 
+class _Staging:
+    """Page-locked host memory, mapped into the device's address space, in which the tables of the launches are
+    written and from which ``fp8gmm_upload`` (a kernel on the launch stream) copies them to device memory.
+
+    Two halves used in turn: pieces are handed out from one half until it is full; before the other half is written
+    again, the host waits for the events recorded, on every stream that read from it, when it was left - so a piece
+    is never overwritten while a copy kernel may still read it, and the host only ever waits when the GPU is a whole
+    half (hundreds of launches) behind.  One per device, shared by all threads."""
+
+    HALF = 16 << 20
+
+    def __init__(self):
+        # zeroed, not just allocated: the first write to each page of fresh page-locked memory costs the host a
+        # page fault (0.15 ms per MB of tables, for the first 2 x HALF bytes of uploads)
+        self.host = torch.zeros(2 * self.HALF, dtype=torch.uint8, pin_memory=True)
+        self.bytes = self.host.numpy()
+        self.base = self.host.data_ptr()
+        self.lock = threading.Lock()
+        self.half, self.used = 0, 0
+        self.readers = [{}, {}]     # per half: stream handle -> torch stream object that read from it
+        self.left = [[], []]        # per half: events recorded when it was left
+
+    def reserve(self, nbytes, stream):
+        """Offset of ``nbytes`` (rounded up to 256) of staging memory that ``stream`` will read, or None when the
+        request is larger than a half."""
+        n = (nbytes + 255) & ~255
+        if n > self.HALF:
+            return None
+        with self.lock:
+            if self.used + n > self.HALF:
+                for s in self.readers[self.half].values():
+                    ev = torch.cuda.Event()
+                    ev.record(s)
+                    self.left[self.half].append(ev)
+                self.readers[self.half] = {}
+                self.half ^= 1
+                self.used = 0
+                for ev in self.left[self.half]:
+                    ev.synchronize()
+                self.left[self.half] = []
+            offset = self.half * self.HALF + self.used
+            self.used += n
+            self.readers[self.half].setdefault(stream.cuda_stream, stream)
+        return offset
+
+    def give_back(self, offset, reserved, used):
+        """The piece at ``offset`` needs only ``used`` of its ``reserved`` bytes: the rest is handed out again if
+        nothing was reserved after it."""
+        reserved, used = (reserved + 255) & ~255, (used + 255) & ~255
+        with self.lock:
+            if offset + reserved == self.half * self.HALF + self.used:
+                self.used -= reserved - used
+
+
+_staging = {}
+
+
+def _staging_of(device):
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    st = _staging.get(index)
+    if st is None:
+        st = _staging.setdefault(index, _Staging())
+    return st
+
+
+def _to_device(device, room, fill):
+    """Device copy (uint8 tensor) of the tables that ``fill(host address, numpy view of the host bytes)`` writes
+    into ``room`` bytes of staging memory; ``fill`` returns how many of them it used (None: all; 0: nothing to
+    copy, the result is None).  The copy is enqueued on the current stream of ``device``."""
+    room = (room + 15) & ~15
+    with _on_device(device):
+        stream = torch.cuda.current_stream(device)
+        st = _staging_of(device) if options.upload == "kernel" else None
+        offset = st.reserve(room, stream) if st is not None else None
+        if offset is None:   # larger than the staging area, or by choice: a pinned buffer of its own and torch's copy
+            pinned = torch.empty(room, dtype=torch.uint8, pin_memory=True)
+            used = fill(pinned.data_ptr(), pinned.numpy())
+            used = room if used is None else (used + 15) & ~15
+            return pinned[:used].to(device, non_blocking=True) if used else None
+        used = fill(st.base + offset, st.bytes[offset: offset + room])
+        used = room if used is None else (used + 15) & ~15
+        if used < room:
+            st.give_back(offset, room, used)
+        if not used:
+            return None
+        out = torch.empty(used, dtype=torch.uint8, device=device)
+        _lib.check(_lib.load().fp8gmm_upload(out.data_ptr(), st.base + offset, used, stream.cuda_stream))
+    return out
+
+
 def _upload(table, device):
     """Host table (numpy structured array) -> device bytes, asynchronously on the current stream."""
-    host = torch.from_numpy(table.view(np.uint8).reshape(-1))
-    pinned = torch.empty(host.numel(), dtype=torch.uint8, pin_memory=True)
-    pinned.copy_(host)
-    return pinned.to(device, non_blocking=True)
+    raw = table.view(np.uint8).reshape(-1)
+
+    def fill(_, host):
+        host[: raw.size] = raw
+        host[raw.size:] = 0
+
+    return _to_device(device, raw.size, fill)
 
 
-# A launch needs its table in device memory, and every upload is a small copy kernel with a dispatch gap on
-# either side (about 20 us per launch on an otherwise busy GPU).  Inside ``batched_uploads()`` the entry
-# points only plan and queue their launch; at the end of the block all queued tables travel in ONE copy
-# and the kernels are launched back to back, in the order they were queued.
+# A launch needs its table in device memory, and every upload is a small copy kernel in front of it.  Inside
+# ``batched_uploads()`` the entry points only plan and queue their launch; at the end of the block all queued
+# tables travel in ONE copy and the kernels are launched back to back, in the order they were queued.
 _pending = threading.local()
 
 
@@ -227,11 +338,11 @@ def _flush(items):
         for table, _, _, _ in group:
             offsets.append(total)
             total += (table.nbytes + 127) // 128 * 128   # every table on its own cache lines
-        pinned = torch.empty(total, dtype=torch.uint8, pin_memory=True)
-        host = pinned.numpy()
-        for (table, _, _, _), off in zip(group, offsets):
-            host[off: off + table.nbytes] = table.view(np.uint8).reshape(-1)
-        dev_tables = pinned.to(device, non_blocking=True)
+        def fill(_, host, group=group, offsets=offsets):
+            for (table, _, _, _), off in zip(group, offsets):
+                host[off: off + table.nbytes] = table.view(np.uint8).reshape(-1)
+
+        dev_tables = _to_device(device, total, fill)
         base = dev_tables.data_ptr()
         for (_, _, launch, _), off in zip(group, offsets):
             launch(base + off)
@@ -644,7 +755,8 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
             ws = _gemm_workspace(device, plan.n_slots)
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
             with _timed("grouped_gemm", lambda: _algorithmic_flops(table),
-                        lambda: _algorithmic_gemm_bytes(table, 2 if c_dtype == torch.bfloat16 else 1)):
+                        lambda: _algorithmic_gemm_bytes(table, 2 if c_dtype == torch.bfloat16 else 1),
+                        lambda: gemm_form(fmts[0], fmts[3])):
                 fix_ptr = dev_ptr + off_fix if plan.n_fixups else None
                 rc = _lib.load().fp8gmm_grouped_gemm(dev_ptr, n, dev_ptr + off_items, fix_ptr, plan, *fmts, ws_ptr,
                                                      ws_bytes, _stream(device))
@@ -673,16 +785,19 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
 # scratch memory for partial sums and a second, small launch; options.stream_k = False plans every launch without it.
 class GemmOptions:
     """Launch policy of the grouped GEMMs of this process: ``tile`` "auto" | "256" | "128", ``stream_k`` (share the
-    tail tiles of a launch along K), ``wgrad`` "in_place" | "copy".  The defaults can be preset with the
-    environment variables FP8GMM_TILE, FP8GMM_STREAMK (0 turns sharing off) and FP8GMM_WGRAD, read once when the
-    module is imported; afterwards assign the attributes or use ``gemm_options(...)`` for a block."""
+    tail tiles of a launch along K), ``wgrad`` "in_place" | "copy", ``upload`` "kernel" (tables reach the device
+    through staging memory and a copy kernel of the library) | "copy" (a pinned buffer per upload and torch's
+    asynchronous copy).  The defaults can be preset with the environment variables FP8GMM_TILE, FP8GMM_STREAMK
+    (0 turns sharing off), FP8GMM_WGRAD and FP8GMM_UPLOAD, read once when the module is imported; afterwards assign
+    the attributes or use ``gemm_options(...)`` for a block."""
 
-    __slots__ = ("tile", "stream_k", "wgrad")
+    __slots__ = ("tile", "stream_k", "wgrad", "upload")
 
     def __init__(self, env=os.environ):
         self.tile = env.get("FP8GMM_TILE", "auto")
         self.stream_k = env.get("FP8GMM_STREAMK", "1") != "0"
         self.wgrad = env.get("FP8GMM_WGRAD", "in_place")
+        self.upload = env.get("FP8GMM_UPLOAD", "kernel")
 
 
 options = GemmOptions()
@@ -747,15 +862,17 @@ def release_workspaces():
 
 def warm_up(device=None):
     """Do everything a first launch on `device` would do besides the launch itself - the library's per-device
-    initialisation and the allocation of a tail-balancing workspace of the largest size a launch can need
-    (2 x grid slots of 256 KB: 128 MiB on 256 compute units) for the current stream - so that none of it falls
-    into a timed or captured region."""
+    initialisation, the allocation of a tail-balancing workspace of the largest size a launch can need
+    (2 x grid slots of 256 KB: 128 MiB on 256 compute units) for the current stream, and of the page-locked staging
+    memory of the table uploads - so that none of it falls into a timed or captured region."""
     device = torch.device("cuda") if device is None else torch.device(device)
     if device.index is None:
         device = torch.device("cuda", torch.cuda.current_device())
     grid = _lib.gemm_grid(_lib.init(device.index))
     with _on_device(device):
         _gemm_workspace(device, 2 * grid)
+        if options.upload == "kernel":
+            _staging_of(device)
 
 
 # ------------------------------------------------------------------------------------------------
@@ -795,15 +912,21 @@ def linear_pass(device, backward=False, **fields):
     bound = 4096 + desc.experts * (2 * 128 + 3 * 96) + 3 * (tiles + 8 * grid) * 64 + 3 * 32 * 2 * grid
     plan = _lib.PassPlan()
     fn = L.fp8gmm_plan_linear_backward if backward else L.fp8gmm_plan_linear_forward
-    pinned = torch.empty(bound, dtype=torch.uint8, pin_memory=True)
-    rc = fn(ctypes.byref(desc), pinned.data_ptr(), bound, ctypes.byref(plan))
-    if rc == -8:   # FP8GMM_ERR_BUFFER_TOO_SMALL: the plan says how much room it needs
-        bound = int(plan.blob_bytes)
-        pinned = torch.empty(bound, dtype=torch.uint8, pin_memory=True)
-        rc = fn(ctypes.byref(desc), pinned.data_ptr(), bound, ctypes.byref(plan))
-    _lib.check(rc)
+    # the planner writes the tables straight into staging memory
+    while True:
+        def fill(address, _):
+            fill.rc = fn(ctypes.byref(desc), address, bound, ctypes.byref(plan))
+            return int(plan.blob_bytes) if fill.rc == 0 else 0
+
+        blob = _to_device(device, bound, fill)
+        if fill.rc == -8 and plan.blob_bytes > bound:   # FP8GMM_ERR_BUFFER_TOO_SMALL: the plan says how much room it needs
+            bound = int(plan.blob_bytes)
+            continue
+        _lib.check(fill.rc)
+        break
+    if blob is None:
+        return plan
     with _on_device(device):
-        blob = pinned[: plan.blob_bytes].to(device, non_blocking=True)
         base, stream = blob.data_ptr(), _stream(device)
         for i in range(plan.n_launches):
             rec = plan.launch[i]
@@ -811,10 +934,11 @@ def linear_pass(device, backward=False, **fields):
                 continue
             ws = _gemm_workspace(device, rec.plan.n_slots) if rec.kind == _lib.PASS_GEMM else None
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
-            with _timed(_PASS_KERNEL_NAMES[rec.kind], lambda: rec.work, lambda: rec.bytes):
+            with _timed(_PASS_KERNEL_NAMES[rec.kind], lambda: rec.work, lambda: rec.bytes,
+                        (lambda: gemm_form(rec.a_fmt, rec.epilogue)) if rec.kind == _lib.PASS_GEMM else None):
                 rc = L.fp8gmm_run_planned(base, ctypes.byref(rec), ws_ptr, ws_bytes, stream)
             _lib.check(rc)
-    return plan, pinned
+    return plan
 
 
 def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False, keep_scale_inv=None):

@@ -208,6 +208,18 @@ int launch_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int 
 }
 }  // namespace
 
+namespace fp8gmm {
+// Tables travel host -> device through this kernel: it reads page-locked host memory that is mapped into the
+// device's address space, 16 bytes per thread, and writes device memory.  A copy enqueued with hipMemcpyAsync runs
+// as a transfer of its own whose hand-over to the next kernel of the stream took 25 - 30 us on this machine; a
+// kernel of the stream hands over like any other kernel.
+__global__ void __launch_bounds__(256) upload_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src,
+                                                     unsigned pieces) {
+  const unsigned i = blockIdx.x * 256u + threadIdx.x;
+  if (i < pieces) dst[i] = src[i];
+}
+}  // namespace fp8gmm
+
 extern "C" {
 
 int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scale_inv, int history_len, int slots,
@@ -239,6 +251,19 @@ int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total
   if (descs_dev == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipLaunchKernelGGL(fp8gmm::multi_scale_mul_kernel, dim3(total_blocks), dim3(fp8gmm::kPwThreads), 0,
                      static_cast<hipStream_t>(stream), descs_dev, n);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_upload(void* dst_dev, const void* src_host, size_t bytes, void* stream) {
+  if (bytes == 0) return FP8GMM_OK;
+  if (dst_dev == nullptr || src_host == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  if (((reinterpret_cast<uintptr_t>(dst_dev) | reinterpret_cast<uintptr_t>(src_host) | bytes) & 15) != 0)
+    return FP8GMM_ERR_ALIGNMENT;
+  if (bytes > (size_t(1) << 30)) return FP8GMM_ERR_BAD_ARGUMENT;
+  const unsigned pieces = (unsigned)(bytes / 16);
+  hipLaunchKernelGGL(fp8gmm::upload_kernel, dim3((pieces + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<uint4*>(dst_dev),
+                     static_cast<const uint4*>(src_host), pieces);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 

@@ -417,6 +417,17 @@ int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scal
                                   float fp8_max, int margin, int most_recent, int keep_period, int keep_phase,
                                   void* stream);
 
+/*
+ * Copy `bytes` of tables from page-locked host memory that the device can address (hipHostMalloc; torch's
+ * pin_memory) to device memory with a kernel on `stream`: dst_dev, src_host and bytes multiples of 16, at most
+ * 1 GiB.  The host memory must stay as it is until the stream has passed this point.  Every launch entry point of
+ * this header reads its tables from device memory; the reference hands the same tables over as launch arguments
+ * (csrc/multi_pad_fusion.cu:14-35,495-501, csrc/multi_pointwise.cu) or with one synchronous copy per array
+ * (cutlass::DeviceAllocation::copy_from_host, csrc/fp8_gmm.cu:116-135).  A hipMemcpyAsync on the stream does the
+ * same job; measured here its hand-over to the next kernel costs 25 - 30 us per copy, a kernel's 2 - 4.
+ */
+int fp8gmm_upload(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+
 /* ---- token routing around the expert layers ----------------------------------------------- */
 /*
  * The reference's example MoE layers (fp8_gmm/example.py:15-32,50-59,86-94,113-119) take these steps from the

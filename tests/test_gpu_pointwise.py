@@ -358,3 +358,36 @@ def test_delayed_scaling_update_matches_the_torch_rule(dev, history_len, slots, 
         bump = torch.rand(slots, generator=g) * 3.0
         cpu.amax_history[0] += bump
         gpu.amax_history[0] += bump.to(dev)
+
+
+def test_tables_reach_the_device_through_the_staging_memory(dev, monkeypatch):
+    """Tables are written into page-locked staging memory and copied by a kernel of the library (fp8gmm_upload).
+    With the staging area shrunk to 2 x 8 KiB its halves are reused every few uploads: every device copy must hold
+    its own table, also those made while earlier copies are still queued behind a long kernel, on two streams, and
+    a table larger than a half goes through a buffer of its own."""
+    import numpy as np
+
+    backend = _backend()
+    monkeypatch.setattr(backend._Staging, "HALF", 8192)
+    monkeypatch.setattr(backend, "_staging", {})
+    rng = np.random.default_rng(5)
+    busy = torch.randn(4096, 4096, device=dev)
+    side = torch.cuda.Stream(device=dev)
+    copies = []
+    for i in range(300):
+        n = int(rng.choice([1, 16, 100, 1000, 3000, 8192, 20000]))
+        table = rng.integers(0, 256, size=n, dtype=np.uint8)
+        if i % 25 == 0:
+            busy = busy @ busy * 1e-4      # keeps the stream busy, so that copies queue up behind it
+        if i % 7 == 3:
+            side.wait_stream(torch.cuda.current_stream(dev))
+            with torch.cuda.stream(side):
+                copies.append((table, backend._upload(table, dev)))
+        else:
+            copies.append((table, backend._upload(table, dev)))
+    torch.cuda.synchronize()
+    for i, (table, on_device) in enumerate(copies):
+        assert on_device.numel() == (len(table) + 15) // 16 * 16
+        got = on_device.cpu().numpy()
+        assert np.array_equal(got[: len(table)], table), f"upload {i} of {len(table)} bytes"
+        assert not got[len(table):].any()
