@@ -169,19 +169,29 @@ __global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __re
   if (c >= slots) return;
   float* col = history + c;
   const float first = col[0];
+  float sc = scale[c];
   float amax = first;
-  if (!most_recent) {
-    // torch.max semantics: a NaN anywhere in the column wins
-    for (int i = 1; i < history_len; ++i) {
-      const float v = col[(size_t)i * slots];
-      amax = (v > amax || v != v) ? v : amax;
+  // The column is walked once, eight rows at a time: the loads of a group are issued together (one round trip to
+  // memory per group, not per row - the rows are written through the same pointer they are read from, so the
+  // compiler keeps loads and stores of a row-by-row loop in order), the maximum is taken, and the rows are written
+  // one place up.  A group's stores end one row below its loads and the next group's loads start above them.
+  constexpr int kGroup = 8;
+  for (int base = 1; base < history_len; base += kGroup) {
+    float v[kGroup];
+#pragma unroll
+    for (int j = 0; j < kGroup; ++j) v[j] = base + j < history_len ? col[(size_t)(base + j) * slots] : 0.f;
+#pragma unroll
+    for (int j = 0; j < kGroup; ++j) {
+      if (base + j < history_len) {
+        // torch.max semantics: a NaN anywhere in the column wins
+        if (!most_recent) amax = (v[j] > amax || v[j] != v[j]) ? v[j] : amax;
+        col[(size_t)(base + j - 1) * slots] = v[j];
+      }
     }
   }
-  float sc = scale[c];
   if (amax > 0.f && amax <= 3.4028234663852886e38f) sc = ((1.0f / amax) * fp8_max) * margin_factor;
   scale[c] = sc;
   if (!(keep_period > 0 && c % keep_period == keep_phase)) scale_inv[c] = 1.0f / sc;
-  for (int i = 0; i + 1 < history_len; ++i) col[(size_t)i * slots] = col[(size_t)(i + 1) * slots];
   if (history_len > 1) col[(size_t)(history_len - 1) * slots] = first;
   col[0] = 0.f;
 }
