@@ -86,6 +86,12 @@ __device__ __forceinline__ void global_store(void* p, T v) {
   *reinterpret_cast<__attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)) = v;
 }
 
+// The same with the streaming hint: data that is written once and read once, soon, by another launch.
+template <typename T>
+__device__ __forceinline__ void global_store_stream(void* p, T v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<__attribute__((address_space(1))) T*>(reinterpret_cast<uintptr_t>(p)));
+}
+
 // Raw buffer descriptors: offsets past `bytes` read as zero and are dropped on store, so the fast paths
 // of the HBM-bound kernels need no per-lane branches and can issue all their loads back to back.
 constexpr uint32_t kOobOffset = 0xffffffffu;

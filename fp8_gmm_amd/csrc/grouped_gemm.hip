@@ -46,14 +46,14 @@ __global__ __launch_bounds__(kFixupThreads) void grouped_gemm_fixup_kernel(
     const f32x4* first = reinterpret_cast<const f32x4*>(workspace + (size_t)fx.first_slot * kPartialBytes) +
                          (size_t)part * NT * kFixupThreads + threadIdx.x;
 #pragma unroll
-    for (int q = 0; q < NT; ++q) sum[q] = first[q * kFixupThreads];
+    for (int q = 0; q < NT; ++q) sum[q] = __builtin_nontemporal_load(first + q * kFixupThreads);
   }
   for (int w = 1; w < fx.n_pieces; ++w) {
     const f32x4* next = reinterpret_cast<const f32x4*>(workspace + (size_t)(fx.first_slot + w) * kPartialBytes) +
                         (size_t)part * NT * kFixupThreads + threadIdx.x;
     f32x4 piece[NT];
 #pragma unroll
-    for (int q = 0; q < NT; ++q) piece[q] = next[q * kFixupThreads];
+    for (int q = 0; q < NT; ++q) piece[q] = __builtin_nontemporal_load(next + q * kFixupThreads);
 #pragma unroll
     for (int q = 0; q < NT; ++q) sum[q] += piece[q];
   }

@@ -390,7 +390,10 @@ __device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int 
 #pragma unroll
           for (int it = 0; it < 4; ++it) {
             const uint32_t row_off = (uint32_t)((wave_m * WM + i * 32 + 8 * it) * (int)ldc);
-            buf_store16_stream(rb[it], rc, lane_off8 + row_off);
+            // plain stores, unlike the bf16 copy above: the fp8 activation is the next launch's operand, and what the
+            // memory-side cache keeps of it that launch does not fetch from HBM (config 4: this launch -8 us, the
+            // weight gradients that read it -4 us each)
+            __builtin_amdgcn_raw_buffer_store_b128(rb[it], rc, (int)(lane_off8 + row_off), 0, 0);
           }
         }
       });
@@ -571,6 +574,10 @@ __device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int 
 
 // Accumulators <-> workspace slot.  Register group r4 = (i * NT + j) * 4 + g of lane t sits at
 // (r4 * NTHREADS + t) * 16 bytes: every wavefront instruction moves 1 KB of contiguous memory.
+// Written here and read by the fix-up launch with the streaming hint: partial sums are used once, and as ordinary
+// traffic they took the place of operands in the memory-side cache that later launches of the step would have
+// found there (config 3: 19 MB of them after the forward GEMM made the weight gradient, two launches later, 40 us
+// slower; the same 19 MB written and read by any other kernel did the same).
 template <int TILE>
 __device__ __forceinline__ void partial_store(uint8_t* slot) {
   constexpr int MT = TILE / 64, NT = TILE / 64;
@@ -581,7 +588,7 @@ __device__ __forceinline__ void partial_store(uint8_t* slot) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const f32x4 v = {t[4 * g + 0], t[4 * g + 1], t[4 * g + 2], t[4 * g + 3]};
-      global_store(base + (ij * 4 + g) * (NTHREADS * 4), v);
+      global_store_stream(base + (ij * 4 + g) * (NTHREADS * 4), v);
     }
   });
 }
