@@ -353,8 +353,7 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   bool dangling_piece = false;
   auto write_record = [&](const Item& it, size_t index) {
     const fp8gmm_gemm_problem& p = probs[it.prob];
-    fp8gmm_gemm_item& o = items[index];
-    o = fp8gmm_gemm_item{};
+    fp8gmm_gemm_item o{};   // assembled in registers and stored once: stores into the list could alias anything
     const int64_t rows = p.m - it.m0 < BM ? p.m - it.m0 : BM;
     const int64_t cols = p.n - it.n0 < BN ? p.n - it.n0 : BN;
     if (p.k > 0) {
@@ -392,34 +391,68 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
     } else if (rows <= BM / 2) {
       o.flags = FP8GMM_ITEM_HALF_HEIGHT;      // a whole tile with at most 128 valid rows
     }
+    items[index] = o;
   };
+  // The strided part, which holds nearly all records, round by round: record r of workgroup w sits at
+  // items[r * grid + w], so this order writes the list front to back (one workgroup after the other writes a cache
+  // line every 64 * grid bytes, which takes several times as long on lists of a few thousand records in fresh
+  // memory).  The tiles and their order are those cursor_valid / cursor_item / cursor_advance give: a workgroup's
+  // position in the round advances by kRoundRotation, modulo the workgroups of the XCD.
+  struct Walk { int pos, prob; };
+  std::vector<Walk> walk(grid);
+  // problem and origin of every tile, filled in tile order without the divisions of tile_origin (its arithmetic,
+  // walked: groups of kRasterRows rows of tiles, inside a group the row runs fastest)
+  struct Where { int32_t prob, m0, n0; };
+  std::vector<Where> where(items != nullptr ? total_tiles : 0);
+  if (items != nullptr)
+    for (int p = 0; p < n; ++p) {
+      const int tiles_m = (probs[p].m + BM - 1) / BM, tiles_n = (probs[p].n + BN - 1) / BN;
+      Where* w = where.data() + probs[p].tile_begin;
+      for (int first = 0; first < tiles_m; first += kRasterRows) {
+        const int rows = tiles_m - first < kRasterRows ? tiles_m - first : kRasterRows;
+        for (int col = 0; col < tiles_n; ++col)
+          for (int row = 0; row < rows; ++row) *w++ = Where{p, (first + row) * BM, col * BN};
+      }
+    }
+  int strided_rounds = 0;
+  const int rotation = kRoundRotation % wgs;   // every XCD has wgs workgroups
+  for (int wg = 0; wg < grid; ++wg) {
+    const Sched& sx = sched[wg % kNumXcd];
+    walk[wg] = Walk{(wg / kNumXcd) % wgs, 0};
+    if (sx.dp_rounds > strided_rounds) strided_rounds = sx.dp_rounds;
+  }
+  for (int r = 0; r < strided_rounds; ++r)
+    for (int wg = 0; wg < grid; ++wg) {
+      const Sched& sx = sched[wg % kNumXcd];
+      if (count[wg] != r || r >= sx.dp_rounds) continue;   // this workgroup's strided part has ended
+      Walk& w = walk[wg];
+      const int tile = sx.range_begin + sx.wgs * r + w.pos;
+      if (tile >= sx.sk_begin) continue;
+      w.pos += rotation;
+      if (w.pos >= wgs) w.pos -= wgs;
+      count[wg] = r + 1;
+      const size_t index = (size_t)r * grid + wg;
+      if (index >= (size_t)max_items) continue;
+      const Where& at = where[tile];
+      w.prob = at.prob;
+      Item it;
+      it.tile = tile;
+      it.prob = at.prob;
+      it.m0 = at.m0;
+      it.n0 = at.n0;
+      it.k_begin = 0;
+      it.nk = (probs[at.prob].k + 127) / 128;
+      it.slot = -1;
+      write_record(it, index);
+    }
+  // what is left: the pieces of the shared remainder
   for (int wg = 0; wg < grid; ++wg) {
     const int x = wg % kNumXcd, j = wg / kNumXcd;
     const Sched& sx = sched[x];
     Cursor c;
     cursor_init(sx, j, c);
-    int r = 0, prob = 0;
-    // The strided part, which holds nearly all records, without the cursor's repeated index arithmetic: the same
-    // tiles in the same order as cursor_valid / cursor_item / cursor_advance give (dp_tile's position in the
-    // round advances by kRoundRotation, modulo the workgroups of the XCD).
-    for (int pos = j % sx.wgs; c.dp_i < sx.dp_rounds; ++c.dp_i, ++r) {
-      const int tile = sx.range_begin + sx.wgs * c.dp_i + pos;
-      if (tile >= sx.sk_begin) break;
-      pos += kRoundRotation % sx.wgs;
-      if (pos >= sx.wgs) pos -= sx.wgs;
-      const size_t index = (size_t)r * grid + wg;
-      if (index >= (size_t)max_items) continue;
-      while (prob + 1 < n && probs[prob + 1].tile_begin <= tile) ++prob;
-      Item it;
-      it.tile = tile;
-      it.prob = prob;
-      tile_origin(probs[prob].m, probs[prob].n, tile - probs[prob].tile_begin, &it.m0, &it.n0);
-      it.k_begin = 0;
-      it.nk = (probs[prob].k + 127) / 128;
-      it.slot = -1;
-      write_record(it, index);
-    }
-    // what is left: the pieces of the shared remainder
+    c.dp_i = count[wg];
+    int r = count[wg], prob = walk[wg].prob;
     for (; cursor_valid(sx, j, c); cursor_advance(sx, j, c), ++r) {
       const size_t index = (size_t)r * grid + wg;
       if (index >= (size_t)max_items) continue;
@@ -429,18 +462,21 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
     }
     count[wg] = r;
     if (r > rounds) rounds = r;
-    // records without K steps repeat the height of the next record that has some (see FP8GMM_ITEM_HALF_HEIGHT)
-    int next_height = 0;
-    for (int q = r - 1; q >= 0; --q) {
-      const size_t index = (size_t)q * grid + wg;
-      if (index >= (size_t)max_items) continue;
-      fp8gmm_gemm_item& o = items[index];
-      if (o.nk == 0) {
-        o.flags |= next_height << 1;
-      } else {
-        next_height = o.flags & FP8GMM_ITEM_HALF_HEIGHT;
+  }
+  // records without K steps repeat the height of the next record that has some (see FP8GMM_ITEM_HALF_HEIGHT)
+  {
+    std::vector<uint8_t> next_height(grid, 0);
+    for (int r = rounds - 1; r >= 0; --r)
+      for (int wg = 0; wg < grid; ++wg) {
+        const size_t index = (size_t)r * grid + wg;
+        if (r >= count[wg] || index >= (size_t)max_items) continue;
+        fp8gmm_gemm_item& o = items[index];
+        if (o.nk == 0) {
+          o.flags |= next_height[wg] << 1;
+        } else {
+          next_height[wg] = (uint8_t)(o.flags & FP8GMM_ITEM_HALF_HEIGHT);
+        }
       }
-    }
   }
   rounds += 1;  // every list ends with a record whose prob is -1
   const int n_fixups = (int)fix.size();
@@ -456,8 +492,9 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   fp8gmm_gemm_item end_record{};
   end_record.prob = -1;
   end_record.slot = -1;
-  for (int wg = 0; wg < grid; ++wg)
-    for (int r = count[wg]; r < rounds; ++r) items[(size_t)r * grid + wg] = end_record;
+  for (int r = 0; r < rounds; ++r)
+    for (int wg = 0; wg < grid; ++wg)
+      if (r >= count[wg]) items[(size_t)r * grid + wg] = end_record;
   return FP8GMM_OK;
 }
 
