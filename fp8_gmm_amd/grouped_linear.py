@@ -282,14 +282,9 @@ class _GroupedLinear(torch.autograd.Function):
         else:
             multi_quantize(row_slices(grad_out, cumsums), row_slices(grad_out_fp8, cumsums), g_scales, g_amaxes)
 
-        grad_input = None
-        if ctx.input_requires_grad:
-            grad_input = fp8_gmm(
-                grad_out_fp8, weight_for_dgrad, ctx.group_sizes, g_scale_invs,
-                meta.get_meta_pointers(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
-                backward=True, cutlass=ctx.cutlass, b_transposed=not ctx.reference_layout,
-            )
-
+        # the weight gradient first (the reference runs it second, grouped_linear.py:153-184): its operands are what
+        # the casts have just written, and behind the data gradient's pass over all the weights less of them is left in
+        # the memory-side cache
         grad_weight = None
         if ctx.weight_requires_grad:
             grad_weight = torch.empty(ctx.weight_shape, dtype=torch.bfloat16, device=dev)
@@ -303,6 +298,14 @@ class _GroupedLinear(torch.autograd.Function):
             else:  # dW[i] = dY_i^T . X_i on the row-major slices, contraction over the expert's rows
                 grouped_gemm(row_slices(grad_out_fp8, cumsums), row_slices(input_for_wgrad, cumsums),
                              TensorBatch.stack_of(grad_weight), g_scale_invs, x_scale_invs, transposed=True)
+
+        grad_input = None
+        if ctx.input_requires_grad:
+            grad_input = fp8_gmm(
+                grad_out_fp8, weight_for_dgrad, ctx.group_sizes, g_scale_invs,
+                meta.get_meta_pointers(Fp8TensorType.kForwardWeightGroup1, MetaTensorType.kScaleInv),
+                backward=True, cutlass=ctx.cutlass, b_transposed=not ctx.reference_layout,
+            )
         return grad_input, grad_weight, None, None, None, None, None, None
 
 

@@ -108,6 +108,9 @@ class _GroupedMlp(torch.autograd.Function):
             plain, with_t)
 
         if plain[0]:
+            # fc2's weights first, the input last: the launch walks its table in order, and what it wrote last is
+            # what the memory-side cache still holds when fc1's GEMM starts reading (config 4: that GEMM -14 us)
+            plain = tuple(lst[::-1] for lst in plain)
             multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
                            np.concatenate(plain[3]))
         if with_t[0]:

@@ -326,8 +326,8 @@ int fp8gmm_grouped_gemm_static(const fp8gmm_gemm_problem* probs_dev, int n, cons
  * the default data flow: activations, gradients and weights are cast to fp8 once, row-major, and every GEMM reads
  * them in place.
  *   forward : cast x (and, unless cast_weights == 0, the weights) ; y[rows_i] = x_fp8[rows_i] . w_fp8[i]^T
- *   backward: cast dy ; dx[rows_i] = dy_fp8[rows_i] . w_fp8[i]  (dgrad != 0) ; dw[i] = dy_fp8[rows_i]^T . x_fp8[rows_i]
- *             (wgrad != 0)
+ *   backward: cast dy ; dw[i] = dy_fp8[rows_i]^T . x_fp8[rows_i]  (wgrad != 0) ; dx[rows_i] = dy_fp8[rows_i] . w_fp8[i]
+ *             (dgrad != 0)
  * replaces, for that data flow, the per-expert host loops of fp8_gmm/grouped_linear.py:109-188 and the argument
  * packing of csrc/fp8_gmm.cu:115-135 and csrc/multi_pad_fusion.cu:455-502.  The scaling metadata is addressed
  * through the bases of the flat fp32 arrays in TransformerEngine's slot layout, which the reference indexes in
