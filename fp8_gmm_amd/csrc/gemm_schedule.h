@@ -25,7 +25,7 @@ namespace fp8gmm {
 // of such a tile in K order and runs the normal epilogue.  No workgroup ever waits for another one.
 constexpr int kSkMinPairs = 4;        // never cut pieces shorter than this many K = 128 steps
 constexpr int kSkMaxPieces = 8;       // average pieces per tile the region may be cut into
-constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost 4 %
+constexpr int kSkMaxRounds = 24;      // with more full rounds than this the tail cannot cost enough to share it
 // The second launch, which completes the shared tiles, costs about kSkFixupLaunch K = 128 steps of time (5 us:
 // the gap between two launches) plus kSkFixupPerTile / 100 steps per shared tile of the XCD (four workgroups per
 // tile on 256 compute units, a megabyte of partial sums each), three times that when it has the GELU epilogue to
@@ -123,8 +123,12 @@ FP8GMM_HD void sched_init(Sched& s, const fp8gmm_gemm_problem* probs, int nprob,
   s.sk_cost = 0;
   const int full = n_x / W, rem = n_x % W;
   if (!sk_enable || rem == 0 || full > kSkMaxRounds) return;
-  // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves 4 % ...
-  if ((int64_t)(W - rem) * 25 < (int64_t)W * (full + 1)) return;
+  // striding needs full + 1 rounds, sharing the remainder full + rem / W: take it when that saves a twelfth of the
+  // launch by this count.  Measured, sharing returns about half of what the count promises (workgroups do not
+  // finish their rounds in step, so part of a last round is hidden anyway), and it costs the second launch and a
+  // round trip of the partial sums through memory: config 2's 4.25 rounds (15 % by the count) gain 6.5 %, launches
+  // of 14 rounds with a short tail (4 - 6.5 % by the count; the reference's example layer) lost 1 % of their step.
+  if ((int64_t)(W - rem) * 12 < (int64_t)W * (full + 1)) return;
   const int n_sk = rem;
   const int rounds = full;
   const int sk_begin = s.range_begin + rounds * W;
