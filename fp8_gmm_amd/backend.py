@@ -252,7 +252,10 @@ def _to_device(device, room, fill):
     room = (room + 15) & ~15
     with _on_device(device):
         stream = torch.cuda.current_stream(device)
-        st = _staging_of(device) if options.upload == "kernel" else None
+        # (under stream capture the tables go the other way: a captured copy kernel would read, at every replay,
+        # whatever the staging memory holds by then)
+        staged = options.upload == "kernel" and not torch.cuda.is_current_stream_capturing()
+        st = _staging_of(device) if staged else None
         offset = st.reserve(room, stream) if st is not None else None
         if offset is None:   # larger than the staging area, or by choice: a pinned buffer of its own and torch's copy
             pinned = torch.empty(room, dtype=torch.uint8, pin_memory=True)
