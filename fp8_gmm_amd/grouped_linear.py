@@ -130,7 +130,8 @@ class _GroupedLinear(torch.autograd.Function):
         fp8_dtype = to_torch_dtype(fwd_dtype)
         dev = input.device
 
-        if fp8_meta.get("planned_passes", True) and not reference_layout and not cutlass and input.is_cuda and input.is_contiguous() and weight.is_contiguous() \
+        if fp8_meta.get("planned_passes", True) and not reference_layout and not cutlass and input.is_cuda \
+                and input.is_contiguous() and weight.is_contiguous() \
                 and input.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16:
             # The default data flow as one planned pass: every table of the cast launch and of the GEMM comes out of
             # one library call (with 64 experts the array arithmetic below costs more host time than the kernels run).

@@ -304,8 +304,8 @@ class GroupedMlp(Fp8GroupedModuleBase):
     """E expert MLPs ``in_features -> out_features -> in_features`` with tanh-GELU, no biases.
 
     ``forward(input[tokens, in_features], group_sizes[E], has_tp=False, tp_group=None, is_first_microbatch=None)``;
-    ``reference_layout`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True / False: cast into / reuse
-    the module's fp8 weight buffers).
+    ``reference_layout`` and ``is_first_microbatch`` as for GroupedLinear (None: cast the weights every pass; True /
+    False: cast into / reuse the module's fp8 weight buffers).
     ``fused_dgelu=True`` (default layout only): the fc2 data-gradient GEMM applies the GELU's derivative and the cast to
     fp8 in its epilogue, from the fp32 accumulators (one rounding, where the separate pass rounds to bf16 first), and
     the pass over ``[tokens, out_features]`` that the reference runs behind that GEMM (grouped_mlp.py:243-287) is gone.
