@@ -69,6 +69,18 @@ __device__ __forceinline__ void buf_store16_stream(u32x4 v, __amdgpu_buffer_rsrc
   __builtin_amdgcn_raw_buffer_store_b128(v, r, (int)off, 0, 2);
 }
 
+// A buffer descriptor of a tile's result, made of values that are the same in every lane.  The compiler does not
+// always know that: when it has moved the address arithmetic of a tile to the vector unit (it does, where scalar
+// registers are short), a descriptor built from the outcome sits in vector registers, and every store through it
+// becomes a loop that reads the four words back lane by lane - a dozen instructions and a branch per store, 32
+// stores per wavefront and tile.  Reading the words back once, here, costs three instructions per tile.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_uniform_rsrc(const void* base, uint32_t bytes) {
+  const uint64_t a = reinterpret_cast<uintptr_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return make_rsrc(reinterpret_cast<const void*>(((uint64_t)hi << 32) | lo), __builtin_amdgcn_readfirstlane(bytes));
+}
+
 constexpr int kPartialBytes = FP8GMM_GEMM_SLOT_BYTES;  // one workspace slot: the fp32 accumulators of one tile
 static_assert(kPartialBytes == BM * BN * 4, "a slot holds one tile of fp32 accumulators");
 
@@ -246,7 +258,7 @@ __device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int 
       // Two 4 KB staging buffers alternate, so that the read-back of one unit is under way while the next unit is
       // converted: the round trip through LDS, a third of the epilogue when exposed, hides behind the arithmetic.
       uint16_t* const C = static_cast<uint16_t*>(pr.c) + (int64_t)m0 * ldc + n0;
-      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
+      const __amdgpu_buffer_rsrc_t rc = make_uniform_rsrc(C, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       // (the small tile's staging area holds one unit per wavefront: a wavefront's LDS operations complete in
       // order, so the read-back of a unit is done before the next unit's writes land in the same place)
       uint8_t* mine = stage + wave * kStageBytes;
@@ -302,8 +314,8 @@ __device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int 
       // zero (oob_zero), and gelu(0) = 0 leaves the amax alone.
       uint8_t* const C = static_cast<uint8_t*>(pr.c) + (int64_t)m0 * ldc + n0;
       uint16_t* const AUX = static_cast<uint16_t*>(pr.aux) + (int64_t)m0 * ldc + n0;
-      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
-      const __amdgpu_buffer_rsrc_t ra = make_rsrc(AUX, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
+      const __amdgpu_buffer_rsrc_t rc = make_uniform_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
+      const __amdgpu_buffer_rsrc_t ra = make_uniform_rsrc(AUX, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       uint8_t* mine = stage + wave * 8192;
       const int wr = l32 * 256 + khalf * 8;   // bf16 block: + ((4 j + g) ^ (l32 & 15)) * 16
       const int wr8 = l32 * 128 + khalf * 4;  // fp8 block:  + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
@@ -409,8 +421,8 @@ __device__ __forceinline__ int tile_epilogue(const fp8gmm_gemm_problem& pr, int 
       // alone and the stores fall outside the result's descriptor.
       uint8_t* const C = static_cast<uint8_t*>(pr.c) + (int64_t)m0 * ldc + n0;
       const uint16_t* const PRE = static_cast<const uint16_t*>(pr.aux) + (int64_t)m0 * ldc + n0;
-      const __amdgpu_buffer_rsrc_t rc = make_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
-      const __amdgpu_buffer_rsrc_t rp = make_rsrc(PRE, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
+      const __amdgpu_buffer_rsrc_t rc = make_uniform_rsrc(C, (uint32_t)((rv - 1) * (int)ldc + cv));
+      const __amdgpu_buffer_rsrc_t rp = make_uniform_rsrc(PRE, (uint32_t)(((rv - 1) * (int)ldc + cv) * 2));
       uint8_t* mine = stage + wave * 8192;
       const int wr8 = l32 * 128 + khalf * 4;  // + ((2 j + g / 2) ^ ((l32 >> 1) & 7)) * 16 + (g & 1) * 8
       const int rrow8 = lane >> 3, rchunk8 = lane & 7;
