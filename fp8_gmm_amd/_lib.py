@@ -127,6 +127,19 @@ class LinearPass(ctypes.Structure):
                 ("bwd_amax", ctypes.c_void_p)]
 
 
+class MlpPass(ctypes.Structure):
+    """struct fp8gmm_mlp_pass: one pass of a grouped MLP, as the pass planner takes it"""
+
+    _fields_ = [("experts", ctypes.c_int32), ("hidden", ctypes.c_int32), ("ffn", ctypes.c_int32),
+                ("fwd_fmt", ctypes.c_int32), ("bwd_fmt", ctypes.c_int32), ("cast_weights", ctypes.c_int32),
+                ("dgrad", ctypes.c_int32), ("wgrad", ctypes.c_int32), ("grid", ctypes.c_int32),
+                ("stream_k", ctypes.c_int32), ("tile_policy", ctypes.c_int32), ("reserved", ctypes.c_int32),
+                ("tokens", ctypes.c_int64), ("group_sizes", ctypes.c_void_p)] + \
+        [(name, ctypes.c_void_p) for name in (
+            "x", "x_fp8", "w1", "w1_fp8", "w2", "w2_fp8", "pre", "act_fp8", "y", "dy", "dy_fp8", "dact", "dpre_fp8",
+            "dx", "dw1", "dw2", "fwd_scale", "fwd_scale_inv", "fwd_amax", "bwd_scale", "bwd_scale_inv", "bwd_amax")]
+
+
 class PassLaunch(ctypes.Structure):
     """struct fp8gmm_pass_launch"""
 
@@ -142,7 +155,7 @@ class PassPlan(ctypes.Structure):
     """struct fp8gmm_pass_plan"""
 
     _fields_ = [("n_launches", ctypes.c_int32), ("reserved", ctypes.c_int32), ("blob_bytes", ctypes.c_int64),
-                ("launch", PassLaunch * 4)]
+                ("launch", PassLaunch * 8)]
 
 
 PASS_CAST = 1
@@ -160,6 +173,9 @@ EXPORTS = (
     "fp8gmm_grouped_gemm_static",
     "fp8gmm_plan_linear_forward",
     "fp8gmm_plan_linear_backward",
+    "fp8gmm_plan_mlp_forward",
+    "fp8gmm_plan_mlp_backward",
+    "fp8gmm_sizeof_mlp_pass",
     "fp8gmm_run_planned",
     "fp8gmm_sizeof_linear_pass",
     "fp8gmm_sizeof_pass_plan",
@@ -254,6 +270,11 @@ def load():
     for fn in (L.fp8gmm_plan_linear_forward, L.fp8gmm_plan_linear_backward):
         fn.restype = ci
         fn.argtypes = [ctypes.POINTER(LinearPass), vp, ctypes.c_size_t, ctypes.POINTER(PassPlan)]
+    for fn in (L.fp8gmm_plan_mlp_forward, L.fp8gmm_plan_mlp_backward):
+        fn.restype = ci
+        fn.argtypes = [ctypes.POINTER(MlpPass), vp, ctypes.c_size_t, ctypes.POINTER(PassPlan)]
+    L.fp8gmm_sizeof_mlp_pass.restype = ctypes.c_size_t
+    L.fp8gmm_sizeof_mlp_pass.argtypes = []
     L.fp8gmm_run_planned.restype = ci
     L.fp8gmm_run_planned.argtypes = [vp, ctypes.POINTER(PassLaunch), vp, ctypes.c_size_t, vp]
     L.fp8gmm_sizeof_linear_pass.restype = ctypes.c_size_t
@@ -283,6 +304,7 @@ def load():
     if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize \
             or L.fp8gmm_sizeof_gemm_item() != GEMM_ITEM.itemsize or ctypes.sizeof(GemmPlan) != 32 \
             or L.fp8gmm_sizeof_linear_pass() != ctypes.sizeof(LinearPass) \
+            or L.fp8gmm_sizeof_mlp_pass() != ctypes.sizeof(MlpPass) \
             or L.fp8gmm_sizeof_pass_plan() != ctypes.sizeof(PassPlan):
         raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
     _lib = L

@@ -881,19 +881,13 @@ def warm_up(device=None):
 # ------------------------------------------------------------------------------------------------
 # a whole pass of a grouped linear layer, planned by one library call
 # ------------------------------------------------------------------------------------------------
-_PASS_KERNEL_NAMES = {_lib.PASS_CAST: "multi_quantize", _lib.PASS_GEMM: "grouped_gemm"}
-
-
-def linear_pass(device, backward=False, **fields):
-    """Plans one pass of a grouped linear layer with ONE library call (fp8gmm_plan_linear_forward / _backward),
-    uploads its tables with one copy and enqueues its launches.  ``fields`` are the members of
-    ``fp8gmm_linear_pass`` (include/fp8gmm.h): tensors are given as tensors (their addresses are taken here),
-    ``group_sizes`` as an int64 numpy array.  The tables are the ones the per-launch entry points of this module
-    build for the same tensors; what this call saves is the host time of building them in Python."""
+def _run_pass(device, desc, fields, plan_fn, bound_fn):
+    """Fill the pass description `desc` from `fields`, plan it with `plan_fn` straight into staging memory (of
+    `bound_fn(desc, grid)` bytes at first; the planner says how much it needs when that is too little), upload the
+    tables and enqueue the launches."""
     L = _lib.load()
     flush_uploads()   # launches queued before this pass come first
     keep = []
-    desc = _lib.LinearPass()
     for name, value in fields.items():
         if isinstance(value, torch.Tensor):
             keep.append(value)
@@ -907,22 +901,15 @@ def linear_pass(device, backward=False, **fields):
     desc.grid = grid
     desc.stream_k = int(bool(options.stream_k))
     desc.tile_policy = {"auto": 0, "256": 256, "128": 128}[options.tile]
-    # room for the tables: descriptors, problem tables and, per GEMM, a work list of at most one record per
-    # 128 x 128 tile plus a few rounds of end records
-    widest = max(desc.in_features, desc.out_features)
-    tiles = (desc.tokens // 128 + desc.experts) * ((widest + 127) // 128) + \
-        desc.experts * ((desc.in_features + 127) // 128) * ((desc.out_features + 127) // 128)
-    bound = 4096 + desc.experts * (2 * 128 + 3 * 96) + 3 * (tiles + 8 * grid) * 64 + 3 * 32 * 2 * grid
+    bound = bound_fn(desc, grid)
     plan = _lib.PassPlan()
-    fn = L.fp8gmm_plan_linear_backward if backward else L.fp8gmm_plan_linear_forward
-    # the planner writes the tables straight into staging memory
     while True:
         def fill(address, _):
-            fill.rc = fn(ctypes.byref(desc), address, bound, ctypes.byref(plan))
+            fill.rc = plan_fn(ctypes.byref(desc), address, bound, ctypes.byref(plan))
             return int(plan.blob_bytes) if fill.rc == 0 else 0
 
         blob = _to_device(device, bound, fill)
-        if fill.rc == -8 and plan.blob_bytes > bound:   # FP8GMM_ERR_BUFFER_TOO_SMALL: the plan says how much room it needs
+        if fill.rc == -8 and plan.blob_bytes > bound:   # FP8GMM_ERR_BUFFER_TOO_SMALL
             bound = int(plan.blob_bytes)
             continue
         _lib.check(fill.rc)
@@ -935,13 +922,48 @@ def linear_pass(device, backward=False, **fields):
             rec = plan.launch[i]
             if rec.kind == 0:
                 continue
-            ws = _gemm_workspace(device, rec.plan.n_slots) if rec.kind == _lib.PASS_GEMM else None
+            gemm = rec.kind == _lib.PASS_GEMM
+            ws = _gemm_workspace(device, rec.plan.n_slots) if gemm else None
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
-            with _timed(_PASS_KERNEL_NAMES[rec.kind], lambda: rec.work, lambda: rec.bytes,
-                        (lambda: gemm_form(rec.a_fmt, rec.epilogue)) if rec.kind == _lib.PASS_GEMM else None):
+            with _timed("grouped_gemm" if gemm else _OP_NAMES[rec.op], lambda: rec.work, lambda: rec.bytes,
+                        (lambda: gemm_form(rec.a_fmt, rec.epilogue)) if gemm else None):
                 rc = L.fp8gmm_run_planned(base, ctypes.byref(rec), ws_ptr, ws_bytes, stream)
             _lib.check(rc)
     return plan
+
+
+def _pass_room(experts, tokens, shapes, casts, grid):
+    """Bytes that surely hold the tables of a pass with GEMMs over ``shapes`` (pairs of feature counts; every GEMM
+    is token-sliced in one dimension or per expert in both) and ``casts`` cast descriptors: per GEMM a problem table
+    and a work list of at most one record per 128 x 128 tile plus a few rounds of end records and the shared-tile
+    records."""
+    room = 4096 + casts * 128
+    for a, b in shapes:
+        widest = max(a, b)
+        tiles = (tokens // 128 + experts) * ((widest + 127) // 128) + experts * ((a + 127) // 128) * ((b + 127) // 128)
+        room += experts * 96 + 256 + (tiles + 8 * grid) * 64 + 32 * 2 * grid
+    return room
+
+
+def linear_pass(device, backward=False, **fields):
+    """Plans one pass of a grouped linear layer with ONE library call (fp8gmm_plan_linear_forward / _backward),
+    uploads its tables with one copy and enqueues its launches.  ``fields`` are the members of
+    ``fp8gmm_linear_pass`` (include/fp8gmm.h): tensors are given as tensors (their addresses are taken here),
+    ``group_sizes`` as an int64 numpy array.  The tables are the ones the per-launch entry points of this module
+    build for the same tensors; what this call saves is the host time of building them in Python."""
+    L = _lib.load()
+    return _run_pass(
+        device, _lib.LinearPass(), fields, L.fp8gmm_plan_linear_backward if backward else L.fp8gmm_plan_linear_forward,
+        lambda d, grid: _pass_room(d.experts, d.tokens, [(d.in_features, d.out_features)] * 3, 2 * d.experts, grid))
+
+
+def mlp_pass(device, backward=False, **fields):
+    """The same for one pass of a grouped MLP in its default data flow (fp8gmm_plan_mlp_forward / _backward, members
+    of ``fp8gmm_mlp_pass``): three launches forward, up to six backward, from one library call and one upload."""
+    L = _lib.load()
+    return _run_pass(
+        device, _lib.MlpPass(), fields, L.fp8gmm_plan_mlp_backward if backward else L.fp8gmm_plan_mlp_forward,
+        lambda d, grid: _pass_room(d.experts, d.tokens, [(d.hidden, d.ffn)] * 4, 3 * d.experts, grid))
 
 
 def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, most_recent=False, keep_scale_inv=None):

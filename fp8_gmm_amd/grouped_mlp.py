@@ -17,19 +17,23 @@ copy its gradient GEMM takes (weights ``[E, K, N]``; activations, the GELU outpu
 gradients zero-padded per expert), as grouped_mlp.py:60-150,196-262 does; by default the
 gradient GEMMs read the row-major fp8 tensors in place and no such copy exists.
 
-Experts with zero tokens are allowed; each wgrad is one grouped launch.
+Experts with zero tokens are allowed; each wgrad is one grouped launch.  In the default layout a whole pass is
+planned by one library call (``backend.mlp_pass``); the launch-by-launch code below it builds the same tables and
+serves the other layouts and options.
 """
 import math
 
 import numpy as np
 import torch
 
+from . import _lib
 from .backend import (
     TensorBatch,
     batched_uploads,
     flush_uploads,
     fp8_gmm,
     grouped_gemm,
+    mlp_pass,
     multi_cast_transpose,
     multi_cast_dgelu,
     multi_cast_transpose_dgelu,
@@ -79,6 +83,50 @@ class _GroupedMlp(torch.autograd.Function):
         fp8_dtype = to_torch_dtype(get_fp8_te_dtype(fp8_meta["recipe"], fprop_tensor=True))
         dev = input.device
         tokens, ffn = input.size(0), fc1_weight.size(1)
+
+        if fp8_meta.get("planned_passes", True) and not reference_layout and input.is_cuda \
+                and input.is_contiguous() and fc1_weight.is_contiguous() and fc2_weight.is_contiguous() \
+                and input.dtype == fc1_weight.dtype == fc2_weight.dtype == torch.bfloat16:
+            # The default data flow as one planned pass: the tables of the cast launch and of both GEMMs come out of
+            # one library call and reach the device in one upload (the same tables, to the byte, that the code below
+            # builds array by array - which with 64 experts costs more host time than the kernels run)
+            sizes = np.diff(np.asarray(cumsums, dtype=np.int64))
+            input_fp8 = torch.empty(input.shape, dtype=fp8_dtype, device=dev)
+            weights_fp8 = []
+            cast_weights = True
+            for weight, cache in zip((fc1_weight, fc2_weight), weight_caches):
+                if cache is None:
+                    weights_fp8.append(torch.empty(weight.shape, dtype=fp8_dtype, device=dev))
+                    continue
+                weights_fp8.append(cache.buffers(weight, fp8_dtype, False)[0])
+                cast_weights = bool(update_fp8_weights)
+                if cast_weights:
+                    cache.valid, cache.valid_t = True, False
+                else:
+                    cache.require(False)
+            fc1_weight_fp8, fc2_weight_fp8 = weights_fp8
+            pre_gelu_out = torch.empty(tokens, ffn, dtype=torch.bfloat16, device=dev)
+            gelu_out_fp8 = torch.empty(tokens, ffn, dtype=fp8_dtype, device=dev)
+            out = torch.empty(tokens, input.size(1), dtype=torch.bfloat16, device=dev)
+            fwd = fp8_meta["scaling_fwd"]
+            mlp_pass(dev, False, experts=num_groups, hidden=input.size(1), ffn=ffn,
+                     fwd_fmt=_lib.E4M3 if fp8_dtype == torch.float8_e4m3fn else _lib.E5M2, cast_weights=cast_weights,
+                     tokens=tokens, group_sizes=sizes, x=input, x_fp8=input_fp8, w1=fc1_weight, w1_fp8=fc1_weight_fp8,
+                     w2=fc2_weight, w2_fp8=fc2_weight_fp8, pre=pre_gelu_out, act_fp8=gelu_out_fp8, y=out,
+                     fwd_scale=fwd.scale, fwd_scale_inv=fwd.scale_inv, fwd_amax=fwd.amax_history)
+            capture = fp8_meta.get("capture")
+            if capture is not None:  # see GroupedMlp.capture_intermediates
+                capture.update(pre_gelu_out=pre_gelu_out, gelu_out_fp8=gelu_out_fp8)
+            if is_grad_enabled:
+                ctx.save_for_backward(input_fp8 if wgrad_needed else None,
+                                      fc1_weight_fp8 if (dgrad_needed and input_requires_grad) else None,
+                                      fc2_weight_fp8 if dgrad_needed else None, pre_gelu_out,
+                                      gelu_out_fp8 if wgrad_needed else None)
+                ctx.planned = True
+                ctx.sizes = sizes
+                _GroupedMlp._remember(ctx, False, group_sizes, meta, num_groups, padded, cumsums, padded_cumsums, fp8_meta,
+                                      fc1_weight, fc2_weight, input_requires_grad, weight_requires_grad, has_tp, tp_group)
+            return out
 
         plain = ([], [], [], [])
         with_t = ([], [], [], [], [])
@@ -151,24 +199,33 @@ class _GroupedMlp(torch.autograd.Function):
                 w1_dgrad = fc1_weight_fp8 if (dgrad_needed and input_requires_grad) else None
                 w2_dgrad = fc2_weight_fp8 if dgrad_needed else None
             ctx.save_for_backward(x_wgrad, w1_dgrad, w2_dgrad, pre_gelu_out, gelu_out_fp8)
-            ctx.reference_layout = reference_layout
-            ctx.group_sizes = group_sizes
-            meta.set_forward_scale_inv_cloned()
-            ctx.meta = meta
-            ctx.num_groups = num_groups
-            ctx.padded = padded
-            ctx.cumsums = cumsums
-            ctx.padded_cumsums = padded_cumsums
-            ctx.fp8_meta = fp8_meta
-            ctx.fc1_weight_shape = fc1_weight.shape
-            ctx.fc2_weight_shape = fc2_weight.shape
-            ctx.input_requires_grad = input_requires_grad
-            ctx.weight_requires_grad = weight_requires_grad
-            ctx.has_tp = has_tp
-            if has_tp:
-                assert tp_group is not None
-            ctx.tp_group = tp_group
+            ctx.planned = False
+            _GroupedMlp._remember(ctx, reference_layout, group_sizes, meta, num_groups, padded, cumsums, padded_cumsums,
+                                  fp8_meta, fc1_weight, fc2_weight, input_requires_grad, weight_requires_grad, has_tp,
+                                  tp_group)
         return out
+
+    @staticmethod
+    def _remember(ctx, reference_layout, group_sizes, meta, num_groups, padded, cumsums, padded_cumsums, fp8_meta,
+                  fc1_weight, fc2_weight, input_requires_grad, weight_requires_grad, has_tp, tp_group):
+        """What the backward pass needs besides the saved tensors."""
+        ctx.reference_layout = reference_layout
+        ctx.group_sizes = group_sizes
+        meta.set_forward_scale_inv_cloned()
+        ctx.meta = meta
+        ctx.num_groups = num_groups
+        ctx.padded = padded
+        ctx.cumsums = cumsums
+        ctx.padded_cumsums = padded_cumsums
+        ctx.fp8_meta = fp8_meta
+        ctx.fc1_weight_shape = fc1_weight.shape
+        ctx.fc2_weight_shape = fc2_weight.shape
+        ctx.input_requires_grad = input_requires_grad
+        ctx.weight_requires_grad = weight_requires_grad
+        ctx.has_tp = has_tp
+        if has_tp:
+            assert tp_group is not None
+        ctx.tp_group = tp_group
 
     @staticmethod
     def _backward(ctx, grad_out):
@@ -182,6 +239,35 @@ class _GroupedMlp(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         dev = grad_out.device
         wgrad = ctx.weight_requires_grad
+
+        if ctx.planned and not ctx.has_tp and grad_out.dtype == torch.bfloat16 \
+                and not ctx.fp8_meta.get("fused_dgelu", False) \
+                and not wgrad_wants_transposed_gradient(cumsums[-1], ctx.num_groups):
+            # the whole pass from one library call (with a tensor-parallel group the collective between the launches
+            # wants the first data gradient flushed on its own: that case takes the per-launch path below)
+            bwd = ctx.fp8_meta["scaling_bwd"]
+            fwd_dtype = to_torch_dtype(get_fp8_te_dtype(ctx.fp8_meta["recipe"], fprop_tensor=True))
+            tokens, ffn = pre_gelu_out.shape
+            grad_out_fp8 = torch.empty(grad_out.shape, dtype=grad_dtype, device=dev)
+            grad_gelu_out = torch.empty(tokens, ffn, dtype=torch.bfloat16, device=dev)
+            grad_pre_fp8 = torch.empty(tokens, ffn, dtype=grad_dtype, device=dev)
+            grad_input = torch.empty(grad_out.shape, dtype=torch.bfloat16, device=dev) \
+                if ctx.input_requires_grad else None
+            grad_fc1_weight = torch.empty(ctx.fc1_weight_shape, dtype=torch.bfloat16, device=dev) if wgrad else None
+            grad_fc2_weight = torch.empty(ctx.fc2_weight_shape, dtype=torch.bfloat16, device=dev) if wgrad else None
+            mlp_pass(dev, True, experts=ctx.num_groups, hidden=grad_out.size(1), ffn=ffn,
+                     fwd_fmt=_lib.E4M3 if fwd_dtype == torch.float8_e4m3fn else _lib.E5M2,
+                     bwd_fmt=_lib.E4M3 if grad_dtype == torch.float8_e4m3fn else _lib.E5M2,
+                     dgrad=int(ctx.input_requires_grad), wgrad=int(wgrad), tokens=tokens, group_sizes=ctx.sizes,
+                     x_fp8=input_for_wgrad, w1_fp8=fc1_weight_dgrad, w2_fp8=fc2_weight_dgrad, pre=pre_gelu_out,
+                     act_fp8=gelu_out_fp8, dy=grad_out, dy_fp8=grad_out_fp8, dact=grad_gelu_out, dpre_fp8=grad_pre_fp8,
+                     dx=grad_input, dw1=grad_fc1_weight, dw2=grad_fc2_weight,
+                     fwd_scale_inv=meta._forward_scale_inv_cloned, bwd_scale=bwd.scale, bwd_scale_inv=bwd.scale_inv,
+                     bwd_amax=bwd.amax_history)
+            capture = ctx.fp8_meta.get("capture")
+            if capture is not None:
+                capture.update(grad_gelu_out=grad_gelu_out, grad_pre_fp8=grad_pre_fp8)
+            return grad_input, grad_fc1_weight, grad_fc2_weight, None, None, None, None, None, None, None
 
         g1_scales = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kScale)
         g1_amaxes = meta.get_meta_pointers(_T.kGradOutputGroup1, _M.kAmax)
@@ -311,11 +397,14 @@ class GroupedMlp(Fp8GroupedModuleBase):
     the pass over ``[tokens, out_features]`` that the reference runs behind that GEMM (grouped_mlp.py:243-287) is gone.
     Off by default: with one wavefront per SIMD the epilogue's arithmetic costs the GEMM more than the pass it
     replaces.
+    ``planned_passes=False`` builds the tables of every launch in Python through the per-launch entry points of
+    ``backend`` instead of one library call per pass (same tables, same launches, more host time).
     """
 
     def __init__(self, in_features, out_features, num_groups, dtype, device="cuda",
-                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False, fused_dgelu=False):
+                 pad_multiple=MODULE_PAD_MULTIPLE, reference_layout=False, fused_dgelu=False, planned_passes=True):
         super().__init__()
+        self.fp8_meta["planned_passes"] = planned_passes
         self.fp8_meta["pad_multiple"] = pad_multiple
         self.fp8_meta["reference_layout"] = reference_layout
         self.fp8_meta["fused_dgelu"] = fused_dgelu

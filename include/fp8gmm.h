@@ -386,7 +386,7 @@ typedef struct fp8gmm_pass_plan {
   int32_t n_launches;
   int32_t reserved;
   int64_t blob_bytes;            /* bytes of the blob in use: what has to be uploaded */
-  fp8gmm_pass_launch launch[4];
+  fp8gmm_pass_launch launch[8];
 } fp8gmm_pass_plan;
 size_t fp8gmm_sizeof_linear_pass(void);
 size_t fp8gmm_sizeof_pass_plan(void);
@@ -402,6 +402,56 @@ int fp8gmm_plan_linear_backward(const fp8gmm_linear_pass* pass, void* blob, size
  * descriptors, so every pass uploads afresh); workspace as for fp8gmm_grouped_gemm. */
 int fp8gmm_run_planned(const void* blob_dev, const fp8gmm_pass_launch* launch, void* workspace, size_t workspace_bytes,
                        void* stream);
+
+/*
+ * The same for a grouped MLP (E experts, hidden -> ffn -> hidden with the tanh GELU between, token-sorted rows) in
+ * its default data flow:
+ *   forward : cast w2, w1 (unless cast_weights == 0) and x ;
+ *             act_fp8[rows_i], pre[rows_i] = gelu epilogue of x_fp8[rows_i] . w1_fp8[i]^T (FP8GMM_EPI_GELU) ;
+ *             y[rows_i] = act_fp8[rows_i] . w2_fp8[i]^T
+ *   backward: cast dy ; dw2[i] = dy_fp8[rows_i]^T . act_fp8[rows_i] (wgrad != 0) ; dact[rows_i] = dy_fp8[rows_i] . w2_fp8[i] ;
+ *             dpre_fp8 = fp8(dact * dgelu(pre)) (FP8GMM_OP_CAST_DGELU) ; dx[rows_i] = dpre_fp8[rows_i] . w1_fp8[i] (dgrad != 0) ;
+ *             dw1[i] = dpre_fp8[rows_i]^T . x_fp8[rows_i] (wgrad != 0)
+ * replaces, for that data flow, the host side of fp8_gmm/grouped_mlp.py:18-325.  Scaling slots as the reference
+ * indexes them (fp8_gmm/utils.py:98-103) with 2 E GEMMs, fc1 of expert i being GEMM i and fc2 GEMM E + i: forward
+ * slots 3 g (input of GEMM g), 3 g + 1 (its weight); backward slots 2 i for dy and 2 E + 2 i for the gradient of pre
+ * (the reference's kGradOutputGroup1 / kGradOutputGroup2, fp8_gmm/grouped_mlp.py:183-184,278-279).  fwd_scale_inv is
+ * the live array in the forward pass and the copy taken after it in the backward pass.
+ */
+typedef struct fp8gmm_mlp_pass {
+  int32_t experts, hidden, ffn;
+  int32_t fwd_fmt, bwd_fmt;
+  int32_t cast_weights;              /* forward: 0 when w1_fp8 / w2_fp8 already hold the cast weights */
+  int32_t dgrad, wgrad;              /* backward: gradient of the input / of the weights wanted */
+  int32_t grid, stream_k, tile_policy, reserved;   /* as in fp8gmm_linear_pass */
+  int64_t tokens;
+  const int64_t* group_sizes;        /* HOST array [experts] */
+  const void* x;                     /* bf16 [tokens, hidden] */
+  void* x_fp8;                       /* fp8, same shape */
+  const void* w1;                    /* bf16 [experts, ffn, hidden] */
+  void* w1_fp8;
+  const void* w2;                    /* bf16 [experts, hidden, ffn] */
+  void* w2_fp8;
+  void* pre;                         /* bf16 [tokens, ffn]: pre-GELU activation (written forward, read backward) */
+  void* act_fp8;                     /* fp8  [tokens, ffn]: gelu(pre) */
+  void* y;                           /* bf16 [tokens, hidden] */
+  const void* dy;                    /* bf16 [tokens, hidden] */
+  void* dy_fp8;
+  void* dact;                        /* bf16 [tokens, ffn]: gradient of gelu(pre) */
+  void* dpre_fp8;                    /* fp8  [tokens, ffn]: gradient of pre */
+  void* dx;                          /* bf16 [tokens, hidden] */
+  void* dw1;                         /* bf16 [experts, ffn, hidden] */
+  void* dw2;                         /* bf16 [experts, hidden, ffn] */
+  const float* fwd_scale;
+  const float* fwd_scale_inv;
+  float* fwd_amax;
+  const float* bwd_scale;
+  const float* bwd_scale_inv;
+  float* bwd_amax;
+} fp8gmm_mlp_pass;
+size_t fp8gmm_sizeof_mlp_pass(void);
+int fp8gmm_plan_mlp_forward(const fp8gmm_mlp_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
+int fp8gmm_plan_mlp_backward(const fp8gmm_mlp_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
 
 /*
  * Delayed-scaling update of one direction, in place, for `slots` scaling factors:

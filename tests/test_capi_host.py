@@ -237,3 +237,160 @@ def test_launch_plan_reports_sizes_before_it_writes():
     assert len(blob) == off_fix
     assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 12, 0, None, 0, None, 0, ctypes.byref(plan)) == -6
     assert lib.fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 2, 0, 16, 0, None, 0, None, 0, None) == -1
+
+
+def _mlp_pass(sizes, h, f, **over):
+    """An fp8gmm_mlp_pass over made-up addresses (the planners are host code and never follow them)."""
+    e = len(sizes)
+    gs = np.asarray(sizes, dtype=np.int64)
+    names = ("x", "x_fp8", "w1", "w1_fp8", "w2", "w2_fp8", "pre", "act_fp8", "y", "dy", "dy_fp8", "dact", "dpre_fp8",
+             "dx", "dw1", "dw2", "fwd_scale", "fwd_scale_inv", "fwd_amax", "bwd_scale", "bwd_scale_inv", "bwd_amax")
+    addr = {n: (i + 1) << 36 for i, n in enumerate(names)}
+    fields = dict(experts=e, hidden=h, ffn=f, fwd_fmt=_lib.E4M3, bwd_fmt=_lib.E5M2, cast_weights=1, dgrad=1, wgrad=1,
+                  grid=64, stream_k=1, tile_policy=0, tokens=int(gs.sum()), group_sizes=gs.ctypes.data, **addr)
+    fields.update(over)
+    return _lib.MlpPass(**fields), addr, gs
+
+
+def test_mlp_pass_planner_lays_out_the_reference_data_flow():
+    """fp8gmm_plan_mlp_forward / _backward against the data flow of the reference's grouped MLP stated launch by
+    launch (fp8_gmm/grouped_mlp.py:60-150 forward, :183-318 backward): operand addresses of every expert, shapes,
+    pitches and the scaling slots (forward 3 g / 3 g + 1 with fc2's GEMMs from g = E, backward 2 i and 2 E + 2 i)."""
+    lib = _lib.load()
+    assert lib.fp8gmm_sizeof_mlp_pass() == ctypes.sizeof(_lib.MlpPass) == 240
+    sizes, h, f = [300, 0, 77, 513, 1], 256, 512
+    e = len(sizes)
+    desc, A, gs = _mlp_pass(sizes, h, f)
+    row0 = np.concatenate([[0], np.cumsum(gs)[:-1]]).astype(np.uint64)
+    idx = np.arange(e, dtype=np.uint64)
+    slot = lambda name, first, stride: np.uint64(A[name] + 4 * first) + idx * np.uint64(4 * stride)
+    blob = np.zeros(1 << 22, dtype=np.uint8)
+    plan = _lib.PassPlan()
+
+    def table(rec, dtype):
+        return blob[rec.table_offset: rec.table_offset + rec.n * dtype.itemsize].view(dtype)
+
+    def rows_problem(t, a, b, c, c_bytes, n, k, kmajor, a_si, b_si, aux=None):
+        assert (t["a"] == np.uint64(A[a]) + row0 * np.uint64(k)).all()
+        assert (t["b"] == np.uint64(A[b]) + idx * np.uint64(n * k)).all()
+        assert (t["c"] == np.uint64(A[c]) + row0 * np.uint64(n * c_bytes)).all()
+        assert (t["aux"] == (np.uint64(A[aux]) + row0 * np.uint64(2 * n) if aux else 0)).all()
+        assert (t["m"] == gs).all() and (t["n"] == n).all() and (t["k"] == k).all()
+        assert (t["lda"] == k).all() and (t["ldb"] == (n if kmajor else k)).all() and (t["ldc"] == n).all()
+        assert (t["a_scale_inv"] == a_si).all() and (t["b_scale_inv"] == b_si).all()
+
+    def wgrad_problem(t, a, b, c, m, n, a_si, b_si):
+        assert (t["a"] == np.uint64(A[a]) + row0 * np.uint64(m)).all()
+        assert (t["b"] == np.uint64(A[b]) + row0 * np.uint64(n)).all()
+        assert (t["c"] == np.uint64(A[c]) + idx * np.uint64(2 * m * n)).all()
+        assert (t["m"] == m).all() and (t["n"] == n).all() and (t["k"] == gs).all()
+        assert (t["lda"] == m).all() and (t["ldb"] == n).all() and (t["ldc"] == n).all()
+        assert (t["a_scale_inv"] == a_si).all() and (t["b_scale_inv"] == b_si).all()
+        assert (t["aux"] == 0).all() and (t["c_scale"] == 0).all()
+
+    def row_casts(t, src, dst, cols, scale, amax, src2=None):
+        assert (t["in"] == np.uint64(A[src]) + row0 * np.uint64(2 * cols)).all()
+        assert (t["out"] == np.uint64(A[dst]) + row0 * np.uint64(cols)).all()
+        assert (t["in2"] == (np.uint64(A[src2]) + row0 * np.uint64(2 * cols) if src2 else 0)).all()
+        assert (t["cols"] == gs * cols).all() and (t["rows"] == (gs > 0)).all()
+        assert (t["scale"] == scale).all() and (t["amax"] == amax).all()
+
+    _lib.check(lib.fp8gmm_plan_mlp_forward(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+    assert plan.n_launches == 3 and [plan.launch[i].kind for i in range(3)] == [_lib.PASS_CAST, _lib.PASS_GEMM, _lib.PASS_GEMM]
+    t = table(plan.launch[0], _lib.TENSOR_DESC)
+    assert len(t) == 3 * e
+    for part, (src, dst, first) in enumerate((("w2", "w2_fp8", 3 * e + 1), ("w1", "w1_fp8", 1))):
+        w = t[part * e: (part + 1) * e]
+        assert (w["in"] == np.uint64(A[src]) + idx * np.uint64(2 * h * f)).all()
+        assert (w["out"] == np.uint64(A[dst]) + idx * np.uint64(h * f)).all()
+        assert (w["rows"] == 1).all() and (w["cols"] == h * f).all()
+        assert (w["scale"] == slot("fwd_scale", first, 3)).all() and (w["amax"] == slot("fwd_amax", first, 3)).all()
+    row_casts(t[2 * e:], "x", "x_fp8", h, slot("fwd_scale", 0, 3), slot("fwd_amax", 0, 3))
+    fc1 = table(plan.launch[1], _lib.GEMM_PROBLEM)
+    rows_problem(fc1, "x_fp8", "w1_fp8", "act_fp8", 1, f, h, False, slot("fwd_scale_inv", 0, 3),
+                 slot("fwd_scale_inv", 1, 3), aux="pre")
+    assert (fc1["c_scale"] == slot("fwd_scale", 3 * e, 3)).all() and (fc1["c_amax"] == slot("fwd_amax", 3 * e, 3)).all()
+    assert (plan.launch[1].out_kind, plan.launch[1].epilogue, plan.launch[1].plan.tile) == (_lib.E4M3, _lib.EPI_GELU, 256)
+    fc2 = table(plan.launch[2], _lib.GEMM_PROBLEM)
+    rows_problem(fc2, "act_fp8", "w2_fp8", "y", 2, h, f, False, slot("fwd_scale_inv", 3 * e, 3),
+                 slot("fwd_scale_inv", 3 * e + 1, 3))
+    assert (fc2["c_scale"] == 0).all() and plan.launch[2].out_kind == _lib.OUT_BF16
+    # algorithmic bytes of the GELU launch: both operands, the fp8 result and the bf16 pre-activation
+    m = gs.astype(np.float64)
+    assert plan.launch[1].bytes == float(((m + f) * h + m * f * 3).sum())
+    assert plan.launch[1].work == float((2 * m * f * h).sum())
+
+    _lib.check(lib.fp8gmm_plan_mlp_backward(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+    assert plan.n_launches == 6
+    assert [(plan.launch[i].kind, plan.launch[i].op) for i in range(6)] == [
+        (_lib.PASS_CAST, _lib.OP_QUANTIZE), (_lib.PASS_GEMM, 0), (_lib.PASS_GEMM, 0),
+        (_lib.PASS_CAST, _lib.OP_CAST_DGELU), (_lib.PASS_GEMM, 0), (_lib.PASS_GEMM, 0)]
+    g1 = (slot("bwd_scale", 0, 2), slot("bwd_amax", 0, 2), slot("bwd_scale_inv", 0, 2))
+    g2 = (slot("bwd_scale", 2 * e, 2), slot("bwd_amax", 2 * e, 2), slot("bwd_scale_inv", 2 * e, 2))
+    row_casts(table(plan.launch[0], _lib.TENSOR_DESC), "dy", "dy_fp8", h, g1[0], g1[1])
+    wgrad_problem(table(plan.launch[1], _lib.GEMM_PROBLEM), "dy_fp8", "act_fp8", "dw2", h, f, g1[2],
+                  slot("fwd_scale_inv", 3 * e, 3))
+    rows_problem(table(plan.launch[2], _lib.GEMM_PROBLEM), "dy_fp8", "w2_fp8", "dact", 2, f, h, True, g1[2],
+                 slot("fwd_scale_inv", 3 * e + 1, 3))
+    row_casts(table(plan.launch[3], _lib.TENSOR_DESC), "dact", "dpre_fp8", f, g2[0], g2[1], src2="pre")
+    rows_problem(table(plan.launch[4], _lib.GEMM_PROBLEM), "dpre_fp8", "w1_fp8", "dx", 2, h, f, True, g2[2],
+                 slot("fwd_scale_inv", 1, 3))
+    wgrad_problem(table(plan.launch[5], _lib.GEMM_PROBLEM), "dpre_fp8", "x_fp8", "dw1", f, h, g2[2],
+                  slot("fwd_scale_inv", 0, 3))
+    kk = _lib.GEMM_A_KMAJOR | _lib.GEMM_B_KMAJOR
+    assert [plan.launch[i].epilogue for i in (1, 2, 4, 5)] == [kk, _lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR, kk]
+    assert [(plan.launch[i].a_fmt, plan.launch[i].b_fmt) for i in (1, 2, 4, 5)] == [(_lib.E5M2, _lib.E4M3)] * 4
+    assert plan.launch[3].bytes == float((m * f * 5).sum()) and plan.launch[3].out_fmt == _lib.E5M2
+    # every table on its own cache line, none overlapping the next
+    ends = 0
+    for i in range(6):
+        rec = plan.launch[i]
+        assert rec.table_offset % 128 == 0 and rec.table_offset >= ends
+        ends = rec.table_offset + rec.n * (128 if rec.kind == _lib.PASS_CAST else 96)
+        if rec.kind == _lib.PASS_GEMM:
+            assert rec.items_offset % 128 == 0 and rec.items_offset >= ends
+            ends = rec.items_offset + rec.plan.rounds * rec.plan.grid * 64
+            assert rec.fixups_offset >= ends
+            ends = rec.fixups_offset + rec.plan.n_fixups * 32
+    assert ends <= plan.blob_bytes
+
+
+def test_mlp_pass_planner_options_and_errors():
+    lib = _lib.load()
+    sizes, h, f = [300, 0, 77], 256, 512
+    e = len(sizes)
+    blob = np.zeros(1 << 21, dtype=np.uint8)
+    plan = _lib.PassPlan()
+    fwd, bwd = lib.fp8gmm_plan_mlp_forward, lib.fp8gmm_plan_mlp_backward
+    run = lambda fn, d, room=blob.nbytes: fn(ctypes.byref(d), blob.ctypes.data, room, ctypes.byref(plan))
+    # cached weights: only the input is cast
+    d, _, _ = _mlp_pass(sizes, h, f, cast_weights=0, w1=0, w2=0)
+    assert run(fwd, d) == 0 and plan.launch[0].n == e
+    # gradients of the input only / of the weights only
+    d, _, _ = _mlp_pass(sizes, h, f, wgrad=0, dw1=0, dw2=0, x_fp8=0, act_fp8=0)
+    assert run(bwd, d) == 0 and plan.n_launches == 4
+    assert [plan.launch[i].kind for i in range(4)] == [_lib.PASS_CAST, _lib.PASS_GEMM, _lib.PASS_CAST, _lib.PASS_GEMM]
+    d, _, _ = _mlp_pass(sizes, h, f, dgrad=0, dx=0, w1_fp8=0)
+    assert run(bwd, d) == 0 and plan.n_launches == 5
+    # no tokens at all: nothing to do but the weight gradients, which are written as zeros
+    d, _, _ = _mlp_pass([0, 0], h, f)
+    assert run(bwd, d) == 0 and [plan.launch[i].kind for i in range(plan.n_launches)] == [0, _lib.PASS_GEMM, 0, 0, 0, _lib.PASS_GEMM]
+    assert run(fwd, d) == 0 and [plan.launch[i].kind for i in range(3)] == [_lib.PASS_CAST, 0, 0]   # the weights
+    # too little room: the size the pass needs, and nothing written past the room given
+    d, _, _ = _mlp_pass(sizes, h, f)
+    blob[:] = 0x55
+    assert run(bwd, d, 4096) == -8 and (blob[4096:] == 0x55).all()
+    need = plan.blob_bytes
+    assert run(bwd, d, need) == 0 and plan.blob_bytes == need
+    assert run(bwd, d, need - 128) == -8
+    # errors
+    for over, status in ((dict(hidden=250), -4), (dict(ffn=0), -6), (dict(tokens=5), -2), (dict(tile_policy=64), -6),
+                         (dict(grid=0), -6), (dict(pre=0), -1), (dict(dact=0), -1), (dict(dw2=0), -1)):
+        d, _, _ = _mlp_pass(sizes, h, f, **over)
+        assert run(bwd, d) == status, over
+    for over, status in ((dict(w1=0), -1), (dict(act_fp8=0), -1), (dict(fwd_amax=0), -1)):
+        d, _, _ = _mlp_pass(sizes, h, f, **over)
+        assert run(fwd, d) == status, over
+    d, _, _ = _mlp_pass([-1, 1], h, f)
+    assert run(fwd, d) == -2
+    assert lib.fp8gmm_plan_mlp_forward(None, blob.ctypes.data, blob.nbytes, ctypes.byref(plan)) == -1

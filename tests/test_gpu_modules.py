@@ -569,6 +569,149 @@ def test_planned_pass_tables_are_those_of_the_per_launch_entry_points(dev, monke
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("sizes", [[137, 0, 59, 403, 1, 700], [0, 0, 16], [300] * 9])
+@pytest.mark.parametrize("grads", ["both", "input", "weights"])
+def test_planned_mlp_passes_equal_the_per_launch_path(dev, sizes, grads):
+    """GroupedMlp plans a whole pass with one library call (fp8gmm_plan_mlp_forward / _backward).  Outputs, gradients,
+    the intermediates between the kernels, fp8 scaling state and amax history must equal, bit for bit, what the
+    per-launch entry points give over three steps (ragged, empty and equal experts; cached fp8 weights on the last
+    step; gradients wanted for the input, the weights or both)."""
+    import fp8_gmm_amd as pkg
+
+    e, h, f = len(sizes), 256, 384
+    g = torch.Generator(device=dev).manual_seed(6)
+    w1 = (torch.randn(e, f, h, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    w2 = (torch.randn(e, h, f, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    xs = [torch.randn(sum(sizes), h, generator=g, device=dev).to(torch.bfloat16) for _ in range(3)]
+    dys = [(torch.randn(sum(sizes), h, generator=g, device=dev) * 1e-2).to(torch.bfloat16) for _ in range(3)]
+    results = []
+    for planned in (True, False):
+        module = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev, planned_passes=planned)
+        module.fc1_weight.data.copy_(w1)
+        module.fc2_weight.data.copy_(w2)
+        for p in module.parameters():
+            p.requires_grad_(grads != "input")
+        cap = {}
+        module.capture_intermediates(cap)
+        recipe = pkg.DelayedScaling(amax_history_len=2)
+        trace = []
+        for step, first in enumerate((None, True, False)):
+            x = xs[step].clone().requires_grad_(grads != "weights")
+            module.zero_grad(set_to_none=True)
+            with pkg.fp8_autocast(enabled=True, fp8_recipe=recipe):
+                out = module(x, torch.tensor(sizes), is_first_microbatch=first)
+            out.backward(dys[step])
+            torch.cuda.synchronize()
+            fwd, bwd = module.fp8_meta["scaling_fwd"], module.fp8_meta["scaling_bwd"]
+            got = {"out": out.detach(), "grad_input": x.grad, "grad_fc1": module.fc1_weight.grad,
+                   "grad_fc2": module.fc2_weight.grad, "fwd scale": fwd.scale, "fwd amax history": fwd.amax_history,
+                   "bwd scale": bwd.scale, "bwd amax history": bwd.amax_history}
+            got.update(cap)
+            trace.append({k: v.clone() for k, v in got.items() if v is not None})
+        results.append(trace)
+    bits = {torch.bfloat16: torch.int16, torch.float8_e4m3fn: torch.uint8, torch.float8_e5m2: torch.uint8}
+    for step, (a, b) in enumerate(zip(*results)):
+        assert a.keys() == b.keys()
+        assert {"pre_gelu_out", "gelu_out_fp8", "grad_gelu_out", "grad_pre_fp8"} <= a.keys()
+        assert ("grad_input" in a) == (grads != "weights") and ("grad_fc1" in a) == (grads != "input")
+        for name in a:
+            ta, tb = a[name], b[name]
+            assert ta.dtype == tb.dtype and ta.shape == tb.shape, name
+            assert torch.equal(ta.view(bits.get(ta.dtype, ta.dtype)), tb.view(bits.get(tb.dtype, tb.dtype))), \
+                f"step {step}: {name}"
+
+
+@pytest.mark.gpu
+def test_planned_mlp_pass_tables_are_those_of_the_per_launch_entry_points(dev, monkeypatch):
+    """The tables fp8gmm_plan_mlp_forward / _backward write for given buffers must be, byte for byte, the tensor
+    descriptors, problem tables, work lists and shared-tile records that backend.multi_quantize / fp8_gmm /
+    grouped_gemm / multi_cast_dgelu build for the same buffers in the order GroupedMlp calls them (captured here
+    without launching anything)."""
+    import ctypes
+
+    import numpy as np
+
+    from fp8_gmm_amd import _lib, backend
+
+    sizes = [700, 0, 33, 1291, 5, 256]
+    e, h, f, tokens = len(sizes), 512, 768, sum(sizes)
+    E4, E5, bf = torch.float8_e4m3fn, torch.float8_e5m2, torch.bfloat16
+    z = lambda shape, dtype: torch.zeros(shape, dtype=dtype, device=dev)
+    x, x8 = z((tokens, h), bf), z((tokens, h), E4)
+    w1, w18, dw1 = z((e, f, h), bf), z((e, f, h), E4), z((e, f, h), bf)
+    w2, w28, dw2 = z((e, h, f), bf), z((e, h, f), E4), z((e, h, f), bf)
+    pre, act8, y = z((tokens, f), bf), z((tokens, f), E4), z((tokens, h), bf)
+    dy, dy8, dact, dpre8, dx = z((tokens, h), bf), z((tokens, h), E5), z((tokens, f), bf), z((tokens, f), E5), z((tokens, h), bf)
+    fs, fsi, fa = (torch.ones(6 * e, device=dev) for _ in range(3))
+    bs, bsi, ba = (torch.ones(4 * e, device=dev) for _ in range(3))
+    bounds = np.concatenate([[0], np.cumsum(sizes)])
+    ptr = lambda t, first, stride: np.uint64(t.data_ptr() + 4 * first) + np.arange(e, dtype=np.uint64) * np.uint64(4 * stride)
+    rows, stack = backend.TensorBatch.rows_of, backend.TensorBatch.stack_of
+    g2, b2 = 3 * e, 2 * e   # first forward / backward scaling slot of the fc2 GEMMs
+
+    captured = []
+    monkeypatch.setattr(backend, "_flush", lambda items: captured.extend(bytes(it[0].view(np.uint8).reshape(-1)) for it in items))
+    with backend.batched_uploads():
+        # forward: casts (fc2's weights, fc1's weights, the input), fc1 with the GELU epilogue, fc2
+        backend.multi_quantize(stack(w2) + stack(w1) + rows(x, bounds), stack(w28) + stack(w18) + rows(x8, bounds),
+                               np.concatenate([ptr(fs, g2 + 1, 3), ptr(fs, 1, 3), ptr(fs, 0, 3)]),
+                               np.concatenate([ptr(fa, g2 + 1, 3), ptr(fa, 1, 3), ptr(fa, 0, 3)]))
+        backend.fp8_gmm(x8, w18, sizes, ptr(fsi, 0, 3), ptr(fsi, 1, 3), c=act8, pre_gelu_out=pre,
+                        c_scales=ptr(fs, g2, 3), c_amaxes=ptr(fa, g2, 3))
+        backend.fp8_gmm(act8, w28, sizes, ptr(fsi, g2, 3), ptr(fsi, g2 + 1, 3), c=y)
+        # backward: cast, fc2 wgrad, fc2 dgrad, dGELU cast, fc1 dgrad, fc1 wgrad
+        backend.multi_quantize(rows(dy, bounds), rows(dy8, bounds), ptr(bs, 0, 2), ptr(ba, 0, 2))
+        backend.grouped_gemm(rows(dy8, bounds), rows(act8, bounds), stack(dw2), ptr(bsi, 0, 2), ptr(fsi, g2, 3), transposed=True)
+        backend.fp8_gmm(dy8, w28, sizes, ptr(bsi, 0, 2), ptr(fsi, g2 + 1, 3), c=dact, backward=True, b_transposed=True)
+        backend.multi_cast_dgelu(rows(dact, bounds), rows(pre, bounds), rows(dpre8, bounds), ptr(bs, b2, 2), ptr(ba, b2, 2))
+        backend.fp8_gmm(dpre8, w18, sizes, ptr(bsi, b2, 2), ptr(fsi, 1, 3), c=dx, backward=True, b_transposed=True)
+        backend.grouped_gemm(rows(dpre8, bounds), rows(x8, bounds), stack(dw1), ptr(bsi, b2, 2), ptr(fsi, 0, 3), transposed=True)
+    assert len(captured) == 9
+
+    grid = _lib.gemm_grid(_lib.init(torch.cuda.current_device()))
+    gs = np.asarray(sizes, dtype=np.int64)
+    desc = _lib.MlpPass(experts=e, hidden=h, ffn=f, fwd_fmt=_lib.E4M3, bwd_fmt=_lib.E5M2, cast_weights=1, dgrad=1, wgrad=1,
+                        grid=grid, stream_k=int(backend.options.stream_k), tile_policy=0, tokens=tokens,
+                        group_sizes=gs.ctypes.data, x=x.data_ptr(), x_fp8=x8.data_ptr(), w1=w1.data_ptr(),
+                        w1_fp8=w18.data_ptr(), w2=w2.data_ptr(), w2_fp8=w28.data_ptr(), pre=pre.data_ptr(),
+                        act_fp8=act8.data_ptr(), y=y.data_ptr(), dy=dy.data_ptr(), dy_fp8=dy8.data_ptr(),
+                        dact=dact.data_ptr(), dpre_fp8=dpre8.data_ptr(), dx=dx.data_ptr(), dw1=dw1.data_ptr(),
+                        dw2=dw2.data_ptr(), fwd_scale=fs.data_ptr(), fwd_scale_inv=fsi.data_ptr(), fwd_amax=fa.data_ptr(),
+                        bwd_scale=bs.data_ptr(), bwd_scale_inv=bsi.data_ptr(), bwd_amax=ba.data_ptr())
+    L = _lib.load()
+    blob = np.zeros(1 << 23, dtype=np.uint8)
+    want = iter(captured)
+    for fn, launches in ((L.fp8gmm_plan_mlp_forward, 3), (L.fp8gmm_plan_mlp_backward, 6)):
+        plan = _lib.PassPlan()
+        assert fn(ctypes.byref(desc), blob.ctypes.data, 1024, ctypes.byref(plan)) == -8
+        need = plan.blob_bytes
+        _lib.check(fn(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+        assert plan.blob_bytes == need and plan.n_launches == launches
+        for i in range(plan.n_launches):
+            rec, ref = plan.launch[i], next(want)
+            if rec.kind == _lib.PASS_CAST:
+                got = bytes(blob[rec.table_offset: rec.table_offset + rec.n * 128])
+                assert got == ref, f"launch {i}: tensor descriptors differ"
+            else:
+                probs = bytes(blob[rec.table_offset: rec.table_offset + rec.n * 96])
+                items = bytes(blob[rec.items_offset: rec.items_offset + rec.plan.rounds * rec.plan.grid * 64])
+                fix = bytes(blob[rec.fixups_offset: rec.fixups_offset + rec.plan.n_fixups * 32])
+                off_items = (rec.n * 96 + 127) // 128 * 128
+                assert probs == ref[: rec.n * 96], f"launch {i}: problem table differs"
+                assert items == ref[off_items: off_items + len(items)], f"launch {i}: work list differs"
+                assert fix == ref[off_items + len(items):], f"launch {i}: shared-tile records differ"
+    # the launch records say what each launch is
+    plan = _lib.PassPlan()
+    _lib.check(L.fp8gmm_plan_mlp_forward(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+    assert (plan.launch[1].out_kind, plan.launch[1].epilogue) == (_lib.E4M3, _lib.EPI_GELU)
+    assert (plan.launch[2].out_kind, plan.launch[2].epilogue) == (_lib.OUT_BF16, 0)
+    _lib.check(L.fp8gmm_plan_mlp_backward(ctypes.byref(desc), blob.ctypes.data, blob.nbytes, ctypes.byref(plan)))
+    assert [plan.launch[i].op for i in (0, 3)] == [_lib.OP_QUANTIZE, _lib.OP_CAST_DGELU]
+    assert [plan.launch[i].epilogue for i in (1, 2, 4, 5)] == [
+        _lib.GEMM_A_KMAJOR | _lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR, _lib.GEMM_A_KMAJOR | _lib.GEMM_B_KMAJOR]
+
+
+@pytest.mark.gpu
 def test_fused_dgelu_backward_against_the_oracle(dev):
     """GroupedMlp(fused_dgelu=True): the fc2 data-gradient GEMM forms d(pre-GELU) = fp8(v * dgelu(pre)) in its
     epilogue, from the fp32 accumulator, and the separate cast + dGELU pass is gone.  Checked against the oracle's
