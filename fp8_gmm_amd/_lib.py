@@ -22,6 +22,7 @@ EPI_DGELU = 8
 GEMM_B_KMAJOR = 2
 GEMM_A_KMAJOR = 4
 GEMM_TILE_128 = 0x100   # planning flag: 128 x 128 tiles, two workgroups per compute unit
+GEMM_TILE_DUAL = 0x200  # planning flag: 128 x 256 tiles for the kernel form with two sets of accumulators
 
 OP_QUANTIZE = 0
 OP_SCALE_MUL = 1
@@ -109,7 +110,7 @@ class GemmPlan(ctypes.Structure):
 
     _fields_ = [("grid", ctypes.c_int32), ("rounds", ctypes.c_int32), ("n_fixups", ctypes.c_int32),
                 ("n_slots", ctypes.c_int32), ("total_tiles", ctypes.c_int32), ("tile", ctypes.c_int32),
-                ("reserved", ctypes.c_int32 * 2)]
+                ("tile_m", ctypes.c_int32), ("reserved", ctypes.c_int32)]
 
 
 class LinearPass(ctypes.Structure):

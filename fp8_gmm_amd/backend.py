@@ -746,6 +746,8 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
     epi = _lib.EPI_GELU if gelu else _lib.EPI_DGELU if dgelu else 0
     if not epi and _small_tiles(table):
         plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | _lib.GEMM_TILE_128, 2 * grid, False)
+    elif not epi and c_dtype == torch.bfloat16 and _dual_tiles(table, a_kmajor):
+        plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | _lib.GEMM_TILE_DUAL, grid, False)
     else:
         plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, layout | epi, grid, options.stream_k)
     if plan.total_tiles == 0:
@@ -787,7 +789,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
 # Tail balancing of the grouped GEMM (the workgroups of an XCD share their range's last tiles along K) needs
 # scratch memory for partial sums and a second, small launch; options.stream_k = False plans every launch without it.
 class GemmOptions:
-    """Launch policy of the grouped GEMMs of this process: ``tile`` "auto" | "256" | "128", ``stream_k`` (share the
+    """Launch policy of the grouped GEMMs of this process: ``tile`` "auto" | "256" | "128" | "dual", ``stream_k`` (share the
     tail tiles of a launch along K), ``wgrad`` "in_place" | "copy", ``upload`` "kernel" (tables reach the device
     through staging memory and a copy kernel of the library) | "copy" (a pinned buffer per upload and torch's
     asynchronous copy).  The defaults can be preset with the environment variables FP8GMM_TILE, FP8GMM_STREAMK
@@ -821,6 +823,26 @@ def gemm_options(**changes):
 
 def wgrad_wants_transposed_gradient(total_rows, num_groups):
     return options.wgrad == "copy" and num_groups > 0 and total_rows > 0
+
+
+# The form with two sets of accumulators (128 x 256 tiles, a finished tile stored between the products of the next
+# one) takes the tile boundaries out of a launch and pays with operand traffic: 1.33 x the bytes from L2 per flop and
+# three quarters of the bytes in flight per compute unit.  It wins where the boundaries are what a launch waits for
+# - contractions of up to 2048 whose operands and result the 256 MB memory-side cache can largely hold, 7 - 17 %
+# there - and loses where the launch streams from HBM (by 15 - 25 % on config 4's launches) or keeps the matrix pipes
+# busy (by 20 - 35 % at K >= 3072).  The weight-gradient form (both operands contraction-major) loses 4 % even
+# then.  options.tile = "dual" forces it wherever it exists (bf16 results, no fused epilogue).
+_DUAL_MAX_K = 2048
+_DUAL_MAX_BYTES = 320 << 20
+
+
+def _dual_tiles(table, a_kmajor):
+    if options.tile != "auto":
+        return options.tile == "dual"
+    if a_kmajor or len(table) == 0:
+        return False
+    m, n, k = (table[f].astype(np.int64) for f in ("m", "n", "k"))
+    return int(k.max()) <= _DUAL_MAX_K and int(((m + n) * k + 2 * m * n).sum()) <= _DUAL_MAX_BYTES
 
 
 def _small_tiles(table):
@@ -900,7 +922,7 @@ def _run_pass(device, desc, fields, plan_fn, bound_fn):
     grid = _lib.gemm_grid(_lib.init(index))
     desc.grid = grid
     desc.stream_k = int(bool(options.stream_k))
-    desc.tile_policy = {"auto": 0, "256": 256, "128": 128}[options.tile]
+    desc.tile_policy = {"auto": 0, "256": 256, "128": 128, "dual": _lib.GEMM_TILE_DUAL}[options.tile]
     bound = bound_fn(desc, grid)
     plan = _lib.PassPlan()
     while True:

@@ -161,15 +161,15 @@ FP8GMM_HD int64_t sk_bound(const Sched& s, int j) { return s.sk_cost * j / s.sk_
 // 8 x 4 block that needs 12 operand slabs, whatever the shape of the problem (a 56 x 16 weight-gradient
 // problem walked with m fastest over all 56 rows would need 33).
 constexpr int kRasterRows = 8;
-FP8GMM_HD void tile_origin(int m, int n, int local, int tile, int* m0, int* n0) {
-  const int tiles_m = (m + tile - 1) / tile, tiles_n = (n + tile - 1) / tile;
+FP8GMM_HD void tile_origin(int m, int n, int local, int tile_m, int tile_n, int* m0, int* n0) {
+  const int tiles_m = (m + tile_m - 1) / tile_m, tiles_n = (n + tile_n - 1) / tile_n;
   const int group = local / (kRasterRows * tiles_n);
   const int within = local - group * (kRasterRows * tiles_n);
   const int rows = tiles_m - group * kRasterRows < kRasterRows ? tiles_m - group * kRasterRows : kRasterRows;
-  *m0 = (group * kRasterRows + within % rows) * tile;
-  *n0 = (within / rows) * tile;
+  *m0 = (group * kRasterRows + within % rows) * tile_m;
+  *n0 = (within / rows) * tile_n;
 }
-FP8GMM_HD void tile_origin(int m, int n, int local, int* m0, int* n0) { tile_origin(m, n, local, BM, m0, n0); }
+FP8GMM_HD void tile_origin(int m, int n, int local, int* m0, int* n0) { tile_origin(m, n, local, BM, BN, m0, n0); }
 
 struct Item {
   int tile, prob, m0, n0;

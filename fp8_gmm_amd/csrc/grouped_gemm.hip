@@ -205,9 +205,15 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
     return FP8GMM_ERR_BAD_FORMAT;
   // e5m2 x e5m2 does not exist (cuBLASLt rejects it too); the contraction-major forms are the gradient GEMMs,
   // whose b is a forward tensor (weight or activation), always e4m3
-  const int tile = plan->tile == 0 ? kGemmTileM : plan->tile;
-  if (tile != kGemmTileM && tile != FP8GMM_GEMM_SMALL_TILE) return FP8GMM_ERR_BAD_ARGUMENT;
-  // the small tile is never shared along K and has no fused GELU epilogue
+  int tile = plan->tile == 0 ? kGemmTileN : plan->tile;
+  if (tile != kGemmTileN && tile != FP8GMM_GEMM_SMALL_TILE) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (plan->tile_m != 0 && plan->tile_m != tile) {
+    // the form with two sets of accumulators: bf16 results only
+    if (tile != kGemmTileN || plan->tile_m != FP8GMM_GEMM_DUAL_TILE_M || out_kind != FP8GMM_OUT_BF16)
+      return FP8GMM_ERR_BAD_ARGUMENT;
+    tile = kTileDual;
+  }
+  // only the large tile is ever shared along K or has the fused epilogues
   if (tile != kGemmTileM &&
       (plan->n_slots != 0 || plan->n_fixups != 0 || (epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU))))
     return FP8GMM_ERR_BAD_ARGUMENT;

@@ -1272,6 +1272,15 @@ __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_ke
 #undef FP8GMM_MF0
 #undef FP8GMM_MF1
 
+}  // namespace fp8gmm
+#include "grouped_gemm_dual.h"
+namespace fp8gmm {
+
+// The template argument that stands for the form with two sets of accumulators (tiles of 128 x 256) wherever a tile
+// size selects a kernel.
+constexpr int kTileDual = FP8GMM_GEMM_DUAL_TILE_M + kGemmTileN;
+static_assert(kTileDual != kGemmTileM && kTileDual != FP8GMM_GEMM_SMALL_TILE, "a code of its own");
+
 // Per device: "the GEMM kernels may use the whole LDS" has been set for this variant.  fp8gmm_init sets it for
 // every variant; a launch on a device that was never initialised sets its own.
 constexpr int kMaxDevices = 64;
@@ -1281,9 +1290,16 @@ int prepare_variant(int dev) {
   static std::atomic<bool> attr_set[kMaxDevices];
   if (dev < 0 || dev >= kMaxDevices) return FP8GMM_ERR_NO_DEVICE;
   if (!attr_set[dev].load(std::memory_order_acquire)) {
-    auto kernel = grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            RING * TILE * BK) != hipSuccess)
+    const void* kernel = nullptr;
+    int lds_bytes = 0;
+    if constexpr (TILE == kTileDual) {
+      kernel = reinterpret_cast<const void*>(grouped_gemm_dual_kernel<A_FMT, B_FMT, A_TR, B_TR>);
+      lds_bytes = RING * BN * BK;
+    } else {
+      kernel = reinterpret_cast<const void*>(grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>);
+      lds_bytes = RING * TILE * BK;
+    }
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess)
       return FP8GMM_ERR_LAUNCH;
     attr_set[dev].store(true, std::memory_order_release);
   }
@@ -1297,8 +1313,14 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item*
   if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
   const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR, TILE>(dev);
   if (rc != FP8GMM_OK) return rc;
-  hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>), dim3(grid), dim3(NTHREADS),
-                     RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace);
+  if constexpr (TILE == kTileDual) {
+    // bf16 results without a fused epilogue only (the caller has checked)
+    hipLaunchKernelGGL((grouped_gemm_dual_kernel<A_FMT, B_FMT, A_TR, B_TR>), dim3(grid), dim3(NTHREADS), RING * BN * BK,
+                       stream, probs_dev, items_dev);
+  } else {
+    hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>), dim3(grid), dim3(NTHREADS),
+                       RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace);
+  }
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
@@ -1318,7 +1340,14 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item*
   X(FP8GMM_E4M3, FP8GMM_E4M3, false, true, 128)   \
   X(FP8GMM_E5M2, FP8GMM_E4M3, false, true, 128)   \
   X(FP8GMM_E4M3, FP8GMM_E4M3, true, true, 128)    \
-  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 128)
+  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true, 128)    \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, false, kTileDual)  \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, false, kTileDual)  \
+  X(FP8GMM_E4M3, FP8GMM_E5M2, false, false, kTileDual)  \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, false, true, kTileDual)   \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, false, true, kTileDual)   \
+  X(FP8GMM_E4M3, FP8GMM_E4M3, true, true, kTileDual)    \
+  X(FP8GMM_E5M2, FP8GMM_E4M3, true, true, kTileDual)
 
 #define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT, TL)                                                                     \
   extern template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                        \

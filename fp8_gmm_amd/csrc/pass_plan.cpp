@@ -35,6 +35,21 @@ bool small_tiles_pay(const fp8gmm_gemm_problem* p, int n) {
   return large != 0 && (large <= 160 || 2 * small <= 5 * large);
 }
 
+// ... and the form with two sets of accumulators (FP8GMM_GEMM_TILE_DUAL): a contraction of up to 2048 whose
+// operands and result the 256 MB memory-side cache can largely hold, operand a row-major; what the tile boundaries
+// cost such a launch is more than the form's extra operand traffic.
+bool dual_tiles_pay(const fp8gmm_gemm_problem* p, int n, int layout) {
+  if ((layout & FP8GMM_GEMM_A_KMAJOR) || n == 0) return false;
+  int64_t bytes = 0;
+  int32_t k_max = 0;
+  for (int i = 0; i < n; ++i) {
+    const int64_t m = p[i].m, nn = p[i].n, k = p[i].k;
+    bytes += (m + nn) * k + 2 * m * nn;
+    if (p[i].k > k_max) k_max = p[i].k;
+  }
+  return k_max <= 2048 && bytes <= ((int64_t)320 << 20);
+}
+
 struct Writer {
   void* blob;
   int64_t capacity;
@@ -84,7 +99,9 @@ int plan_gemm(Writer& w, fp8gmm_gemm_problem* probs, int n, int layout, int tile
   rec->out_kind = out_kind;
   rec->epilogue = layout | epi;
   const bool small = epi == 0 && (tile_policy == 128 || (tile_policy == 0 && small_tiles_pay(probs, n)));
-  const int plan_layout = layout | epi | (small ? FP8GMM_GEMM_TILE_128 : 0);
+  const bool dual = !small && epi == 0 && out_kind == FP8GMM_OUT_BF16 &&
+                    (tile_policy == FP8GMM_GEMM_TILE_DUAL || (tile_policy == 0 && dual_tiles_pay(probs, n, layout)));
+  const int plan_layout = layout | epi | (small ? FP8GMM_GEMM_TILE_128 : dual ? FP8GMM_GEMM_TILE_DUAL : 0);
   const int plan_grid = small ? 2 * grid : grid;
   // room for the work list: whatever is left of the blob
   int64_t items_off = 0;
@@ -94,7 +111,7 @@ int plan_gemm(Writer& w, fp8gmm_gemm_problem* probs, int n, int layout, int tile
   fp8gmm_gemm_item* items = room > 0 ? reinterpret_cast<fp8gmm_gemm_item*>(at(w.blob, w.used)) : nullptr;
   // shared-tile records are few (at most one per workgroup): planned into a local array, appended afterwards
   static thread_local fp8gmm_gemm_fixup_desc fix[4096];
-  int rc = fp8gmm_plan_grouped_gemm_launch(probs, n, plan_layout, plan_grid, small ? 0 : stream_k, items, (int)room, fix,
+  int rc = fp8gmm_plan_grouped_gemm_launch(probs, n, plan_layout, plan_grid, small || dual ? 0 : stream_k, items, (int)room, fix,
                                            4096, &rec->plan);
   if (rc != FP8GMM_OK && rc != FP8GMM_ERR_BUFFER_TOO_SMALL) return rc;
   const int64_t item_bytes = (int64_t)rec->plan.rounds * rec->plan.grid * (int64_t)sizeof(fp8gmm_gemm_item);
@@ -125,7 +142,8 @@ int check_common(const fp8gmm_linear_pass* s, fp8gmm_pass_plan* out) {
   if (s->experts < 0 || s->in_features <= 0 || s->out_features <= 0 || s->grid <= 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (s->experts > 0 && s->group_sizes == nullptr) return FP8GMM_ERR_NULL_POINTER;
   if ((s->in_features % 16) != 0 || (s->out_features % 16) != 0) return FP8GMM_ERR_ALIGNMENT;
-  if (s->tile_policy != 0 && s->tile_policy != 128 && s->tile_policy != 256) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (s->tile_policy != 0 && s->tile_policy != 128 && s->tile_policy != 256 && s->tile_policy != FP8GMM_GEMM_TILE_DUAL)
+    return FP8GMM_ERR_BAD_ARGUMENT;
   int64_t rows = 0;
   for (int i = 0; i < s->experts; ++i) {
     if (s->group_sizes[i] < 0) return FP8GMM_ERR_BAD_SHAPE;
@@ -357,7 +375,8 @@ int check_mlp(const fp8gmm_mlp_pass* s, fp8gmm_pass_plan* out) {
   if (s->experts < 0 || s->hidden <= 0 || s->ffn <= 0 || s->grid <= 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (s->experts > 0 && s->group_sizes == nullptr) return FP8GMM_ERR_NULL_POINTER;
   if ((s->hidden % 16) != 0 || (s->ffn % 16) != 0) return FP8GMM_ERR_ALIGNMENT;
-  if (s->tile_policy != 0 && s->tile_policy != 128 && s->tile_policy != 256) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (s->tile_policy != 0 && s->tile_policy != 128 && s->tile_policy != 256 && s->tile_policy != FP8GMM_GEMM_TILE_DUAL)
+    return FP8GMM_ERR_BAD_ARGUMENT;
   const int64_t widest = s->hidden > s->ffn ? s->hidden : s->ffn;
   int64_t rows = 0;
   for (int i = 0; i < s->experts; ++i) {

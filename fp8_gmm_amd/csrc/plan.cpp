@@ -184,13 +184,14 @@ int fp8gmm_plan_grouped_gemm_layout(fp8gmm_gemm_problem* probs, int n, int layou
 // The work list of a launch: the schedule of gemm_schedule.h written out, one record per (workgroup, item), in
 // the order items[r * grid + workgroup]; the slots in use are renumbered from 0 in the order the workgroups
 // are walked, and the fix-up records name them by their new numbers.
-// The same launch cut into 128 x 128 tiles (FP8GMM_GEMM_TILE_128): whole tiles only, the tile list in 8 contiguous
-// ranges of equal work, the workgroups of an XCD striding through their range.
-static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int grid, fp8gmm_gemm_item* items,
-                            int max_items, fp8gmm_gemm_plan* plan) {
+// The same launch cut into 128 x 128 tiles (FP8GMM_GEMM_TILE_128) or into 128 x 256 tiles for the kernel with two
+// sets of accumulators (FP8GMM_GEMM_TILE_DUAL): whole tiles only, the tile list in 8 contiguous ranges of equal
+// work, the workgroups of an XCD striding through their range.
+// kOverhead: what a tile costs besides its steps, in K = 128 steps: epilogue and switch of a small tile on a
+// workgroup that shares its compute unit; with two sets of accumulators, the slower steps that carry the result.
+static int plan_whole_tiles(const int TM, const int TN, const int kOverhead, fp8gmm_gemm_problem* probs, int n, int layout,
+                            int grid, fp8gmm_gemm_item* items, int max_items, fp8gmm_gemm_plan* plan) {
   using namespace fp8gmm;
-  constexpr int T = FP8GMM_GEMM_SMALL_TILE;
-  constexpr int kOverhead = 3;   // epilogue and switch of a small tile, in K = 128 steps of a workgroup that shares its CU
   int unused = 0;
   const int rc = fp8gmm_plan_grouped_gemm_layout(probs, n, layout, &unused);
   if (rc != FP8GMM_OK) return rc;
@@ -198,7 +199,7 @@ static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int g
   // tiles and work per problem
   std::vector<int64_t> tile_begin((size_t)n + 1, 0), work_begin((size_t)n + 1, 0);
   for (int p = 0; p < n; ++p) {
-    const int64_t tiles = (int64_t)((probs[p].m + T - 1) / T) * ((probs[p].n + T - 1) / T);
+    const int64_t tiles = (int64_t)((probs[p].m + TM - 1) / TM) * ((probs[p].n + TN - 1) / TN);
     const int64_t steps = (probs[p].k + 127) / 128;
     tile_begin[p + 1] = tile_begin[p] + tiles;
     work_begin[p + 1] = work_begin[p] + tiles * ((steps > 0 ? steps : 1) + kOverhead);
@@ -206,7 +207,8 @@ static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int g
   }
   const int total_tiles = (int)tile_begin[n];
   plan->total_tiles = total_tiles;
-  plan->tile = T;
+  plan->tile = TN;
+  plan->tile_m = TM == TN ? 0 : TM;
   if (total_tiles == 0) return FP8GMM_OK;
   {
     const int needed = ((total_tiles + kNumXcd - 1) / kNumXcd) * kNumXcd;
@@ -252,9 +254,9 @@ static int plan_small_tiles(fp8gmm_gemm_problem* probs, int n, int layout, int g
       fp8gmm_gemm_item& o = items[(size_t)r * grid + (size_t)j * kNumXcd + x];
       o = fp8gmm_gemm_item{};
       int m0 = 0, n0 = 0;
-      tile_origin(pr.m, pr.n, (int)(t - tile_begin[p]), T, &m0, &n0);
-      const int64_t rows = pr.m - m0 < T ? pr.m - m0 : T;
-      const int64_t cols = pr.n - n0 < T ? pr.n - n0 : T;
+      tile_origin(pr.m, pr.n, (int)(t - tile_begin[p]), TM, TN, &m0, &n0);
+      const int64_t rows = pr.m - m0 < TM ? pr.m - m0 : TM;
+      const int64_t cols = pr.n - n0 < TN ? pr.n - n0 : TN;
       if (pr.k > 0) {
         if (!a_kmajor) {
           o.a = (uint64_t)reinterpret_cast<uintptr_t>(pr.a) + (uint64_t)m0 * (uint64_t)pr.lda;
@@ -292,9 +294,14 @@ int fp8gmm_plan_grouped_gemm_launch(fp8gmm_gemm_problem* probs, int n, int layou
   if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
   *plan = fp8gmm_gemm_plan{};
   if (grid <= 0 || (grid % kNumXcd) != 0 || max_items < 0 || max_fixups < 0) return FP8GMM_ERR_BAD_ARGUMENT;
-  if (layout & FP8GMM_GEMM_TILE_128) {
+  if (layout & (FP8GMM_GEMM_TILE_128 | FP8GMM_GEMM_TILE_DUAL)) {
     if (layout & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU)) return FP8GMM_ERR_BAD_ARGUMENT;
-    return plan_small_tiles(probs, n, layout & ~FP8GMM_GEMM_TILE_128, grid, items, max_items, plan);
+    if ((layout & FP8GMM_GEMM_TILE_128) && (layout & FP8GMM_GEMM_TILE_DUAL)) return FP8GMM_ERR_BAD_ARGUMENT;
+    const int operands = layout & ~(FP8GMM_GEMM_TILE_128 | FP8GMM_GEMM_TILE_DUAL);
+    if (layout & FP8GMM_GEMM_TILE_128)
+      return plan_whole_tiles(FP8GMM_GEMM_SMALL_TILE, FP8GMM_GEMM_SMALL_TILE, 3, probs, n, operands, grid, items,
+                              max_items, plan);
+    return plan_whole_tiles(FP8GMM_GEMM_DUAL_TILE_M, kGemmTileN, 2, probs, n, operands, grid, items, max_items, plan);
   }
   plan->tile = kGemmTileM;
   const int layout_given = layout, grid_given = grid;

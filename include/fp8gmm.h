@@ -167,6 +167,14 @@ typedef struct fp8gmm_gemm_problem {
  * csrc/fp8_gmm.cu:82-110). */
 #define FP8GMM_GEMM_TILE_128 0x100
 #define FP8GMM_GEMM_SMALL_TILE 128
+/* Planning flag (`layout` of fp8gmm_plan_grouped_gemm_launch only): cut the outputs into tiles of 128 rows x 256
+ * columns for the kernel form with two sets of accumulators per wavefront, which stores a finished tile in pieces
+ * between the products of the next one (one workgroup per compute unit, the usual grid).  For launches with a short
+ * contraction (up to about 2048) that fill the machine, which otherwise spend as long at their tile boundaries as in
+ * their main loops; costs 1.33 x the operand traffic from L2 per flop.  bf16 results without FP8GMM_EPI_* only; never
+ * shares tiles along K (stream_k is ignored).  No counterpart in the reference. */
+#define FP8GMM_GEMM_TILE_DUAL 0x200
+#define FP8GMM_GEMM_DUAL_TILE_M 128
 
 /*
  * Work list of a grouped-GEMM launch, written by fp8gmm_plan_grouped_gemm_launch on the host and read by the
@@ -215,8 +223,9 @@ typedef struct fp8gmm_gemm_plan {
   int32_t n_fixups;    /* tiles shared along K = workgroups of the fix-up launch (0: no such launch) */
   int32_t n_slots;     /* workspace slots the launch writes: it needs n_slots * FP8GMM_GEMM_SLOT_BYTES bytes */
   int32_t total_tiles;
-  int32_t tile;        /* rows = columns of a tile: 256, or 128 when planned with FP8GMM_GEMM_TILE_128 (0 reads as 256) */
-  int32_t reserved[2];
+  int32_t tile;        /* columns of a tile: 256, or 128 when planned with FP8GMM_GEMM_TILE_128 (0 reads as 256) */
+  int32_t tile_m;      /* rows of a tile where they differ from `tile`: 128 when planned with FP8GMM_GEMM_TILE_DUAL (0: as `tile`) */
+  int32_t reserved;
 } fp8gmm_gemm_plan;    /* 32 bytes */
 
 #define FP8GMM_GEMM_SLOT_BYTES 262144  /* fp32 accumulators of one 256 x 256 tile */
@@ -342,7 +351,8 @@ typedef struct fp8gmm_linear_pass {
   int32_t dgrad, wgrad;              /* backward: which gradients are wanted */
   int32_t grid;                      /* fp8gmm_gemm_grid() of the device */
   int32_t stream_k;                  /* as for fp8gmm_plan_grouped_gemm_launch */
-  int32_t tile_policy;               /* 0: the library chooses per launch; 256 or 128: that tile for every launch */
+  int32_t tile_policy;               /* 0: the library chooses per launch; 256 or 128: that tile for every launch;
+                                        FP8GMM_GEMM_TILE_DUAL: the 128 x 256 form for every launch that can take it */
   int32_t reserved;
   int64_t tokens;                    /* rows of x / dy: must equal the sum of group_sizes */
   const int64_t* group_sizes;        /* HOST array [experts] */

@@ -265,10 +265,12 @@ def test_consecutive_tiles_form_compact_blocks():
             assert len(rows) + len(cols) <= 12, (shape, start, len(rows), len(cols))
 
 
-def test_small_tile_plan():
-    """FP8GMM_GEMM_TILE_128: the same launch cut into 128 x 128 tiles, whole tiles only.  Every 128 x 128 block of
-    every output exactly once, records with the addresses and extents of a 128-row / 128-column slab, XCD ranges
-    contiguous and in order, no workspace, no fix-up launch; not available together with the GELU epilogue."""
+@pytest.mark.parametrize("flag,tm,tn", [(_lib.GEMM_TILE_128, 128, 128), (_lib.GEMM_TILE_DUAL, 128, 256)])
+def test_whole_tile_plans(flag, tm, tn):
+    """FP8GMM_GEMM_TILE_128 / FP8GMM_GEMM_TILE_DUAL: the same launch cut into 128 x 128 / 128 x 256 tiles, whole tiles
+    only.  Every such block of every output exactly once, records with the addresses and extents of a slab of that
+    many rows / columns, XCD ranges contiguous and in order, no workspace, no fix-up launch; not available together
+    with the GELU epilogue."""
     rng = np.random.default_rng(7)
     cases = [[(137, 512, 256), (401, 512, 256), (0, 512, 256), (59, 512, 256)],
              [(64, 1408, 2048)] * 64,
@@ -291,10 +293,11 @@ def test_small_tile_plan():
                 t[i]["ldb"] = max(n if layout & _lib.GEMM_B_KMAJOR else k, 16)
                 t[i]["ldc"] = max(n, 1)
             grid = 512
-            plan, items, fixups = _lib.plan_grouped_gemm_launch(t.copy(), layout | _lib.GEMM_TILE_128, grid, True)
-            want = {(p, i * 128, j * 128) for p in range(len(t))
-                    for i in range((int(t["m"][p]) + 127) // 128) for j in range((int(t["n"][p]) + 127) // 128)}
-            assert plan.tile == 128 and plan.total_tiles == len(want) and plan.n_slots == 0 and plan.n_fixups == 0
+            plan, items, fixups = _lib.plan_grouped_gemm_launch(t.copy(), layout | flag, grid, True)
+            want = {(p, i * tm, j * tn) for p in range(len(t))
+                    for i in range((int(t["m"][p]) + tm - 1) // tm) for j in range((int(t["n"][p]) + tn - 1) // tn)}
+            assert plan.tile == tn and plan.tile_m == (0 if tm == tn else tm)
+            assert plan.total_tiles == len(want) and plan.n_slots == 0 and plan.n_fixups == 0
             assert len(fixups) == 0
             if not want:
                 continue
@@ -316,11 +319,11 @@ def test_small_tile_plan():
                         if layout & _lib.GEMM_A_KMAJOR:
                             assert r["a"] == 0x10000 + m0 and r["a_bytes"] == (k - 1) * lda + (m - m0)
                         else:
-                            assert r["a"] == 0x10000 + m0 * lda and r["a_bytes"] == (min(m - m0, 128) - 1) * lda + k
+                            assert r["a"] == 0x10000 + m0 * lda and r["a_bytes"] == (min(m - m0, tm) - 1) * lda + k
                         if layout & _lib.GEMM_B_KMAJOR:
                             assert r["b"] == 0x20000 + n0 and r["b_bytes"] == (k - 1) * ldb + (n - n0)
                         else:
-                            assert r["b"] == 0x20000 + n0 * ldb and r["b_bytes"] == (min(n - n0, 128) - 1) * ldb + k
+                            assert r["b"] == 0x20000 + n0 * ldb and r["b_bytes"] == (min(n - n0, tn) - 1) * ldb + k
             assert seen == want
             # the XCD ranges follow the problem order
             last = -1
@@ -328,12 +331,13 @@ def test_small_tile_plan():
                 if x in order:
                     assert min(order[x]) >= last
                     last = max(order[x])
-    # no fused GELU epilogue with the small tile
+    # no fused GELU epilogue with these tiles, and one tile flag at a time
     t, _ = make_table([(256, 256, 128)])
     import ctypes
     plan = _lib.GemmPlan()
-    assert _lib.load().fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 1, _lib.GEMM_TILE_128 | _lib.EPI_GELU, 16, 0,
-                                                       None, 0, None, 0, ctypes.byref(plan)) < 0
+    for bad in (flag | _lib.EPI_GELU, _lib.GEMM_TILE_128 | _lib.GEMM_TILE_DUAL):
+        assert _lib.load().fp8gmm_plan_grouped_gemm_launch(t.ctypes.data, 1, bad, 16, 0, None, 0, None, 0,
+                                                           ctypes.byref(plan)) < 0
 
 
 def test_half_height_flag_marks_the_ragged_last_row_of_tiles():

@@ -433,7 +433,7 @@ def test_random_problem_lists_are_exact(dev):
 def test_random_launches_of_every_form_are_exact(dev, monkeypatch):
     """240 random launches over everything a caller can choose: the four operand layouts (row-major, weights read
     contraction-major, both operands contraction-major, a padded transposed copy with the other operand in place),
-    both gradient formats, the tile size forced either way or left to the launch, tail balancing on and off, bf16
+    both gradient formats, the tile forced to each of its three forms or left to the launch, tail balancing on and off, bf16
     and e4m3 outputs, row counts around the tile edges, contractions of any length.  Exactly summable operands
     ({0, +-0.25 .. +-2}, power-of-two scales): bf16 results must equal torch's fp32 matmul bit for bit, e4m3
     results its saturating cast, and the recorded amax the exact maximum."""
@@ -457,7 +457,7 @@ def test_random_launches_of_every_form_are_exact(dev, monkeypatch):
 
     for trial in range(240):
         form = int(rng.integers(0, 5))
-        monkeypatch.setattr(backend.options, "tile", str(rng.choice(["auto", "128", "256"])))
+        monkeypatch.setattr(backend.options, "tile", str(rng.choice(["auto", "128", "256", "dual"])))
         monkeypatch.setattr(backend.options, "stream_k", bool(rng.integers(0, 2)))
         a_dtype = E5M2 if rng.integers(0, 2) else E4M3
         e = int(rng.integers(1, 12))
