@@ -17,12 +17,14 @@
 // accumulators, one rounding.
 //
 // Layout.  Wavefront (wave_m, wave_n) owns rows wave_m * 64 + 32 i + l32 (i < 2) and columns wave_n * 128 + 32 j ..
-// (j < 4) of the tile; MFMA block (i, j) of set S accumulates in a[16 (4 (i + 2 S) + j) ..+15].  The ring is the
-// one of the large tile (five units of 32 KB); a token unit holds 128 rows x 128 B (contraction-major: 128
-// contraction rows x 128 B) in its LOWER 16 KB, in the layout of the small tile's units.  The upper 16 KB of the unit
-// that holds the NEXT step's tokens are free for the whole step (they were last read as weights three steps
-// earlier and receive weights again one step later): 4 KB per wavefront stage the result pieces, 32 rows x 64
-// columns at a time, so that every store instruction writes whole 128-byte lines.
+// (j < 4) of the tile; MFMA block (i, j) of set S accumulates in a[16 (4 (i + 2 S) + j) ..+15].  LDS holds THREE
+// whole steps: stage t = 16 KB of tokens (128 rows x 128 B, or 128 contraction rows x 128 B, in the layout of the
+// small tile's units) followed by 32 KB of weights (the large tile's unit), 48 KB each, and behind them 4 KB per
+// wavefront that stage the result pieces, 32 rows x 64 columns at a time, so that every store instruction writes
+// whole 128-byte lines.  The smaller steps leave room for a longer run-up than the large tile's two and a half
+// steps: a step's loads are issued two and a half to three steps before it is computed (its first half behind the
+// barrier of the step three before it, which frees the stage; the rest during the low K half of the step two before
+// it).  These launches wait for memory, not for the matrix pipes: what a compute unit has in flight is what it gets.
 #pragma once
 
 namespace fp8gmm {
@@ -59,9 +61,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
     const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int TM = kDualRows, TN = BN;
-  constexpr int US = BN * BK;            // ring unit: 32 KB (a token unit fills the lower half)
-  constexpr int kStageOffset = TM * BK;  // the upper half of a token unit
-  constexpr int kStageBytes = 4096;      // per wavefront: 32 rows x 128 B
+  constexpr int kUnitA = TM * BK, kUnitB = TN * BK;   // 16 KB of tokens, 32 KB of weights
+  constexpr int kStep = kUnitA + kUnitB;              // one stage of the ring: 48 KB
+  constexpr int kStages = 3;
+  constexpr int kPieceOffset = kStages * kStep;       // the result pieces' staging area: the last 16 KB
+  constexpr int kStageBytes = 4096;                   // ... per wavefront: 32 rows x 128 B
+  static_assert(kPieceOffset + NWAVES * kStageBytes == RING * BN * BK, "all of the LDS the large tile has");
   constexpr int MT = 2, NT = 4;          // MFMA blocks of a wavefront's 64 x 128 sub-tile
   constexpr int kPartsA = 4, kPartsB = 8;  // load instructions (1 KB each) per wavefront and unit
 
@@ -175,16 +180,17 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
     rsrc_a[2] = 0;
     rsrc_b[2] = 0;
   };
-  auto dma_a = [&](int unit, int j) {   // j < kPartsA
+  // part j of the tokens / weights of the step the load cursor points at, into stage `stage`
+  auto dma_a = [&](int stage, int j) {   // j < kPartsA
     uint32_t v = a_k + j * a_step;
     if constexpr (!A_TR) v = k_ok ? v : 0xffffffffu;
-    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
+    const uint32_t l = lds_base + stage * kStep + (wave + NWAVES * j) * 1024;
     FP8GMM_DMA(l, v, rsrc_a);
   };
-  auto dma_b = [&](int unit, int j) {   // j < kPartsB
+  auto dma_b = [&](int stage, int j) {   // j < kPartsB
     uint32_t v = b_k + j * b_step;
     if constexpr (!B_TR) v = k_ok ? v : 0xffffffffu;
-    const uint32_t l = lds_base + unit * US + (wave + NWAVES * j) * 1024;
+    const uint32_t l = lds_base + stage * kStep + kUnitA + (wave + NWAVES * j) * 1024;
     FP8GMM_DMA(l, v, rsrc_b);
   };
   auto dma_advance = [&]() {
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
       step_setup();
     }
   };
-  auto ring_inc = [](int x) { return x + 1 == RING ? 0 : x + 1; };
+  auto stage_inc = [](int x) { return x + 1 == kStages ? 0 : x + 1; };
 
   i32x8 fa0[MT], fb0[NT], fa1[MT], fb1[NT];
   typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -240,26 +246,32 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
     half_a(f, unit, i, hh, 1);
   };
 
-  // ---- fill: steps 0 and 1 of the stream into units 0..3, the first fragments into registers ----
+  // ---- fill: steps 0 and 1 of the stream and the first half of step 2's loads; the first fragments into registers ----
+  constexpr int kFirstLoads = kPartsA + 2;                 // of a step's 12 loads: the tokens and two parts of the weights
+  constexpr int kLastLoads = kPartsB - 2;
   load_setup();
 #pragma unroll
   for (int j = 0; j < kPartsA; ++j) dma_a(0, j);
+#pragma unroll
+  for (int j = 0; j < kPartsB; ++j) dma_b(0, j);
+  dma_advance();
+#pragma unroll
+  for (int j = 0; j < kPartsA; ++j) dma_a(1, j);
 #pragma unroll
   for (int j = 0; j < kPartsB; ++j) dma_b(1, j);
   dma_advance();
 #pragma unroll
   for (int j = 0; j < kPartsA; ++j) dma_a(2, j);
-#pragma unroll
-  for (int j = 0; j < kPartsB; ++j) dma_b(3, j);
-  dma_advance();
-  FP8GMM_WAIT_VM(kPartsA + kPartsB);
+  dma_b(2, 0);
+  dma_b(2, 1);
+  FP8GMM_WAIT_VM(kPartsA + kPartsB + kFirstLoads);
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int j = 0; j < NT; ++j) frag_b(fb0[j], lds + US, j, 0);
+  for (int j = 0; j < NT; ++j) frag_b(fb0[j], lds + kUnitA, j, 0);
 #pragma unroll
   for (int i = 0; i < MT; ++i) frag_a(fa0[i], lds, i, 0);
-  int ua = 0;        // ring unit of the current step's tokens
-  int relaxed = 0;   // stores issued at the very end of the previous step: they may stay in flight at the next barrier
+  int cur = 0;       // stage of the current step
+  int relaxed = 0;   // stores that the previous step issued (a lower bound will do): free to stay in flight at the next barrier
 
   asm volatile("" ::: FP8GMM_ALL_ACC_256);   // the accumulation registers belong to the statements of this file
 
@@ -301,7 +313,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
   // pieces [U0, U1) of the waiting tile, one after the other (where no steps are left to carry them)
   auto flush = [&](auto set_c, auto u0_c, auto u1_c) {
     constexpr int U0 = decltype(u0_c)::value, U1 = decltype(u1_c)::value;
-    uint8_t* buf = lds + ua * US + kStageOffset + wave * kStageBytes;   // see the layout note at the top
+    uint8_t* buf = lds + kPieceOffset + wave * kStageBytes;
     static_for<U1 - U0>([&](auto d) {
       constexpr int u = U0 + decltype(d)::value;
       static_for<8>([&](auto qc) { piece_quarter(set_c, std::integral_constant<int, u>{}, qc, buf); });
@@ -334,32 +346,36 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
     constexpr int E = decltype(epi_c)::value;
     constexpr int UL = E == 2 ? 2 : 0, UH = UL + 1;   // the pieces of the low and the high half
     FP8GMM_SB(); FP8GMM_DMF0(0, 0); FP8GMM_SB();
-    const int ub = ring_inc(ua), na = ring_inc(ub), nb = ring_inc(na), fa = ring_inc(nb);
-    [[maybe_unused]] uint8_t* const buf = lds + na * US + kStageOffset + wave * kStageBytes;
+    const int nxt = stage_inc(cur), nn = stage_inc(nxt);
+    [[maybe_unused]] uint8_t* const buf = lds + kPieceOffset + wave * kStageBytes;
     [[maybe_unused]] u32x4 pv[4];
     {
-      // ---- low K half: fragments in fa0 / fb0; the high half's are read from the same units
-      const uint8_t* qa = lds + ua * US;
-      const uint8_t* qb = lds + ub * US;
-      dma_a(fa, 0);
+      // ---- low K half: fragments in fa0 / fb0; the high half's are read from the same stage.  The load cursor
+      // points two steps ahead: the second half of that step's loads goes out (its stage was free since the
+      // previous step's barrier)
+      const uint8_t* qa = lds + cur * kStep;
+      const uint8_t* qb = qa + kUnitA;
+      dma_b(nn, 2);
       frag_b(fb1[0], qb, 0, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 0); FP8GMM_DQ(UL, 1); }
       FP8GMM_SB(); FP8GMM_DMF0(0, 1); FP8GMM_SB();
-      dma_a(fa, 1);
+      dma_b(nn, 3);
       frag_b(fb1[1], qb, 1, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 2); }
       FP8GMM_SB(); FP8GMM_DMF0(0, 2); FP8GMM_SB();
-      dma_a(fa, 2);
+      dma_b(nn, 4);
       frag_b(fb1[2], qb, 2, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 3); }
       FP8GMM_SB(); FP8GMM_DMF0(0, 3); FP8GMM_SB();
-      dma_a(fa, 3);
+      dma_b(nn, 5);
       frag_b(fb1[3], qb, 3, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 4); }
       FP8GMM_SB(); FP8GMM_DMF0(1, 0); FP8GMM_SB();
+      dma_b(nn, 6);
       frag_a(fa1[0], qa, 0, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 5); }
       FP8GMM_SB(); FP8GMM_DMF0(1, 1); FP8GMM_SB();
+      dma_b(nn, 7);
       frag_a(fa1[1], qa, 1, 1);
       if constexpr (E != 0) { FP8GMM_DQ(UL, 6); FP8GMM_DQ(UL, 7); }
       FP8GMM_SB(); FP8GMM_DMF0(1, 2); FP8GMM_SB();
@@ -367,60 +383,59 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
       FP8GMM_SB(); FP8GMM_DMF0(1, 3); FP8GMM_SB();
       if constexpr (E != 0) piece_store(std::integral_constant<int, UL>{}, pv);
     }
-    // ---- the barrier: every wavefront has read this step's units, and the next step's have landed.  Younger than
-    // those loads, and free to stay in flight: the token loads of this half, its piece's stores, and the stores
-    // that the previous step issued behind its last load
+    // ---- the barrier: every wavefront has read this step's stage, and the next step's has landed.  Younger than
+    // the next step's loads, and free to stay in flight: the second half of the loads of the step after it (this
+    // low half's), the first half (the previous step's high half), and the stores of pieces in between
     FP8GMM_SB();
     if (relaxed != 0) {
-      FP8GMM_WAIT_VM_LGKM(kPartsA + (E != 0 ? kDualStores : 0) + kDualStores);
+      FP8GMM_WAIT_VM_LGKM(kFirstLoads + kLastLoads + (E != 0 ? kDualStores : 0) + 2 * kDualStores);
     } else {
-      FP8GMM_WAIT_VM_LGKM(kPartsA + (E != 0 ? kDualStores : 0));
+      FP8GMM_WAIT_VM_LGKM(kFirstLoads + kLastLoads + (E != 0 ? kDualStores : 0));
     }
-    relaxed = E != 0 ? kDualStores : 0;
+    relaxed = E != 0 ? 2 * kDualStores : 0;
     __builtin_amdgcn_s_barrier();
     {
-      // ---- high K half: fragments in fa1 / fb1; the next step's low-half fragments are read from its units
-      const uint8_t* qa = lds + na * US;
-      const uint8_t* qb = lds + nb * US;
+      // ---- high K half: fragments in fa1 / fb1; the next step's low-half fragments are read from its stage.  The
+      // load cursor moves on to the step three ahead, whose stage is the one this barrier has just freed
+      const uint8_t* qa = lds + nxt * kStep;
+      const uint8_t* qb = qa + kUnitA;
       FP8GMM_SB(); FP8GMM_DMF1(0, 0); FP8GMM_SB();
-      dma_b(ua, 0);
-      frag_b(fb0[0], qb, 0, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 0); FP8GMM_DQ(UH, 1); }
-      FP8GMM_SB(); FP8GMM_DMF1(0, 1); FP8GMM_SB();
-      dma_b(ua, 1);
-      frag_b(fb0[1], qb, 1, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 2); }
-      FP8GMM_SB(); FP8GMM_DMF1(0, 2); FP8GMM_SB();
-      dma_b(ua, 2);
-      frag_b(fb0[2], qb, 2, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 3); }
-      FP8GMM_SB(); FP8GMM_DMF1(0, 3); FP8GMM_SB();
-      dma_b(ua, 3);
-      frag_b(fb0[3], qb, 3, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 4); }
-      FP8GMM_SB(); FP8GMM_DMF1(1, 0); FP8GMM_SB();
-      dma_b(ua, 4);
-      frag_a(fa0[0], qa, 0, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 5); }
-      FP8GMM_SB(); FP8GMM_DMF1(1, 1); FP8GMM_SB();
-      dma_b(ua, 5);
-      frag_a(fa0[1], qa, 1, 0);
-      if constexpr (E != 0) { FP8GMM_DQ(UH, 6); FP8GMM_DQ(UH, 7); }
-      FP8GMM_SB(); FP8GMM_DMF1(1, 2); FP8GMM_SB();
-      dma_b(ua, 6);
-      dma_b(ua, 7);
-      if constexpr (E != 0) piece_read_back(pv, buf);
       if constexpr (SAME) {
         ++ld_kt;
         step_setup();
       } else {
         dma_advance();
       }
+      dma_a(cur, 0);
+      frag_b(fb0[0], qb, 0, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 0); FP8GMM_DQ(UH, 1); }
+      FP8GMM_SB(); FP8GMM_DMF1(0, 1); FP8GMM_SB();
+      dma_a(cur, 1);
+      frag_b(fb0[1], qb, 1, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 2); }
+      FP8GMM_SB(); FP8GMM_DMF1(0, 2); FP8GMM_SB();
+      dma_a(cur, 2);
+      frag_b(fb0[2], qb, 2, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 3); }
+      FP8GMM_SB(); FP8GMM_DMF1(0, 3); FP8GMM_SB();
+      dma_a(cur, 3);
+      frag_b(fb0[3], qb, 3, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 4); }
+      FP8GMM_SB(); FP8GMM_DMF1(1, 0); FP8GMM_SB();
+      dma_b(cur, 0);
+      frag_a(fa0[0], qa, 0, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 5); }
+      FP8GMM_SB(); FP8GMM_DMF1(1, 1); FP8GMM_SB();
+      dma_b(cur, 1);
+      frag_a(fa0[1], qa, 1, 0);
+      if constexpr (E != 0) { FP8GMM_DQ(UH, 6); FP8GMM_DQ(UH, 7); }
+      FP8GMM_SB(); FP8GMM_DMF1(1, 2); FP8GMM_SB();
+      if constexpr (E != 0) piece_read_back(pv, buf);
       FP8GMM_SB(); FP8GMM_DMF1(1, 3); FP8GMM_SB();
       if constexpr (E != 0) piece_store(std::integral_constant<int, UH>{}, pv);
       FP8GMM_SB();
     }
-    ua = na;
+    cur = nxt;
   };
 
   // One tile in set S; the tile that waits (pe_on) is in the other set.  Returns false at the end of the list.
@@ -454,10 +469,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
     for (; kt + 3 < nk; ++kt) k_step(T{}, F{}, SetC{}, E0{});
     for (; kt < nk; ++kt) k_step(F{}, F{}, SetC{}, E0{});
     // what the steps could not carry of the waiting tile
-    // (a flush ends with the four stores of its last piece, like a step that carried one)
+    // (`relaxed` stays what it is: the stores of a flush only add to those in flight)
     if (carry && nk == 0) flush(Waiting{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 4>{});
     if (carry && nk == 1) flush(Waiting{}, std::integral_constant<int, 2>{}, std::integral_constant<int, 4>{});
-    if (carry && nk < 2) relaxed = kDualStores;
     // ---- this tile's result: it waits in set S for the next tile's steps, if it can take the staged form
     const int m0 = g.m0, n0 = g.n0;
     const int M = pr.m, N = pr.n;
