@@ -723,8 +723,9 @@ def test_edge_tiles_store_nothing_outside_the_problem(dev, form, monkeypatch):
 @pytest.mark.gpu
 @pytest.mark.parametrize("a_dtype", [E4M3, E5M2], ids=["e4m3", "e5m2"])
 def test_small_tile_gives_the_same_bits_as_the_large_tile(dev, a_dtype, monkeypatch):
-    """The 128 x 128 tile (two workgroups per compute unit) is chosen per launch when the launch is planned; it walks K
-    in the same order with the same MFMA, so every output must equal the 256 x 256 tile's bit for bit: row-major
+    """The 128 x 128 tile (two workgroups per compute unit) and the 128 x 256 tile with two sets of accumulators are
+    chosen per launch when the launch is planned; they walk K in the same order with the same MFMA, so every output
+    must equal the 256 x 256 tile's bit for bit: row-major
     operands, a contraction-major b (data gradient), both contraction-major (weight gradient, ragged K), ragged and
     empty problems, unaligned outputs, an fp8 output with its amax.  Compared with tail balancing off: a large tile
     that is shared along K is the sum of fp32 partial sums, associated differently from the small tile's one running
@@ -733,13 +734,22 @@ def test_small_tile_gives_the_same_bits_as_the_large_tile(dev, a_dtype, monkeypa
     monkeypatch.setattr(backend.options, "stream_k", False)
     g = torch.Generator(device=dev).manual_seed(321)
 
+    def same(x, y):
+        if isinstance(x, tuple):
+            return all(same(p, q) for p, q in zip(x, y))
+        bits = torch.int16 if x.dtype == torch.bfloat16 else torch.uint8 if x.element_size() == 1 else x.dtype
+        return torch.equal(x.view(bits), y.view(bits))
+
     def both(fn):
         out = {}
-        for tile in ("256", "128"):
+        for tile in ("256", "128", "dual"):
             monkeypatch.setattr(backend.options, "tile", tile)
             out[tile] = fn()
         monkeypatch.setattr(backend.options, "tile", "auto")
         auto = fn()
+        # the form with two sets of accumulators (128 x 256 tiles; where a launch cannot take it - an fp8 result -
+        # the large tile runs): the same bits again
+        assert same(out["256"], out["dual"]), "two sets of accumulators"
         return out["256"], out["128"], auto
 
     for sizes, n, k in [([64, 1, 0, 128, 129], 1408, 2048), ([300, 0, 513, 90], 512, 1040), ([1, 15], 16, 16),
