@@ -5,16 +5,16 @@
 //
 // Why: with one set (grouped_gemm_kernel) a workgroup's matrix pipes idle and its ring stays full of the next tile's
 // first steps through every epilogue, and all workgroups of a launch reach their epilogues together, so that the
-// stores come in bursts at the memory system's write bandwidth and nothing moves in between.  Launches with a short
-// contraction (a tile of 4 - 16 steps) spend as long at their tile boundaries as in their steps.  Here a tile's result
-// leaves in 32 pieces spread over the first two steps of the next tile.
+// stores come in bursts and nothing overlaps them (a quarter to a third of a launch with a short contraction).
+// Here a tile's result leaves in four pieces of eight quarters, spread over the first two steps of the next tile.
 //
 // The price: a wavefront's sub-tile is 64 x 128 instead of 128 x 128, so a product needs 1.5 x the fragment reads
-// from LDS and the launch 1.33 x the operand bytes from L2 per flop.  Launches that keep the matrix pipes busy
-// (long contractions) are better off with the large tile; which form a launch takes is decided when it is planned
-// (FP8GMM_GEMM_TILE_DUAL).  bf16 results without a fused epilogue only; whole tiles only (no sharing along K).
-// Every tile gets the same bits as from the other forms: the same products in the same order into fp32
-// accumulators, one rounding.
+// from LDS and 1.5 x the operand bytes through the load path (1.33 x from L2, where neighbouring tiles share).  The
+// load path is what launches with a short contraction wait for most, so the form only pays where the operands come
+// from the memory-side cache rather than from HBM, and never where the matrix pipes are busy (long contractions);
+// which form a launch takes is decided when it is planned (FP8GMM_GEMM_TILE_DUAL).  bf16 results without a fused
+// epilogue only; whole tiles only (no sharing along K).  Every tile gets the same bits as from the other forms: the
+// same products in the same order into fp32 accumulators, one rounding.
 //
 // Layout.  Wavefront (wave_m, wave_n) owns rows wave_m * 64 + 32 i + l32 (i < 2) and columns wave_n * 128 + 32 j ..
 // (j < 4) of the tile; MFMA block (i, j) of set S accumulates in a[16 (4 (i + 2 S) + j) ..+15].  LDS holds THREE

@@ -805,6 +805,71 @@ def test_small_tile_gives_the_same_bits_as_the_large_tile(dev, a_dtype, monkeypa
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("grid", [8, 16])
+def test_two_sets_of_accumulators_on_long_work_lists(dev, grid):
+    """The form with two sets of accumulators (FP8GMM_GEMM_TILE_DUAL) through the C ABI on a grid of 8 / 16 workgroups,
+    so that every workgroup walks a list of a dozen tiles in which everything that can follow anything does: tiles of
+    no K step at all (k = 0: zeros), of one step (the waiting tile's last two pieces are flushed), of two and more
+    (the steps carry all four pieces), results that 16-byte stores can take next to results with an odd pitch or a
+    base address off by one element (written element by element when their tile ends, with no tile left waiting),
+    ragged rows and a column count that ends inside a tile.  Exactly summable operands: every element must equal
+    torch's fp32 matmul bit for bit, and nothing may be written outside a result (guard columns stay NaN)."""
+    import ctypes
+
+    import numpy as np
+
+    from fp8_gmm_amd import _lib
+
+    L = _lib.load()
+    _lib.init(dev.index)
+    vals = torch.tensor([0.0, 0.5, -0.5, 1.0, -1.0, 2.0, -2.0, 0.25], device=dev)
+    g = torch.Generator(device=dev).manual_seed(77 + grid)
+    rng = np.random.default_rng(grid)
+
+    def exact(shape):
+        return vals[torch.randint(0, 8, shape, generator=g, device=dev)].to(E4M3)
+
+    shapes = []
+    for k in (0, 16, 128, 144, 256, 400, 1024):
+        for kind in ("staged", "odd pitch", "odd base"):
+            shapes.append((int(rng.choice([1, 100, 128, 129, 300])), int(rng.choice([256, 272, 520])), k, kind))
+    order = rng.permutation(len(shapes))
+    shapes = [shapes[i] for i in order]
+    e = len(shapes)
+    table = np.zeros(e, dtype=_lib.GEMM_PROBLEM)
+    a_list, b_list, c_list, views = [], [], [], []
+    for i, (m, n, k, kind) in enumerate(shapes):
+        a, b = exact((m, max(k, 16))), exact((n, max(k, 16)))
+        pitch = n + (3 if kind == "odd pitch" else 8)
+        c = torch.full((m, pitch), float("nan"), dtype=torch.bfloat16, device=dev)
+        first = 1 if kind == "odd base" else 0
+        view = c[:, first: first + n]
+        a_list.append(a), b_list.append(b), c_list.append(c), views.append(view)
+        table[i]["a"], table[i]["b"], table[i]["c"] = a.data_ptr(), b.data_ptr(), view.data_ptr()
+        table[i]["m"], table[i]["n"], table[i]["k"] = m, n, k
+        table[i]["lda"] = table[i]["ldb"] = max(k, 16)
+        table[i]["ldc"] = pitch
+    plan, blob, off_items, off_fix = _lib.plan_grouped_gemm_blob(table, _lib.GEMM_TILE_DUAL, grid, False)
+    assert (plan.tile, plan.tile_m, plan.grid, plan.n_fixups) == (256, 128, grid, 0) and plan.rounds > 4
+    dev_blob = torch.from_numpy(blob).to(dev)
+    p = dev_blob.data_ptr()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    _lib.check(L.fp8gmm_grouped_gemm(p, e, p + off_items, None, plan, _lib.E4M3, _lib.E4M3, _lib.OUT_BF16, 0, None, 0,
+                                     stream))
+    # an fp8 result is not something this form has
+    assert L.fp8gmm_grouped_gemm(p, e, p + off_items, None, plan, _lib.E4M3, _lib.E4M3, _lib.E4M3, 0, None, 0, stream) == -6
+    torch.cuda.synchronize()
+    for i, (m, n, k, kind) in enumerate(shapes):
+        want = (a_list[i][:, :k].float() @ b_list[i][:, :k].float().t()).to(torch.bfloat16)
+        got = views[i]
+        assert torch.equal(got.contiguous().view(torch.int16), want.view(torch.int16)), f"problem {i}: {shapes[i]}"
+        guard = torch.ones_like(c_list[i], dtype=torch.bool)
+        first = 1 if kind == "odd base" else 0
+        guard[:, first: first + n] = False
+        assert torch.isnan(c_list[i][guard].float()).all(), f"problem {i}: {shapes[i]} wrote outside its result"
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("tile", ["256", "128"])
 def test_weight_gradient_with_a_transposed_gradient_copy_gives_the_same_bits(dev, tile, monkeypatch):
     """grouped_gemm(..., transposed="b"): a is a zero-padded transposed copy [m, kpad], b the activation slice
