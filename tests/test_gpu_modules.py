@@ -537,8 +537,9 @@ def test_planned_pass_tables_are_those_of_the_per_launch_entry_points(dev, monke
 
     grid = _lib.gemm_grid(_lib.init(torch.cuda.current_device()))
     gs = np.asarray(sizes, dtype=np.int64)
+    policy = {"auto": 0, "256": 256, "128": 128, "dual": _lib.GEMM_TILE_DUAL}[backend.options.tile]   # as backend does
     desc = _lib.LinearPass(experts=e, in_features=k, out_features=n, fwd_fmt=_lib.E4M3, bwd_fmt=_lib.E5M2, cast_weights=1,
-                           dgrad=1, wgrad=1, grid=grid, stream_k=int(backend.options.stream_k), tile_policy=0, tokens=tokens,
+                           dgrad=1, wgrad=1, grid=grid, stream_k=int(backend.options.stream_k), tile_policy=policy, tokens=tokens,
                            group_sizes=gs.ctypes.data, x=x.data_ptr(), x_fp8=x8.data_ptr(), w=w.data_ptr(),
                            w_fp8=w8.data_ptr(), y=y.data_ptr(), dy=dy.data_ptr(), dy_fp8=dy8.data_ptr(), dx=dx.data_ptr(),
                            dw=dw.data_ptr(), fwd_scale=fs.data_ptr(), fwd_scale_inv=fsi.data_ptr(), fwd_amax=fa.data_ptr(),
@@ -670,8 +671,9 @@ def test_planned_mlp_pass_tables_are_those_of_the_per_launch_entry_points(dev, m
 
     grid = _lib.gemm_grid(_lib.init(torch.cuda.current_device()))
     gs = np.asarray(sizes, dtype=np.int64)
+    policy = {"auto": 0, "256": 256, "128": 128, "dual": _lib.GEMM_TILE_DUAL}[backend.options.tile]   # as backend does
     desc = _lib.MlpPass(experts=e, hidden=h, ffn=f, fwd_fmt=_lib.E4M3, bwd_fmt=_lib.E5M2, cast_weights=1, dgrad=1, wgrad=1,
-                        grid=grid, stream_k=int(backend.options.stream_k), tile_policy=0, tokens=tokens,
+                        grid=grid, stream_k=int(backend.options.stream_k), tile_policy=policy, tokens=tokens,
                         group_sizes=gs.ctypes.data, x=x.data_ptr(), x_fp8=x8.data_ptr(), w1=w1.data_ptr(),
                         w1_fp8=w18.data_ptr(), w2=w2.data_ptr(), w2_fp8=w28.data_ptr(), pre=pre.data_ptr(),
                         act_fp8=act8.data_ptr(), y=y.data_ptr(), dy=dy.data_ptr(), dy_fp8=dy8.data_ptr(),
