@@ -141,6 +141,18 @@ class MlpPass(ctypes.Structure):
             "dx", "dw1", "dw2", "fwd_scale", "fwd_scale_inv", "fwd_amax", "bwd_scale", "bwd_scale_inv", "bwd_amax")]
 
 
+class ScalingUpdate(ctypes.Structure):
+    """struct fp8gmm_scaling_update"""
+
+    _fields_ = [("amax_history", ctypes.c_void_p), ("scale", ctypes.c_void_p), ("scale_inv", ctypes.c_void_p),
+                ("history_len", ctypes.c_int32), ("slots", ctypes.c_int32), ("fp8_max", ctypes.c_float),
+                ("margin", ctypes.c_int32), ("most_recent", ctypes.c_int32), ("keep_period", ctypes.c_int32),
+                ("keep_phase", ctypes.c_int32), ("reserved", ctypes.c_int32)]
+
+
+MAX_SCALING_UPDATES = 4
+
+
 class PassLaunch(ctypes.Structure):
     """struct fp8gmm_pass_launch"""
 
@@ -178,6 +190,7 @@ EXPORTS = (
     "fp8gmm_plan_mlp_backward",
     "fp8gmm_sizeof_mlp_pass",
     "fp8gmm_run_planned",
+    "fp8gmm_delayed_scaling_updates",
     "fp8gmm_sizeof_linear_pass",
     "fp8gmm_sizeof_pass_plan",
     "fp8gmm_gemm_tile_shape",
@@ -284,6 +297,8 @@ def load():
     L.fp8gmm_sizeof_pass_plan.argtypes = []
     L.fp8gmm_delayed_scaling_update.restype = ci
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
+    L.fp8gmm_delayed_scaling_updates.restype = ci
+    L.fp8gmm_delayed_scaling_updates.argtypes = [ctypes.POINTER(ScalingUpdate), ci, vp]
     L.fp8gmm_upload.restype = ci
     L.fp8gmm_upload.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t
@@ -305,7 +320,7 @@ def load():
     if L.fp8gmm_sizeof_tensor_desc() != TENSOR_DESC.itemsize or L.fp8gmm_sizeof_gemm_problem() != GEMM_PROBLEM.itemsize \
             or L.fp8gmm_sizeof_gemm_item() != GEMM_ITEM.itemsize or ctypes.sizeof(GemmPlan) != 32 \
             or L.fp8gmm_sizeof_linear_pass() != ctypes.sizeof(LinearPass) \
-            or L.fp8gmm_sizeof_mlp_pass() != ctypes.sizeof(MlpPass) \
+            or L.fp8gmm_sizeof_mlp_pass() != ctypes.sizeof(MlpPass) or ctypes.sizeof(ScalingUpdate) != 56 \
             or L.fp8gmm_sizeof_pass_plan() != ctypes.sizeof(PassPlan):
         raise ImportError("struct layout mismatch between fp8_gmm_amd/_lib.py and include/fp8gmm.h")
     _lib = L

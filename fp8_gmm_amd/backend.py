@@ -1007,6 +1007,35 @@ def delayed_scaling_update(amax_history, scale, scale_inv, fp8_max, margin=0, mo
     _lib.check(rc)
 
 
+def delayed_scaling_updates(updates):
+    """Several ``delayed_scaling_update`` calls (tuples of its arguments, all tensors on one device) in ONE kernel
+    launch: a module's forward and backward scaling state in front of every step."""
+    if not updates:
+        return
+    if len(updates) > _lib.MAX_SCALING_UPDATES:
+        _fail(f"fp8_gmm_amd: at most {_lib.MAX_SCALING_UPDATES} scaling updates per launch")
+    table = (_lib.ScalingUpdate * len(updates))()
+    tensors = []
+    for u, args in zip(table, updates):
+        amax_history, scale, scale_inv, fp8_max = args[:4]
+        margin, most_recent, keep = (tuple(args[4:]) + (0, False, None)[len(args) - 4:])[:3]
+        for t, what in ((amax_history, "amax_history"), (scale, "scale"), (scale_inv, "scale_inv")):
+            if t.dtype != torch.float32 or not t.is_contiguous():
+                _fail(f"fp8_gmm_amd: {what} must be a contiguous fp32 tensor")
+        if amax_history.dim() != 2 or scale.numel() != amax_history.shape[1] or scale_inv.numel() != scale.numel():
+            _fail("fp8_gmm_amd: amax_history must be [history, slots] and scale / scale_inv [slots]")
+        period, phase = keep if keep is not None else (0, 0)
+        u.amax_history, u.scale, u.scale_inv = amax_history.data_ptr(), scale.data_ptr(), scale_inv.data_ptr()
+        u.history_len, u.slots = amax_history.shape
+        u.fp8_max, u.margin, u.most_recent = float(fp8_max), int(margin), int(bool(most_recent))
+        u.keep_period, u.keep_phase = int(period), int(phase)
+        tensors += [amax_history, scale, scale_inv]
+    dev = _device_of(tensors)
+    with _on_device(dev):
+        rc = _lib.load().fp8gmm_delayed_scaling_updates(table, len(updates), _stream(dev))
+    _lib.check(rc)
+
+
 def grouped_gemm(a_list, b_list, c_list, a_scale_invs, b_scale_invs, pre_gelu_outs=None, c_scales=None,
                  c_amaxes=None, transposed=False):
     """c_list[i][m, n] = epilogue(a_list[i][m, k] . b_list[i][n, k]^T) for all i in ONE launch.

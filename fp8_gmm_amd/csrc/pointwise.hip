@@ -159,13 +159,10 @@ __global__ __launch_bounds__(kPwThreads) void multi_scale_mul_kernel(const fp8gm
 //   history   : row i <- row i + 1, last row <- old row 0, then row 0 <- 0 (a history of one row is just cleared)
 // The factor is formed as reciprocal times fp8_max, which is what `fp8_max / amax` on a torch tensor
 // evaluates to; the two differ in the last bit for some inputs.
-__global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __restrict__ history,
-                                                                     float* __restrict__ scale,
-                                                                     float* __restrict__ scale_inv, int history_len,
-                                                                     int slots, float fp8_max, float margin_factor,
-                                                                     int most_recent, int keep_period,
-                                                                     int keep_phase) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+__device__ __forceinline__ void delayed_scaling_update_column(float* __restrict__ history, float* __restrict__ scale,
+                                                               float* __restrict__ scale_inv, int history_len, int slots,
+                                                               float fp8_max, float margin_factor, int most_recent,
+                                                               int keep_period, int keep_phase, int c) {
   if (c >= slots) return;
   float* col = history + c;
   const float first = col[0];
@@ -194,6 +191,33 @@ __global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __re
   if (!(keep_period > 0 && c % keep_period == keep_phase)) scale_inv[c] = 1.0f / sc;
   if (history_len > 1) col[(size_t)(history_len - 1) * slots] = first;
   col[0] = 0.f;
+}
+
+__global__ __launch_bounds__(256) void delayed_scaling_update_kernel(float* __restrict__ history,
+                                                                     float* __restrict__ scale,
+                                                                     float* __restrict__ scale_inv, int history_len,
+                                                                     int slots, float fp8_max, float margin_factor,
+                                                                     int most_recent, int keep_period,
+                                                                     int keep_phase) {
+  delayed_scaling_update_column(history, scale, scale_inv, history_len, slots, fp8_max, margin_factor, most_recent,
+                                keep_period, keep_phase, blockIdx.x * blockDim.x + threadIdx.x);
+}
+
+// Several directions (a module's forward and backward scaling state) in one launch: the workgroups of update u
+// follow those of update u - 1.  The updates travel as a kernel argument.
+struct ScalingUpdates {
+  fp8gmm_scaling_update u[FP8GMM_MAX_SCALING_UPDATES];
+  float margin_factor[FP8GMM_MAX_SCALING_UPDATES];
+  int first_block[FP8GMM_MAX_SCALING_UPDATES + 1];
+  int n;
+};
+__global__ __launch_bounds__(256) void delayed_scaling_updates_kernel(const ScalingUpdates all) {
+  int i = 0;
+  while (i + 1 < all.n && (int)blockIdx.x >= all.first_block[i + 1]) ++i;
+  const fp8gmm_scaling_update& u = all.u[i];
+  delayed_scaling_update_column(u.amax_history, u.scale, u.scale_inv, u.history_len, u.slots, u.fp8_max,
+                                all.margin_factor[i], u.most_recent, u.keep_period, u.keep_phase,
+                                ((int)blockIdx.x - all.first_block[i]) * (int)blockDim.x + (int)threadIdx.x);
 }
 
 }  // namespace
@@ -244,6 +268,32 @@ int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scal
   hipLaunchKernelGGL(fp8gmm::delayed_scaling_update_kernel, dim3((slots + 255) / 256), dim3(256), 0,
                      static_cast<hipStream_t>(stream), amax_history, scale, scale_inv, history_len, slots, fp8_max,
                      margin_factor, most_recent != 0, keep_period, keep_phase);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_delayed_scaling_updates(const fp8gmm_scaling_update* updates, int n, void* stream) {
+  if (n < 0 || n > FP8GMM_MAX_SCALING_UPDATES) return FP8GMM_ERR_BAD_ARGUMENT;
+  if (n == 0) return FP8GMM_OK;
+  if (updates == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  fp8gmm::ScalingUpdates all{};
+  int blocks = 0;
+  for (int i = 0; i < n; ++i) {
+    const fp8gmm_scaling_update& u = updates[i];
+    if (u.history_len < 1 || u.slots < 0 || u.margin < -126 || u.margin > 126) return FP8GMM_ERR_BAD_ARGUMENT;
+    if (u.keep_period < 0 || (u.keep_period > 0 && (u.keep_phase < 0 || u.keep_phase >= u.keep_period)))
+      return FP8GMM_ERR_BAD_ARGUMENT;
+    if (u.slots > 0 && (u.amax_history == nullptr || u.scale == nullptr || u.scale_inv == nullptr))
+      return FP8GMM_ERR_NULL_POINTER;
+    all.u[i] = u;
+    all.margin_factor[i] = __builtin_ldexpf(1.0f, -u.margin);
+    all.first_block[i] = blocks;
+    blocks += (u.slots + 255) / 256;
+  }
+  all.first_block[n] = blocks;
+  all.n = n;
+  if (blocks == 0) return FP8GMM_OK;
+  hipLaunchKernelGGL(fp8gmm::delayed_scaling_updates_kernel, dim3(blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     all);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 

@@ -229,11 +229,20 @@ class Fp8GroupedModuleBase(torch.nn.Module):
         self._apply_pending_state()
         if self.training and torch.is_grad_enabled():
             if self._fp8_steps > 0 and self._fp8_steps % fp8_recipe.interval == 0:
+                fwd, bwd = self.fp8_meta["scaling_fwd"], self.fp8_meta["scaling_bwd"]
+                keep = None if update_weights else (self.FWD_SLOTS_PER_GEMM, self.WEIGHT_SLOT)
                 with torch.no_grad():
-                    amax_and_scale_update(
-                        self.fp8_meta["scaling_fwd"], self.fp8_meta["fp8_max_fwd"], fp8_recipe,
-                        None if update_weights else (self.FWD_SLOTS_PER_GEMM, self.WEIGHT_SLOT))
-                    amax_and_scale_update(self.fp8_meta["scaling_bwd"], self.fp8_meta["fp8_max_bwd"], fp8_recipe)
+                    if fwd.amax_history.is_cuda and float(fp8_recipe.margin) == int(fp8_recipe.margin):
+                        # both directions in one kernel launch (the rule is amax_and_scale_update's)
+                        from . import backend
+
+                        margin, recent = int(fp8_recipe.margin), fp8_recipe.amax_compute_algo != "max"
+                        backend.delayed_scaling_updates([
+                            (fwd.amax_history, fwd.scale, fwd.scale_inv, self.fp8_meta["fp8_max_fwd"], margin, recent, keep),
+                            (bwd.amax_history, bwd.scale, bwd.scale_inv, self.fp8_meta["fp8_max_bwd"], margin, recent)])
+                    else:
+                        amax_and_scale_update(fwd, self.fp8_meta["fp8_max_fwd"], fp8_recipe, keep)
+                        amax_and_scale_update(bwd, self.fp8_meta["fp8_max_bwd"], fp8_recipe)
             self._fp8_steps += 1
         yield
 

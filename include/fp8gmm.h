@@ -477,6 +477,20 @@ int fp8gmm_delayed_scaling_update(float* amax_history, float* scale, float* scal
                                   float fp8_max, int margin, int most_recent, int keep_period, int keep_phase,
                                   void* stream);
 
+/* The same for up to FP8GMM_MAX_SCALING_UPDATES directions in ONE launch (a module's forward and backward state are
+ * updated at the same point, in front of a forward pass: one kernel instead of two per step).  `updates` is a HOST
+ * array; its contents travel as a kernel argument. */
+#define FP8GMM_MAX_SCALING_UPDATES 4
+typedef struct fp8gmm_scaling_update {
+  float* amax_history;   /* [history_len, slots] */
+  float* scale;          /* [slots] */
+  float* scale_inv;      /* [slots] */
+  int32_t history_len, slots;
+  float fp8_max;
+  int32_t margin, most_recent, keep_period, keep_phase, reserved;
+} fp8gmm_scaling_update;   /* 56 bytes */
+int fp8gmm_delayed_scaling_updates(const fp8gmm_scaling_update* updates, int n, void* stream);
+
 /*
  * Copy `bytes` of tables from page-locked host memory that the device can address (hipHostMalloc; torch's
  * pin_memory) to device memory with a kernel on `stream`: dst_dev, src_host and bytes multiples of 16, at most

@@ -360,6 +360,41 @@ def test_delayed_scaling_update_matches_the_torch_rule(dev, history_len, slots, 
         gpu.amax_history[0] += bump.to(dev)
 
 
+def test_several_scaling_updates_in_one_launch_equal_one_launch_each(dev):
+    """fp8gmm_delayed_scaling_updates: up to four directions in one kernel launch (a module's forward and backward
+    state go together) must leave every tensor exactly as one launch per direction does: different history
+    lengths and slot counts (more than one workgroup's worth, and none), margins, both amax rules, a kept
+    scale_inv phase; a fifth update is refused."""
+    from fp8_gmm_amd import fp8
+
+    backend = _backend()
+    g = gen(88)
+    specs = [(16, 771, 448.0, 0, False, (3, 1)), (1, 5, 57344.0, 2, True, None), (7, 0, 448.0, 0, False, None),
+             (1024, 130, 57344.0, 1, False, None)]
+    single, together = [], []
+    for history_len, slots, fp8_max, margin, recent, keep in specs:
+        hist = torch.rand(history_len, slots, generator=g) * 10.0 ** torch.randint(-6, 6, (1, slots), generator=g).float()
+        if slots > 3:
+            hist[:, 0], hist[0, 1], hist[history_len // 2, 2] = 0.0, float("inf"), float("nan")
+        scale, scale_inv = torch.rand(slots, generator=g) + 0.5, torch.rand(slots, generator=g) + 0.5
+        for group in (single, together):
+            group.append((hist.to(dev), scale.to(dev), scale_inv.to(dev), fp8_max, margin, recent, keep))
+    for step in range(2):
+        for args in single:
+            backend.delayed_scaling_update(*args[:6], keep_scale_inv=args[6])
+        backend.delayed_scaling_updates(together)
+        for i, (a, b) in enumerate(zip(single, together)):
+            for t, u, name in zip(a[:3], b[:3], ("amax_history", "scale", "scale_inv")):
+                assert torch.equal(t.view(torch.int32), u.view(torch.int32)), f"update {i} {name} at step {step}"
+        for a, b in zip(single, together):
+            if a[0].shape[1]:
+                bump = torch.rand(a[0].shape[1], generator=g).to(dev)
+                a[0][0] += bump
+                b[0][0] += bump
+    with pytest.raises(RuntimeError):
+        backend.delayed_scaling_updates(together + together[:1])
+
+
 def test_tables_reach_the_device_through_the_staging_memory(dev, monkeypatch):
     """Tables are written into page-locked staging memory and copied by a kernel of the library (fp8gmm_upload).
     With the staging area shrunk to 2 x 8 KiB its halves are reused every few uploads: every device copy must hold
