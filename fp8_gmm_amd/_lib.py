@@ -159,8 +159,9 @@ class PassLaunch(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int32), ("op", ctypes.c_int32), ("n", ctypes.c_int32),
                 ("total_blocks", ctypes.c_int32), ("out_fmt", ctypes.c_int32), ("a_fmt", ctypes.c_int32),
                 ("b_fmt", ctypes.c_int32), ("out_kind", ctypes.c_int32), ("epilogue", ctypes.c_int32),
-                ("reserved", ctypes.c_int32), ("table_offset", ctypes.c_int64), ("items_offset", ctypes.c_int64),
-                ("fixups_offset", ctypes.c_int64), ("plan", GemmPlan), ("work", ctypes.c_double),
+                ("merge_n", ctypes.c_int32), ("table_offset", ctypes.c_int64), ("items_offset", ctypes.c_int64),
+                ("fixups_offset", ctypes.c_int64), ("merge_offset", ctypes.c_int64), ("plan", GemmPlan),
+                ("work", ctypes.c_double),
                 ("bytes", ctypes.c_double)]
 
 

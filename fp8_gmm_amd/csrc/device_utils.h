@@ -162,13 +162,18 @@ __device__ __forceinline__ void block_amax_merge(float local, uint32_t* target, 
 }
 
 // Second pass of the calls that record amax: one lane per tensor merges the tensor's partial into the
-// caller's slot.  n atomics in total, against one per workgroup of the main kernel.
+// caller's slot.  n atomics in total, against one per workgroup of the main kernel.  Run by a launch of its own
+// behind the cast, or - inside a planned pass - by the first workgroup of the GEMM launch that follows the cast.
+__device__ __forceinline__ void merge_amax_partials(const fp8gmm_tensor_desc* __restrict__ descs, int n, int first,
+                                                    int stride) {
+  for (int i = first; i < n; i += stride) {
+    const float p = __builtin_bit_cast(float, descs[i].amax_partial);
+    float* amax = descs[i].amax;
+    if (amax != nullptr && p > 0.f) atomic_max_nonneg(amax, p);
+  }
+}
 [[maybe_unused]] static __global__ __launch_bounds__(256) void amax_merge_kernel(const fp8gmm_tensor_desc* __restrict__ descs, int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float p = __builtin_bit_cast(float, descs[i].amax_partial);
-  float* amax = descs[i].amax;
-  if (amax != nullptr && p > 0.f) atomic_max_nonneg(amax, p);
+  merge_amax_partials(descs, n, blockIdx.x * blockDim.x + threadIdx.x, gridDim.x * blockDim.x);
 }
 
 // exp(-2a) and 1 / (1 + exp(-2a)) for a >= 0, from a fixed sequence of IEEE single-precision operations (add, mul,

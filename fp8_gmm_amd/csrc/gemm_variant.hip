@@ -14,7 +14,7 @@ namespace fp8gmm {
 #define FP8GMM_INSTANTIATE(AF, BF, AT, BT, TL)                                                                     \
   template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                           \
   template int launch_variant<AF, BF, AT, BT, TL>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, \
-                                                  uint8_t*, hipStream_t);
+                                                  uint8_t*, const fp8gmm_tensor_desc*, int, hipStream_t);
 
 #define FP8GMM_V0 FP8GMM_INSTANTIATE(FP8GMM_E4M3, FP8GMM_E4M3, false, false, 256)
 #define FP8GMM_V1 FP8GMM_INSTANTIATE(FP8GMM_E5M2, FP8GMM_E4M3, false, false, 256)

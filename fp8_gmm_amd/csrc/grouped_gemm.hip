@@ -5,6 +5,7 @@
 // (fp8_gmm/backend.py:84-96, grouped_linear.py:173-182, grouped_mlp.py:234-242,313-322) with ONE launch over
 // device-side tables written by the host planner (plan.cpp).
 #include "grouped_gemm_kernel.h"
+#include "internal.h"
 
 // Scratch of fp8gmm_grouped_gemm_static: the tail-balancing workspace for callers that cannot allocate one.
 // Every GPU the library runs on holds its own copy of this array, at its own address, until the process ends.
@@ -176,7 +177,8 @@ int scratch_for(int dev, uint8_t** out) {
   return FP8GMM_OK;
 }
 
-typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*, hipStream_t);
+typedef int (*launch_fn)(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, int, uint8_t*,
+                         const fp8gmm_tensor_desc*, int, hipStream_t);
 
 // the variant for a format / layout combination, or null when the combination does not exist
 launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor, int tile) {
@@ -190,8 +192,10 @@ launch_fn variant_for(int a_fmt, int b_fmt, bool a_kmajor, bool b_kmajor, int ti
 
 int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
                    const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
-                   int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream) {
+                   int out_kind, int epilogue, void* workspace, size_t workspace_bytes, void* stream,
+                   const fp8gmm_tensor_desc* merge_descs = nullptr, int merge_n = 0) {
   if (plan == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  if (merge_n < 0 || (merge_n > 0 && merge_descs == nullptr)) return FP8GMM_ERR_BAD_ARGUMENT;
   if (n < 0 || plan->total_tiles < 0 || plan->rounds < 0 || plan->n_fixups < 0 || plan->n_slots < 0)
     return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_kind != FP8GMM_OUT_BF16 && out_kind != FP8GMM_E4M3 && out_kind != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
@@ -219,7 +223,7 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
     return FP8GMM_ERR_BAD_ARGUMENT;
   const launch_fn launch = variant_for(a_fmt, b_fmt, a_kmajor, b_kmajor, tile);
   if (launch == nullptr) return FP8GMM_ERR_BAD_FORMAT;
-  if (n == 0 || plan->total_tiles == 0) return FP8GMM_OK;
+  if (n == 0 || plan->total_tiles == 0) return merge_n > 0 ? FP8GMM_ERR_BAD_ARGUMENT : FP8GMM_OK;   // nothing would merge
   if (plan->grid <= 0 || (plan->grid % kNumXcd) != 0 || plan->rounds < 1) return FP8GMM_ERR_BAD_ARGUMENT;
   if (probs_dev == nullptr || items_dev == nullptr || (plan->n_fixups > 0 && fixups_dev == nullptr))
     return FP8GMM_ERR_NULL_POINTER;
@@ -228,7 +232,7 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
     return FP8GMM_ERR_WORKSPACE;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int rc = launch(probs_dev, items_dev, plan->grid, out_kind, epilogue & (FP8GMM_EPI_GELU | FP8GMM_EPI_DGELU),
-                        static_cast<uint8_t*>(workspace), s);
+                        static_cast<uint8_t*>(workspace), merge_descs, merge_n, s);
   if (rc != FP8GMM_OK) return rc;
   if (plan->n_fixups > 0) {
     hipLaunchKernelGGL(grouped_gemm_fixup_kernel, dim3(plan->n_fixups * kFixupSplit), dim3(kFixupThreads), 0, s, probs_dev,
@@ -240,6 +244,15 @@ int launch_checked(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gem
 }
 
 }  // namespace
+
+int launch_gemm_merging(const fp8gmm_gemm_problem* probs_dev, int n, const fp8gmm_gemm_item* items_dev,
+                        const fp8gmm_gemm_fixup_desc* fixups_dev, const fp8gmm_gemm_plan* plan, int a_fmt, int b_fmt,
+                        int out_kind, int epilogue, void* workspace, size_t workspace_bytes,
+                        const fp8gmm_tensor_desc* merge_descs, int merge_n, void* stream) {
+  return launch_checked(probs_dev, n, items_dev, fixups_dev, plan, a_fmt, b_fmt, out_kind, epilogue, workspace,
+                        workspace_bytes, stream, merge_descs, merge_n);
+}
+
 }  // namespace fp8gmm
 
 extern "C" {

@@ -58,8 +58,10 @@ __device__ __forceinline__ f32x4 acc_quad() {   // four consecutive accumulators
 
 template <int A_FMT, int B_FMT, bool A_TR, bool B_TR>
 __global__ __launch_bounds__(NTHREADS, 1) void grouped_gemm_dual_kernel(
-    const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items) {
+    const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items,
+    const fp8gmm_tensor_desc* __restrict__ merge_descs, int merge_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  if (merge_n > 0 && blockIdx.x == 0) merge_amax_partials(merge_descs, merge_n, threadIdx.x, NTHREADS);
   constexpr int TM = kDualRows, TN = BN;
   constexpr int kUnitA = TM * BK, kUnitB = TN * BK;   // 16 KB of tokens, 32 KB of weights
   constexpr int kStep = kUnitA + kUnitB;              // one stage of the ring: 48 KB

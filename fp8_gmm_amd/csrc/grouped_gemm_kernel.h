@@ -637,8 +637,10 @@ static_assert(offsetof(fp8gmm_gemm_item, k) == 32 && offsetof(fp8gmm_gemm_item, 
 template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 __global__ __launch_bounds__(NTHREADS, TILE == 256 ? 1 : 2) void grouped_gemm_kernel(
     const fp8gmm_gemm_problem* __restrict__ probs, const fp8gmm_gemm_item* __restrict__ items, int out_kind,
-    int epilogue, uint8_t* __restrict__ workspace) {
+    int epilogue, uint8_t* __restrict__ workspace, const fp8gmm_tensor_desc* __restrict__ merge_descs, int merge_n) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // the amax merge of the cast launch in front of this one, where the pass planner has moved it here
+  if (merge_n > 0 && blockIdx.x == 0) merge_amax_partials(merge_descs, merge_n, threadIdx.x, NTHREADS);
   // the tile's extents shadow the namespace's (which are those of the 256 x 256 tile)
   [[maybe_unused]] constexpr int BM = TILE;
   constexpr int BN = TILE, US = TILE * BK, WM = TILE / 2, WN = TILE / 2, MT = WM / 32, NT = WN / 32;
@@ -1308,7 +1310,8 @@ int prepare_variant(int dev) {
 
 template <int A_FMT, int B_FMT, bool A_TR, bool B_TR, int TILE>
 int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item* items_dev, int grid, int out_kind,
-                   int epilogue, uint8_t* workspace, hipStream_t stream) {
+                   int epilogue, uint8_t* workspace, const fp8gmm_tensor_desc* merge_descs, int merge_n,
+                   hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return FP8GMM_ERR_NO_DEVICE;
   const int rc = prepare_variant<A_FMT, B_FMT, A_TR, B_TR, TILE>(dev);
@@ -1316,10 +1319,10 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item*
   if constexpr (TILE == kTileDual) {
     // bf16 results without a fused epilogue only (the caller has checked)
     hipLaunchKernelGGL((grouped_gemm_dual_kernel<A_FMT, B_FMT, A_TR, B_TR>), dim3(grid), dim3(NTHREADS), RING * BN * BK,
-                       stream, probs_dev, items_dev);
+                       stream, probs_dev, items_dev, merge_descs, merge_n);
   } else {
     hipLaunchKernelGGL((grouped_gemm_kernel<A_FMT, B_FMT, A_TR, B_TR, TILE>), dim3(grid), dim3(NTHREADS),
-                       RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace);
+                       RING * TILE * BK, stream, probs_dev, items_dev, out_kind, epilogue, workspace, merge_descs, merge_n);
   }
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
@@ -1352,7 +1355,7 @@ int launch_variant(const fp8gmm_gemm_problem* probs_dev, const fp8gmm_gemm_item*
 #define FP8GMM_DECLARE_VARIANT(AF, BF, AT, BT, TL)                                                                     \
   extern template int prepare_variant<AF, BF, AT, BT, TL>(int);                                                        \
   extern template int launch_variant<AF, BF, AT, BT, TL>(const fp8gmm_gemm_problem*, const fp8gmm_gemm_item*, int, int, \
-                                                         int, uint8_t*, hipStream_t);
+                                                         int, uint8_t*, const fp8gmm_tensor_desc*, int, hipStream_t);
 #ifndef FP8GMM_VARIANT_INDEX
 FP8GMM_FOR_EACH_GEMM_VARIANT(FP8GMM_DECLARE_VARIANT)
 #endif

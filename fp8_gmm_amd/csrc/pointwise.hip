@@ -8,6 +8,7 @@
 // (one 128-bit load per lane, all steps issued before the first conversion), the wave reduces amax with cross-lane shuffles and the
 // workgroup issues a single integer atomic max.
 #include "device_utils.h"
+#include "internal.h"
 #include "tiling.h"
 
 namespace fp8gmm {
@@ -225,7 +226,7 @@ __global__ __launch_bounds__(256) void delayed_scaling_updates_kernel(const Scal
 
 namespace {
 template <bool DGELU>
-int launch_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream) {
+int launch_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, void* stream, bool merge = true) {
   if (n < 0 || total_blocks < 0) return FP8GMM_ERR_BAD_ARGUMENT;
   if (out_fmt != FP8GMM_E4M3 && out_fmt != FP8GMM_E5M2) return FP8GMM_ERR_BAD_FORMAT;
   if (n == 0 || total_blocks == 0) return FP8GMM_OK;
@@ -237,10 +238,17 @@ int launch_quantize(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int 
   else
     hipLaunchKernelGGL((fp8gmm::multi_quantize_kernel<FP8GMM_E5M2, DGELU>), dim3(total_blocks),
                        dim3(fp8gmm::kPwThreads), 0, s, descs_dev, n);
-  hipLaunchKernelGGL(fp8gmm::amax_merge_kernel, dim3((n + 255) / 256), dim3(256), 0, s, descs_dev, n);
+  if (merge) hipLaunchKernelGGL(fp8gmm::amax_merge_kernel, dim3((n + 255) / 256), dim3(256), 0, s, descs_dev, n);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 }  // namespace
+
+namespace fp8gmm {
+int launch_cast_unmerged(fp8gmm_tensor_desc* descs_dev, int n, int total_blocks, int out_fmt, bool dgelu, void* stream) {
+  return dgelu ? launch_quantize<true>(descs_dev, n, total_blocks, out_fmt, stream, false)
+               : launch_quantize<false>(descs_dev, n, total_blocks, out_fmt, stream, false);
+}
+}  // namespace fp8gmm
 
 namespace fp8gmm {
 // Tables travel host -> device through this kernel: it reads page-locked host memory that is mapped into the

@@ -384,10 +384,12 @@ typedef struct fp8gmm_pass_launch {
   int32_t total_blocks;          /* cast: workgroups */
   int32_t out_fmt;               /* cast: fp8 format written */
   int32_t a_fmt, b_fmt, out_kind, epilogue;   /* GEMM: the arguments of fp8gmm_grouped_gemm */
-  int32_t reserved;
+  int32_t merge_n;               /* cast: != 0: its amax merge is left to the GEMM launch behind it, whose first
+                                    workgroup runs it.  GEMM: descriptors of the cast in front whose merge it runs (0: none) */
   int64_t table_offset;          /* descriptors / problem table */
   int64_t items_offset;          /* GEMM: work list */
   int64_t fixups_offset;         /* GEMM: shared-tile records */
+  int64_t merge_offset;          /* GEMM with merge_n != 0: the descriptors of that cast */
   fp8gmm_gemm_plan plan;         /* GEMM */
   double work;                   /* algorithmic flops (GEMM) or bytes (cast) of the launch */
   double bytes;                  /* algorithmic bytes: every operand read once, every result written once */

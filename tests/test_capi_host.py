@@ -339,6 +339,10 @@ def test_mlp_pass_planner_lays_out_the_reference_data_flow():
                   slot("fwd_scale_inv", 0, 3))
     kk = _lib.GEMM_A_KMAJOR | _lib.GEMM_B_KMAJOR
     assert [plan.launch[i].epilogue for i in (1, 2, 4, 5)] == [kk, _lib.GEMM_B_KMAJOR, _lib.GEMM_B_KMAJOR, kk]
+    # a cast leaves the merge of its running maxima to the GEMM launch right behind it, which finds the cast's table
+    assert [plan.launch[i].merge_n for i in range(6)] == [e, e, 0, e, e, 0]
+    assert plan.launch[1].merge_offset == plan.launch[0].table_offset
+    assert plan.launch[4].merge_offset == plan.launch[3].table_offset
     assert [(plan.launch[i].a_fmt, plan.launch[i].b_fmt) for i in (1, 2, 4, 5)] == [(_lib.E5M2, _lib.E4M3)] * 4
     assert plan.launch[3].bytes == float((m * f * 5).sum()) and plan.launch[3].out_fmt == _lib.E5M2
     # every table on its own cache line, none overlapping the next
@@ -376,6 +380,7 @@ def test_mlp_pass_planner_options_and_errors():
     d, _, _ = _mlp_pass([0, 0], h, f)
     assert run(bwd, d) == 0 and [plan.launch[i].kind for i in range(plan.n_launches)] == [0, _lib.PASS_GEMM, 0, 0, 0, _lib.PASS_GEMM]
     assert run(fwd, d) == 0 and [plan.launch[i].kind for i in range(3)] == [_lib.PASS_CAST, 0, 0]   # the weights
+    assert plan.launch[0].merge_n == 0   # ... whose cast merges its own maxima: no GEMM follows
     # too little room: the size the pass needs, and nothing written past the room given
     d, _, _ = _mlp_pass(sizes, h, f)
     blob[:] = 0x55
