@@ -97,15 +97,21 @@ class kernel_timing:
         return out
 
 
-def gemm_form(a_fmt, flags):
+def gemm_form(a_fmt, flags, plan=None):
     """Name of a grouped-GEMM launch by what it reads: the format of operand a (0 = e4m3, 1 = e5m2: a gradient) and
-    which operands are stored contraction-major (the launch's FP8GMM_GEMM_*_KMAJOR flags)."""
+    which operands are stored contraction-major (the launch's FP8GMM_GEMM_*_KMAJOR flags); with the launch's plan,
+    also the tile where it is not the 256 x 256 one."""
     fmt = "e5m2" if a_fmt == _lib.E5M2 else "e4m3"
+    tile = ""
+    if plan is not None and plan.tile_m not in (0, plan.tile):
+        tile = f"; {plan.tile_m} x {plan.tile} tiles, two sets of accumulators"
+    elif plan is not None and plan.tile not in (0, 256):
+        tile = f"; {plan.tile} x {plan.tile} tiles"
     if flags & _lib.GEMM_A_KMAJOR:
-        return f"{fmt} a and b contraction-major (weight gradient in place)"
+        return f"{fmt} a and b contraction-major (weight gradient in place)" + tile
     if flags & _lib.GEMM_B_KMAJOR:
-        return f"{fmt} a row-major, b contraction-major"
-    return f"{fmt} a and b row-major" + (", GELU epilogue" if flags & _lib.EPI_GELU else "")
+        return f"{fmt} a row-major, b contraction-major" + tile
+    return f"{fmt} a and b row-major" + (", GELU epilogue" if flags & _lib.EPI_GELU else "") + tile
 
 
 class _timed:
@@ -761,7 +767,7 @@ def _launch_gemm(table, a_dtype, b_dtype, c_dtype, gelu, device, keep, b_kmajor=
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
             with _timed("grouped_gemm", lambda: _algorithmic_flops(table),
                         lambda: _algorithmic_gemm_bytes(table, 2 if c_dtype == torch.bfloat16 else 1),
-                        lambda: gemm_form(fmts[0], fmts[3])):
+                        lambda: gemm_form(fmts[0], fmts[3], plan)):
                 fix_ptr = dev_ptr + off_fix if plan.n_fixups else None
                 rc = _lib.load().fp8gmm_grouped_gemm(dev_ptr, n, dev_ptr + off_items, fix_ptr, plan, *fmts, ws_ptr,
                                                      ws_bytes, _stream(device))
@@ -948,7 +954,7 @@ def _run_pass(device, desc, fields, plan_fn, bound_fn):
             ws = _gemm_workspace(device, rec.plan.n_slots) if gemm else None
             ws_ptr, ws_bytes = (ws.data_ptr(), ws.numel()) if ws is not None else (None, 0)
             with _timed("grouped_gemm" if gemm else _OP_NAMES[rec.op], lambda: rec.work, lambda: rec.bytes,
-                        (lambda: gemm_form(rec.a_fmt, rec.epilogue)) if gemm else None):
+                        (lambda: gemm_form(rec.a_fmt, rec.epilogue, rec.plan)) if gemm else None):
                 rc = L.fp8gmm_run_planned(base, ctypes.byref(rec), ws_ptr, ws_bytes, stream)
             _lib.check(rc)
     return plan
