@@ -191,6 +191,8 @@ EXPORTS = (
     "fp8gmm_plan_mlp_backward",
     "fp8gmm_sizeof_mlp_pass",
     "fp8gmm_run_planned",
+    "fp8gmm_host_alloc",
+    "fp8gmm_host_free",
     "fp8gmm_delayed_scaling_updates",
     "fp8gmm_sizeof_linear_pass",
     "fp8gmm_sizeof_pass_plan",
@@ -300,6 +302,10 @@ def load():
     L.fp8gmm_delayed_scaling_update.argtypes = [vp, vp, vp, ci, ci, ctypes.c_float, ci, ci, ci, ci, vp]
     L.fp8gmm_delayed_scaling_updates.restype = ci
     L.fp8gmm_delayed_scaling_updates.argtypes = [ctypes.POINTER(ScalingUpdate), ci, vp]
+    L.fp8gmm_host_alloc.restype = vp
+    L.fp8gmm_host_alloc.argtypes = [ctypes.c_size_t]
+    L.fp8gmm_host_free.restype = None
+    L.fp8gmm_host_free.argtypes = [vp]
     L.fp8gmm_upload.restype = ci
     L.fp8gmm_upload.argtypes = [vp, vp, ctypes.c_size_t, vp]
     L.fp8gmm_route_workspace_bytes.restype = ctypes.c_size_t

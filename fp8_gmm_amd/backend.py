@@ -240,6 +240,39 @@ class _Staging:
                 self.used -= reserved - used
 
 
+class _CaptureArena:
+    """Page-locked memory for the tables of launches that are being captured into a graph.  A replay runs the
+    captured copy kernel again, which reads its source again: the tables must stay where they are, unchanged, for as
+    long as the graph may be replayed, so this memory is handed out once and never recycled (a captured step of a
+    module takes 0.1 - 1.5 MB of it).  Allocated through the library, which can do so while a stream is capturing."""
+
+    CHUNK = 4 << 20
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.chunks = []        # (address, numpy view): alive until the process ends
+        self.used = self.CHUNK  # of the last chunk
+
+    def take(self, nbytes):
+        n = (nbytes + 255) & ~255
+        with self.lock:
+            if self.used + n > self.CHUNK or not self.chunks:
+                size = max(self.CHUNK, n)
+                address = _lib.load().fp8gmm_host_alloc(size)
+                if not address:
+                    _fail("fp8_gmm_amd: could not allocate page-locked memory for the tables of a captured launch")
+                view = np.ctypeslib.as_array((ctypes.c_uint8 * size).from_address(address))
+                self.chunks.append((address, view))
+                self.used = 0 if size == self.CHUNK else self.CHUNK
+                if size != self.CHUNK:
+                    return address, view[:nbytes]
+            address, view = self.chunks[-1]
+            offset = self.used
+            self.used += n
+        return address + offset, view[offset: offset + nbytes]
+
+
+_capture_arena = _CaptureArena()
 _staging = {}
 
 
@@ -258,9 +291,17 @@ def _to_device(device, room, fill):
     room = (room + 15) & ~15
     with _on_device(device):
         stream = torch.cuda.current_stream(device)
-        # (under stream capture the tables go the other way: a captured copy kernel would read, at every replay,
-        # whatever the staging memory holds by then)
-        staged = options.upload == "kernel" and not torch.cuda.is_current_stream_capturing()
+        if torch.cuda.is_current_stream_capturing():
+            # the captured copy kernel reads its source again at every replay: memory of its own, kept for good
+            address, host = _capture_arena.take(room)
+            used = fill(address, host)
+            used = room if used is None else (used + 15) & ~15
+            if not used:
+                return None
+            out = torch.empty(used, dtype=torch.uint8, device=device)
+            _lib.check(_lib.load().fp8gmm_upload(out.data_ptr(), address, used, stream.cuda_stream))
+            return out
+        staged = options.upload == "kernel"
         st = _staging_of(device) if staged else None
         offset = st.reserve(room, stream) if st is not None else None
         if offset is None:   # larger than the staging area, or by choice: a pinned buffer of its own and torch's copy

@@ -322,6 +322,30 @@ int fp8gmm_multi_scale_mul(const fp8gmm_tensor_desc* descs_dev, int n, int total
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
+void* fp8gmm_host_alloc(size_t bytes) {
+  if (bytes == 0) return nullptr;
+  // while a stream is being captured the runtime refuses allocations from any thread; this one is safe there (it
+  // touches no stream), so the calling thread's capture mode is relaxed for its duration
+  hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+  const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+  void* p = nullptr;
+  const hipError_t e = hipHostMalloc(&p, bytes, hipHostMallocDefault);
+  if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return p;
+}
+
+void fp8gmm_host_free(void* p) {
+  if (p == nullptr) return;
+  hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+  const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+  (void)hipHostFree(p);
+  if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+}
+
 int fp8gmm_upload(void* dst_dev, const void* src_host, size_t bytes, void* stream) {
   if (bytes == 0) return FP8GMM_OK;
   if (dst_dev == nullptr || src_host == nullptr) return FP8GMM_ERR_NULL_POINTER;

@@ -494,6 +494,16 @@ typedef struct fp8gmm_scaling_update {
 int fp8gmm_delayed_scaling_updates(const fp8gmm_scaling_update* updates, int n, void* stream);
 
 /*
+ * Page-locked host memory that the device can read (for fp8gmm_upload's source), allocated also while a stream is
+ * being captured into a graph, when the runtime refuses ordinary allocations: the tables of a captured launch are
+ * read again at every replay, so they need memory that outlives the capture and is not recycled, which a staging
+ * ring cannot give.  The caller keeps it unchanged and alive as long as the graph.  NULL when the allocation fails.
+ * No counterpart in the reference (whose launches take their tables as kernel arguments).
+ */
+void* fp8gmm_host_alloc(size_t bytes);
+void fp8gmm_host_free(void* p);
+
+/*
  * Copy `bytes` of tables from page-locked host memory that the device can address (hipHostMalloc; torch's
  * pin_memory) to device memory with a kernel on `stream`: dst_dev, src_host and bytes multiples of 16, at most
  * 1 GiB.  The host memory must stay as it is until the stream has passed this point.  Every launch entry point of
