@@ -839,7 +839,8 @@ class GemmOptions:
     """Launch policy of the grouped GEMMs of this process: ``tile`` "auto" | "256" | "128" | "dual", ``stream_k`` (share the
     tail tiles of a launch along K), ``wgrad`` "in_place" | "copy", ``upload`` "kernel" (tables reach the device
     through staging memory and a copy kernel of the library) | "copy" (a pinned buffer per upload and torch's
-    asynchronous copy).  The defaults can be preset with the environment variables FP8GMM_TILE, FP8GMM_STREAMK
+    asynchronous copy; while a stream is being captured into a graph the tables always take the first way, from
+    memory that is kept for the replays).  The defaults can be preset with the environment variables FP8GMM_TILE, FP8GMM_STREAMK
     (0 turns sharing off), FP8GMM_WGRAD and FP8GMM_UPLOAD, read once when the module is imported; afterwards assign
     the attributes or use ``gemm_options(...)`` for a block."""
 

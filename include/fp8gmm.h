@@ -411,7 +411,9 @@ size_t fp8gmm_sizeof_pass_plan(void);
 int fp8gmm_plan_linear_forward(const fp8gmm_linear_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
 int fp8gmm_plan_linear_backward(const fp8gmm_linear_pass* pass, void* blob, size_t blob_bytes, fp8gmm_pass_plan* out);
 /* Enqueue one launch of a planned pass; blob_dev is the DEVICE copy of the blob (the cast launch writes into its
- * descriptors, so every pass uploads afresh); workspace as for fp8gmm_grouped_gemm. */
+ * descriptors, so every pass uploads afresh); workspace as for fp8gmm_grouped_gemm.  Run the launches of a pass in
+ * their order, all of them, on one stream: a cast whose record has merge_n != 0 has left the merge of its tensors'
+ * maxima into the amax slots to the GEMM launch behind it. */
 int fp8gmm_run_planned(const void* blob_dev, const fp8gmm_pass_launch* launch, void* workspace, size_t workspace_bytes,
                        void* stream);
 
