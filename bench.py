@@ -643,13 +643,15 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="skip the pass that captures the step into a HIP graph")
     ap.add_argument("--headline-only", action="store_true",
                     help="skip the extra passes after the timed region (clock / power sampling, cached-weights "
-                         "step, the other workloads): what a profiler should see")
+                         "step, the HIP-graph replays, the other workloads): what a profiler should see")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy (reads 256 MiB, writes 256 MiB) so that hardware "
                          "byte counters collected around this command can be scaled against a known transfer")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it")
+    if args.headline_only:
+        args.no_graph = True   # a profiler should see the timed steps, not their replays
     if args.workload == "config5":
         print(json.dumps(measure_cast_pad(args)))
         return
