@@ -32,20 +32,16 @@ class _RoutedModule(torch.nn.Module):
 
     def compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins, top_k):
         x = x.view(-1, x.size(-1))
-        # The host needs the split to plan the expert launches.  On the GPU its copy is enqueued ahead of the gather,
+        # The host needs the split to plan the expert launches.  Its copy is enqueued ahead of the gather,
         # which needs nothing from the host, so the rows move while the host waits for the counts.
-        if tokens_per_expert.is_cuda:
-            if self._counts_host is None or self._counts_host.numel() != tokens_per_expert.numel():
-                self._counts_host = torch.empty(tokens_per_expert.shape, dtype=tokens_per_expert.dtype, pin_memory=True)
-                self._counts_ready = torch.cuda.Event()
-            self._counts_host.copy_(tokens_per_expert, non_blocking=True)
-            self._counts_ready.record()
-            x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
-            self._counts_ready.synchronize()
-            batch_sizes = self._counts_host.to(torch.long, copy=True)   # the page-locked buffer is reused by the next step
-        else:
-            x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
-            batch_sizes = tokens_per_expert.to(torch.long)
+        if self._counts_host is None or self._counts_host.numel() != tokens_per_expert.numel():
+            self._counts_host = torch.empty(tokens_per_expert.shape, dtype=tokens_per_expert.dtype, pin_memory=True)
+            self._counts_ready = torch.cuda.Event()
+        self._counts_host.copy_(tokens_per_expert, non_blocking=True)
+        self._counts_ready.record()
+        x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
+        self._counts_ready.synchronize()
+        batch_sizes = self._counts_host.to(torch.long, copy=True)   # the page-locked buffer is reused by the next step
         out = self.experts(x, batch_sizes)
         return moe_ops.scatter(out, indices, bin_ids, expert_weights, bins, top_k)
 

@@ -199,3 +199,53 @@ def test_routed_mlp_layer_trains_like_a_dense_fp32_model(dev):
     assert cos(layer.grouped_mlp.fc1_weight.grad, w1.grad) > 0.99
     assert cos(layer.grouped_mlp.fc2_weight.grad, w2.grad) > 0.99
     assert cos(layer.gating_network.weight.grad, gate.grad) > 0.98
+
+
+def test_example_bf16_layer_against_a_dense_fp32_model(dev):
+    """The bf16 layer of the example recipe (one vendor GEMM per expert on its row slice, hand-written gradients)
+    against an fp32 autograd model of the same routed layer with the same routing decisions."""
+    import fp8_gmm_amd as pkg
+    from fp8_gmm_amd import example
+
+    tokens, h, f, e, top_k = 384, 128, 256, 6, 2
+    torch.manual_seed(21)
+    layer = example.Bf16Module(h, f, e, top_k, device=dev)
+    x = torch.randn(tokens, h, device=dev).to(torch.bfloat16)
+    dy = torch.randn(tokens, h, device=dev).to(torch.bfloat16)
+    xd = x.clone().requires_grad_()
+    out = layer(xd)
+    out.backward(dy)
+
+    xr = x.float().requires_grad_()
+    gate = layer.gating_network.weight.detach().float().requires_grad_()
+    w1 = layer.w1.detach().float().requires_grad_()
+    w2 = layer.w2.detach().float().requires_grad_()
+    _, selected = pkg.moe_ops.topk(layer.gating_network(x).float(), top_k)
+    probs = torch.softmax(xr @ gate.t(), dim=1)
+    ref = torch.zeros(tokens, h, device=dev)
+    for k in range(top_k):
+        ek = selected[:, k]
+        hidden = torch.nn.functional.gelu(torch.einsum("th,tfh->tf", xr, w1[ek]))
+        ref = ref + probs.gather(1, ek[:, None]) * torch.einsum("tf,thf->th", hidden, w2[ek])
+    ref.backward(dy.float())
+
+    def cos(a, b):
+        a, b = a.detach().float().flatten(), b.detach().float().flatten()
+        return (torch.dot(a, b) / (a.norm() * b.norm())).item()
+
+    assert cos(out, ref) > 0.9995
+    assert cos(xd.grad, xr.grad) > 0.999
+    assert cos(layer.w1.grad, w1.grad) > 0.999
+    assert cos(layer.w2.grad, w2.grad) > 0.999
+    assert cos(layer.gating_network.weight.grad, gate.grad) > 0.995
+
+
+def test_example_recipe_runs_every_kind_of_layer(dev, capsys):
+    """``python -m fp8_gmm_amd.example`` at a small size: four timed kinds, one printed line each."""
+    from fp8_gmm_amd import example
+
+    times = example.main(["--tokens", "512", "--hidden", "256", "--inner", "512", "--experts", "8", "--warmup", "1",
+                          "--steps", "2"])
+    assert list(times) == list(example.KINDS) and all(t > 0 for t in times.values())
+    lines = [line for line in capsys.readouterr().out.splitlines() if " run: " in line]
+    assert len(lines) == 4 and lines[0].startswith("Bf16Module run: ") and lines[3].startswith("Fp8MlpModule run: ")
