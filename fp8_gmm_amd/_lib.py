@@ -227,8 +227,11 @@ class Fp8GmmError(RuntimeError):
 _lib = None
 
 
+ABI_VERSION = 3   # FP8GMM_VERSION of include/fp8gmm.h that the structures and argument lists below were written for
+
+
 def load():
-    """Load the shared library once; raise loudly when it is absent or incomplete."""
+    """Load the shared library once; raise loudly when it is absent, incomplete or of another interface version."""
     global _lib
     if _lib is not None:
         return _lib
@@ -245,6 +248,9 @@ def load():
     ip = ctypes.POINTER(ctypes.c_int)
     L.fp8gmm_version.restype = ci
     L.fp8gmm_version.argtypes = []
+    if L.fp8gmm_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH} speaks version {L.fp8gmm_version()} of the interface, this package version "
+                          f"{ABI_VERSION}: rebuild it (`make -C fp8_gmm_amd/csrc -j8`)")
     L.fp8gmm_status_string.restype = ctypes.c_char_p
     L.fp8gmm_status_string.argtypes = [ci]
     L.fp8gmm_sizeof_tensor_desc.restype = ctypes.c_size_t

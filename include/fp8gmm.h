@@ -34,7 +34,9 @@
 extern "C" {
 #endif
 
-#define FP8GMM_VERSION 2
+/* Counts the incompatible changes of this interface (a struct layout, the meaning of a field or an argument): a
+ * binding compares fp8gmm_version() of the library it loaded with the value it was written against. */
+#define FP8GMM_VERSION 3
 
 /* fp8 formats (OCP): e4m3fn = torch.float8_e4m3fn, e5m2 = torch.float8_e5m2 */
 #define FP8GMM_E4M3 0

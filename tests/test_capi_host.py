@@ -40,7 +40,7 @@ def test_struct_layouts_match_the_binding():
     assert _lib.GEMM_ITEM.fields["lda"][1] == 24 and _lib.GEMM_ITEM.fields["k"][1] == 32
     assert _lib.GEMM_ITEM.fields["prob"][1] == 52
     assert ctypes.sizeof(_lib.GemmPlan) == 32
-    assert lib.fp8gmm_version() == 2
+    assert lib.fp8gmm_version() == _lib.ABI_VERSION == 3
     assert _lib.gemm_tile_shape() == (256, 256)
     assert lib.fp8gmm_status_string(0) == b"ok"
     assert b"NULL" in lib.fp8gmm_status_string(-1)
