@@ -190,6 +190,7 @@ class Fp8GroupedModuleBase(torch.nn.Module):
         self.fp8_meta = {}
         self._fp8_steps = 0
         self._weight_caches = []  # Fp8WeightCache objects of the subclass; dropped whenever the scales are replaced
+        self._ahead = None        # fp8 weights that cast_weights_ahead() made for the next forward pass
 
     def _invalidate_weight_caches(self):
         for cache in self._weight_caches:
@@ -245,6 +246,43 @@ class Fp8GroupedModuleBase(torch.nn.Module):
                         amax_and_scale_update(bwd, self.fp8_meta["fp8_max_bwd"], fp8_recipe)
             self._fp8_steps += 1
         yield
+
+    def _cast_ahead(self, weights_and_groups):
+        """The part of a forward pass that needs no group sizes, run now: the delayed-scaling update and the cast of
+        the weight stacks ``[(weight, Fp8TensorType of its scaling slots), ...]`` into fp8 tensors of their own, one
+        launch.  Returns False (and does nothing) where the pass would use the reference's transposed layout."""
+        from .backend import TensorBatch, multi_quantize
+        from .grouped_linear import stage_weight_cast
+        from .utils import Fp8MetaWrapper, MetaTensorType, to_torch_dtype
+
+        first = weights_and_groups[0][0]
+        if self.fp8_meta.get("reference_layout") or not first.is_cuda \
+                or any(w.size(1) % 16 or w.size(2) % 16 or not w.is_contiguous() for w, _ in weights_and_groups):
+            return False
+        self._ahead = None
+        with self.prepare_forward(first, None, self.num_groups * len(weights_and_groups)):
+            import numpy as np
+
+            meta = Fp8MetaWrapper(self.num_groups, self.fp8_meta)
+            fp8_dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
+            caches = tuple(Fp8WeightCache() for _ in weights_and_groups)
+            plain, with_t = ([], [], [], []), ([], [], [], [], [])
+            for (weight, group), cache in reversed(list(zip(weights_and_groups, caches))):
+                stage_weight_cast(weight, fp8_dtype, False, False, cache, True,
+                                  meta.get_meta_pointers(group, MetaTensorType.kScale),
+                                  meta.get_meta_pointers(group, MetaTensorType.kAmax), plain, with_t)
+            with torch.no_grad():
+                multi_quantize(TensorBatch.concat(plain[0]), TensorBatch.concat(plain[1]), np.concatenate(plain[2]),
+                               np.concatenate(plain[3]))
+        self._ahead = caches
+        return True
+
+    def _take_ahead(self, is_first_microbatch):
+        ahead, self._ahead = self._ahead, None
+        if ahead is not None and is_first_microbatch is not None:
+            raise RuntimeError("cast_weights_ahead() has cast this pass's weights: call forward without "
+                               "is_first_microbatch")
+        return ahead
 
     # checkpointing of the scaling state (TransformerEngine exposes it the same way)
     def get_extra_state(self):

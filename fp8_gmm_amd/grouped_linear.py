@@ -19,6 +19,7 @@ gradient is zero), wgrad is a single launch instead of a per-expert loop, and th
 grouped GEMM is the same HIP kernel whatever ``cutlass`` says (``cutlass=True`` keeps
 the two-rounding data flow of the reference's CUTLASS path, see ``backend.fp8_gmm``).
 """
+import contextlib
 import math
 
 import numpy as np
@@ -353,11 +354,23 @@ class GroupedLinear(Fp8GroupedModuleBase):
         dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
         return list(self._weight_cache.buffers(self.weight_tensor, dtype, self.fp8_meta["reference_layout"]))
 
+    def cast_weights_ahead(self):
+        """Start the next forward pass before its group sizes are known: the delayed-scaling update and the cast of
+        the weights to fp8 are enqueued now, and the next ``forward(input, group_sizes)`` runs only what is left, with
+        the same results.  For callers whose sizes come from the device (a router): the GPU works on the weights
+        while the host waits for the sizes and plans the launches.  No counterpart in the reference.  Returns False,
+        having done nothing, for a module in the reference's layout."""
+        return self._cast_ahead([(self.weight_tensor, Fp8TensorType.kWeightGroup1)])
+
     def forward(self, input, group_sizes, is_first_microbatch=None):
-        with self.prepare_forward(input, is_first_microbatch, self.num_groups):
+        ahead = self._take_ahead(is_first_microbatch)
+        with (contextlib.nullcontext() if ahead is not None else
+              self.prepare_forward(input, is_first_microbatch, self.num_groups)):
             grad = torch.is_grad_enabled()
             args = (input, self.weight_tensor, group_sizes, self.fp8_meta, grad, self.cutlass)
-            if is_first_microbatch is not None:
+            if ahead is not None:
+                args += (ahead[0], False)
+            elif is_first_microbatch is not None:
                 args += (self._weight_cache, bool(is_first_microbatch))
             if grad:
                 return _GroupedLinear.apply(*args)

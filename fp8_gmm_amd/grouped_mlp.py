@@ -21,6 +21,7 @@ Experts with zero tokens are allowed; each wgrad is one grouped launch.  In the 
 planned by one library call (``backend.mlp_pass``); the launch-by-launch code below it builds the same tables and
 serves the other layouts and options.
 """
+import contextlib
 import math
 
 import numpy as np
@@ -440,11 +441,20 @@ class GroupedMlp(Fp8GroupedModuleBase):
         return list(self._weight_caches[0].buffers(self.fc1_weight, dtype, tw)) + \
             list(self._weight_caches[1].buffers(self.fc2_weight, dtype, tw))
 
+    def cast_weights_ahead(self):
+        """As ``GroupedLinear.cast_weights_ahead``: the scaling update and the casts of both weight stacks are enqueued
+        now, the next ``forward(input, group_sizes)`` runs the rest."""
+        return self._cast_ahead([(self.fc1_weight, _T.kWeightGroup1), (self.fc2_weight, _T.kWeightGroup2)])
+
     def forward(self, input, group_sizes, has_tp=False, tp_group=None, is_first_microbatch=None):
-        with self.prepare_forward(input, is_first_microbatch, self.num_groups * 2):
+        ahead = self._take_ahead(is_first_microbatch)
+        with (contextlib.nullcontext() if ahead is not None else
+              self.prepare_forward(input, is_first_microbatch, self.num_groups * 2)):
             grad = torch.is_grad_enabled()
             args = (input, self.fc1_weight, self.fc2_weight, group_sizes, self.fp8_meta, grad, has_tp, tp_group)
-            if is_first_microbatch is not None:
+            if ahead is not None:
+                args += (ahead, False)
+            elif is_first_microbatch is not None:
                 args += (tuple(self._weight_caches), bool(is_first_microbatch))
             if grad:
                 return _GroupedMlp.apply(*args)

@@ -30,16 +30,21 @@ class _RoutedModule(torch.nn.Module):
     def experts(self, x, batch_sizes):
         raise NotImplementedError
 
+    def start_experts(self):
+        """Enqueue what the experts' pass can do before the host knows the split (nothing, by default)."""
+
     def compute(self, x, tokens_per_expert, indices, bin_ids, expert_weights, bins, top_k):
         x = x.view(-1, x.size(-1))
-        # The host needs the split to plan the expert launches.  Its copy is enqueued ahead of the gather,
-        # which needs nothing from the host, so the rows move while the host waits for the counts.
+        # The host needs the split to plan the expert launches.  Its copy is enqueued ahead of the gather and of the
+        # experts' weight casts, which need nothing from the host: the GPU has that work to do while the host waits
+        # for the counts and plans the launches.
         if self._counts_host is None or self._counts_host.numel() != tokens_per_expert.numel():
             self._counts_host = torch.empty(tokens_per_expert.shape, dtype=tokens_per_expert.dtype, pin_memory=True)
             self._counts_ready = torch.cuda.Event()
         self._counts_host.copy_(tokens_per_expert, non_blocking=True)
         self._counts_ready.record()
         x = moe_ops.gather(x, indices, bin_ids, bins, top_k)
+        self.start_experts()
         self._counts_ready.synchronize()
         batch_sizes = self._counts_host.to(torch.long, copy=True)   # the page-locked buffer is reused by the next step
         out = self.experts(x, batch_sizes)
@@ -66,6 +71,10 @@ class Fp8LinearModule(_RoutedModule):
         self.grouped_linear2 = GroupedLinear(n_inner, n_embd, n_experts, dtype=dtype, cutlass=cutlass, device=device)
         self.act = torch.nn.GELU()
 
+    def start_experts(self):
+        self.grouped_linear1.cast_weights_ahead()
+        self.grouped_linear2.cast_weights_ahead()
+
     def experts(self, x, batch_sizes):
         return self.grouped_linear2(self.act(self.grouped_linear1(x, batch_sizes)), batch_sizes)
 
@@ -76,6 +85,9 @@ class Fp8MlpModule(_RoutedModule):
     def __init__(self, n_embd, n_inner, n_experts, top_k, dtype=torch.bfloat16, device="cuda"):
         super().__init__(n_embd, n_inner, n_experts, top_k, dtype, device)
         self.grouped_mlp = GroupedMlp(n_embd, n_inner, n_experts, dtype=dtype, device=device)
+
+    def start_experts(self):
+        self.grouped_mlp.cast_weights_ahead()
 
     def experts(self, x, batch_sizes):
         return self.grouped_mlp(x, batch_sizes)

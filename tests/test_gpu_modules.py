@@ -359,6 +359,68 @@ def test_grouped_mlp_cached_weights_equal_recast_weights(dev, frozen):
         assert torch.equal(mods[0].fp8_meta["scaling_bwd"].amax_history, mods[1].fp8_meta["scaling_bwd"].amax_history)
 
 
+@pytest.mark.parametrize("kind", ["linear", "linear-cutlass", "mlp"])
+def test_weights_cast_ahead_of_the_pass_give_the_same_bits(dev, kind):
+    """``cast_weights_ahead()`` moves the scaling update and the weight casts in front of the moment the group sizes
+    are known; outputs, gradients and the whole scaling state must equal those of a module that does everything
+    inside ``forward``, step after step with changing weights and sizes - also with two forward passes in flight
+    before their backward passes, and back on the plain path afterwards."""
+    pkg = _pkg()
+    e, h, f = 5, 256, 512
+    g = gen(3105)
+    mods = []
+    for _ in range(2):
+        if kind == "mlp":
+            mod = pkg.GroupedMlp(h, f, e, torch.bfloat16, device=dev)
+        else:
+            mod = pkg.GroupedLinear(h, f, e, torch.bfloat16, device=dev, cutlass=kind == "linear-cutlass")
+        mods.append(mod)
+    mods[1].load_state_dict(mods[0].state_dict())
+    params = [[p for _, p in sorted(mod.named_parameters())] for mod in mods]
+    fp8_recipe = pkg.DelayedScaling(amax_history_len=3)
+    out_features = h if kind == "mlp" else f
+    splits = [[137, 0, 401, 59, 403], [1, 999, 0, 0, 0], [200] * 5, [64, 64, 0, 64, 808]]
+
+    def passes(mod, ahead, batches):
+        """Forward passes over all batches first, then their backward passes in reverse order."""
+        outs = []
+        for x, sizes, _ in batches:
+            with pkg.fp8_autocast(fp8_recipe=fp8_recipe):
+                if ahead:
+                    assert mod.cast_weights_ahead()
+                outs.append(mod(x, torch.tensor(sizes)))
+        for out, (_, _, dy) in reversed(list(zip(outs, batches))):
+            out.backward(dy)
+        return outs
+
+    for step, ahead in enumerate([True, True, True, False, True]):
+        n = 2 if step == 2 else 1    # step 2: two passes in flight
+        data = []
+        for i in range(n):
+            sizes = splits[(step + i) % len(splits)]
+            m = sum(sizes)
+            data.append((randn_bf16((m, h), g).to(dev), sizes, randn_bf16((m, out_features), g, 1e-2).to(dev)))
+        res = []
+        for mod, use in zip(mods, (ahead, False)):
+            mod.zero_grad()
+            batches = [(x.clone().requires_grad_(), sizes, dy) for x, sizes, dy in data]
+            outs = passes(mod, use, batches)
+            res.append(outs + [b[0].grad for b in batches] + [p.grad for _, p in sorted(mod.named_parameters())])
+        for i, (a, b) in enumerate(zip(*res)):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), f"step {step}: result {i} differs"
+        for name in ("scaling_fwd", "scaling_bwd"):
+            sa, sb = mods[0].fp8_meta[name], mods[1].fp8_meta[name]
+            assert torch.equal(sa.scale, sb.scale) and torch.equal(sa.scale_inv, sb.scale_inv), f"step {step} {name}"
+            assert torch.equal(sa.amax_history, sb.amax_history), f"step {step} {name}"
+        with torch.no_grad():   # an optimizer step: the weights change, so do their scales
+            for pa, pb in zip(*params):
+                pa.add_(pa.grad, alpha=-0.5)
+                pb.add_(pb.grad, alpha=-0.5)
+    with pytest.raises(RuntimeError, match="cast_weights_ahead"):
+        mods[0].cast_weights_ahead()
+        mods[0](data[0][0], torch.tensor(data[0][1]), is_first_microbatch=True)
+
+
 def test_grouped_mlp_frozen_weights_against_the_oracle(dev):
     """No weight gradients: padded transposes are skipped and d(pre-GELU) goes through the cast-only dGELU
     kernel; output and grad_input must still be the oracle's."""
