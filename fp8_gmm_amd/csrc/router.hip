@@ -20,7 +20,8 @@
 namespace fp8gmm {
 namespace {
 
-constexpr int kRouteChunk = 1024;       // list entries per workgroup of the counting sort
+constexpr int kRouteChunk = 512;        // list entries per workgroup of the counting sort
+constexpr int kRouteSteps = kRouteChunk / 64;
 constexpr int kRouteMaxExperts = 4096;  // size of the per-workgroup expert table in LDS (16 KB)
 constexpr int kRowWaves = 4;            // wavefronts (= rows in flight) per workgroup of the row movers
 
@@ -36,10 +37,15 @@ __global__ __launch_bounds__(64) void route_count_kernel(const int32_t* __restri
   for (int e = lane; e < num_experts; e += 64) table[e] = 0;
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * kRouteChunk;
-  for (int r = 0; r < kRouteChunk; r += 64) {
-    const int64_t i = base + r + lane;
-    if (i < n) atomicAdd(&table[clamp_expert(expert_of[i], num_experts)], 1);
+  int32_t ids[kRouteSteps];  // all loads of the chunk in flight at once
+#pragma unroll
+  for (int r = 0; r < kRouteSteps; ++r) {
+    const int64_t i = base + r * 64 + lane;
+    ids[r] = i < n ? expert_of[i] : -1;
   }
+#pragma unroll
+  for (int r = 0; r < kRouteSteps; ++r)
+    if (base + r * 64 + lane < n) atomicAdd(&table[clamp_expert(ids[r], num_experts)], 1);
   __syncthreads();
   for (int e = lane; e < num_experts; e += 64) counts[(size_t)blockIdx.x * num_experts + e] = table[e];
 }
@@ -52,14 +58,34 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ c
   __shared__ int32_t total[kRouteMaxExperts];
   __shared__ int32_t part[256];
   const int tid = threadIdx.x;
-  for (int e = tid; e < num_experts; e += 256) {
-    int32_t run = 0;
-    for (int b = 0; b < chunks; ++b) {
-      const int32_t c = counts[(size_t)b * num_experts + e];
-      counts[(size_t)b * num_experts + e] = run;  // exclusive prefix over the chunks
-      run += c;
+  if (num_experts >= 256) {  // many experts: a thread per expert walks the chunks
+    for (int e = tid; e < num_experts; e += 256) {
+      int32_t run = 0;
+      for (int b = 0; b < chunks; ++b) {
+        const int32_t c = counts[(size_t)b * num_experts + e];
+        counts[(size_t)b * num_experts + e] = run;  // exclusive prefix over the chunks
+        run += c;
+      }
+      total[e] = run;
     }
-    total[e] = run;
+  } else {  // few experts: a wavefront per expert, its lanes over 64 chunks at a time
+    const int lane = tid % 64;
+    for (int e = tid / 64; e < num_experts; e += 4) {
+      int32_t run = 0;
+      for (int b0 = 0; b0 < chunks; b0 += 64) {
+        const int b = b0 + lane;
+        const int32_t c = b < chunks ? counts[(size_t)b * num_experts + e] : 0;
+        int32_t incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int32_t below = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += below;
+        }
+        if (b < chunks) counts[(size_t)b * num_experts + e] = run + incl - c;
+        run += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) total[e] = run;
+    }
   }
   __syncthreads();
   // exclusive scan of the totals over the experts: thread t owns experts [t * per, (t + 1) * per)
@@ -88,15 +114,14 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t* __restrict__ c
     if (bins != nullptr) bins[e] = start;
   }
   __syncthreads();
-  for (int e = tid; e < num_experts; e += 256) {
-    const int32_t s = total[e];
-    for (int b = 0; b < chunks; ++b) counts[(size_t)b * num_experts + e] += s;
-  }
+  const int64_t cells = (int64_t)chunks * num_experts;
+  for (int64_t i = tid; i < cells; i += 256) counts[i] += total[i % num_experts];
 }
 
 // Stable placement: the single wavefront of a workgroup walks its chunk 64 entries at a time, in order; within
 // a group of 64 an entry's rank among the entries of the same expert is the number of lower lanes that hold
-// that expert.
+// that expert.  The lanes that hold the same expert are found bit by bit of the expert id: one ballot per bit,
+// ceil(log2(num_experts)) of them, whatever the number of distinct experts in the group.
 __global__ __launch_bounds__(64) void route_place_kernel(const int32_t* __restrict__ expert_of, int n,
                                                          int num_experts, const int32_t* __restrict__ offsets,
                                                          int32_t* __restrict__ bin_ids,
@@ -108,22 +133,30 @@ __global__ __launch_bounds__(64) void route_place_kernel(const int32_t* __restri
   __syncthreads();
   const int64_t base = (int64_t)blockIdx.x * kRouteChunk;
   const uint64_t below = (1ull << lane) - 1ull;
-  for (int r = 0; r < kRouteChunk; r += 64) {
-    const int64_t i = base + r + lane;
+  int bits = 0;
+  while ((1 << bits) < num_experts) ++bits;
+  int32_t ids[kRouteSteps];  // all loads of the chunk in flight at once
+#pragma unroll
+  for (int r = 0; r < kRouteSteps; ++r) {
+    const int64_t i = base + r * 64 + lane;
+    ids[r] = i < n ? expert_of[i] : 0;
+  }
+#pragma unroll
+  for (int r = 0; r < kRouteSteps; ++r) {
+    const int64_t i = base + r * 64 + lane;
     const bool valid = i < n;
-    const int e = valid ? clamp_expert(expert_of[i], num_experts) : -1;
-    int pos = 0;
-    uint64_t todo = __ballot(valid);
-    while (todo != 0) {  // one round per distinct expert among the 64 entries; `todo` is the same in every lane
-      const int leader = __ffsll((unsigned long long)todo) - 1;
-      const int el = __shfl(e, leader, 64);
-      const uint64_t same = __ballot(e == el);
-      if (e == el) pos = next[el] + __popcll(same & below);
-      __syncthreads();
-      if (lane == leader) next[el] += __popcll(same);
-      __syncthreads();
-      todo &= ~same;
+    const int e = valid ? clamp_expert(ids[r], num_experts) : 0;
+    uint64_t same = __ballot(valid);
+    for (int k = 0; k < bits; ++k) {
+      const bool set = (e >> k) & 1;
+      const uint64_t has = __ballot(valid && set);
+      same &= set ? has : ~has;
     }
+    // for a valid lane `same` now marks the valid lanes with its expert
+    const int pos = valid ? next[e] + __popcll(same & below) : 0;
+    __syncthreads();
+    if (valid && (same & below) == 0) next[e] += __popcll(same);  // the lowest lane of every expert's group
+    __syncthreads();
     if (valid) {
       if (bin_ids != nullptr) bin_ids[pos] = e;
       if (indices != nullptr) indices[pos] = (int32_t)i;
