@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_wgrad_kernel(const
                                                                            const uint16_t* __restrict__ grad_out,
                                                                            const int32_t* __restrict__ indices,
                                                                            float* __restrict__ grad_w, int rows,
-                                                                           int hidden, int top_k) {
+                                                                           int hidden, int top_k, int vec) {
   const int lane = threadIdx.x % 64;
   const int row = blockIdx.x * kRowWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   if (row >= rows) return;
@@ -293,7 +293,30 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_wgrad_kernel(const
   const uint16_t* a = x + (size_t)row * hidden;
   const uint16_t* b = grad_out + (size_t)(idx / top_k) * hidden;
   float acc = 0.f;
-  for (int c = lane; c < hidden; c += 64) acc = __builtin_fmaf(bf16_to_f32(a[c]), bf16_to_f32(b[c]), acc);
+  if (vec) {  // 16 bytes per lane and load, four loads of each row in flight; reads past the row deliver zeros
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(a, (uint32_t)hidden * 2u);
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(b, (uint32_t)hidden * 2u);
+    for (int c0 = 0; c0 < hidden; c0 += 64 * 8 * 4) {
+      u32x4 va[4], vb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        va[u] = buf_load16_stream(ra, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+        vb[u] = buf_load16_stream(rb, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t pa[4] = {va[u].x, va[u].y, va[u].z, va[u].w};
+        const uint32_t pb[4] = {vb[u].x, vb[u].y, vb[u].z, vb[u].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc = __builtin_fmaf(bf16_lo_to_f32(pa[q]), bf16_lo_to_f32(pb[q]), acc);
+          acc = __builtin_fmaf(bf16_hi_to_f32(pa[q]), bf16_hi_to_f32(pb[q]), acc);
+        }
+      }
+    }
+  } else {
+    for (int c = lane; c < hidden; c += 64) acc = __builtin_fmaf(bf16_to_f32(a[c]), bf16_to_f32(b[c]), acc);
+  }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
   if (lane == 0) grad_w[idx] = acc;
@@ -378,7 +401,8 @@ int fp8gmm_moe_scatter_wgrad(const void* x, const void* grad_out, const int32_t*
   if (x == nullptr || grad_out == nullptr || indices == nullptr || grad_w == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipLaunchKernelGGL(moe_scatter_wgrad_kernel, dim3((rows + kRowWaves - 1) / kRowWaves), dim3(kRowWaves * 64), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x),
-                     static_cast<const uint16_t*>(grad_out), indices, grad_w, rows, hidden, top_k);
+                     static_cast<const uint16_t*>(grad_out), indices, grad_w, rows, hidden, top_k,
+                     (int)rows_vectorisable(x, grad_out, hidden));
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 
