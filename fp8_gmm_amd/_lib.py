@@ -212,6 +212,8 @@ EXPORTS = (
     "fp8gmm_route_workspace_bytes",
     "fp8gmm_route_sort",
     "fp8gmm_route_invert",
+    "fp8gmm_route_topk",
+    "fp8gmm_route_topk_backward",
     "fp8gmm_moe_gather",
     "fp8gmm_moe_scatter",
     "fp8gmm_moe_scatter_wgrad",
@@ -320,6 +322,10 @@ def load():
     L.fp8gmm_route_sort.argtypes = [vp, ci, ci, vp, vp, vp, vp, vp, vp, vp]
     L.fp8gmm_route_invert.restype = ci
     L.fp8gmm_route_invert.argtypes = [vp, ci, vp, vp]
+    L.fp8gmm_route_topk.restype = ci
+    L.fp8gmm_route_topk.argtypes = [vp, ci, ci, ci, ci, vp, vp, vp, vp]
+    L.fp8gmm_route_topk_backward.restype = ci
+    L.fp8gmm_route_topk_backward.argtypes = [vp, vp, vp, ci, ci, ci, vp, ci, vp]
     L.fp8gmm_moe_gather.restype = ci
     L.fp8gmm_moe_gather.argtypes = [vp, vp, vp, vp, ci, ci, ci, vp]
     L.fp8gmm_moe_scatter.restype = ci

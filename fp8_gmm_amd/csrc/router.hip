@@ -322,6 +322,106 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_wgrad_kernel(const
   if (lane == 0) grad_w[idx] = acc;
 }
 
+constexpr int kTopKMax = 8;  // choices per token that the selection keeps in registers
+
+template <bool BF16>
+__device__ __forceinline__ float score_at(const void* row, int e) {
+  if constexpr (BF16) return bf16_to_f32(static_cast<const uint16_t*>(row)[e]);
+  return static_cast<const float*>(row)[e];
+}
+
+// One wavefront per token, its lanes over the experts.  probs[t, :] = softmax(scores[t, :]) in fp32 (max, exp of
+// the differences, their sum lane by lane and then across lanes, one division per expert); the top_k choices are
+// made on the scores themselves, largest first, the lower expert on equal scores, so that they do not depend on how
+// an exponential rounds.
+template <bool BF16>
+__global__ __launch_bounds__(kRowWaves * 64) void route_topk_kernel(const void* __restrict__ scores, int tokens,
+                                                                    int num_experts, int top_k,
+                                                                    float* __restrict__ probs,
+                                                                    float* __restrict__ weights,
+                                                                    int64_t* __restrict__ selected) {
+  const int lane = threadIdx.x % 64;
+  const int t = blockIdx.x * kRowWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  if (t >= tokens) return;
+  const void* row = static_cast<const char*>(scores) + (size_t)t * num_experts * (BF16 ? 2 : 4);
+  float m = -INFINITY;
+  for (int e = lane; e < num_experts; e += 64) m = fmaxf(m, score_at<BF16>(row, e));
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  float sum = 0.f;
+  for (int e = lane; e < num_experts; e += 64) sum += expf(score_at<BF16>(row, e) - m);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  float* p = probs + (size_t)t * num_experts;
+  for (int e = lane; e < num_experts; e += 64) p[e] = expf(score_at<BF16>(row, e) - m) / sum;
+  int taken[kTopKMax];  // fixed trip counts below keep it in registers
+#pragma unroll
+  for (int k = 0; k < kTopKMax; ++k) taken[k] = -1;
+#pragma unroll
+  for (int k = 0; k < kTopKMax; ++k) {
+    if (k >= top_k) break;
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < num_experts; e += 64) {
+      bool free_ = true;
+#pragma unroll
+      for (int j = 0; j < kTopKMax; ++j) free_ = free_ && taken[j] != e;
+      const float v = score_at<BF16>(row, e);
+      if (free_ && (at == 0x7fffffff || v > best)) {  // the first free expert of the lane, then only larger scores
+        best = v;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, 64);
+      const int oa = __shfl_xor(at, off, 64);
+      if (oa != 0x7fffffff && (at == 0x7fffffff || ob > best || (ob == best && oa < at))) {
+        best = ob;
+        at = oa;
+      }
+    }
+    taken[k] = at;  // the same in every lane
+    if (lane == 0) {
+      weights[(size_t)t * top_k + k] = expf(best - m) / sum;
+      selected[(size_t)t * top_k + k] = at;
+    }
+  }
+}
+
+// grad_scores[t, j] = p_j * (g_j - sum_i g_i p_i) with g the gradient of the chosen weights scattered to their
+// experts: the chain through the softmax for the top_k outputs of route_topk_kernel.
+template <bool BF16>
+__global__ __launch_bounds__(kRowWaves * 64) void route_topk_backward_kernel(const float* __restrict__ probs,
+                                                                             const int64_t* __restrict__ selected,
+                                                                             const float* __restrict__ grad_weights,
+                                                                             int tokens, int num_experts, int top_k,
+                                                                             void* __restrict__ grad_scores) {
+  const int lane = threadIdx.x % 64;
+  const int t = blockIdx.x * kRowWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  if (t >= tokens) return;
+  const float* p = probs + (size_t)t * num_experts;
+  int at[kTopKMax];
+  float g[kTopKMax];
+  float dot = 0.f;
+#pragma unroll
+  for (int k = 0; k < kTopKMax; ++k) {
+    const bool used = k < top_k;
+    at[k] = used ? (int)selected[(size_t)t * top_k + k] : -1;
+    g[k] = used ? grad_weights[(size_t)t * top_k + k] : 0.f;
+    if ((uint32_t)at[k] >= (uint32_t)num_experts) at[k] = -1, g[k] = 0.f;  // not an expert: no gradient
+    if (at[k] >= 0) dot = __builtin_fmaf(g[k], p[at[k]], dot);
+  }
+  for (int e = lane; e < num_experts; e += 64) {
+    float ge = 0.f;
+#pragma unroll
+    for (int k = 0; k < kTopKMax; ++k) ge += at[k] == e ? g[k] : 0.f;
+    const float v = p[e] * (ge - dot);
+    if constexpr (BF16) static_cast<uint16_t*>(grad_scores)[(size_t)t * num_experts + e] = (uint16_t)f32_to_bf16_bits(v);
+    else static_cast<float*>(grad_scores)[(size_t)t * num_experts + e] = v;
+  }
+}
+
 bool rows_vectorisable(const void* a, const void* b, int hidden) {
   return hidden % 8 == 0 && ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
 }
@@ -364,6 +464,43 @@ int fp8gmm_route_invert(const int32_t* indices, int n, int32_t* inverse, void* s
   if (indices == nullptr || inverse == nullptr) return FP8GMM_ERR_NULL_POINTER;
   hipLaunchKernelGGL(fp8gmm::route_invert_kernel, dim3((n + 255) / 256), dim3(256), 0,
                      static_cast<hipStream_t>(stream), indices, n, inverse);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_route_topk(const void* scores, int scores_bf16, int tokens, int num_experts, int top_k, float* probs,
+                      float* weights, int64_t* selected, void* stream) {
+  using namespace fp8gmm;
+  if (tokens < 0 || num_experts < 1 || top_k < 1 || top_k > kTopKMax || top_k > num_experts)
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if (tokens == 0) return FP8GMM_OK;
+  if (scores == nullptr || probs == nullptr || weights == nullptr || selected == nullptr) return FP8GMM_ERR_NULL_POINTER;
+  const dim3 grid((tokens + kRowWaves - 1) / kRowWaves), block(kRowWaves * 64);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (scores_bf16)
+    hipLaunchKernelGGL(route_topk_kernel<true>, grid, block, 0, s, scores, tokens, num_experts, top_k, probs, weights,
+                       selected);
+  else
+    hipLaunchKernelGGL(route_topk_kernel<false>, grid, block, 0, s, scores, tokens, num_experts, top_k, probs, weights,
+                       selected);
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_route_topk_backward(const float* probs, const int64_t* selected, const float* grad_weights, int tokens,
+                               int num_experts, int top_k, void* grad_scores, int grad_bf16, void* stream) {
+  using namespace fp8gmm;
+  if (tokens < 0 || num_experts < 1 || top_k < 1 || top_k > kTopKMax || top_k > num_experts)
+    return FP8GMM_ERR_BAD_ARGUMENT;
+  if (tokens == 0) return FP8GMM_OK;
+  if (probs == nullptr || selected == nullptr || grad_weights == nullptr || grad_scores == nullptr)
+    return FP8GMM_ERR_NULL_POINTER;
+  const dim3 grid((tokens + kRowWaves - 1) / kRowWaves), block(kRowWaves * 64);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (grad_bf16)
+    hipLaunchKernelGGL(route_topk_backward_kernel<true>, grid, block, 0, s, probs, selected, grad_weights, tokens,
+                       num_experts, top_k, grad_scores);
+  else
+    hipLaunchKernelGGL(route_topk_backward_kernel<false>, grid, block, 0, s, probs, selected, grad_weights, tokens,
+                       num_experts, top_k, grad_scores);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 

@@ -88,10 +88,49 @@ def indices_and_bins(top_expert, sort_end_bit, n_experts):
     return indices, bin_ids, bins, tokens_per_expert
 
 
+MAX_TOP_K = 8
+
+
+class _TopK(torch.autograd.Function):
+    """softmax over the experts + the top_k largest in one launch, and the chain back to the scores in another."""
+
+    @staticmethod
+    def forward(ctx, scores, top_k):
+        tokens, experts = scores.shape
+        probs = torch.empty(tokens, experts, dtype=torch.float32, device=scores.device)
+        weights = torch.empty(tokens, top_k, dtype=torch.float32, device=scores.device)
+        selected = torch.empty(tokens, top_k, dtype=torch.int64, device=scores.device)
+        _lib.check(_lib.load().fp8gmm_route_topk(scores.data_ptr(), int(scores.dtype == torch.bfloat16), tokens,
+                                                experts, top_k, probs.data_ptr(), weights.data_ptr(),
+                                                selected.data_ptr(), _stream(scores.device)))
+        ctx.save_for_backward(probs, selected)
+        ctx.dtype = scores.dtype
+        ctx.mark_non_differentiable(selected)
+        return weights, selected
+
+    @staticmethod
+    def backward(ctx, grad_weights, _):
+        probs, selected = ctx.saved_tensors
+        tokens, experts = probs.shape
+        grad_weights = grad_weights.contiguous().float()
+        grad = torch.empty(tokens, experts, dtype=ctx.dtype, device=probs.device)
+        _lib.check(_lib.load().fp8gmm_route_topk_backward(probs.data_ptr(), selected.data_ptr(), grad_weights.data_ptr(),
+                                                         tokens, experts, selected.shape[1], grad.data_ptr(),
+                                                         int(ctx.dtype == torch.bfloat16), _stream(probs.device)))
+        return grad, None
+
+
 def topk(scores, top_k, moe_renorm=False):
-    """Softmax over experts in fp32, then the ``top_k`` largest (fp8_gmm/example.py:15-23)."""
-    weights = torch.nn.functional.softmax(scores, dim=1, dtype=torch.float)
-    multiplier, selected_experts = torch.topk(weights, top_k)
+    """Softmax over experts in fp32, then the ``top_k`` largest (fp8_gmm/example.py:15-23): weights fp32
+    ``[tokens, top_k]`` and expert ids int64.  One kernel for 2-D bf16 / fp32 scores on the GPU with ``top_k`` up to 8
+    (equal scores: the lower expert first); torch's operators otherwise."""
+    if scores.is_cuda and scores.dim() == 2 and scores.dtype in (torch.bfloat16, torch.float32) \
+            and 1 <= top_k <= min(MAX_TOP_K, scores.shape[1]):
+        with torch.cuda.device(scores.device):
+            multiplier, selected_experts = _TopK.apply(scores.contiguous(), top_k)
+    else:
+        weights = torch.nn.functional.softmax(scores, dim=1, dtype=torch.float)
+        multiplier, selected_experts = torch.topk(weights, top_k)
     if moe_renorm:
         multiplier = multiplier / multiplier.sum(dim=-1, keepdim=True)
     return multiplier, selected_experts

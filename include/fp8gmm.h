@@ -538,6 +538,19 @@ int fp8gmm_upload(void* dst_dev, const void* src_host, size_t bytes, void* strea
 size_t fp8gmm_route_workspace_bytes(int n, int num_experts);
 int fp8gmm_route_sort(const int32_t* expert_of, int n, int num_experts, int32_t* bin_ids, int32_t* indices,
                       int32_t* inverse, int32_t* tokens_per_expert, int32_t* bins, void* workspace, void* stream);
+/*
+ * The router's choice, replacing `topk` of fp8_gmm/example.py:15-23 (softmax over the experts in fp32, then
+ * torch.topk; without its moe_renorm option): probs[t, :] = softmax(scores[t, :]) and, for k < top_k (at most 8),
+ * selected[t, k] = the expert with the k-th largest score of token t (the lower expert on equal scores) and
+ * weights[t, k] = its probability.  scores: [tokens, num_experts] bf16 (scores_bf16 != 0) or fp32, contiguous;
+ * probs: fp32 [tokens, num_experts], kept for the backward pass.
+ */
+int fp8gmm_route_topk(const void* scores, int scores_bf16, int tokens, int num_experts, int top_k, float* probs,
+                      float* weights, int64_t* selected, void* stream);
+/* grad_scores[t, j] = probs[t, j] * (g_j - sum_i g_i probs[t, i]), g = grad_weights[t, :] scattered to the selected
+ * experts: the gradient of `weights` above with respect to `scores`, written as bf16 (grad_bf16 != 0) or fp32. */
+int fp8gmm_route_topk_backward(const float* probs, const int64_t* selected, const float* grad_weights, int tokens,
+                               int num_experts, int top_k, void* grad_scores, int grad_bf16, void* stream);
 /* inverse[indices[i]] = i for a permutation `indices` of 0..n-1 (entries outside that range are skipped) */
 int fp8gmm_route_invert(const int32_t* indices, int n, int32_t* inverse, void* stream);
 /*

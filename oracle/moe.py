@@ -5,6 +5,7 @@ fp8_gmm/example.py:4,15-32,52,59,88,94,115,119), a dependency that is neither ve
 pinned to a version there.  What is restated here is the published meaning of the operators, on plain torch /
 numpy CPU arithmetic:
 
+    topk               softmax over the experts in fp32 + the top_k largest (the example's own function, torch ops)
     sort(x)            stable ascending sort: (sorted ids, original positions)
     histogram, inclusive_cumsum
     gather             out[i] = x[indices[i] // top_k]
@@ -39,6 +40,27 @@ def indices_and_bins(top_expert, n_experts):
     bin_ids, indices = sort(top_expert)
     tokens_per_expert = histogram(top_expert, n_experts)
     return indices, bin_ids, inclusive_cumsum(tokens_per_expert), tokens_per_expert
+
+
+def topk(scores, top_k):
+    """(weights fp32 [tokens, top_k], expert ids int64) - fp8_gmm/example.py:15-23 without moe_renorm: softmax over
+    the experts in fp32, then the top_k largest.  The choice is made on the scores (softmax is monotone), the lower
+    expert first on equal scores - torch.topk leaves the order of equal elements open."""
+    z = np.asarray(scores, dtype=np.float32)
+    ex = np.exp(z - z.max(axis=1, keepdims=True), dtype=np.float32)
+    p = ex / ex.sum(axis=1, keepdims=True, dtype=np.float32)
+    order = np.argsort(-z, axis=1, kind="stable")[:, :top_k]
+    return np.take_along_axis(p, order, axis=1), order.astype(np.int64)
+
+
+def topk_backward(scores, selected, grad_weights):
+    """Gradient of topk's weights with respect to the scores, in float64."""
+    z = np.asarray(scores, dtype=np.float64)
+    ex = np.exp(z - z.max(axis=1, keepdims=True))
+    p = ex / ex.sum(axis=1, keepdims=True)
+    g = np.zeros_like(p)
+    np.put_along_axis(g, np.asarray(selected), np.asarray(grad_weights, dtype=np.float64), axis=1)
+    return p * (g - (g * p).sum(axis=1, keepdims=True))
 
 
 def invert(indices):

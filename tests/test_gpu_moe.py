@@ -104,6 +104,41 @@ def test_gather_scatter_and_their_gradients(dev, tokens, top_k, hidden, e):
             assert ((wd.grad.cpu() - want_gw).abs() <= 1e-5 * bound + 1e-30).all()
 
 
+@pytest.mark.parametrize("tokens,e,top_k,dtype", [(1, 1, 1, torch.float32), (1000, 16, 2, torch.bfloat16),
+                                                   (16384, 16, 2, torch.bfloat16), (513, 64, 8, torch.float32),
+                                                   (300, 200, 3, torch.bfloat16), (77, 4096, 4, torch.float32),
+                                                   (0, 8, 2, torch.bfloat16)])
+def test_topk_against_the_oracle(dev, tokens, e, top_k, dtype):
+    """softmax + top-k in one launch: the chosen experts equal the oracle's (bf16 scores are full of equal values,
+    so this also holds the rule for ties), the weights agree to a few ulp of fp32, and the gradient with respect to
+    the scores agrees with the oracle's float64 chain to fp32 / bf16 rounding."""
+    ops = _ops()
+    rng = np.random.default_rng(900 + tokens + e)
+    z = torch.from_numpy(rng.standard_normal((tokens, e)).astype(np.float32) * 2).to(dtype)
+    zd = z.to(dev).requires_grad_()
+    w, sel = ops.topk(zd, top_k)
+    assert w.dtype == torch.float32 and sel.dtype == torch.int64 and w.shape == sel.shape == (tokens, top_k)
+    want_w, want_sel = orc.topk(z.float().numpy(), top_k)
+    assert (sel.cpu().numpy() == want_sel).all()
+    np.testing.assert_allclose(w.detach().cpu().numpy(), want_w, rtol=4e-6, atol=1e-30)
+    gw = torch.from_numpy(rng.standard_normal((tokens, top_k)).astype(np.float32))
+    w.backward(gw.to(dev))
+    want_g = orc.topk_backward(z.float().numpy(), want_sel, gw.numpy())
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-5
+    assert zd.grad.dtype == dtype
+    np.testing.assert_allclose(zd.grad.float().cpu().numpy(), want_g, rtol=tol, atol=tol * 1e-2)
+
+
+def test_topk_falls_back_to_torch_and_renormalises(dev):
+    ops = _ops()
+    z = torch.randn(50, 8, device=dev, dtype=torch.float64)    # not a dtype of the kernel: torch's operators
+    w, sel = ops.topk(z, 2)
+    tw, tsel = torch.topk(torch.softmax(z, dim=1, dtype=torch.float), 2)
+    assert torch.equal(sel, tsel) and torch.equal(w, tw)
+    w, _ = ops.topk(z.float(), 2, moe_renorm=True)
+    assert torch.allclose(w.sum(dim=1), torch.ones(50, device=dev))
+
+
 def test_bad_arguments_are_rejected(dev):
     ops = _ops()
     x = torch.zeros(4, 8, dtype=torch.bfloat16, device=dev)

@@ -71,3 +71,25 @@ def test_backward_rules_against_autograd():
     x = torch.tensor(rng.integers(-4, 5, size=(tokens, hidden)) / 4.0, dtype=torch.float64, requires_grad=True)
     x[idx // top_k].backward(y.detach())
     assert torch.equal(moe.gather_backward(y.detach().to(torch.bfloat16), indices, top_k).double(), x.grad)
+
+
+def test_topk_is_softmax_then_the_largest():
+    """The oracle's topk against the reference's own formulation in torch operators (fp8_gmm/example.py:15-23) on
+    scores without ties, its tie rule on a hand-made row, and its gradient against autograd."""
+    rng = np.random.default_rng(5)
+    z = rng.standard_normal((300, 16)).astype(np.float32)
+    w, sel = moe.topk(z, 2)
+    tw, tsel = torch.topk(torch.softmax(torch.from_numpy(z), dim=1, dtype=torch.float), 2)
+    assert (sel == tsel.numpy()).all()
+    np.testing.assert_allclose(w, tw.numpy(), rtol=2e-6, atol=0)
+    tie = np.array([[1.0, 3.0, 3.0, 0.5, 3.0]], dtype=np.float32)
+    w, sel = moe.topk(tie, 3)
+    assert sel.tolist() == [[1, 2, 4]] and w[0, 0] == w[0, 1] == w[0, 2]
+    zt = torch.from_numpy(z).double().requires_grad_()
+    gw = rng.standard_normal((300, 2))
+    (torch.softmax(zt, dim=1).gather(1, torch.from_numpy(sel_of(z))) * torch.from_numpy(gw)).sum().backward()
+    np.testing.assert_allclose(moe.topk_backward(z, sel_of(z), gw), zt.grad.numpy(), rtol=1e-9, atol=1e-12)
+
+
+def sel_of(z):
+    return moe.topk(z, 2)[1]
