@@ -1,4 +1,6 @@
 """Shared helpers of the test-suite: seeded inputs, shape lists, comparisons."""
+import os
+
 import torch
 
 from oracle import ref
@@ -34,7 +36,9 @@ def transpose_shapes(shapes, padded, pad=16):
 
 
 def gen(seed):
-    return torch.Generator().manual_seed(seed)
+    """The tests' random inputs: a generator seeded per call site.  FP8GMM_TEST_SEED_OFFSET (an integer, 0 by default)
+    shifts every seed, to run the whole suite over other draws."""
+    return torch.Generator().manual_seed(seed + int(os.environ.get("FP8GMM_TEST_SEED_OFFSET", "0")))
 
 
 def randn_bf16(shape, g, std=1.0):

@@ -183,7 +183,9 @@ def test_fp8_gmm(dev, a_dtype, c_dtype, backward, cutlass, group_sizes, k, n):
         assert (dist != 0).float().mean() <= 2e-3
     for i in range(e):
         if group_sizes[i]:
-            assert torch.allclose(d_amax[i].cpu(), o_amax[i], rtol=1e-5, atol=0), f"amax expert {i}"
+            # the largest |gelu(acc)|: the accumulation order and the hardware's exp2 / rcp move its last digits
+            # (1e-5 was seen over other seeds); an fp8 code step is 6 %
+            assert torch.allclose(d_amax[i].cpu(), o_amax[i], rtol=1e-4, atol=0), f"amax expert {i}"
         else:
             assert_scalar_bits_equal(d_amax[i], o_amax[i], "amax of an empty expert stays untouched")
 
@@ -214,7 +216,7 @@ def test_cublas_fp8_gemm(dev, a_shape, a_dtype, b_shape, c_dtype):
     ref.cublas_fp8_gemm(a, b, o_c, a_inv, b_inv, o_pre, c_scale, o_amax)
     assert_gemm_close(d_pre, ref_f32, 1e-2, "pre_gelu_out")
     assert _fp8_code_distance(dc.cpu(), o_c).max() <= 1
-    assert torch.allclose(d_amax.cpu(), o_amax, rtol=1e-5, atol=0)
+    assert torch.allclose(d_amax.cpu(), o_amax, rtol=1e-4, atol=0)   # see test_fp8_gmm
     # the erf-GELU the reference's own test compares with (test.py:162) is within its atol=rtol=2 of this
     erf = torch.nn.functional.gelu(ref_f32) * c_scale
     assert torch.allclose(dc.cpu().float(), erf, atol=2, rtol=2)
