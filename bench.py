@@ -19,7 +19,7 @@ delayed-scaling update.  Prints ONE JSON line.
   also      the step time of a later micro-batch that reuses the first one's fp8 weights (not the headline:
             the reference casts the weights on every pass), the step on the reference's buffers, one dense GEMM
             of the step's size next to the vendor library's, and - under `configs` - short passes of the other
-            workloads (config 1, 3, 4 and 5) with their own roofline fractions and parity gates
+            workloads (config 1, 3, 4 and 5 and the reference's example layer) with their own roofline fractions and parity gates
   hip_graph_replay  the step captured into a HIP graph once and replayed: its time with the host out of the way
   cpu_baseline  the per-expert quantize-dequantize-fp32-matmul loop (oracle/cpu_baseline.py) over
             the workload's own split, timed on this machine's host cores
@@ -104,6 +104,34 @@ def seeded_normal(shape, seed, std, dev, dtype=torch.bfloat16):
 def _fp8_cast(t, scale, dtype):
     fmax = 448.0 if dtype == torch.float8_e4m3fn else 57344.0
     return (t.float() * scale).clamp(-fmax, fmax).to(dtype)
+
+
+def routed_parity_check(module, x, run_step):
+    """One more step of the routed layer, then 64 sampled tokens of its output against an fp32 model of the same layer
+    built from the module's bf16 parameters (same routing decisions; tanh-GELU): the relative rms error over the
+    sampled block, which for two FP8 GEMMs in a row is a few per cent, and its cosine similarity."""
+    from fp8_gmm_amd import moe_ops
+
+    out, _ = run_step()
+    torch.cuda.synchronize()
+    tokens = torch.arange(0, x.shape[0], max(1, x.shape[0] // 64), device=x.device)[:64]
+    with torch.no_grad():
+        xs = x[tokens]
+        weights, selected = moe_ops.topk(module.gating_network(xs), module.top_k)
+        w1, w2 = module.grouped_mlp.fc1_weight, module.grouped_mlp.fc2_weight
+        ref = torch.zeros(len(tokens), x.shape[1], device=x.device)
+        for t in range(len(tokens)):
+            for k in range(module.top_k):
+                e = int(selected[t, k])
+                hidden = torch.nn.functional.gelu(w1[e].float() @ xs[t].float(), approximate="tanh")
+                ref[t] += weights[t, k] * (w2[e].float() @ hidden)
+        got = out[tokens].float()
+        rel_rms = ((got - ref).pow(2).mean().sqrt() / ref.pow(2).mean().sqrt()).item()
+        cos = (torch.dot(got.flatten(), ref.flatten()) / (got.norm() * ref.norm())).item()
+    return {"rel_rms_err": round(rel_rms, 5), "cosine": round(cos, 6), "tolerance": {"rel_rms_err": 0.08, "cosine": 0.995},
+            "ok": bool(rel_rms <= 0.08 and cos >= 0.995),
+            "checked": "64 sampled tokens of the layer's output against an fp32 model of the routed layer on the bf16 "
+                       "parameters (quantisation error included)"}
 
 
 def parity_check(module, kind, x, dy, sizes, run_step):
@@ -543,6 +571,8 @@ def measure_module(args):
     parity = None
     if gs is not None and not args.no_parity:
         parity = parity_check(module, kind, x, dy, sizes, step)
+    elif kind == "routed_mlp" and not args.no_parity:
+        parity = routed_parity_check(module, x, step)
 
     cpu = None
     if not args.no_cpu_baseline:
@@ -665,7 +695,7 @@ def main():
     if args.workload == "config2" and not args.headline_only:
         # every other workload in the same record: short passes, each with its own correctness gate
         gc_configs = {}
-        for w in ("config1", "config3", "config4", "config5"):
+        for w in ("config1", "config3", "config4", "config5", "example"):
             gc_configs[w] = short_pass(args, w)
         line["also"] = dict(line.get("also") or {})
         line["also"]["configs"] = gc_configs
