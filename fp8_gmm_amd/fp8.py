@@ -35,6 +35,7 @@ import threading
 from dataclasses import dataclass
 from enum import Enum
 
+import numpy as np
 import torch
 
 from .utils import DType
@@ -261,8 +262,6 @@ class Fp8GroupedModuleBase(torch.nn.Module):
             return False
         self._ahead = None
         with self.prepare_forward(first, None, self.num_groups * len(weights_and_groups)):
-            import numpy as np
-
             meta = Fp8MetaWrapper(self.num_groups, self.fp8_meta)
             fp8_dtype = to_torch_dtype(get_fp8_te_dtype(self.fp8_meta["recipe"], fprop_tensor=True))
             caches = tuple(Fp8WeightCache() for _ in weights_and_groups)
