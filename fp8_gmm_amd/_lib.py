@@ -212,6 +212,7 @@ EXPORTS = (
     "fp8gmm_route_workspace_bytes",
     "fp8gmm_route_sort",
     "fp8gmm_route_invert",
+    "fp8gmm_moe_scatter_backward",
     "fp8gmm_route_topk",
     "fp8gmm_route_topk_backward",
     "fp8gmm_moe_gather",
@@ -322,6 +323,8 @@ def load():
     L.fp8gmm_route_sort.argtypes = [vp, ci, ci, vp, vp, vp, vp, vp, vp, vp]
     L.fp8gmm_route_invert.restype = ci
     L.fp8gmm_route_invert.argtypes = [vp, ci, vp, vp]
+    L.fp8gmm_moe_scatter_backward.restype = ci
+    L.fp8gmm_moe_scatter_backward.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, vp]
     L.fp8gmm_route_topk.restype = ci
     L.fp8gmm_route_topk.argtypes = [vp, ci, ci, ci, ci, vp, vp, vp, vp]
     L.fp8gmm_route_topk_backward.restype = ci

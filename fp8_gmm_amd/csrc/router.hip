@@ -322,6 +322,57 @@ __global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_wgrad_kernel(const
   if (lane == 0) grad_w[idx] = acc;
 }
 
+// Both gradients of scatter in one pass over the rows: for sorted row i with idx = indices[i], token idx / top_k and
+// w = weights[idx],  grad_x[i, :] = bf16(w * grad_out[token, :])  (what moe_gather_kernel writes with weights) and
+// grad_w[idx] = < x[i, :], grad_out[token, :] >  (what moe_scatter_wgrad_kernel writes): the gradient row is read
+// once for both.
+__global__ __launch_bounds__(kRowWaves * 64) void moe_scatter_backward_kernel(const uint16_t* __restrict__ x,
+                                                                              const uint16_t* __restrict__ grad_out,
+                                                                              const int32_t* __restrict__ indices,
+                                                                              const float* __restrict__ weights,
+                                                                              uint16_t* __restrict__ grad_x,
+                                                                              float* __restrict__ grad_w, int rows,
+                                                                              int hidden, int top_k) {
+  const int lane = threadIdx.x % 64;
+  const int row = blockIdx.x * kRowWaves + __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+  if (row >= rows) return;
+  const int32_t idx = indices[row];
+  const bool ok = (uint32_t)idx < (uint32_t)rows;
+  const float w = ok ? weights[idx] : 1.0f;
+  const __amdgpu_buffer_rsrc_t ra = make_rsrc(x + (size_t)row * hidden, (uint32_t)hidden * 2u);
+  const __amdgpu_buffer_rsrc_t rb = make_rsrc(grad_out + (size_t)(ok ? idx / top_k : 0) * hidden,
+                                              ok ? (uint32_t)hidden * 2u : 0u);   // not a row: zeros
+  const __amdgpu_buffer_rsrc_t rd = make_rsrc(grad_x + (size_t)row * hidden, (uint32_t)hidden * 2u);
+  float acc = 0.f;
+  for (int c0 = 0; c0 < hidden; c0 += 64 * 8 * 4) {
+    u32x4 va[4], vb[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      va[u] = buf_load16_stream(ra, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+      vb[u] = buf_load16_stream(rb, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t pa[4] = {va[u].x, va[u].y, va[u].z, va[u].w};
+      const uint32_t pb[4] = {vb[u].x, vb[u].y, vb[u].z, vb[u].w};
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        acc = __builtin_fmaf(bf16_lo_to_f32(pa[q]), bf16_lo_to_f32(pb[q]), acc);
+        acc = __builtin_fmaf(bf16_hi_to_f32(pa[q]), bf16_hi_to_f32(pb[q]), acc);
+      }
+      u32x4 o;
+      o.x = scale_bf16x2(pb[0], w);
+      o.y = scale_bf16x2(pb[1], w);
+      o.z = scale_bf16x2(pb[2], w);
+      o.w = scale_bf16x2(pb[3], w);
+      buf_store16(o, rd, (uint32_t)(c0 + (u * 64 + lane) * 8) * 2u);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+  if (lane == 0 && ok) grad_w[idx] = acc;
+}
+
 constexpr int kTopKMax = 8;  // choices per token that the selection keeps in registers
 
 template <bool BF16>
@@ -540,6 +591,28 @@ int fp8gmm_moe_scatter_wgrad(const void* x, const void* grad_out, const int32_t*
                      static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x),
                      static_cast<const uint16_t*>(grad_out), indices, grad_w, rows, hidden, top_k,
                      (int)rows_vectorisable(x, grad_out, hidden));
+  return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
+}
+
+int fp8gmm_moe_scatter_backward(const void* x, const void* grad_out, const int32_t* indices, const float* weights,
+                                void* grad_x, float* grad_w, int rows, int hidden, int top_k, void* stream) {
+  using namespace fp8gmm;
+  if (rows < 0 || hidden < 0 || top_k < 1 || rows % top_k != 0) return FP8GMM_ERR_BAD_ARGUMENT;
+  if ((int64_t)hidden * 2 > 0x7fffffff) return FP8GMM_ERR_BAD_SHAPE;
+  if (rows == 0) return FP8GMM_OK;
+  if (x == nullptr || grad_out == nullptr || indices == nullptr || weights == nullptr || grad_x == nullptr ||
+      grad_w == nullptr)
+    return FP8GMM_ERR_NULL_POINTER;
+  if (!rows_vectorisable(x, grad_out, hidden) || !rows_vectorisable(grad_x, grad_x, hidden)) {
+    // rows that 16-byte accesses cannot take: the two single-purpose kernels
+    int rc = fp8gmm_moe_gather(grad_out, indices, weights, grad_x, rows, hidden, top_k, stream);
+    if (rc != FP8GMM_OK) return rc;
+    return fp8gmm_moe_scatter_wgrad(x, grad_out, indices, grad_w, rows, hidden, top_k, stream);
+  }
+  hipLaunchKernelGGL(moe_scatter_backward_kernel, dim3((rows + kRowWaves - 1) / kRowWaves), dim3(kRowWaves * 64), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x),
+                     static_cast<const uint16_t*>(grad_out), indices, weights, static_cast<uint16_t*>(grad_x), grad_w,
+                     rows, hidden, top_k);
   return hipGetLastError() == hipSuccess ? FP8GMM_OK : FP8GMM_ERR_LAUNCH;
 }
 

@@ -206,6 +206,17 @@ class _Scatter(torch.autograd.Function):
     def backward(ctx, grad):
         x, indices, weights = ctx.saved_tensors
         grad = grad.contiguous()
+        if weights is not None and ctx.needs_input_grad[0] and ctx.needs_input_grad[2]:
+            # both gradients: one pass that reads every gradient row once
+            rows, hidden = x.shape
+            grad_x = torch.empty(rows, hidden, dtype=grad.dtype, device=grad.device)
+            grad_w = torch.zeros_like(weights)
+            with torch.cuda.device(grad.device), _timed("moe_scatter_backward", lambda: 6 * rows * hidden):
+                rc = _lib.load().fp8gmm_moe_scatter_backward(x.data_ptr(), grad.data_ptr(), indices.data_ptr(),
+                                                             weights.data_ptr(), grad_x.data_ptr(), grad_w.data_ptr(),
+                                                             rows, hidden, ctx.top_k, _stream(grad.device))
+            _lib.check(rc)
+            return grad_x, None, grad_w, None
         grad_x = _gather_rows(grad, indices, weights, ctx.top_k) if ctx.needs_input_grad[0] else None
         grad_w = None
         if weights is not None and ctx.needs_input_grad[2]:

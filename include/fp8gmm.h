@@ -572,6 +572,12 @@ int fp8gmm_moe_scatter(const void* x, const int32_t* inverse, const float* weigh
  * to its weights.  x: bf16 [rows, hidden] (sorted order), grad_out: bf16 [rows / top_k, hidden], grad_w: fp32 [rows]. */
 int fp8gmm_moe_scatter_wgrad(const void* x, const void* grad_out, const int32_t* indices, float* grad_w, int rows,
                              int hidden, int top_k, void* stream);
+/* The whole backward pass of ops.scatter (fp8_gmm/example.py:59,94,119) in one launch: grad_x[i, :] =
+ * bf16(weights[indices[i]] * grad_out[indices[i] / top_k, :]) as fp8gmm_moe_gather writes it with weights, and
+ * grad_w as fp8gmm_moe_scatter_wgrad writes it, the gradient rows read once for both.  The same bits as the two
+ * calls.  grad_x: bf16 [rows, hidden]. */
+int fp8gmm_moe_scatter_backward(const void* x, const void* grad_out, const int32_t* indices, const float* weights,
+                                void* grad_x, float* grad_w, int rows, int hidden, int top_k, void* stream);
 
 /* ---- schedule introspection (host only, no GPU needed) ------------------------------------ */
 /*

@@ -139,6 +139,32 @@ def test_topk_falls_back_to_torch_and_renormalises(dev):
     assert torch.allclose(w.sum(dim=1), torch.ones(50, device=dev))
 
 
+@pytest.mark.parametrize("tokens,top_k,hidden,e", [(1000, 2, 256, 4), (513, 1, 4096, 7), (300, 4, 2056, 16),
+                                                    (64, 2, 100, 3)])
+def test_scatter_backward_in_one_pass_equals_the_two_passes(dev, tokens, top_k, hidden, e):
+    """With both gradients wanted scatter's backward pass is one launch; it must write the bits of the two
+    single-purpose launches (weighted gather, per-row dot products), which run when only one gradient is wanted -
+    also on rows that 16-byte accesses cannot take (hidden = 100)."""
+    ops = _ops()
+    rng = np.random.default_rng(40 + tokens)
+    ids = torch.tensor(rng.integers(0, e, size=tokens * top_k), dtype=torch.int32, device=dev)
+    indices, bin_ids, bins, _ = ops.indices_and_bins(ids, 0, e)
+    x = torch.from_numpy(rng.standard_normal((tokens * top_k, hidden)).astype(np.float32)).to(torch.bfloat16).to(dev)
+    w = torch.from_numpy(rng.random(tokens * top_k).astype(np.float32)).to(dev)
+    g = torch.from_numpy(rng.standard_normal((tokens, hidden)).astype(np.float32)).to(torch.bfloat16).to(dev)
+
+    def grads(need_x, need_w):
+        xd, wd = x.clone().requires_grad_(need_x), w.clone().requires_grad_(need_w)
+        ops.scatter(xd, indices, bin_ids, wd, bins, top_k).backward(g)
+        return xd.grad, wd.grad
+
+    both_x, both_w = grads(True, True)
+    only_x, _ = grads(True, False)
+    _, only_w = grads(False, True)
+    assert torch.equal(both_x.view(torch.int16), only_x.view(torch.int16))
+    assert torch.equal(both_w.view(torch.int32), only_w.view(torch.int32))
+
+
 def test_bad_arguments_are_rejected(dev):
     ops = _ops()
     x = torch.zeros(4, 8, dtype=torch.bfloat16, device=dev)
